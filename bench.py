@@ -1,0 +1,299 @@
+#!/usr/bin/env python3
+"""Benchmark of the int4 decode linears on one MI355X.
+
+A "step" is one pass over the Janus-Pro-1B decoder linear set at M=1: per layer
+q/k/v/o 2048->2048, gate and up 2048->5632, down 5632->2048, times 24 layers
+with distinct seeded weights (168 GEMVs, 642,539,520 algorithmic bytes), all
+int4 with group size 128.  Operands are resident in HBM before the timed region.
+
+Prints one JSON line.  ``value`` is the aggregate algorithmic GB/s of the step;
+``roofline`` prices the dominant kernel against the 8 TB/s HBM peak; ``cpu_baseline``
+times the PyTorch dequant + matmul path on the host cores over a bounded sample;
+``detail`` carries the other launch strategies, per-call latencies and the M=32
+rollout-batch figure.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0
+HIDDEN, INTER, LAYERS, GROUP, HEAD = 2048, 5632, 24, 128, 16384
+ROOT = os.path.dirname(os.path.abspath(__file__))
+
+# (name, K, N) in the order the decoder layer applies them
+LAYER_LINEARS = [("q", HIDDEN, HIDDEN), ("k", HIDDEN, HIDDEN), ("v", HIDDEN, HIDDEN),
+                 ("o", HIDDEN, HIDDEN), ("gate", HIDDEN, INTER), ("up", HIDDEN, INTER),
+                 ("down", INTER, HIDDEN)]
+
+
+def make_weights(seed: int, K: int, N: int, G: int, device):
+    """Seeded synthetic packed weights, generated on the device.
+
+    Uniform 32-bit words are eight independent uniform nibbles; scales are
+    |N(0, 0.02)| as bf16 (zeros replaced), zero-point words uniform with the
+    unused high nibbles of the last word cleared.
+    """
+    gen = torch.Generator(device=device).manual_seed(seed)
+    groups = K // G
+    zwords = (groups + 7) // 8
+    qweight = torch.randint(-2 ** 31, 2 ** 31, (N, K // 8), generator=gen, device=device,
+                            dtype=torch.int64).to(torch.int32)
+    scales = (torch.randn((N, groups), generator=gen, device=device) * 0.02).abs()
+    scales = torch.where(scales < 1e-6, torch.full_like(scales, 1e-3), scales).to(torch.bfloat16)
+    qzeros = torch.randint(-2 ** 31, 2 ** 31, (N, zwords), generator=gen, device=device,
+                           dtype=torch.int64).to(torch.int32)
+    used = groups - 8 * (zwords - 1)
+    if used < 8:
+        keep = (1 << (4 * used)) - 1
+        qzeros[:, -1] &= keep
+    return qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+
+
+def make_x(seed: int, M: int, K: int, device):
+    gen = torch.Generator(device=device).manual_seed(seed)
+    return torch.randn((M, K), generator=gen, device=device).to(torch.bfloat16).contiguous()
+
+
+def time_region(fn, steps: int, warmup: int):
+    """ms per call of ``fn`` over ``steps`` calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def build_set(cfg: int, M: int, device, with_head: bool):
+    """All linears of one decode step: list of dicts with operands and byte counts."""
+    from visionrl_amd.int4_format import algorithmic_bytes
+
+    items = []
+    xs = {K: make_x(1000 * cfg + 7, M, K, device) for K in (HIDDEN, INTER)}
+    for layer in range(LAYERS):
+        for proj, (name, K, N) in enumerate(LAYER_LINEARS):
+            qw, sc, qz = make_weights(1000 * cfg + 10 * layer + proj, K, N, GROUP, device)
+            items.append({"name": f"l{layer}.{name}", "layer": layer, "proj": name, "K": K, "N": N,
+                          "x": xs[K], "qweight": qw, "scales": sc, "qzeros": qz,
+                          "bytes": algorithmic_bytes(M, K, N, GROUP)})
+    if with_head:
+        qw, sc, qz = make_weights(1000 * cfg + 999, HIDDEN, HEAD, GROUP, device)
+        items.append({"name": "gen_head", "layer": LAYERS, "proj": "head", "K": HIDDEN, "N": HEAD,
+                      "x": xs[HIDDEN], "qweight": qw, "scales": sc, "qzeros": qz,
+                      "bytes": algorithmic_bytes(M, HIDDEN, HEAD, GROUP)})
+    return items
+
+
+def measure_set(items, steps: int, warmup: int):
+    """Time one decode step's linear set under each launch strategy."""
+    from visionrl_amd import ops
+
+    total_bytes = sum(it["bytes"] for it in items)
+    out = {"launches_per_step": {}, "ms_per_step": {}, "GBps": {}}
+
+    def record(name, ms, launches):
+        out["ms_per_step"][name] = ms
+        out["GBps"][name] = total_bytes / (ms * 1e-3) / 1e9
+        out["launches_per_step"][name] = launches
+
+    # one launch for the whole set
+    grouped = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
+                               for it in items])
+    record("grouped_1_launch", time_region(grouped.launch, steps, warmup), 1)
+
+    # one launch per linear, stream ordered
+    def eager():
+        for it in items:
+            ops.int4_gemv(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP)
+
+    record("per_linear_eager", time_region(eager, max(3, steps // 4), max(1, warmup // 4)), len(items))
+
+    # the same launches replayed from a HIP graph
+    try:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            eager()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            eager()
+        record("per_linear_hip_graph", time_region(graph.replay, steps, warmup), len(items))
+    except Exception as exc:  # graph capture is an extra, never the headline
+        out["hip_graph_error"] = repr(exc)[:200]
+
+    # launches a real decoder layer could issue: q|k|v together, o, gate|up together, down
+    by_layer = {}
+    for it in items:
+        by_layer.setdefault(it["layer"], []).append(it)
+    plans = []
+    for layer in sorted(by_layer):
+        its = {it["proj"]: it for it in by_layer[layer]}
+        for names in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",), ("head",)):
+            sel = [its[n] for n in names if n in its]
+            if sel:
+                plans.append(ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"],
+                                               GROUP, False) for it in sel]))
+
+    def layered():
+        for plan in plans:
+            plan.launch()
+
+    record("per_layer_4_launches", time_region(layered, steps, warmup), len(plans))
+    return out, total_bytes, grouped
+
+
+def per_call_latency(items, steps: int):
+    """us per single-GEMV launch for each distinct shape, rotating over the distinct weights."""
+    from visionrl_amd import ops
+
+    res = {}
+    shapes = {}
+    for it in items:
+        shapes.setdefault((it["K"], it["N"]), []).append(it)
+    for (K, N), group in shapes.items():
+        def rotate():
+            for it in group:
+                ops.int4_gemv(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP)
+        ms = time_region(rotate, max(2, steps // 4), 1) / len(group)
+        res[f"{K}x{N}"] = {"us_per_call": ms * 1e3, "GBps": group[0]["bytes"] / (ms * 1e-3) / 1e9,
+                           "distinct_weights": len(group)}
+    return res
+
+
+def cpu_baseline(seconds: float = 12.0):
+    """PyTorch dequant + matmul on the host cores over one decoder layer's seven linears."""
+    from oracle import int4_oracle as oracle  # the checker, used here as the reported CPU baseline
+
+    cpu = torch.device("cpu")
+    ops_cpu = []
+    nbytes = 0
+    for proj, (name, K, N) in enumerate(LAYER_LINEARS):
+        qw, sc, qz = make_weights(2000 + proj, K, N, GROUP, cpu)
+        ops_cpu.append((make_x(2007, 1, K, cpu), qw, sc, qz))
+        nbytes += oracle.algorithmic_bytes(1, K, N, GROUP)
+
+    def layer():
+        for x, qw, sc, qz in ops_cpu:
+            oracle.torch_cpu_linear(x, qw, sc, qz, GROUP)
+
+    layer()
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        layer()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= seconds or reps >= 200:
+            break
+    return {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{reps} passes over one decoder layer's 7 linears (M=1, {nbytes} B each pass), "
+                      f"torch CPU dequant + F.linear, {el:.1f} s",
+            "host_cpu_count": os.cpu_count()}
+
+
+def load_traffic(kernel: str):
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    try:
+        with open(path) as fh:
+            return json.load(fh).get(kernel)
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-headline", action="store_true",
+                    help="run just the grouped decode-step launches (for profilers)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X: no ROCm device is visible")
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    from visionrl_amd import ops
+
+    items = build_set(2, 1, device, with_head=False)
+    torch.cuda.synchronize()
+
+    if args.only_headline:
+        grouped = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
+                                   for it in items])
+        ms = time_region(grouped.launch, args.steps, args.warmup)
+        print(json.dumps({"ms_per_step": ms}))
+        return
+
+    strat, total_bytes, grouped = measure_set(items, args.steps, args.warmup)
+    latency = per_call_latency(items, args.steps)
+
+    best = max(strat["GBps"], key=lambda k: strat["GBps"][k])
+    headline = "grouped_1_launch"
+    ms = strat["ms_per_step"][headline]
+    value = strat["GBps"][headline]
+
+    # the dominant kernel's own duration: the grouped kernel is the whole step, one launch each
+    kernel_ms = time_region(grouped.launch, args.steps, 2)
+    achieved = total_bytes / (kernel_ms * 1e-3) / 1e9
+
+    del items, grouped
+    torch.cuda.empty_cache()
+
+    # rollout batch M=32 plus the image-token head
+    items32 = build_set(3, 32, device, with_head=True)
+    strat32, bytes32, _ = measure_set(items32, max(10, args.steps // 4), max(2, args.warmup // 4))
+    del items32
+    torch.cuda.empty_cache()
+
+    result = {
+        "metric": "int4 GEMV GB/s (% of HBM peak) + us/call, Janus-1B shapes at M=1 and M=32",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "Janus-Pro-1B decoder linear set, M=1: 24 layers x (4x 2048->2048, "
+                               "2x 2048->5632, 1x 5632->2048), int4 group 128, 168 GEMVs, distinct weights",
+                   "algorithmic_bytes_per_step": total_bytes,
+                   "launch": "one grouped launch per step (all 168 GEMVs in one kernel)"},
+        "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": load_traffic("gemv_grouped_kernel"),
+                     "kernel": "gemv_grouped_kernel", "bytes_per_launch": total_bytes,
+                     "avg_launch_ms": kernel_ms},
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(),
+        "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,
+                   "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32},
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

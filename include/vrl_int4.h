@@ -1,0 +1,121 @@
+/*
+ * C ABI of the MI355X (gfx950) int4 weight-only decode linears.
+ *
+ * These entry points replace, for autoregressive rollout decode, the bf16
+ * nn.Linear calls the reference reaches through
+ *   vrl/models/families/janus_pro/policy.py:673-678  (Llama trunk: q/k/v/o_proj,
+ *                                                      gate/up/down_proj)
+ *   vrl/models/families/janus_pro/policy.py:138-160  (gen_head, image-token logits)
+ * The reference has no FFI of its own for this path (it is pure Python on
+ * torch); a binding is a ctypes stub over this header.
+ *
+ * Operand formats (row-major, caller-owned device memory, 16-byte aligned):
+ *   x        bf16  [M, K]            activations
+ *   qweight  int32 [N, K/8]          nibble i (bits 4i..4i+3) of word r = q[n, 8r+i], q in [0,15]
+ *   scales   bf16  [N, K/G]          one scale per group of G consecutive k
+ *   qzeros   int32 [N, ceil(K/G/8)]  zero-points, same nibble order along the group axis,
+ *                                    unused high nibbles of the last word are 0
+ *   y        bf16  [M, N]
+ * Arithmetic:
+ *   w[n,k] = bf16_rne( (float)(q[n,k] - z[n,k/G]) * (float)s[n,k/G] )   (bit-exact)
+ *   y[m,n] = bf16_rne( sum_k (float)x[m,k] * w[n,k] )                   (fp32 accumulate,
+ *                                                                        order unspecified)
+ * Scales must be finite bf16 numbers; zero, negative and subnormal scales are allowed.
+ *
+ * Every call only enqueues work on `hip_stream` (a hipStream_t, NULL = the
+ * default stream) of the current device; it does not allocate, synchronise or
+ * keep state, and is re-entrant.  Return value: 0 on success, a hipError_t
+ * value (1..999) if the launch failed, or one of the VRL_INT4_E* codes below if
+ * the arguments violate a precondition (nothing is enqueued then).
+ * Preconditions: M >= 1, N >= 1, K >= 8, K % 8 == 0, G % 8 == 0, K % G == 0,
+ * non-NULL 16-byte aligned pointers, N * K < 2^40.
+ */
+#ifndef VRL_INT4_H
+#define VRL_INT4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VRL_INT4_ABI_VERSION 1
+
+#define VRL_INT4_OK 0
+#define VRL_INT4_ESHAPE 1001  /* M, N, K or G violates a precondition */
+#define VRL_INT4_EALIGN 1002  /* a pointer is not 16-byte aligned */
+#define VRL_INT4_ENULL 1003   /* a required pointer is NULL */
+#define VRL_INT4_EPLAN 1004   /* malformed or undersized grouped plan */
+
+int vrl_int4_abi_version(void);
+
+/* Static text for a return code of this library ("hip error" for 1..999). */
+const char *vrl_int4_error_string(int code);
+
+/*
+ * y[M,N] = x[M,K] . dequant(qweight, scales, qzeros)^T.
+ * Replaces one nn.Linear.forward of the decode step
+ * (policy.py:673-678 trunk projections; policy.py:160 gen_head).
+ */
+int vrl_int4_gemv_bf16(const void *x, const void *qweight, const void *scales,
+                       const void *qzeros, void *y, int M, int N, int K, int G,
+                       void *hip_stream);
+
+/*
+ * w[N,K] (bf16) = dequant(qweight, scales, qzeros): the canonical weight tile,
+ * bit-exact.  Used by the loader glue and by the train-time replay path that
+ * keeps bf16 weights (policy.py:419-424).
+ */
+int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *qzeros,
+                          void *w, int N, int K, int G, void *hip_stream);
+
+/*
+ * Fused front half of LlamaMLP (down_proj(act_fn(gate_proj(x)) * up_proj(x)),
+ * reached from policy.py:673-678):  y[M,I] = bf16( silu(x.Wg^T) * (x.Wu^T) ),
+ * accumulators, SiLU and product in fp32.  The packed operand has 2*I rows:
+ * rows 0..I-1 are gate_proj, rows I..2I-1 are up_proj.
+ */
+int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void *scales_gu,
+                               const void *qzeros_gu, void *y, int M, int I, int K, int G,
+                               void *hip_stream);
+
+/*
+ * Grouped launch: several independent GEMVs (for example q/k/v of one layer, or
+ * a whole decode step's weight set when the caller streams them back to back)
+ * in ONE kernel launch, so small matrices share the machine instead of paying
+ * one launch latency each.
+ *
+ * A plan is a flat byte blob built on the host, copied by the caller into
+ * device memory once, and reused for every launch while the pointers stay
+ * valid.  vrl_int4_grouped_plan_size() gives its size; vrl_int4_grouped_plan_build()
+ * validates every problem against the preconditions above and fills a host
+ * buffer; vrl_int4_gemv_grouped_bf16() takes the DEVICE copy plus the host
+ * copy's header values (n_problems, total_tiles as returned by _build).
+ */
+typedef struct vrl_int4_problem {
+    const void *x;
+    const void *qweight;
+    const void *scales;
+    const void *qzeros;
+    void *y;
+    int32_t M, N, K, G;
+    int32_t fused_gate_up; /* 0: y[M,N]; 1: rows are gate||up, y[M,N/2] with the SiLU epilogue */
+    int32_t reserved[3];
+} vrl_int4_problem;
+
+size_t vrl_int4_grouped_plan_size(int n_problems);
+
+/* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems));
+ * *total_tiles receives the number of work tiles the launch will walk. */
+int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems,
+                                void *plan_host, size_t plan_bytes, int *total_tiles);
+
+int vrl_int4_gemv_grouped_bf16(const void *plan_dev, int n_problems, int total_tiles,
+                               void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* VRL_INT4_H */

@@ -1,0 +1,113 @@
+"""The C-ABI library loads, exports what the header declares and rejects bad calls.
+
+No kernel is launched here: precondition checks run on the host before any HIP
+call, so these tests need no GPU.
+"""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from visionrl_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "vrl_int4.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vrl_int4_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_symbols()
+    assert set(names) == set(_lib.SYMBOLS)
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_abi_version_and_error_strings(lib):
+    assert lib.vrl_int4_abi_version() == 1
+    assert _lib.error_string(0) == "ok"
+    for code in (1001, 1002, 1003, 1004):
+        assert "unknown" not in _lib.error_string(code)
+    assert "unknown" in _lib.error_string(-5)
+
+
+def test_problem_struct_matches_header():
+    # 5 pointers + 4 ints + flag + 3 reserved ints
+    assert ctypes.sizeof(_lib.Problem) == 5 * 8 + 8 * 4
+
+
+def buf(nbytes, misalign=0):
+    raw = ctypes.create_string_buffer(nbytes + 64)
+    base = (ctypes.addressof(raw) + 15) & ~15
+    return raw, base + misalign
+
+
+@pytest.mark.parametrize("M,N,K,G,code", [
+    (0, 16, 128, 128, 1001),
+    (1, 0, 128, 128, 1001),
+    (1, 16, 0, 128, 1001),
+    (1, 16, 124, 4, 1001),     # K % 8
+    (1, 16, 128, 12, 1001),    # G % 8
+    (1, 16, 128, 48, 1001),    # K % G
+    (1, 16, 128, 0, 1001),
+    (-3, 16, 128, 128, 1001),
+])
+def test_gemv_rejects_bad_shapes(lib, M, N, K, G, code):
+    keep, p = buf(4096)
+    rc = lib.vrl_int4_gemv_bf16(p, p, p, p, p, M, N, K, G, None)
+    assert rc == code
+    with pytest.raises(ValueError):
+        _lib.check(rc, "gemv")
+
+
+def test_null_and_alignment_are_reported(lib):
+    keep, p = buf(4096)
+    assert lib.vrl_int4_gemv_bf16(None, p, p, p, p, 1, 16, 128, 128, None) == 1003
+    assert lib.vrl_int4_gemv_bf16(p, p, p, p, None, 1, 16, 128, 128, None) == 1003
+    assert lib.vrl_int4_gemv_bf16(p + 2, p, p, p, p, 1, 16, 128, 128, None) == 1002
+    assert lib.vrl_int4_gemv_bf16(p, p + 4, p, p, p, 1, 16, 128, 128, None) == 1002
+    assert lib.vrl_int4_dequant_bf16(p, p, None, p, 16, 128, 128, None) == 1003
+    assert lib.vrl_int4_dequant_bf16(p, p, p, p + 8, 16, 128, 128, None) == 1002
+    assert lib.vrl_int4_dequant_bf16(p, p, p, p, 16, 120, 16, None) == 1001
+    assert lib.vrl_int4_gate_up_silu_bf16(p, p, p, p, p, 1, 0, 128, 128, None) == 1001
+    assert lib.vrl_int4_gate_up_silu_bf16(p, p, p, None, p, 1, 8, 128, 128, None) == 1003
+
+
+def test_grouped_plan_validation(lib):
+    keep, p = buf(4096)
+    assert lib.vrl_int4_grouped_plan_size(0) == 0
+    size = lib.vrl_int4_grouped_plan_size(2)
+    assert size >= 2 * ctypes.sizeof(_lib.Problem)
+    probs = (_lib.Problem * 2)()
+    for rec, n in zip(probs, (64, 96)):
+        rec.x = rec.qweight = rec.scales = rec.qzeros = rec.y = p
+        rec.M, rec.N, rec.K, rec.G = 1, n, 256, 128
+    plan = ctypes.create_string_buffer(size)
+    tiles = ctypes.c_int(-1)
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(tiles)) == 0
+    assert tiles.value == 1 + 2   # 64-row tiles: ceil(64/64) + ceil(96/64)
+    # undersized buffer, bad shape inside the list, null list
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size - 1, ctypes.byref(tiles)) == 1004
+    probs[1].K = 100
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(tiles)) == 1001
+    assert lib.vrl_int4_grouped_plan_build(None, 2, plan, size, ctypes.byref(tiles)) == 1003
+    assert lib.vrl_int4_gemv_grouped_bf16(None, 2, 3, None) == 1003
+    assert lib.vrl_int4_gemv_grouped_bf16(p, 0, 3, None) == 1004
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.Int4LibraryError, match="no CPU or PyTorch fallback"):
+        _lib.load()

@@ -1,0 +1,291 @@
+"""Parity of the HIP path against the CPU oracle, on an MI355X.
+
+Every call goes through the torch operators, i.e. through the C ABI.  Dequant is
+checked bit for bit; GEMV outputs against the float64 truth under the operator
+tolerance (see ``tests/_util.assert_gemv_close``); the in-kernel dequant of the
+GEMV is also checked bit for bit through one-hot activations.
+"""
+
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import int4_oracle as o
+from tests._util import assert_gemv_close, bf16_to_bits, bits_to_bf16, to_device
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ops_mod():
+    from visionrl_amd import ops
+    return ops
+
+
+def run_gemv(ops_mod, ops, G):
+    d = to_device(ops, DEV)
+    y = ops_mod.int4_gemv(d["x"], d["qweight"], d["scales"], d["qzeros"], G)
+    torch.cuda.synchronize()
+    return bf16_to_bits(y)
+
+
+# ------------------------------------------------------------------ dequant
+def test_dequant_exhaustive_bit_exact(ops_mod):
+    """All 256 (q, z) pairs x every bf16 mantissa at several exponents."""
+    say("dequant exhaustive")
+    mant = np.arange(128, dtype=np.uint16)
+    scales = np.concatenate([(e << 7) | mant for e in (0x01, 0x60, 0x70, 0x78, 0x7F, 0x90)])
+    scales = np.concatenate([scales, scales | 0x8000]).astype(np.uint16)   # negative scales too
+    G = 16
+    rows = [(int(sb), z) for sb in scales for z in range(16)]
+    N = len(rows)
+    q = np.tile(np.arange(16, dtype=np.uint8), (N, 1))
+    z = np.array([r[1] for r in rows], dtype=np.uint8)[:, None]
+    sb = np.array([r[0] for r in rows], dtype=np.uint16)[:, None]
+    qweight, qzeros = o.pack_nibbles(q), o.pack_nibbles(z)
+    want = o.dequant_bf16(qweight, sb, qzeros, G)
+    got = ops_mod.int4_dequant(torch.from_numpy(qweight).to(DEV), bits_to_bf16(sb, DEV),
+                               torch.from_numpy(qzeros).to(DEV), G)
+    got = bf16_to_bits(got)
+    # +0 and -0 are the same weight
+    same = (got == want) | (((got | want) & 0x7FFF) == 0)
+    assert same.all(), f"{int((~same).sum())} mismatches"
+
+
+@pytest.mark.parametrize("N,K,G,mode", [
+    (64, 2048, 128, "normal"), (33, 5632, 32, "loguniform"), (17, 5632, 64, "loguniform"),
+    (5, 88, 8, "normal"), (256, 4096, 128, "normal"), (7, 48, 24, "normal"),
+])
+def test_dequant_random_bit_exact(ops_mod, N, K, G, mode):
+    say("dequant", N, K, G, mode)
+    ops = o.make_operands(200 + N, 1, K, N, G, mode)
+    d = to_device(ops, DEV)
+    got = bf16_to_bits(ops_mod.int4_dequant(d["qweight"], d["scales"], d["qzeros"], G))
+    want = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    assert (got == want).all()
+
+
+# ------------------------------------------------------------------ GEMV
+TILE_SHAPES = [
+    # M, K, N, G  (K % 128 == 0 and G % 32 == 0: the MFMA tile path)
+    (1, 2048, 2048, 128),      # configuration 1
+    (1, 128, 16, 128),
+    (1, 256, 40, 32),          # ragged N
+    (2, 384, 16, 64),
+    (3, 1024, 100, 128),
+    (7, 2048, 33, 64),
+    (16, 2048, 256, 128),
+    (16, 5632, 64, 128),       # staged activations take several passes
+    (17, 1024, 48, 128),       # second slab of activation rows
+    (32, 2048, 512, 128),      # rollout batch
+    (1, 5632, 2048, 32),       # configuration 5b
+    (1, 5632, 2048, 64),
+    (1, 5632, 2048, 128),
+    (8, 4096, 300, 128),
+    (1, 2048, 5632, 128),
+    (1, 11008, 96, 128),
+]
+
+
+@pytest.mark.parametrize("M,K,N,G", TILE_SHAPES)
+def test_gemv_tile_path(ops_mod, M, K, N, G):
+    say("gemv tile", M, K, N, G)
+    mode = "loguniform" if K == 5632 and N == 2048 else "normal"
+    ops = o.make_operands(1000 + 7 * M + K + N + G, M, K, N, G, mode)
+    be = assert_gemv_close(run_gemv(ops_mod, ops, G), ops, G, f"M{M} K{K} N{N} G{G}")
+    say("  backward error", be)
+    assert be < 2.0 ** -18
+
+
+GENERIC_SHAPES = [
+    (1, 8, 1, 8), (1, 64, 5, 8), (2, 88, 9, 8), (3, 48, 7, 24), (1, 192, 33, 16),
+    (5, 96, 4, 32), (9, 200, 11, 40), (1, 2040, 16, 8),
+]
+
+
+@pytest.mark.parametrize("M,K,N,G", GENERIC_SHAPES)
+def test_gemv_generic_path(ops_mod, M, K, N, G):
+    say("gemv generic", M, K, N, G)
+    ops = o.make_operands(2000 + M + K + N + G, M, K, N, G)
+    assert_gemv_close(run_gemv(ops_mod, ops, G), ops, G, f"M{M} K{K} N{N} G{G}")
+
+
+@pytest.mark.parametrize("M,K,N,G", [(1, 256, 48, 128), (4, 512, 32, 32), (1, 96, 8, 8)])
+def test_gemv_one_hot_is_the_exact_weight_column(ops_mod, M, K, N, G):
+    """x = e_k in every activation row: y must equal column k of the canonical tile bit for bit,
+    which pins the in-register dequant of the GEMV kernels (no summation error is possible)."""
+    say("gemv one-hot", M, K, N, G)
+    ops = o.make_operands(3000 + K, M, K, N, G, "loguniform")
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    ks = sorted(set([0, 1, 4, 7, 8, 31, 32, 33, K // 2 + 5, K - 9, K - 1]))
+    for k0 in ks:
+        x = np.zeros((M, K), dtype=np.float32)
+        for m in range(M):
+            x[m, (k0 + 13 * m) % K] = 1.0
+        ops["x_bits"] = o.f32_to_bf16_bits(x)
+        y = run_gemv(ops_mod, ops, G)
+        for m in range(M):
+            want = w[:, (k0 + 13 * m) % K]
+            same = (y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)
+            assert same.all(), (k0, m)
+
+
+def test_gemv_every_q_z_pair_through_the_kernel(ops_mod):
+    """All 256 (q, z) pairs x 128 mantissas through the tile kernel's dequant, via one-hot x."""
+    say("gemv exhaustive one-hot")
+    G, K = 32, 128
+    mant = np.arange(128, dtype=np.uint16)
+    scales = np.concatenate([(e << 7) | mant for e in (0x70, 0x78)]).astype(np.uint16)
+    rows = [(int(sb), z) for sb in scales for z in range(16)]
+    N = len(rows)
+    q = np.tile(np.arange(16, dtype=np.uint8), (N, K // 16))
+    z = np.repeat(np.array([r[1] for r in rows], dtype=np.uint8)[:, None], K // G, axis=1)
+    sb = np.repeat(np.array([r[0] for r in rows], dtype=np.uint16)[:, None], K // G, axis=1)
+    ops = {"qweight": o.pack_nibbles(q), "scales_bits": sb, "qzeros": o.pack_nibbles(z)}
+    w = o.dequant_bf16(ops["qweight"], sb, ops["qzeros"], G)
+    x = np.zeros((16, K), dtype=np.float32)
+    for m in range(16):
+        x[m, 16 * (m % 8) + m] = 1.0      # activation row m selects k with q = m
+    ops["x_bits"] = o.f32_to_bf16_bits(x)
+    y = run_gemv(ops_mod, ops, G)
+    for m in range(16):
+        want = w[:, 16 * (m % 8) + m]
+        same = (y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)
+        assert same.all(), m
+
+
+def test_gemv_integer_case_is_exact(ops_mod):
+    """s = 1, z = 0, x in {-1,0,1}: an integer matmul, exact in fp32, so only the output rounds."""
+    say("gemv integer")
+    M, K, N, G = 5, 1024, 80, 128
+    rng = np.random.default_rng(5)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    x = rng.integers(-1, 2, (M, K)).astype(np.float32)
+    ops = {"x_bits": o.f32_to_bf16_bits(x), "qweight": o.pack_nibbles(q),
+           "scales_bits": o.f32_to_bf16_bits(np.ones((N, K // G), dtype=np.float32)),
+           "qzeros": o.pack_nibbles(np.zeros((N, K // G), dtype=np.uint8))}
+    want = (x.astype(np.int64) @ q.astype(np.int64).T).astype(np.float32)
+    assert (run_gemv(ops_mod, ops, G) == o.f32_to_bf16_bits(want)).all()
+
+
+def test_gemv_zero_when_q_equals_z(ops_mod):
+    say("gemv q==z")
+    M, K, N, G = 2, 512, 64, 64
+    ops = o.make_operands(6, M, K, N, G)
+    ops["qweight"] = o.pack_nibbles(np.repeat(ops["z"], G, axis=1))
+    assert ((run_gemv(ops_mod, ops, G) & 0x7FFF) == 0).all()
+
+
+def test_gemv_rows_are_independent_of_batch(ops_mod):
+    """Row m of a batched call equals the single-row call (same kernel arithmetic per row)."""
+    say("gemv batch consistency")
+    M, K, N, G = 32, 2048, 128, 128
+    ops = o.make_operands(7, M, K, N, G)
+    full = run_gemv(ops_mod, ops, G)
+    for m in (0, 5, 15, 16, 31):
+        one = dict(ops)
+        one["x_bits"] = ops["x_bits"][m:m + 1]
+        single = run_gemv(ops_mod, one, G)
+        tol_ops = dict(ops)
+        tol_ops["x_bits"] = ops["x_bits"][m:m + 1]
+        assert_gemv_close(single, tol_ops, G, f"row {m} alone")
+        diff = np.abs(o.bf16_bits_to_f32(single[0]).astype(np.float64)
+                      - o.bf16_bits_to_f32(full[m]).astype(np.float64))
+        assert (diff <= o.bf16_ulp(o.bf16_bits_to_f32(full[m]).astype(np.float64))).all()
+
+
+def test_gemv_linearity_in_x(ops_mod):
+    say("gemv linearity")
+    K, N, G = 2048, 256, 128
+    ops = o.make_operands(8, 1, K, N, G)
+    y1 = run_gemv(ops_mod, ops, G)
+    two = dict(ops)
+    two["x_bits"] = o.f32_to_bf16_bits(o.bf16_bits_to_f32(ops["x_bits"]) * 2.0)
+    y2 = run_gemv(ops_mod, two, G)
+    # doubling x doubles every partial sum exactly, so the bf16 results differ by one exponent step
+    assert (o.bf16_bits_to_f32(y2) == 2.0 * o.bf16_bits_to_f32(y1)).all()
+
+
+def test_gemv_is_deterministic(ops_mod):
+    say("gemv determinism")
+    ops = o.make_operands(9, 4, 2048, 2048, 128)
+    a = run_gemv(ops_mod, ops, 128)
+    b = run_gemv(ops_mod, ops, 128)
+    assert (a == b).all()
+
+
+# ------------------------------------------------------------------ fused gate/up
+@pytest.mark.parametrize("M,K,I,G", [
+    (1, 2048, 5632, 128), (8, 4096, 704, 128), (3, 256, 24, 64), (16, 1024, 50, 32),
+    (2, 88, 6, 8), (20, 512, 40, 128),
+])
+def test_gate_up_silu(ops_mod, M, K, I, G):
+    say("gate_up_silu", M, K, I, G)
+    ops = o.make_operands(4000 + M + K + I, M, K, 2 * I, G)
+    d = to_device(ops, DEV)
+    y = bf16_to_bits(ops_mod.int4_gate_up_silu(d["x"], d["qweight"], d["scales"], d["qzeros"], G))
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    ref = o.gate_up_silu_f64(*args)
+    acc = o.gemv_f64(*args)
+    aabs = o.gemv_abs_f64(*args)
+    # first-order propagation of the accumulation noise through silu(g) * u
+    g, u = acc[:, :I], acc[:, I:]
+    sig = 1.0 / (1.0 + np.exp(-g))
+    dsilu = sig * (1.0 + g * (1.0 - sig))
+    noise = 2.0 ** -18 * (np.abs(dsilu * u) * aabs[:, :I] + np.abs(o.silu_f64(g)) * aabs[:, I:])
+    tol = np.maximum(o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + noise
+    err = np.abs(o.bf16_bits_to_f32(y).astype(np.float64) - ref)
+    assert y.shape == (M, I)
+    assert (err <= tol).all(), f"{int((err > tol).sum())} of {err.size} out of tolerance"
+
+
+# ------------------------------------------------------------------ grouped launch
+def test_grouped_launch_matches_single_launches(ops_mod):
+    say("grouped")
+    shapes = [(1, 2048, 2048, 128, False), (1, 2048, 2048, 128, False), (1, 2048, 5632, 128, False),
+              (1, 5632, 2048, 128, False), (4, 2048, 200, 64, False), (2, 1024, 2 * 96, 128, True)]
+    problems, singles, all_ops = [], [], []
+    for i, (M, K, N, G, fused) in enumerate(shapes):
+        ops = o.make_operands(5000 + i, M, K, N, G)
+        d = to_device(ops, DEV)
+        problems.append((d["x"], d["qweight"], d["scales"], d["qzeros"], G, fused))
+        fn = ops_mod.int4_gate_up_silu if fused else ops_mod.int4_gemv
+        singles.append(fn(d["x"], d["qweight"], d["scales"], d["qzeros"], G))
+        all_ops.append((ops, G, fused))
+    grouped = ops_mod.GroupedGemv(problems)
+    for rep in range(2):
+        for y in grouped.outputs:
+            y.zero_()
+        outs = grouped.launch()
+        torch.cuda.synchronize()
+        for y, ref, (ops, G, fused) in zip(outs, singles, all_ops):
+            assert y.shape == ref.shape
+            if not fused:
+                assert_gemv_close(bf16_to_bits(y), ops, G, "grouped")
+            diff = (y.float() - ref.float()).abs()
+            ulp = torch.from_numpy(o.bf16_ulp(ref.float().cpu().numpy().astype(np.float64))).to(DEV)
+            assert (diff <= ulp).all()
+
+
+# ------------------------------------------------------------------ contract violations
+def test_operator_contract_errors(ops_mod):
+    ops = o.make_operands(10, 2, 256, 16, 128)
+    d = to_device(ops, DEV)
+    with pytest.raises(TypeError):
+        ops_mod.int4_gemv(d["x"].float(), d["qweight"], d["scales"], d["qzeros"], 128)
+    with pytest.raises(ValueError):
+        ops_mod.int4_gemv(d["x"][:, :128].contiguous(), d["qweight"], d["scales"], d["qzeros"], 128)
+    with pytest.raises(ValueError):
+        ops_mod.int4_gemv(d["x"].cpu(), d["qweight"], d["scales"], d["qzeros"], 128)
+    with pytest.raises(ValueError):
+        ops_mod.int4_gemv(d["x"], d["qweight"], d["scales"], d["qzeros"], 96)
+    with pytest.raises(ValueError):
+        ops_mod.int4_gemv(d["x"].t().contiguous().t(), d["qweight"], d["scales"], d["qzeros"], 128)

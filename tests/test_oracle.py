@@ -1,0 +1,380 @@
+"""Pins the CPU oracle (numpy and C restatements) by mathematics.
+
+The reference ships no quantised operator and no numeric vector for its decode
+linears, so each oracle function is checked against something that does not
+share its formula: exact integer / rational arithmetic, torch's bf16 rounding,
+special cases that collapse to an integer matmul or to a column of the weight
+tile, and the two restatements against each other.
+"""
+
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import int4_oracle as o
+from tests._util import bits_to_bf16
+
+
+# ---------------------------------------------------------------- exact helpers
+def exact_rne_bf16(fr: Fraction) -> int:
+    """Round a rational to bf16 (8 significant bits, RNE) with integer arithmetic.
+
+    Normal range only (the tests stay inside it).  Returns the bit pattern.
+    """
+    if fr == 0:
+        return 0
+    sign = 0x8000 if fr < 0 else 0
+    a = -fr if fr < 0 else fr
+    e = 0
+    while a >= 2:
+        a /= 2
+        e += 1
+    while a < 1:
+        a *= 2
+        e -= 1
+    scaled = a * 128  # in [128, 256)
+    lo = scaled.numerator // scaled.denominator
+    rem = scaled - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (lo & 1)):
+        lo += 1
+    if lo == 256:
+        lo = 128
+        e += 1
+    assert -126 <= e <= 127
+    return sign | ((e + 127) << 7) | (lo - 128)
+
+
+def bf16_fraction(bits: int) -> Fraction:
+    sign = -1 if bits & 0x8000 else 1
+    e = (bits >> 7) & 0xFF
+    m = bits & 0x7F
+    assert 0 < e < 255
+    return sign * Fraction(128 + m, 128) * Fraction(2) ** (e - 127)
+
+
+# ---------------------------------------------------------------- packing
+def test_pack_known_answers():
+    assert int(o.pack_nibbles(np.arange(8))[0]) == 0x76543210
+    assert int(o.pack_nibbles(np.arange(8, 16))[0]) & 0xFFFFFFFF == 0xFEDCBA98
+    # nibble i alone lands at bits 4i..4i+3
+    for i in range(8):
+        q = np.zeros(8, dtype=np.uint8)
+        q[i] = 0xA
+        assert int(o.pack_nibbles(q)[0]) & 0xFFFFFFFF == 0xA << (4 * i)
+    # a short tail is zero padded into one more word
+    w = o.pack_nibbles(np.array([1, 2, 3, 4, 5, 6, 7, 8, 9, 10], dtype=np.uint8))
+    assert [int(v) & 0xFFFFFFFF for v in w] == [0x87654321, 0x000000A9]
+
+
+def test_pack_unpack_round_trip():
+    rng = np.random.default_rng(0)
+    for shape in [(1, 8), (3, 40), (5, 7, 24), (2, 13)]:
+        q = rng.integers(0, 16, size=shape, dtype=np.uint8)
+        packed = o.pack_nibbles(q)
+        assert packed.dtype == np.int32
+        assert (o.unpack_nibbles(packed, shape[-1]) == q).all()
+    with pytest.raises(ValueError):
+        o.pack_nibbles(np.array([16]))
+
+
+def test_unpack_matches_python_ints():
+    rng = np.random.default_rng(1)
+    words = rng.integers(-2 ** 31, 2 ** 31, size=64, dtype=np.int64).astype(np.int32)
+    got = o.unpack_nibbles(words[None, :], 512)[0]
+    for r, w in enumerate(words):
+        u = int(w) & 0xFFFFFFFF
+        assert [int(v) for v in got[8 * r: 8 * r + 8]] == [(u >> (4 * i)) & 0xF for i in range(8)]
+
+
+# ---------------------------------------------------------------- bf16 rounding
+def test_bf16_rounding_against_torch_and_ties(c_oracle):
+    rng = np.random.default_rng(2)
+    vals = np.concatenate([
+        rng.normal(0, 1, 4096).astype(np.float32),
+        (rng.normal(0, 1, 4096) * 10.0 ** rng.uniform(-30, 30, 4096)).astype(np.float32),
+        # exact ties: mantissa tail 0x8000, even and odd keepers
+        np.array([0x3F808000, 0x3F818000, 0x3FFF8000, 0xBF808000, 0x7F7F8000 - 0x10000,
+                  0x00808000, 0x3F807FFF, 0x3F808001], dtype=np.uint32).view(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, 1.0, 3.0e38], dtype=np.float32),
+    ])
+    mine = o.f32_to_bf16_bits(vals)
+    theirs = torch.from_numpy(vals.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (mine == theirs).all()
+    assert (c_oracle.f32_to_bf16_bits(vals) == theirs).all()
+    # hand-checked ties: 1.00390625 (0x3F808000) -> even keeper 0x3F80; 0x3F818000 -> 0x3F82
+    assert mine[8192] == 0x3F80 and mine[8193] == 0x3F82
+    # widening is exact
+    assert (o.bf16_bits_to_f32(mine).view(np.uint32) == (mine.astype(np.uint32) << 16)).all()
+
+
+def test_bf16_ulp():
+    assert o.bf16_ulp(np.array([1.0]))[0] == 2.0 ** -7
+    assert o.bf16_ulp(np.array([1.99]))[0] == 2.0 ** -7
+    assert o.bf16_ulp(np.array([-2.0]))[0] == 2.0 ** -6
+    assert o.bf16_ulp(np.array([3.0]))[0] == 2.0 ** -6
+    # spacing really is the distance between neighbours
+    b = np.array([0x4049], dtype=np.uint16)  # 3.140625
+    nxt = o.bf16_bits_to_f32(b + 1) - o.bf16_bits_to_f32(b)
+    assert o.bf16_ulp(o.bf16_bits_to_f32(b).astype(np.float64))[0] == float(nxt[0])
+
+
+# ---------------------------------------------------------------- dequant
+def scale_sweep() -> np.ndarray:
+    rng = np.random.default_rng(3)
+    s = [1.0, 2.0 ** -7, 2.0 ** -14, 0.02, 1e-4, 1e-1, 255.0 / 256.0, 1.9921875]
+    s += list(10.0 ** rng.uniform(-4, -1, 40))
+    s += list(np.abs(rng.normal(0, 0.02, 40)))
+    bits = o.f32_to_bf16_bits(np.array(s, dtype=np.float32))
+    # every mantissa pattern, at two exponents: covers all rounding cases of (q-z)*s
+    allm = np.array([(0x3C00 | m) for m in range(128)] + [(0x3880 | m) for m in range(128)],
+                    dtype=np.uint16)
+    return np.unique(np.concatenate([bits, allm]))
+
+
+def test_dequant_exhaustive_against_exact_arithmetic(c_oracle):
+    """All 256 (q, z) pairs x a scale sweep, against integer RNE on exact rationals."""
+    scales = scale_sweep()
+    G = 16
+    # one row per (scale, z): the 16 k of its single group carry q = 0..15
+    rows = [(int(sb), z) for sb in scales for z in range(16)]
+    N = len(rows)
+    q = np.tile(np.arange(16, dtype=np.uint8), (N, 1))
+    z = np.array([r[1] for r in rows], dtype=np.uint8)[:, None]
+    sb = np.array([r[0] for r in rows], dtype=np.uint16)[:, None]
+    qweight, qzeros = o.pack_nibbles(q), o.pack_nibbles(z)
+    got = o.dequant_bf16(qweight, sb, qzeros, G)
+    assert (c_oracle.dequant_bf16(qweight, sb, qzeros, G) == got).all()
+    for n, (sbits, zz) in enumerate(rows):
+        s = bf16_fraction(sbits)
+        for qq in range(16):
+            want = exact_rne_bf16((qq - zz) * s)
+            if qq == zz:
+                assert got[n, qq] in (0x0000, 0x8000)
+            else:
+                assert got[n, qq] == want, (hex(sbits), zz, qq, hex(got[n, qq]), hex(want))
+
+
+def test_dequant_product_is_exact_in_fp32():
+    """(q - z) * s needs at most 12 significant bits: float64 and float32 agree exactly."""
+    scales = o.bf16_bits_to_f32(scale_sweep())
+    d = np.arange(-15, 16, dtype=np.float32)
+    p32 = d[:, None] * scales[None, :]
+    p64 = d[:, None].astype(np.float64) * scales[None, :].astype(np.float64)
+    assert (p32.astype(np.float64) == p64).all()
+
+
+def test_dequant_group_and_zero_indexing(c_oracle):
+    """A hand-built case: scales are powers of two so every weight is an exact integer multiple."""
+    N, K, G = 3, 48, 16
+    rng = np.random.default_rng(4)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    z = rng.integers(0, 16, (N, K // G), dtype=np.uint8)
+    s = np.array([[1.0, 0.5, 4.0], [2.0, 0.25, 8.0], [0.125, 16.0, 1.0]], dtype=np.float32)
+    want = (q.reshape(N, K // G, G).astype(np.float32) - z[:, :, None]) * s[:, :, None]
+    got = o.bf16_bits_to_f32(o.dequant_bf16(o.pack_nibbles(q), o.f32_to_bf16_bits(s),
+                                            o.pack_nibbles(z), G))
+    assert (got == want.reshape(N, K)).all()
+    got_c = c_oracle.dequant_bf16(o.pack_nibbles(q), o.f32_to_bf16_bits(s), o.pack_nibbles(z), G)
+    assert (o.bf16_bits_to_f32(got_c) == want.reshape(N, K)).all()
+
+
+def test_dequant_many_groups_uses_second_zero_word(c_oracle):
+    """More than 8 groups per row: zero-points continue in the next packed word."""
+    N, K, G = 2, 11 * 8, 8
+    rng = np.random.default_rng(5)
+    ops = o.make_operands(5, 1, K, N, G)
+    assert ops["qzeros"].shape == (N, 2)
+    w = o.bf16_bits_to_f32(o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G))
+    s = o.bf16_bits_to_f32(ops["scales_bits"])
+    for n in range(N):
+        for k in range(K):
+            g = k // G
+            exact = (int(ops["q"][n, k]) - int(ops["z"][n, g])) * float(s[n, g])
+            assert w[n, k] == np.float32(torch.tensor(exact, dtype=torch.float32)
+                                         .to(torch.bfloat16).float().item())
+    assert (c_oracle.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+            == o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)).all()
+
+
+def test_dequant_matches_torch_cpu_path():
+    """The PyTorch dequant used as CPU baseline produces the same bits."""
+    ops = o.make_operands(6, 1, 512, 24, 64)
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], 64)
+    tw = o.torch_dequant(torch.from_numpy(ops["qweight"]), bits_to_bf16(ops["scales_bits"]),
+                         torch.from_numpy(ops["qzeros"]), 64)
+    assert (tw.view(torch.int16).numpy().view(np.uint16) == w).all()
+
+
+def test_shape_checks():
+    ops = o.make_operands(7, 1, 64, 4, 32)
+    with pytest.raises(ValueError):
+        o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], 12)
+    with pytest.raises(ValueError):
+        o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], 48)
+    with pytest.raises(ValueError):
+        o.dequant_bf16(ops["qweight"], ops["scales_bits"][:, :1], ops["qzeros"], 32)
+
+
+# ---------------------------------------------------------------- GEMV
+def int_case(seed, M, K, N, G):
+    """s = 1, z = 0, x in {-1, 0, 1}: the GEMV is an exact integer matmul."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    x = rng.integers(-1, 2, (M, K)).astype(np.float32)
+    ops = {
+        "x_bits": o.f32_to_bf16_bits(x),
+        "qweight": o.pack_nibbles(q),
+        "scales_bits": o.f32_to_bf16_bits(np.ones((N, K // G), dtype=np.float32)),
+        "qzeros": o.pack_nibbles(np.zeros((N, K // G), dtype=np.uint8)),
+    }
+    return ops, x.astype(np.int64) @ q.astype(np.int64).T
+
+
+def test_gemv_reduces_to_integer_matmul(c_oracle):
+    ops, want = int_case(8, 3, 128, 16, 32)  # |y| <= 15*128 = 1920 < 2^24: fp32 exact too
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], 32)
+    assert (o.gemv_f64(*args) == want).all()
+    y64, yabs = c_oracle.gemv_f64(*args)
+    assert (y64 == want).all()
+    assert (yabs == np.abs(o.bf16_bits_to_f32(ops["x_bits"]).astype(np.int64))
+            @ o.unpack_nibbles(ops["qweight"], 128).astype(np.int64).T).all()
+    assert (o.gemv_abs_f64(*args) == yabs).all()
+    # bf16 output: exact integers round like torch rounds them
+    want_bits = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy()
+    assert (o.gemv_bf16(*args).view(np.int16) == want_bits).all()
+    assert (c_oracle.gemv_bf16(*args).view(np.int16) == want_bits).all()
+
+
+def test_gemv_one_hot_selects_weight_column(c_oracle):
+    """x = e_k: the output row is column k of the canonical tile, with no rounding left."""
+    K, N, G = 96, 12, 32
+    ops = o.make_operands(9, 1, K, N, G)
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    for k in (0, 7, 31, 32, 95):
+        x = np.zeros((1, K), dtype=np.float32)
+        x[0, k] = 1.0
+        xb = o.f32_to_bf16_bits(x)
+        assert (o.gemv_bf16(xb, ops["qweight"], ops["scales_bits"], ops["qzeros"], G)[0] == w[:, k]).all()
+        assert (c_oracle.gemv_bf16(xb, ops["qweight"], ops["scales_bits"], ops["qzeros"], G)[0]
+                == w[:, k]).all()
+
+
+def test_gemv_zero_when_q_equals_z():
+    K, N, G = 64, 8, 32
+    ops = o.make_operands(10, 2, K, N, G)
+    q = np.repeat(ops["z"], G, axis=1)
+    y = o.gemv_f64(ops["x_bits"], o.pack_nibbles(q), ops["scales_bits"], ops["qzeros"], G)
+    assert (y == 0).all()
+
+
+def test_gemv_restatements_agree_and_track_truth(c_oracle):
+    for seed, (M, K, N, G) in enumerate([(1, 256, 32, 128), (4, 384, 20, 64), (2, 160, 9, 32)]):
+        ops = o.make_operands(100 + seed, M, K, N, G)
+        args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+        y64 = o.gemv_f64(*args)
+        c64, cabs = c_oracle.gemv_f64(*args)
+        # same products, different summation order, both in double
+        assert np.allclose(y64, c64, rtol=0, atol=1e-12 * cabs.max())
+        assert np.allclose(o.gemv_abs_f64(*args), cabs, rtol=1e-12)
+        # an independent evaluation with exact rationals on one output
+        w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+        tot = Fraction(0)
+        for k in range(K):
+            wb, xb = int(w[1, k]), int(ops["x_bits"][0, k])
+            if (wb & 0x7FFF) == 0 or (xb & 0x7FFF) == 0:
+                continue
+            tot += bf16_fraction(wb) * bf16_fraction(xb)
+        assert abs(float(tot) - y64[0, 1]) <= 1e-12 * cabs[0, 1]
+        # both bf16 operators sit inside the stated tolerance of the truth
+        tol = o.gemv_tolerance(y64, cabs)
+        for y_bits in (o.gemv_bf16(*args), c_oracle.gemv_bf16(*args)):
+            assert (np.abs(o.bf16_bits_to_f32(y_bits).astype(np.float64) - y64) <= tol).all()
+
+
+def test_gemv_linearity():
+    K, N, G = 128, 16, 64
+    ops = o.make_operands(11, 2, K, N, G)
+    x = o.bf16_bits_to_f32(ops["x_bits"])
+    x2 = np.stack([x[0] * 2.0, x[0] + 0.0])  # scaling by 2 is exact in bf16
+    y = o.gemv_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    y2 = o.gemv_f64(o.f32_to_bf16_bits(x2), ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    assert (y2[0] == 2.0 * y[0]).all() and (y2[1] == y[0]).all()
+
+
+# ---------------------------------------------------------------- fused gate/up
+def test_gate_up_silu_against_unfused_torch(c_oracle):
+    M, K, I, G = 3, 256, 24, 64
+    ops = o.make_operands(12, M, K, 2 * I, G)
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    acc = o.gemv_f64(*args)
+    want = torch.nn.functional.silu(torch.from_numpy(acc[:, :I])) * torch.from_numpy(acc[:, I:])
+    got64 = o.gate_up_silu_f64(*args)
+    assert np.allclose(got64, want.numpy(), rtol=1e-13, atol=0)
+    for y_bits in (o.gate_up_silu_bf16(*args), c_oracle.gate_up_silu_bf16(*args)):
+        y = o.bf16_bits_to_f32(y_bits).astype(np.float64)
+        assert y.shape == (M, I)
+        assert (np.abs(y - got64) <= np.maximum(o.bf16_ulp(got64), 1e-2 * np.abs(got64)) + 1e-6).all()
+    # silu(0) * u = 0 and silu is odd-ish: a sign flip of the gate rows changes the output as torch says
+    assert o.silu_f64(np.array([0.0]))[0] == 0.0
+    assert abs(o.silu_f64(np.array([1.0]))[0] - 0.7310585786300049) < 1e-15
+
+
+# ---------------------------------------------------------------- quantiser
+def test_quantizer_reconstruction_bound():
+    rng = np.random.default_rng(13)
+    w = rng.normal(0, 0.05, (16, 256)).astype(np.float32)
+    G = 64
+    q, s_bits, z = o.quantize_minmax(w, G)
+    s = o.bf16_bits_to_f32(s_bits)
+    deq = (q.reshape(16, 4, G).astype(np.float32) - z[:, :, None]) * s[:, :, None]
+    err = np.abs(deq.reshape(16, 256) - w).reshape(16, 4, G)
+    # inside the representable range the error is at most half a step; the rounded
+    # zero-point and scale can push the extreme values one further half step out
+    assert (err <= 1.01 * s[:, :, None]).all()
+    assert (np.quantile(err / s[:, :, None], 0.9) <= 0.5 + 1e-3)
+    assert q.min() >= 0 and q.max() <= 15 and z.min() >= 0 and z.max() <= 15
+    # a zero weight dequantises to exactly zero (the range always contains 0)
+    w0 = w.copy()
+    w0[:, ::5] = 0.0
+    q0, s0, z0 = o.quantize_minmax(w0, G)
+    assert (q0[:, ::5] == np.repeat(z0, G, axis=1)[:, ::5]).all()
+
+
+def test_quantizer_is_fixed_point_on_its_own_output():
+    """Quantising an already quantised tile that spans the full 0..15 range reproduces it."""
+    N, K, G = 4, 128, 32
+    rng = np.random.default_rng(14)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    q.reshape(N, K // G, G)[:, :, 0] = 0
+    q.reshape(N, K // G, G)[:, :, 1] = 15
+    z = rng.integers(1, 15, (N, K // G), dtype=np.uint8)
+    s_bits = o.f32_to_bf16_bits(np.full((N, K // G), 0.015625, dtype=np.float32))  # 2^-6
+    w = o.bf16_bits_to_f32(o.dequant_bf16(o.pack_nibbles(q), s_bits, o.pack_nibbles(z), G))
+    q2, s2, z2 = o.quantize_minmax(w, G)
+    assert (q2 == q).all() and (s2 == s_bits).all() and (z2 == z).all()
+
+
+# ---------------------------------------------------------------- bookkeeping
+def test_algorithmic_bytes_match_published_table():
+    assert o.algorithmic_bytes(1, 2048, 2048, 128) == 2_187_264
+    per_layer = 4 * o.algorithmic_bytes(1, 2048, 2048, 128) + \
+        2 * o.algorithmic_bytes(1, 2048, 5632, 128) + o.algorithmic_bytes(1, 5632, 2048, 128)
+    assert per_layer == 26_772_480 and 24 * per_layer == 642_539_520
+    assert o.algorithmic_bytes(32, 2048, 16384, 128) == 18_612_224
+    assert o.algorithmic_bytes(8, 4096, 2 * 11008, 128, fused_gate_up=True) == 47_091_712
+    assert [o.algorithmic_bytes(1, 5632, 2048, g) for g in (32, 64, 128)] == \
+        [6_683_648, 6_233_088, 6_007_808]
+
+
+def test_make_operands_is_seeded_and_in_range():
+    a = o.make_operands(42, 2, 256, 8, 128)
+    b = o.make_operands(42, 2, 256, 8, 128)
+    c = o.make_operands(43, 2, 256, 8, 128)
+    assert all((a[k] == b[k]).all() for k in a)
+    assert not (a["qweight"] == c["qweight"]).all()
+    assert (a["scales_bits"] != 0).all() and (a["scales_bits"] < 0x8000).all()
+    lg = o.make_operands(44, 1, 256, 64, 32, scale_mode="loguniform")
+    s = o.bf16_bits_to_f32(lg["scales_bits"])
+    assert s.min() >= 0.99e-4 and s.max() <= 1.01e-1

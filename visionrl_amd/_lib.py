@@ -1,0 +1,118 @@
+"""ctypes binding of ``include/vrl_int4.h``.
+
+The library is loaded from the package tree (``csrc/libvrl_int4.so``); nothing
+is compiled at import or call time.  A missing library is an error, never a
+reason to fall back to another implementation.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+from .build import LIB_PATH
+
+ABI_VERSION = 1
+
+SYMBOLS = (
+    "vrl_int4_abi_version",
+    "vrl_int4_error_string",
+    "vrl_int4_gemv_bf16",
+    "vrl_int4_dequant_bf16",
+    "vrl_int4_gate_up_silu_bf16",
+    "vrl_int4_grouped_plan_size",
+    "vrl_int4_grouped_plan_build",
+    "vrl_int4_gemv_grouped_bf16",
+)
+
+
+class Int4LibraryError(RuntimeError):
+    """The HIP library is missing, stale, or returned an error code."""
+
+
+class Problem(ctypes.Structure):
+    """Mirror of ``vrl_int4_problem``."""
+
+    _fields_ = [
+        ("x", ctypes.c_void_p),
+        ("qweight", ctypes.c_void_p),
+        ("scales", ctypes.c_void_p),
+        ("qzeros", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("M", ctypes.c_int32),
+        ("N", ctypes.c_int32),
+        ("K", ctypes.c_int32),
+        ("G", ctypes.c_int32),
+        ("fused_gate_up", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 3),
+    ]
+
+
+_lock = threading.Lock()
+_lib = None
+
+
+def _bind(lib):
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.vrl_int4_abi_version.restype = ci
+    lib.vrl_int4_abi_version.argtypes = []
+    lib.vrl_int4_error_string.restype = ctypes.c_char_p
+    lib.vrl_int4_error_string.argtypes = [ci]
+    lib.vrl_int4_gemv_bf16.restype = ci
+    lib.vrl_int4_gemv_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.vrl_int4_dequant_bf16.restype = ci
+    lib.vrl_int4_dequant_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
+    lib.vrl_int4_gate_up_silu_bf16.restype = ci
+    lib.vrl_int4_gate_up_silu_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.vrl_int4_grouped_plan_size.restype = ctypes.c_size_t
+    lib.vrl_int4_grouped_plan_size.argtypes = [ci]
+    lib.vrl_int4_grouped_plan_build.restype = ci
+    lib.vrl_int4_grouped_plan_build.argtypes = [
+        ctypes.POINTER(Problem), ci, vp, ctypes.c_size_t, ctypes.POINTER(ci)]
+    lib.vrl_int4_gemv_grouped_bf16.restype = ci
+    lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ci, ci, vp]
+
+
+def load():
+    """Return the loaded library, raising ``Int4LibraryError`` if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise Int4LibraryError(
+                    f"{LIB_PATH} is missing: build it with `python -m visionrl_amd.build` "
+                    "(there is no CPU or PyTorch fallback for the int4 operators)")
+            try:
+                lib = ctypes.CDLL(LIB_PATH)
+            except OSError as exc:
+                raise Int4LibraryError(f"cannot load {LIB_PATH}: {exc}") from exc
+            for name in SYMBOLS:
+                if not hasattr(lib, name):
+                    raise Int4LibraryError(f"{LIB_PATH} does not export {name}")
+            _bind(lib)
+            got = lib.vrl_int4_abi_version()
+            if got != ABI_VERSION:
+                raise Int4LibraryError(f"{LIB_PATH} has ABI {got}, this package needs {ABI_VERSION}")
+            _lib = lib
+    return _lib
+
+
+def error_string(code: int) -> str:
+    return load().vrl_int4_error_string(int(code)).decode()
+
+
+def check(code: int, what: str) -> None:
+    """Turn a non-zero return code into a Python exception.
+
+    Precondition violations (codes >= 1000) are the caller's mistake and raise
+    ``ValueError``; HIP launch failures raise ``Int4LibraryError``.
+    """
+    if code == 0:
+        return
+    msg = f"{what}: {error_string(code)} (code {code})"
+    if code >= 1000:
+        raise ValueError(msg)
+    raise Int4LibraryError(msg)

@@ -1,0 +1,659 @@
+// int4 weight-only decode linears for MI355X (gfx950 / CDNA4).
+//
+// Replaces the bf16 nn.Linear calls of the rollout decode step that the
+// reference reaches at vrl/models/families/janus_pro/policy.py:673-678 (Llama
+// trunk projections) and policy.py:138-160 (gen_head).  Operand formats and the
+// arithmetic contract are stated in include/vrl_int4.h.
+//
+// Kernels
+//   dequant_kernel        packed int4 -> bf16 [N,K], bit-exact, write-bound.
+//   gemv_tile_kernel      the hot path.  A workgroup owns TILE_ROWS weight rows;
+//                         its waves split K in 128-wide chunks.  Each lane
+//                         streams 16-byte pieces of "its" row (lane%16) with
+//                         global_load_dwordx4, rebuilds the exactly rounded bf16
+//                         weights in registers and feeds them to
+//                         v_mfma_f32_16x16x32_bf16 as the B operand; the
+//                         activations are staged once per workgroup in LDS (in
+//                         the k-order the unpack produces) and read as the A
+//                         operand.  Partial sums of the K split meet in LDS.
+//   gemv_generic_kernel   any legal shape (K%8, G%8): one wave per row, VALU
+//                         dot product, DPP/shuffle reduction.  Correctness
+//                         fallback for shapes the tile kernel does not take.
+//
+// In-register dequant, exact by construction: nibble pairs (i, i+4) of a packed
+// word are turned into two bf16 numbers 128+q with one shift and one and-or
+// ((v >> 4i) & 0x000F000F | 0x43004300), then
+//   v_dot2_f32_bf16(pair, (s,0) or (0,s), c)   with  c = -(128+z)*s  (fp32, exact)
+// gives (q-z)*s exactly (16-bit products, 12-bit result), and
+// v_cvt_pk_bf16_f32 applies the one round-to-nearest-even the contract asks for.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../include/vrl_int4.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+constexpr int WAVE = 64;
+constexpr int KCHUNK = 128;          // k covered by one wave step (4 lanes x 32 k per row)
+constexpr uint32_t PAIR_MASK = 0x000F000Fu;
+constexpr uint32_t PAIR_BIAS = 0x43004300u;  // two bf16 128.0
+
+// Device-side problem record (72 bytes).  Also the element type of a grouped plan.
+struct DevProblem {
+    const uint16_t *x;
+    const uint32_t *qweight;
+    const uint16_t *scales;
+    const uint32_t *qzeros;
+    uint16_t *y;
+    int32_t M, N, K, G;
+    int32_t fused;       // gate||up rows with SiLU epilogue
+    int32_t tile_begin;  // first tile index of this problem inside a grouped launch
+    int32_t kc;          // k extent of x staged in LDS per pass (multiple of KCHUNK)
+    int32_t pad;
+};
+static_assert(sizeof(DevProblem) == 72, "plan record layout is part of the plan format");
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) {
+    return __builtin_bit_cast(float, bits << 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
+    bf16x2_t r;
+    r[0] = (__bf16)lo;  // v_cvt_pk_bf16_f32: round-to-nearest-even
+    r[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bias) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(bias));
+    return r;
+}
+
+// fp32  a.lo*b.lo + a.hi*b.hi + c  on bf16 pairs
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    float r;
+    asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Per-(row, group) dequant constants held by a lane.
+struct GroupConst {
+    uint32_t s_lo;  // bf16 pair (s, 0)
+    uint32_t s_hi;  // bf16 pair (0, s)
+    float c;        // -(128 + z) * s, exact in fp32
+};
+
+__device__ __forceinline__ GroupConst make_group_const(uint32_t scale_bits, uint32_t z) {
+    GroupConst g;
+    g.s_lo = scale_bits & 0xFFFFu;
+    g.s_hi = scale_bits << 16;
+    g.c = -(128.0f + (float)z) * bf16_bits_to_f32(scale_bits & 0xFFFFu);
+    return g;
+}
+
+// One packed word -> 8 exactly rounded bf16 weights in the order
+// (w0,w4),(w1,w5),(w2,w6),(w3,w7): four dwords.
+__device__ __forceinline__ void dequant_word(uint32_t v, const GroupConst &g, uint32_t bias,
+                                             uint32_t out[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t p = and_or(i == 0 ? v : (v >> (4 * i)), PAIR_MASK, bias);
+        float lo = dot2_bf16(p, g.s_lo, g.c);
+        float hi = dot2_bf16(p, g.s_hi, g.c);
+        out[i] = pack_bf16_rne(lo, hi);
+    }
+}
+
+// -------------------------------------------------------------------------
+// dequant: one thread per packed word, natural k order out
+// -------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dequant_kernel(const uint32_t *__restrict__ qweight,
+                                                      const uint16_t *__restrict__ scales,
+                                                      const uint32_t *__restrict__ qzeros,
+                                                      uint16_t *__restrict__ w, int N, int K, int G) {
+    const int kwords = K >> 3;
+    const int groups = K / G;
+    const int zwords = (groups + 7) >> 3;
+    const long total = (long)N * kwords;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int n = (int)(idx / kwords);
+        const int r = (int)(idx - (long)n * kwords);
+        const int g = (r << 3) / G;
+        const uint32_t v = qweight[idx];
+        const float s = bf16_bits_to_f32(scales[(long)n * groups + g]);
+        const int z = (qzeros[(long)n * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xF;
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q0 = (v >> (8 * i)) & 0xF;
+            const int q1 = (v >> (8 * i + 4)) & 0xF;
+            o[i] = pack_bf16_rne((float)(q0 - z) * s, (float)(q1 - z) * s);
+        }
+        u32x4_t ov = {o[0], o[1], o[2], o[3]};
+        *reinterpret_cast<u32x4_t *>(w + idx * 8) = ov;
+    }
+}
+
+// -------------------------------------------------------------------------
+// generic GEMV: one wave per output row (pair of rows when fused)
+// -------------------------------------------------------------------------
+constexpr int GEN_MT = 4;  // activation rows per pass
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ void generic_row_dot(const DevProblem &p, int n, int m0, int mt,
+                                                float acc[GEN_MT]) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int kwords = p.K >> 3;
+    const int groups = p.K / p.G;
+    const int zwords = (groups + 7) >> 3;
+#pragma unroll
+    for (int j = 0; j < GEN_MT; ++j) acc[j] = 0.0f;
+    for (int r = lane; r < kwords; r += WAVE) {
+        const int g = (r << 3) / p.G;
+        const uint32_t v = p.qweight[(long)n * kwords + r];
+        const float s = bf16_bits_to_f32(p.scales[(long)n * groups + g]);
+        const int z = (p.qzeros[(long)n * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xF;
+        float wv[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q0 = (v >> (8 * i)) & 0xF;
+            const int q1 = (v >> (8 * i + 4)) & 0xF;
+            const uint32_t pk = pack_bf16_rne((float)(q0 - z) * s, (float)(q1 - z) * s);
+            wv[2 * i] = bf16_bits_to_f32(pk & 0xFFFFu);
+            wv[2 * i + 1] = bf16_bits_to_f32(pk >> 16);
+        }
+#pragma unroll
+        for (int j = 0; j < GEN_MT; ++j) {
+            if (j < mt) {
+                const u32x4_t xv =
+                    *reinterpret_cast<const u32x4_t *>(p.x + (long)(m0 + j) * p.K + (r << 3));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[j] = __builtin_fmaf(bf16_bits_to_f32(xv[i] & 0xFFFFu), wv[2 * i], acc[j]);
+                    acc[j] = __builtin_fmaf(bf16_bits_to_f32(xv[i] >> 16), wv[2 * i + 1], acc[j]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < GEN_MT; ++j) acc[j] = wave_sum(acc[j]);
+}
+
+__global__ __launch_bounds__(256) void gemv_generic_kernel(DevProblem p) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const int out_cols = p.fused ? p.N / 2 : p.N;
+    const int n = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (n >= out_cols) return;  // whole wave leaves together
+    for (int m0 = 0; m0 < p.M; m0 += GEN_MT) {
+        const int mt = min(GEN_MT, p.M - m0);
+        float a[GEN_MT], b[GEN_MT];
+        generic_row_dot(p, n, m0, mt, a);
+        if (p.fused) generic_row_dot(p, out_cols + n, m0, mt, b);
+        if (lane == 0) {
+            for (int j = 0; j < mt; ++j) {
+                float v = a[j];
+                if (p.fused) v = (v / (1.0f + __expf(-v))) * b[j];
+                p.y[(long)(m0 + j) * out_cols + n] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+            }
+        }
+    }
+}
+
+// -------------------------------------------------------------------------
+// tile GEMV (MFMA dot, VALU dequant)
+// -------------------------------------------------------------------------
+// R   weight row tiles (16 rows each) per workgroup; fused problems use R/2
+//     gate tiles followed by R/2 up tiles and emit 16*R/2 output columns.
+// MB  16-row blocks of activations (M <= 16*MB).
+// WPB waves per workgroup; wave w owns k-chunks c with c % WPB == w.
+template <int R, int MB, int WPB>
+struct TileCfg {
+    static constexpr int THREADS = WPB * WAVE;
+    static constexpr int RED_FLOATS = WPB * R * MB * 256;
+};
+
+constexpr int XPAD = 8;  // bf16 elements of padding per staged activation row (16 bytes)
+
+template <int R>
+struct Prefetch {
+    u32x4_t w[R];
+    uint32_t sbits[R];
+    uint32_t zword[R];
+};
+
+template <int R, int MB, int WPB>
+__device__ __forceinline__ void tile_body(const DevProblem &p, int tile, uint8_t *smem) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid >> 6;
+    const int lc = lane & 15;  // weight row within a tile / activation row within a block
+    const int kq = lane >> 4;  // which 32-k quarter of the chunk this lane streams
+
+    const int K = p.K, G = p.G, M = p.M;
+    const int kwords = K >> 3;
+    const int groups = K / G;
+    const int zwords = (groups + 7) >> 3;
+    const bool fused = p.fused != 0;
+    const int out_cols = fused ? p.N / 2 : p.N;
+    const int cols_per_tile = fused ? 16 * (R / 2) : 16 * R;
+    const int col0 = tile * cols_per_tile;
+
+    // weight row streamed by this lane for each of the R tiles (clamped: rows past
+    // the end are loaded from the last row and their results never stored)
+    long row_off[R];
+    long sc_off[R];
+    long z_off[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int row;
+        if (fused) {
+            constexpr int H = R > 1 ? R / 2 : 1;  // fused launches always have R >= 2
+            const int half = r / H;
+            const int c = col0 + 16 * (r % H) + lc;
+            row = half * out_cols + min(c, out_cols - 1);
+        } else {
+            row = min(col0 + 16 * r + lc, p.N - 1);
+        }
+        row_off[r] = (long)row * kwords;
+        sc_off[r] = (long)row * groups;
+        z_off[r] = (long)row * zwords;
+    }
+
+    f32x4_t acc[R][MB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int kc = p.kc;                 // staged k extent
+    const int xstride = kc + XPAD;       // bf16 elements per staged row
+    const uint32_t bias = PAIR_BIAS;
+
+    auto issue = [&](int chunk, Prefetch<R> &pf) {
+        const int k0 = chunk * KCHUNK + 32 * kq;
+        const int g = k0 / G;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            pf.w[r] = *reinterpret_cast<const u32x4_t *>(p.qweight + row_off[r] + (k0 >> 3));
+            pf.sbits[r] = p.scales[sc_off[r] + g];
+            pf.zword[r] = p.qzeros[z_off[r] + (g >> 3)];
+        }
+        return g;
+    };
+
+    for (int kbase = 0; kbase < K; kbase += kc) {
+        const int kext = min(kc, K - kbase);
+        // ---- stage x[:, kbase : kbase+kext] into LDS, pair-interleaved per 8 k ----
+        if (kbase != 0) __syncthreads();
+        {
+            const int words_per_row = kext >> 3;  // 16-byte pieces
+            const int total = M * words_per_row;
+            for (int idx = tid; idx < total; idx += WPB * WAVE) {
+                const int m = idx / words_per_row;
+                const int j = idx - m * words_per_row;
+                const u32x4_t d =
+                    *reinterpret_cast<const u32x4_t *>(p.x + (long)m * K + kbase + (j << 3));
+                u32x4_t o;
+                o[0] = (d[0] & 0xFFFFu) | (d[2] << 16);          // x0, x4
+                o[1] = (d[0] >> 16) | (d[2] & 0xFFFF0000u);      // x1, x5
+                o[2] = (d[1] & 0xFFFFu) | (d[3] << 16);          // x2, x6
+                o[3] = (d[1] >> 16) | (d[3] & 0xFFFF0000u);      // x3, x7
+                *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = o;
+            }
+        }
+        __syncthreads();
+
+        const int c_begin = kbase / KCHUNK;
+        const int c_end = (kbase + kext) / KCHUNK;
+        int chunk = c_begin + wave;
+        Prefetch<R> cur, nxt;
+        int g_cur = 0, g_nxt = 0;
+        if (chunk < c_end) g_cur = issue(chunk, cur);
+        for (; chunk < c_end; chunk += WPB) {
+            const bool more = chunk + WPB < c_end;
+            if (more) g_nxt = issue(chunk + WPB, nxt);
+
+            // activations for this chunk: A operands, 4 k-steps x MB row blocks
+            bf16x8_t xa[4][MB];
+            const int kloc = chunk * KCHUNK - kbase + 32 * kq;
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = min(16 * b + lc, M - 1);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const u32x4_t raw =
+                        *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * t);
+                    xa[t][b] = __builtin_bit_cast(bf16x8_t, raw);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t z = (cur.zword[r] >> (4 * (g_cur & 7))) & 0xFu;
+                const GroupConst gc = make_group_const(cur.sbits[r], z);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    uint32_t wb[4];
+                    dequant_word(cur.w[r][t], gc, bias, wb);
+                    const u32x4_t wv = {wb[0], wb[1], wb[2], wb[3]};
+                    const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+                    for (int b = 0; b < MB; ++b)
+                        acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[t][b], bop,
+                                                                            acc[r][b], 0, 0, 0);
+                }
+            }
+            if (more) {
+                cur = nxt;
+                g_cur = g_nxt;
+            }
+        }
+    }
+
+    // ---- meet the K split: partial tiles -> LDS -> sum -> epilogue ----
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(smem);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[((wave * R + r) * MB + b) * 256 + i * WAVE + lane] = acc[r][b][i];
+    __syncthreads();
+
+    // element e of a (tile r, block b) slab: i = e / 64, lane = e % 64 ->
+    //   activation row m = 16 b + 4 (lane / 16) + i, column = lane % 16
+    const int RO = fused ? R / 2 : R;
+    const int count = RO * MB * 256;
+    for (int e = tid; e < count; e += WPB * WAVE) {
+        const int slab = e >> 8;
+        const int r = slab / MB;
+        const int b = slab - r * MB;
+        const int within = e & 255;
+        const int i = within >> 6;
+        const int ln = within & 63;
+        const int m = 16 * b + 4 * (ln >> 4) + i;
+        const int col = col0 + 16 * r + (ln & 15);
+        if (m >= M || col >= out_cols) continue;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < WPB; ++w) v += red[((w * R + r) * MB + b) * 256 + within];
+        if (fused) {
+            float u = 0.f;
+#pragma unroll
+            for (int w = 0; w < WPB; ++w) u += red[((w * R + r + R / 2) * MB + b) * 256 + within];
+            v = (v / (1.0f + __expf(-v))) * u;
+        }
+        p.y[(long)m * out_cols + col] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+    }
+}
+
+template <int R, int MB, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_tile_kernel(DevProblem p) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    tile_body<R, MB, WPB>(p, blockIdx.x, smem);
+}
+
+// Grouped launch: blocks walk the tile list with a grid stride; every wave of a
+// block sees the same uniform loop bounds, so all of them reach the end.
+template <int R, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_grouped_kernel(const DevProblem *__restrict__ plan,
+                                                                 int n_problems, int total_tiles) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        // largest i with plan[i].tile_begin <= t
+        int lo = 0, hi = n_problems - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (plan[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
+        }
+        const DevProblem p = plan[lo];
+        if (t != blockIdx.x) __syncthreads();  // LDS of the previous tile is free again
+        tile_body<R, 1, WPB>(p, t - p.tile_begin, smem);
+    }
+}
+
+// -------------------------------------------------------------------------
+// host side
+// -------------------------------------------------------------------------
+constexpr int TILE_WPB = 8;
+constexpr int GROUPED_R = 4;
+constexpr int MAX_TILE_M = 16;                  // activation rows one tile-kernel launch takes
+constexpr size_t LDS_X_BUDGET = 40 * 1024;      // staged activations per workgroup
+constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // staged extents shorter than K are multiples of this
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_problem(const void *x, const void *qw, const void *sc, const void *qz, const void *y,
+                  long M, long N, long K, long G) {
+    if (!x || !qw || !sc || !qz || !y) return VRL_INT4_ENULL;
+    if (M < 1 || N < 1 || K < 8 || G < 8) return VRL_INT4_ESHAPE;
+    if (K % 8 != 0 || G % 8 != 0 || K % G != 0) return VRL_INT4_ESHAPE;
+    if (N * K >= (1L << 40) || M * K >= (1L << 31) || M * N >= (1L << 31)) return VRL_INT4_ESHAPE;
+    if (!aligned16(x) || !aligned16(qw) || !aligned16(sc) || !aligned16(qz) || !aligned16(y))
+        return VRL_INT4_EALIGN;
+    return VRL_INT4_OK;
+}
+
+bool tile_path_ok(const DevProblem &p) {
+    return p.K % KCHUNK == 0 && p.G % 32 == 0 && p.M <= MAX_TILE_M;
+}
+
+// k extent of x staged per pass: all of K when M rows of it fit the budget,
+// else the largest multiple of STAGE_STEP that does (M <= 16 always fits one step)
+int staged_k(int M, int K) {
+    if ((size_t)M * (K + XPAD) * 2 <= LDS_X_BUDGET) return K;
+    long kc = (long)(LDS_X_BUDGET / ((size_t)M * 2)) - XPAD;
+    kc -= kc % STAGE_STEP;
+    if (kc < STAGE_STEP) kc = STAGE_STEP;
+    return (int)(kc < K ? kc : K);
+}
+
+template <int R, int MB>
+size_t tile_smem_bytes(int M, int kc) {
+    const size_t xbytes = (size_t)M * (kc + XPAD) * 2;
+    const size_t rbytes = (size_t)TileCfg<R, MB, TILE_WPB>::RED_FLOATS * 4;
+    return xbytes > rbytes ? xbytes : rbytes;
+}
+
+int device_cu_count() {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            cus = v;
+    }
+    return cus;
+}
+
+template <int R, int MB>
+int launch_tile(const DevProblem &p, hipStream_t stream) {
+    const int out_cols = p.fused ? p.N / 2 : p.N;
+    const int cols_per_tile = p.fused ? 16 * (R / 2) : 16 * R;
+    const int tiles = (out_cols + cols_per_tile - 1) / cols_per_tile;
+    const size_t smem = tile_smem_bytes<R, MB>(p.M, p.kc);
+    hipLaunchKernelGGL((gemv_tile_kernel<R, MB, TILE_WPB>), dim3(tiles), dim3(TILE_WPB * WAVE), smem,
+                       stream, p);
+    return (int)hipGetLastError();
+}
+
+int launch_problem(DevProblem p, hipStream_t stream) {
+    const int out_cols = p.fused ? p.N / 2 : p.N;
+    if (!tile_path_ok(p)) {
+        // the generic kernel walks activation rows itself, any M
+        const int waves = 4;
+        hipLaunchKernelGGL(gemv_generic_kernel, dim3((out_cols + waves - 1) / waves),
+                           dim3(waves * WAVE), 0, stream, p);
+        return (int)hipGetLastError();
+    }
+    p.kc = staged_k(p.M, p.K);
+    // widest tile that still gives every CU two workgroups; narrow tiles otherwise
+    const int cus = device_cu_count();
+    const int cols_r4 = p.fused ? 32 : 64;
+    if ((out_cols + cols_r4 - 1) / cols_r4 >= 2 * cus) return launch_tile<4, 1>(p, stream);
+    if (p.fused || (out_cols + 31) / 32 >= 2 * cus) return launch_tile<2, 1>(p, stream);
+    return launch_tile<1, 1>(p, stream);
+}
+
+int run_rows(const void *x, const void *qw, const void *sc, const void *qz, void *y, int M, int N,
+             int K, int G, int fused, void *hip_stream) {
+    int rc = check_problem(x, qw, sc, qz, y, M, N, K, G);
+    if (rc != VRL_INT4_OK) return rc;
+    if (fused && (N % 2 != 0)) return VRL_INT4_ESHAPE;
+    const int out_cols = fused ? N / 2 : N;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    // activation rows go in slabs of MAX_TILE_M (weights are re-read per slab)
+    for (int m0 = 0; m0 < M; m0 += MAX_TILE_M) {
+        DevProblem p;
+        memset(&p, 0, sizeof p);
+        p.x = static_cast<const uint16_t *>(x) + (long)m0 * K;
+        p.qweight = static_cast<const uint32_t *>(qw);
+        p.scales = static_cast<const uint16_t *>(sc);
+        p.qzeros = static_cast<const uint32_t *>(qz);
+        p.y = static_cast<uint16_t *>(y) + (long)m0 * out_cols;
+        p.M = (M - m0 < MAX_TILE_M) ? (M - m0) : MAX_TILE_M;
+        p.N = N;
+        p.K = K;
+        p.G = G;
+        p.fused = fused;
+        rc = launch_problem(p, stream);
+        if (rc != 0) return rc;
+    }
+    return VRL_INT4_OK;
+}
+
+struct PlanHeader {
+    uint32_t magic;
+    int32_t n_problems;
+    int32_t total_tiles;
+    int32_t max_smem;
+};
+static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
+constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
+
+}  // namespace
+
+extern "C" {
+
+int vrl_int4_abi_version(void) { return VRL_INT4_ABI_VERSION; }
+
+const char *vrl_int4_error_string(int code) {
+    switch (code) {
+        case VRL_INT4_OK: return "ok";
+        case VRL_INT4_ESHAPE: return "shape violates a precondition (M,N>=1; K%8==0; G%8==0; K%G==0)";
+        case VRL_INT4_EALIGN: return "pointer is not 16-byte aligned";
+        case VRL_INT4_ENULL: return "required pointer is NULL";
+        case VRL_INT4_EPLAN: return "malformed or undersized grouped plan";
+        default: break;
+    }
+    if (code > 0 && code < 1000) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error code";
+}
+
+int vrl_int4_gemv_bf16(const void *x, const void *qweight, const void *scales, const void *qzeros,
+                       void *y, int M, int N, int K, int G, void *hip_stream) {
+    return run_rows(x, qweight, scales, qzeros, y, M, N, K, G, 0, hip_stream);
+}
+
+int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void *scales_gu,
+                               const void *qzeros_gu, void *y, int M, int I, int K, int G,
+                               void *hip_stream) {
+    if (I < 1 || I > (1 << 29)) return VRL_INT4_ESHAPE;
+    return run_rows(x, qweight_gu, scales_gu, qzeros_gu, y, M, 2 * I, K, G, 1, hip_stream);
+}
+
+int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *qzeros, void *w,
+                          int N, int K, int G, void *hip_stream) {
+    int rc = check_problem(qweight, qweight, scales, qzeros, w, 1, N, K, G);
+    if (rc != VRL_INT4_OK) return rc;
+    const long total = (long)N * (K >> 3);
+    long blocks = (total + 255) / 256;
+    const long cap = (long)device_cu_count() * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(hip_stream),
+                       static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
+                       static_cast<const uint32_t *>(qzeros), static_cast<uint16_t *>(w), N, K, G);
+    return (int)hipGetLastError();
+}
+
+size_t vrl_int4_grouped_plan_size(int n_problems) {
+    if (n_problems < 1) return 0;
+    return sizeof(PlanHeader) + (size_t)n_problems * sizeof(DevProblem);
+}
+
+int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems, void *plan_host,
+                                size_t plan_bytes, int *total_tiles) {
+    if (!problems || !plan_host || !total_tiles) return VRL_INT4_ENULL;
+    if (n_problems < 1 || plan_bytes < vrl_int4_grouped_plan_size(n_problems)) return VRL_INT4_EPLAN;
+    PlanHeader hdr;
+    hdr.magic = PLAN_MAGIC;
+    hdr.n_problems = n_problems;
+    hdr.max_smem = 0;
+    DevProblem *recs = reinterpret_cast<DevProblem *>(static_cast<uint8_t *>(plan_host) + sizeof hdr);
+    long tiles = 0;
+    for (int i = 0; i < n_problems; ++i) {
+        const vrl_int4_problem &q = problems[i];
+        int rc = check_problem(q.x, q.qweight, q.scales, q.qzeros, q.y, q.M, q.N, q.K, q.G);
+        if (rc != VRL_INT4_OK) return rc;
+        if (q.fused_gate_up && q.N % 2 != 0) return VRL_INT4_ESHAPE;
+        DevProblem p;
+        memset(&p, 0, sizeof p);
+        p.x = static_cast<const uint16_t *>(q.x);
+        p.qweight = static_cast<const uint32_t *>(q.qweight);
+        p.scales = static_cast<const uint16_t *>(q.scales);
+        p.qzeros = static_cast<const uint32_t *>(q.qzeros);
+        p.y = static_cast<uint16_t *>(q.y);
+        p.M = q.M; p.N = q.N; p.K = q.K; p.G = q.G;
+        p.fused = q.fused_gate_up ? 1 : 0;
+        if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take tile-path shapes only
+        p.kc = staged_k(p.M, p.K);
+        p.tile_begin = (int)tiles;
+        const int out_cols = p.fused ? p.N / 2 : p.N;
+        const int cols_per_tile = p.fused ? 16 * (GROUPED_R / 2) : 16 * GROUPED_R;
+        tiles += (out_cols + cols_per_tile - 1) / cols_per_tile;
+        if (tiles >= (1L << 30)) return VRL_INT4_ESHAPE;
+        const size_t smem = tile_smem_bytes<GROUPED_R, 1>(p.M, p.kc);
+        if ((int)smem > hdr.max_smem) hdr.max_smem = (int)smem;
+        recs[i] = p;
+    }
+    hdr.total_tiles = (int)tiles;
+    memcpy(plan_host, &hdr, sizeof hdr);
+    *total_tiles = (int)tiles;
+    return VRL_INT4_OK;
+}
+
+int vrl_int4_gemv_grouped_bf16(const void *plan_dev, int n_problems, int total_tiles,
+                               void *hip_stream) {
+    if (!plan_dev) return VRL_INT4_ENULL;
+    if (n_problems < 1 || total_tiles < 1 || !aligned16(plan_dev)) return VRL_INT4_EPLAN;
+    const DevProblem *recs =
+        reinterpret_cast<const DevProblem *>(static_cast<const uint8_t *>(plan_dev) + sizeof(PlanHeader));
+    // LDS: the most any record can need (staged activations never exceed the budget)
+    size_t smem = tile_smem_bytes<GROUPED_R, 1>(1, 0);
+    if (LDS_X_BUDGET > smem) smem = LDS_X_BUDGET;
+    int blocks = device_cu_count() * 2;
+    if (blocks > total_tiles) blocks = total_tiles;
+    hipLaunchKernelGGL((gemv_grouped_kernel<GROUPED_R, TILE_WPB>), dim3(blocks),
+                       dim3(TILE_WPB * WAVE), smem, reinterpret_cast<hipStream_t>(hip_stream), recs,
+                       n_problems, total_tiles);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,0 +1,133 @@
+"""``Int4Linear``: drop-in for the bf16 ``nn.Linear`` layers of rollout decode.
+
+The reference calls its decode linears as plain modules, ``module(x[..., K]) ->
+[..., N]`` in the model dtype, under ``torch.no_grad()``
+(``vrl/models/families/janus_pro/policy.py:673-678`` for the Llama trunk,
+``policy.py:138-160`` for ``gen_head``).  These modules keep that calling
+convention and route the arithmetic to the HIP library; the weights are frozen
+(no gradient flows into the packed tensors).
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from . import ops
+from .int4_format import check_packed, pack_nibbles, quantize_minmax
+
+
+def _rows(x: torch.Tensor, in_features: int) -> torch.Tensor:
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"Int4Linear runs in bfloat16 like the policy it replaces, got {x.dtype}")
+    if x.shape[-1] != in_features:
+        raise ValueError(f"last dimension {x.shape[-1]} != in_features {in_features}")
+    return x.reshape(-1, in_features).contiguous()
+
+
+class Int4Linear(nn.Module):
+    """int4 weight-only linear: ``y = x . dequant(qweight, scales, qzeros)^T (+ bias)``.
+
+    Buffers (saved in ``state_dict``): ``qweight`` int32 ``[N, K/8]``, ``scales`` bf16
+    ``[N, K/G]``, ``qzeros`` int32 ``[N, ceil(K/G/8)]``, optional ``bias`` bf16 ``[N]``.
+    """
+
+    def __init__(self, in_features: int, out_features: int, group_size: int = 128,
+                 bias: bool = False, device=None):
+        super().__init__()
+        if group_size % 8 != 0 or in_features % group_size != 0:
+            raise ValueError("group_size must be a multiple of 8 that divides in_features")
+        self.in_features = int(in_features)
+        self.out_features = int(out_features)
+        self.group_size = int(group_size)
+        groups = in_features // group_size
+        self.register_buffer("qweight", torch.zeros((out_features, in_features // 8),
+                                                    dtype=torch.int32, device=device))
+        self.register_buffer("scales", torch.ones((out_features, groups), dtype=torch.bfloat16,
+                                                  device=device))
+        self.register_buffer("qzeros", torch.zeros((out_features, (groups + 7) // 8),
+                                                   dtype=torch.int32, device=device))
+        if bias:
+            self.register_buffer("bias", torch.zeros(out_features, dtype=torch.bfloat16, device=device))
+        else:
+            self.bias = None
+
+    @classmethod
+    def from_packed(cls, qweight, scales, qzeros, group_size: int, bias=None) -> "Int4Linear":
+        N, K, _ = check_packed(qweight, scales, qzeros, group_size)
+        mod = cls(K, N, group_size, bias=bias is not None, device=qweight.device)
+        mod.qweight, mod.scales, mod.qzeros = qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+        if bias is not None:
+            mod.bias = bias.detach().to(torch.bfloat16).contiguous()
+        return mod
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, group_size: int = 128) -> "Int4Linear":
+        """Quantise an ``nn.Linear`` (min/max, asymmetric, per K-group) on its own device."""
+        qweight, scales, qzeros = quantize_minmax(linear.weight.data, group_size)
+        return cls.from_packed(qweight, scales, qzeros, group_size,
+                               None if linear.bias is None else linear.bias.data)
+
+    @classmethod
+    def from_unpacked_zeros(cls, qweight, scales, zeros_u8, group_size: int, bias=None):
+        """Accepts zero-points as an unpacked ``uint8 [N, K/G]`` tensor and packs them."""
+        return cls.from_packed(qweight, scales, pack_nibbles(zeros_u8.to(torch.int32)), group_size, bias)
+
+    def dequantize(self) -> torch.Tensor:
+        """The canonical bf16 weight ``[N, K]`` (bit-exact tile), e.g. for the train-time replay."""
+        return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rows = _rows(x, self.in_features)
+        y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*x.shape[:-1], self.out_features)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"group_size={self.group_size}, bias={self.bias is not None}")
+
+
+class Int4GateUpSiLU(nn.Module):
+    """Fused ``silu(gate_proj(x)) * up_proj(x)`` over one packed gate||up operand."""
+
+    def __init__(self, gate: Int4Linear, up: Int4Linear):
+        super().__init__()
+        if (gate.in_features, gate.out_features, gate.group_size) != \
+                (up.in_features, up.out_features, up.group_size):
+            raise ValueError("gate_proj and up_proj must have the same shape and group size")
+        if gate.bias is not None or up.bias is not None:
+            raise ValueError("the fused gate/up operator takes bias-free projections")
+        self.in_features = gate.in_features
+        self.intermediate_size = gate.out_features
+        self.group_size = gate.group_size
+        self.register_buffer("qweight", torch.cat([gate.qweight, up.qweight], dim=0).contiguous())
+        self.register_buffer("scales", torch.cat([gate.scales, up.scales], dim=0).contiguous())
+        self.register_buffer("qzeros", torch.cat([gate.qzeros, up.qzeros], dim=0).contiguous())
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        rows = _rows(x, self.in_features)
+        y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        return y.reshape(*x.shape[:-1], self.intermediate_size)
+
+
+class Int4LlamaMLP(nn.Module):
+    """``down_proj(silu(gate_proj(x)) * up_proj(x))`` with both halves in int4.
+
+    Built from a Hugging Face ``LlamaMLP``-shaped module (attributes ``gate_proj``,
+    ``up_proj``, ``down_proj``; SiLU activation).
+    """
+
+    def __init__(self, mlp: nn.Module, group_size: int = 128):
+        super().__init__()
+        act = getattr(mlp, "act_fn", None)
+        if act is not None and not isinstance(act, nn.SiLU) and \
+                getattr(act, "__name__", type(act).__name__).lower() not in ("silu", "siluactivation"):
+            raise ValueError(f"fused MLP needs a SiLU activation, found {act!r}")
+        as_int4 = lambda m: m if isinstance(m, Int4Linear) else Int4Linear.from_linear(m, group_size)
+        self.gate_up = Int4GateUpSiLU(as_int4(mlp.gate_proj), as_int4(mlp.up_proj))
+        self.down_proj = as_int4(mlp.down_proj)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(self.gate_up(x))

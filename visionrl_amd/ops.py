@@ -1,0 +1,179 @@
+"""Torch operators over the HIP library (namespace ``vrl_hip``).
+
+``vrl_hip::int4_gemv``          y[M,N]  = x[M,K] . dequant(W)^T
+``vrl_hip::int4_dequant``       W[N,K]  bf16, bit-exact canonical tile
+``vrl_hip::int4_gate_up_silu``  y[M,I]  = silu(x . Wg^T) * (x . Wu^T)
+
+They stand where the reference calls bf16 ``nn.Linear`` modules during rollout
+decode (``vrl/models/families/janus_pro/policy.py:673-678`` trunk,
+``policy.py:138-160`` head).  Contract violations raise ``ValueError`` /
+``TypeError`` before anything is enqueued, in the raise-on-violation style of the
+reference's step functions (``policy.py:585-601``).  The operators run only on a
+ROCm device through the HIP library: there is no CPU implementation, and a
+missing library raises ``Int4LibraryError``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .int4_format import check_packed
+
+__all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "GroupedGemv"]
+
+
+def _stream_handle(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_device(name: str, t: torch.Tensor, device: torch.device | None = None) -> torch.device:
+    if t.device.type != "cuda":
+        raise ValueError(
+            f"{name} must live on a ROCm device (got {t.device}); the int4 operators have no CPU path")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name} is on {t.device}, expected {device}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t.device
+
+
+def _check_call(x, qweight, scales, qzeros, group_size):
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"x must be bfloat16, got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError("x must be [M, K]")
+    N, K, _ = check_packed(qweight, scales, qzeros, group_size)
+    if x.shape[1] != K:
+        raise ValueError(f"x has K={x.shape[1]}, packed weights have K={K}")
+    if x.shape[0] < 1:
+        raise ValueError("x needs at least one row")
+    dev = _require_device("x", x)
+    for name, t in (("qweight", qweight), ("scales", scales), ("qzeros", qzeros)):
+        _require_device(name, t, dev)
+    return x.shape[0], N, K, dev
+
+
+@torch.library.custom_op("vrl_hip::int4_gemv", mutates_args=())
+def int4_gemv(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+              qzeros: torch.Tensor, group_size: int) -> torch.Tensor:
+    M, N, K, dev = _check_call(x, qweight, scales, qzeros, group_size)
+    lib = _lib.load()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.vrl_int4_gemv_bf16(x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                    qzeros.data_ptr(), y.data_ptr(), M, N, K, int(group_size),
+                                    _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_gemv_bf16")
+    return y
+
+
+@int4_gemv.register_fake
+def _(x, qweight, scales, qzeros, group_size):
+    return x.new_empty((x.shape[0], qweight.shape[0]))
+
+
+@torch.library.custom_op("vrl_hip::int4_dequant", mutates_args=())
+def int4_dequant(qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
+                 group_size: int) -> torch.Tensor:
+    N, K, _ = check_packed(qweight, scales, qzeros, group_size)
+    dev = _require_device("qweight", qweight)
+    _require_device("scales", scales, dev)
+    _require_device("qzeros", qzeros, dev)
+    lib = _lib.load()
+    w = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.vrl_int4_dequant_bf16(qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+                                       w.data_ptr(), N, K, int(group_size), _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_dequant_bf16")
+    return w
+
+
+@int4_dequant.register_fake
+def _(qweight, scales, qzeros, group_size):
+    return scales.new_empty((qweight.shape[0], qweight.shape[1] * 8))
+
+
+@torch.library.custom_op("vrl_hip::int4_gate_up_silu", mutates_args=())
+def int4_gate_up_silu(x: torch.Tensor, qweight_gu: torch.Tensor, scales_gu: torch.Tensor,
+                      qzeros_gu: torch.Tensor, group_size: int) -> torch.Tensor:
+    M, N2, K, dev = _check_call(x, qweight_gu, scales_gu, qzeros_gu, group_size)
+    if N2 % 2 != 0:
+        raise ValueError("gate||up operand needs an even number of rows")
+    inter = N2 // 2
+    lib = _lib.load()
+    y = torch.empty((M, inter), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.vrl_int4_gate_up_silu_bf16(x.data_ptr(), qweight_gu.data_ptr(), scales_gu.data_ptr(),
+                                            qzeros_gu.data_ptr(), y.data_ptr(), M, inter, K,
+                                            int(group_size), _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_gate_up_silu_bf16")
+    return y
+
+
+@int4_gate_up_silu.register_fake
+def _(x, qweight_gu, scales_gu, qzeros_gu, group_size):
+    return x.new_empty((x.shape[0], qweight_gu.shape[0] // 2))
+
+
+class GroupedGemv:
+    """Several independent int4 GEMVs enqueued as one kernel launch.
+
+    ``problems`` is a list of ``(x, qweight, scales, qzeros, group_size, fused)``
+    tuples; outputs are allocated once here and overwritten by every
+    :meth:`launch`.  The plan (pointer table) is validated and built on the host
+    by the library, copied to the device once, and stays valid while the tensors
+    captured here are alive and not reallocated.
+    """
+
+    MAX_ROWS = 16  # activation rows one record of the plan may carry
+
+    def __init__(self, problems):
+        if not problems:
+            raise ValueError("GroupedGemv needs at least one problem")
+        lib = _lib.load()
+        self._keep = []
+        self.outputs = []
+        dev = None
+        records = []
+        for x, qweight, scales, qzeros, group_size, fused in problems:
+            M, N, K, d = _check_call(x, qweight, scales, qzeros, group_size)
+            if dev is None:
+                dev = d
+            elif d != dev:
+                raise ValueError("all problems of a grouped launch must share one device")
+            if fused and N % 2 != 0:
+                raise ValueError("gate||up operand needs an even number of rows")
+            y = torch.empty((M, N // 2 if fused else N), dtype=torch.bfloat16, device=dev)
+            self._keep.append((x, qweight, scales, qzeros))
+            self.outputs.append(y)
+            # one record per slab of MAX_ROWS activation rows (row slices stay contiguous)
+            for m0 in range(0, M, self.MAX_ROWS):
+                m1 = min(M, m0 + self.MAX_ROWS)
+                records.append((x[m0:m1].data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                qzeros.data_ptr(), y[m0:m1].data_ptr(), m1 - m0, N, K,
+                                int(group_size), 1 if fused else 0))
+        n = len(records)
+        table = (_lib.Problem * n)()
+        for rec, vals in zip(table, records):
+            (rec.x, rec.qweight, rec.scales, rec.qzeros, rec.y,
+             rec.M, rec.N, rec.K, rec.G, rec.fused_gate_up) = vals
+        size = lib.vrl_int4_grouped_plan_size(n)
+        host = torch.empty(size, dtype=torch.uint8)
+        tiles = ctypes.c_int(0)
+        rc = lib.vrl_int4_grouped_plan_build(table, n, host.data_ptr(), size, ctypes.byref(tiles))
+        _lib.check(rc, "vrl_int4_grouped_plan_build")
+        self.device = dev
+        self.n_problems = n
+        self.total_tiles = int(tiles.value)
+        self.plan = host.to(dev)
+
+    def launch(self):
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            rc = lib.vrl_int4_gemv_grouped_bf16(self.plan.data_ptr(), self.n_problems,
+                                                self.total_tiles, _stream_handle(self.device))
+        _lib.check(rc, "vrl_int4_gemv_grouped_bf16")
+        return self.outputs

@@ -1,0 +1,162 @@
+"""Loader glue: swap a Janus-Pro style policy's decode linears for int4 modules.
+
+Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
+
+* ``policy.py:240-266``  ``JanusProPolicy._lm_trunk()`` returns the Hugging Face
+  ``LlamaModel`` whose ``layers[i].self_attn.{q,k,v,o}_proj`` and
+  ``layers[i].mlp.{gate,up,down}_proj`` are ``nn.Linear``.
+* ``policy.py:226-238``, ``:138-160``  ``_base().gen_head`` maps hidden states to
+  image-token logits.
+* ``policy.py:298-324``  LoRA: PEFT wraps target linears; the wrapper keeps the
+  frozen weight in ``base_layer`` and adds ``scaling * B(A(x))``.  Only
+  ``base_layer`` is replaced, so the adapter keeps working on top of int4.
+* ``builder.py:11-33``, ``:77-113`` and ``vrl/distributed/ray/rollout/worker.py:143-163``:
+  rollout workers build the policy from a ``RuntimeBuildSpec`` whose ``extra``
+  dict is the only channel for new scalar options; ``extra["int4"]`` carries
+  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true}``.
+
+Nothing here imports the reference; the policy is duck-typed.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Callable, Iterable
+
+from torch import nn
+
+from .linear import Int4Linear, Int4LlamaMLP
+
+ATTN_TARGETS = ("q_proj", "k_proj", "v_proj", "o_proj")
+MLP_TARGETS = ("gate_proj", "up_proj", "down_proj")
+DEFAULT_TARGETS = ATTN_TARGETS + MLP_TARGETS
+
+
+def _trunk(policy: Any) -> nn.Module:
+    if hasattr(policy, "_lm_trunk"):
+        return policy._lm_trunk()
+    if isinstance(policy, nn.Module) and hasattr(policy, "layers"):
+        return policy
+    raise TypeError("expected a policy exposing _lm_trunk() or a LlamaModel-like trunk with .layers")
+
+
+def _head_owner(policy: Any):
+    base = policy._base() if hasattr(policy, "_base") else policy
+    return base if hasattr(base, "gen_head") else None
+
+
+def _quantizable(linear: nn.Module, group_size: int) -> bool:
+    return isinstance(linear, nn.Linear) and linear.in_features % group_size == 0
+
+
+def _swap_linear(parent: nn.Module, name: str, group_size: int) -> bool:
+    """Replace ``parent.name`` (or its PEFT ``base_layer``) by an ``Int4Linear``."""
+    child = getattr(parent, name, None)
+    if child is None:
+        return False
+    if isinstance(child, Int4Linear):
+        return False
+    inner = getattr(child, "base_layer", None)
+    if inner is not None and not isinstance(child, nn.Linear):
+        # PEFT LoRA wrapper: keep the adapter, quantise the frozen base weight
+        if _quantizable(inner, group_size):
+            child.base_layer = Int4Linear.from_linear(inner, group_size)
+            return True
+        return False
+    if _quantizable(child, group_size):
+        setattr(parent, name, Int4Linear.from_linear(child, group_size))
+        return True
+    return False
+
+
+def _swap_all_linears(module: nn.Module, group_size: int) -> int:
+    n = 0
+    for name, child in list(module.named_children()):
+        if isinstance(child, nn.Linear):
+            n += int(_swap_linear(module, name, group_size))
+        else:
+            n += _swap_all_linears(child, group_size)
+    return n
+
+
+def apply_int4_to_policy(policy: Any, group_size: int = 128,
+                         targets: Iterable[str] = DEFAULT_TARGETS, fuse_mlp: bool = True,
+                         head: bool = True) -> dict:
+    """Quantise the decode linears of ``policy`` in place; returns a count summary.
+
+    ``fuse_mlp`` replaces a whole MLP block by :class:`Int4LlamaMLP` (gate||up with
+    the SiLU epilogue in one launch) when all three projections are targeted and
+    none of them carries a LoRA adapter.
+    """
+    targets = tuple(targets)
+    unknown = set(targets) - set(DEFAULT_TARGETS)
+    if unknown:
+        raise ValueError(f"unknown int4 targets {sorted(unknown)}; choose from {DEFAULT_TARGETS}")
+    trunk = _trunk(policy)
+    summary = {"linears": 0, "fused_mlps": 0, "head_linears": 0, "group_size": int(group_size)}
+    for layer in trunk.layers:
+        attn, mlp = getattr(layer, "self_attn", None), getattr(layer, "mlp", None)
+        if attn is not None:
+            for name in ATTN_TARGETS:
+                if name in targets:
+                    summary["linears"] += int(_swap_linear(attn, name, group_size))
+        if mlp is None:
+            continue
+        wants_all = all(n in targets for n in MLP_TARGETS)
+        plain = all(isinstance(getattr(mlp, n, None), nn.Linear) and
+                    _quantizable(getattr(mlp, n), group_size) and getattr(mlp, n).bias is None
+                    for n in MLP_TARGETS)
+        if fuse_mlp and wants_all and plain:
+            layer.mlp = Int4LlamaMLP(mlp, group_size)
+            summary["fused_mlps"] += 1
+            summary["linears"] += 3
+        else:
+            for name in MLP_TARGETS:
+                if name in targets:
+                    summary["linears"] += int(_swap_linear(mlp, name, group_size))
+    owner = _head_owner(policy)
+    if head and owner is not None:
+        if isinstance(owner.gen_head, nn.Linear):
+            summary["head_linears"] += int(_swap_linear(owner, "gen_head", group_size))
+        else:
+            summary["head_linears"] += _swap_all_linears(owner.gen_head, group_size)
+    return summary
+
+
+def int4_options_from_spec(spec: Any) -> dict | None:
+    """Read ``spec.extra["int4"]``; ``None`` when int4 is not requested.
+
+    Accepts ``True`` (defaults) or a dict of scalars/lists, the only kinds of
+    value the reference lets cross its process boundary.
+    """
+    extra = getattr(spec, "extra", None) or {}
+    opt = extra.get("int4")
+    if opt is None or opt is False:
+        return None
+    if opt is True:
+        opt = {}
+    if not isinstance(opt, dict):
+        raise TypeError('RuntimeBuildSpec.extra["int4"] must be true or a dict of options')
+    allowed = {"group_size", "targets", "fuse_mlp", "head"}
+    unknown = set(opt) - allowed
+    if unknown:
+        raise ValueError(f'unknown keys in extra["int4"]: {sorted(unknown)}')
+    return {"group_size": int(opt.get("group_size", 128)),
+            "targets": tuple(opt.get("targets", DEFAULT_TARGETS)),
+            "fuse_mlp": bool(opt.get("fuse_mlp", True)),
+            "head": bool(opt.get("head", True))}
+
+
+def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
+    """Wrap a family runtime builder (``build_janus_pro_runtime_bundle``-shaped).
+
+    Runs ``builder(spec)``, then quantises ``bundle.policy`` if the spec asks for
+    it, and records what was done in ``bundle.metadata["int4"]``.
+    """
+    bundle = builder(spec)
+    opt = int4_options_from_spec(spec)
+    if opt is not None:
+        summary = apply_int4_to_policy(bundle.policy, **opt)
+        meta = getattr(bundle, "metadata", None)
+        if isinstance(meta, dict):
+            meta["int4"] = summary
+    return bundle
