@@ -71,19 +71,6 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bias) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(bias));
-    return r;
-}
-
-// fp32  a.lo*b.lo + a.hi*b.hi + c  on bf16 pairs
-__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
-    float r;
-    asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-
 // Per-(row, group) dequant constants held by a lane.
 struct GroupConst {
     uint32_t s_lo;  // bf16 pair (s, 0)
@@ -101,15 +88,45 @@ __device__ __forceinline__ GroupConst make_group_const(uint32_t scale_bits, uint
 
 // One packed word -> 8 exactly rounded bf16 weights in the order
 // (w0,w4),(w1,w5),(w2,w6),(w3,w7): four dwords.
+//
+// One asm block on purpose.  On gfx90a and later the result of a DOT instruction
+// may not be read (or overwritten) by a different VALU instruction for three
+// wait states and the hardware does not interlock; the compiler cannot see
+// inside inline asm, so the order below keeps every v_cvt_pk at least three
+// instructions behind the v_dot2 it reads, and the trailing s_nop covers the
+// consumer of the last v_cvt_pk.
 __device__ __forceinline__ void dequant_word(uint32_t v, const GroupConst &g, uint32_t bias,
                                              uint32_t out[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint32_t p = and_or(i == 0 ? v : (v >> (4 * i)), PAIR_MASK, bias);
-        float lo = dot2_bf16(p, g.s_lo, g.c);
-        float hi = dot2_bf16(p, g.s_hi, g.c);
-        out[i] = pack_bf16_rne(lo, hi);
-    }
+    uint32_t p0, p1, p2, p3, d0, d1, d2, d3, d4, d5, d6, d7;
+    asm("v_and_or_b32 %[p0], %[v], %[mask], %[bias]\n\t"
+        "v_lshrrev_b32 %[p1], 4, %[v]\n\t"
+        "v_lshrrev_b32 %[p2], 8, %[v]\n\t"
+        "v_lshrrev_b32 %[p3], 12, %[v]\n\t"
+        "v_and_or_b32 %[p1], %[p1], %[mask], %[bias]\n\t"
+        "v_and_or_b32 %[p2], %[p2], %[mask], %[bias]\n\t"
+        "v_and_or_b32 %[p3], %[p3], %[mask], %[bias]\n\t"
+        "v_dot2_f32_bf16 %[d0], %[p0], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d1], %[p0], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d2], %[p1], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d3], %[p1], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d4], %[p2], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d5], %[p2], %[shi], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d6], %[p3], %[slo], %[c]\n\t"
+        "v_dot2_f32_bf16 %[d7], %[p3], %[shi], %[c]\n\t"
+        "v_cvt_pk_bf16_f32 %[d0], %[d0], %[d1]\n\t"
+        "v_cvt_pk_bf16_f32 %[d2], %[d2], %[d3]\n\t"
+        "v_cvt_pk_bf16_f32 %[d4], %[d4], %[d5]\n\t"
+        "v_cvt_pk_bf16_f32 %[d6], %[d6], %[d7]\n\t"
+        "s_nop 1"
+        : [p0] "=&v"(p0), [p1] "=&v"(p1), [p2] "=&v"(p2), [p3] "=&v"(p3), [d0] "=&v"(d0),
+          [d1] "=&v"(d1), [d2] "=&v"(d2), [d3] "=&v"(d3), [d4] "=&v"(d4), [d5] "=&v"(d5),
+          [d6] "=&v"(d6), [d7] "=&v"(d7)
+        : [v] "v"(v), [slo] "v"(g.s_lo), [shi] "v"(g.s_hi), [c] "v"(g.c), [mask] "s"(PAIR_MASK),
+          [bias] "v"(bias));
+    out[0] = d0;
+    out[1] = d2;
+    out[2] = d4;
+    out[3] = d6;
 }
 
 // -------------------------------------------------------------------------
