@@ -89,9 +89,11 @@ int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void
  * A plan is a flat byte blob built on the host, copied by the caller into
  * device memory once, and reused for every launch while the pointers stay
  * valid.  vrl_int4_grouped_plan_size() gives its size; vrl_int4_grouped_plan_build()
- * validates every problem against the preconditions above and fills a host
- * buffer; vrl_int4_gemv_grouped_bf16() takes the DEVICE copy plus the host
- * copy's header values (n_problems, total_tiles as returned by _build).
+ * validates every problem against the preconditions above (and, in addition,
+ * requires K % 128 == 0, G a power of two >= 32 and M <= 16 per problem),
+ * fills a host buffer and a small launch descriptor; vrl_int4_gemv_grouped_bf16()
+ * takes the DEVICE copy of the blob plus that descriptor.  The plan is built for
+ * the current device (its CU count sizes the launch).
  */
 typedef struct vrl_int4_problem {
     const void *x;
@@ -104,14 +106,22 @@ typedef struct vrl_int4_problem {
     int32_t reserved[3];
 } vrl_int4_problem;
 
+typedef struct vrl_int4_plan_info {
+    int32_t n_problems;    /* records in the blob */
+    int32_t total_tiles;   /* 16-column output tiles over all problems */
+    int32_t grid;          /* workgroups of the launch */
+    int32_t block_threads; /* threads per workgroup */
+    int32_t lds_bytes;     /* dynamic LDS per workgroup */
+    int32_t reserved[3];
+} vrl_int4_plan_info;
+
 size_t vrl_int4_grouped_plan_size(int n_problems);
 
-/* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems));
- * *total_tiles receives the number of work tiles the launch will walk. */
+/* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems)) and *info. */
 int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems,
-                                void *plan_host, size_t plan_bytes, int *total_tiles);
+                                void *plan_host, size_t plan_bytes, vrl_int4_plan_info *info);
 
-int vrl_int4_gemv_grouped_bf16(const void *plan_dev, int n_problems, int total_tiles,
+int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *info,
                                void *hip_stream);
 
 #ifdef __cplusplus

@@ -90,20 +90,32 @@ def test_grouped_plan_validation(lib):
     size = lib.vrl_int4_grouped_plan_size(2)
     assert size >= 2 * ctypes.sizeof(_lib.Problem)
     probs = (_lib.Problem * 2)()
-    for rec, n in zip(probs, (64, 96)):
+    for rec, n in zip(probs, (64, 100)):
         rec.x = rec.qweight = rec.scales = rec.qzeros = rec.y = p
         rec.M, rec.N, rec.K, rec.G = 1, n, 256, 128
     plan = ctypes.create_string_buffer(size)
-    tiles = ctypes.c_int(-1)
-    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(tiles)) == 0
-    assert tiles.value == 1 + 2   # 64-row tiles: ceil(64/64) + ceil(96/64)
-    # undersized buffer, bad shape inside the list, null list
-    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size - 1, ctypes.byref(tiles)) == 1004
+    info = _lib.PlanInfo()
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(info)) == 0
+    assert info.n_problems == 2
+    assert info.total_tiles == 4 + 7        # 16-column tiles: 64/16 and ceil(100/16)
+    assert 1 <= info.grid <= info.total_tiles and info.block_threads % 64 == 0
+    assert info.lds_bytes >= 1 * (256 + 8) * 2
+    # the per-workgroup tile ranges stored after the records cover every tile exactly once
+    import struct
+    rec_bytes = (size - 16 - 4 * 4097) // 2
+    begins = struct.unpack_from(f"{info.grid + 1}i", plan.raw, 16 + 2 * rec_bytes)
+    assert begins[0] == 0 and begins[-1] == info.total_tiles
+    assert all(a <= b for a, b in zip(begins, begins[1:]))
+    # undersized buffer, bad shape inside the list, shapes only the generic kernel takes, nulls
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size - 1, ctypes.byref(info)) == 1004
     probs[1].K = 100
-    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(tiles)) == 1001
-    assert lib.vrl_int4_grouped_plan_build(None, 2, plan, size, ctypes.byref(tiles)) == 1003
-    assert lib.vrl_int4_gemv_grouped_bf16(None, 2, 3, None) == 1003
-    assert lib.vrl_int4_gemv_grouped_bf16(p, 0, 3, None) == 1004
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(info)) == 1001
+    probs[1].K, probs[1].G = 192, 24
+    assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size, ctypes.byref(info)) == 1001
+    assert lib.vrl_int4_grouped_plan_build(None, 2, plan, size, ctypes.byref(info)) == 1003
+    assert lib.vrl_int4_gemv_grouped_bf16(None, ctypes.byref(info), None) == 1003
+    bad = _lib.PlanInfo()
+    assert lib.vrl_int4_gemv_grouped_bf16(p, ctypes.byref(bad), None) == 1004
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

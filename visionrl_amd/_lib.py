@@ -49,6 +49,19 @@ class Problem(ctypes.Structure):
     ]
 
 
+class PlanInfo(ctypes.Structure):
+    """Mirror of ``vrl_int4_plan_info``."""
+
+    _fields_ = [
+        ("n_problems", ctypes.c_int32),
+        ("total_tiles", ctypes.c_int32),
+        ("grid", ctypes.c_int32),
+        ("block_threads", ctypes.c_int32),
+        ("lds_bytes", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 3),
+    ]
+
+
 _lock = threading.Lock()
 _lib = None
 
@@ -69,9 +82,9 @@ def _bind(lib):
     lib.vrl_int4_grouped_plan_size.argtypes = [ci]
     lib.vrl_int4_grouped_plan_build.restype = ci
     lib.vrl_int4_grouped_plan_build.argtypes = [
-        ctypes.POINTER(Problem), ci, vp, ctypes.c_size_t, ctypes.POINTER(ci)]
+        ctypes.POINTER(Problem), ci, vp, ctypes.c_size_t, ctypes.POINTER(PlanInfo)]
     lib.vrl_int4_gemv_grouped_bf16.restype = ci
-    lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ci, ci, vp]
+    lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
 
 
 def load():

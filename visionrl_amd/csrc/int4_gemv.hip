@@ -427,22 +427,209 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_tile_kernel(DevProblem p) {
     tile_body<R, MB, WPB>(p, blockIdx.x, smem);
 }
 
-// Grouped launch: blocks walk the tile list with a grid stride; every wave of a
-// block sees the same uniform loop bounds, so all of them reach the end.
-template <int R, int WPB>
-__global__ __launch_bounds__(WPB *WAVE) void gemv_grouped_kernel(const DevProblem *__restrict__ plan,
-                                                                 int n_problems, int total_tiles) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    for (int t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-        // largest i with plan[i].tile_begin <= t
-        int lo = 0, hi = n_problems - 1;
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (plan[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
+// -------------------------------------------------------------------------
+// stream GEMV (grouped launches): a wave owns 16 weight rows for all of K
+// -------------------------------------------------------------------------
+// The tile list of a plan (16 output columns per tile, all problems back to
+// back) is cut into one contiguous range per workgroup, balanced by bytes.  A
+// workgroup walks its range problem by problem: it stages that problem's
+// activations in LDS once, then each wave streams whole tiles - no K split, so
+// no partial sums to meet - keeping STREAM_DEPTH 128-k chunks of its 16 rows in
+// flight (non-temporal global_load_dwordx4: the weights are read exactly once).
+constexpr int STREAM_WPB = 4;
+constexpr int STREAM_DEPTH = 4;
+
+template <int RS>
+struct Slot {
+    u32x4_t w[RS];
+    uint32_t sbits[RS];
+    uint32_t zword[RS];
+};
+
+__device__ __forceinline__ void stage_x(const DevProblem &p, int kbase, int kext, uint16_t *xs,
+                                        int xstride, int nthreads) {
+    const int words_per_row = kext >> 3;  // 16-byte pieces
+    const int total = p.M * words_per_row;
+    for (int idx = threadIdx.x; idx < total; idx += nthreads) {
+        const int m = idx / words_per_row;
+        const int j = idx - m * words_per_row;
+        const u32x4_t d = *reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + kbase + (j << 3));
+        u32x4_t o;
+        o[0] = (d[0] & 0xFFFFu) | (d[2] << 16);      // x0, x4
+        o[1] = (d[0] >> 16) | (d[2] & 0xFFFF0000u);  // x1, x5
+        o[2] = (d[1] & 0xFFFFu) | (d[3] << 16);      // x2, x6
+        o[3] = (d[1] >> 16) | (d[3] & 0xFFFF0000u);  // x3, x7
+        *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = o;
+    }
+}
+
+// acc += x[:, kbase:kbase+kext] . W[tile rows, kbase:kbase+kext]^T for this wave's tile
+template <int MB, bool FUSED>
+__device__ __forceinline__ void stream_rows(const DevProblem &p, int tile_local, const uint16_t *xs,
+                                            int xstride, int kbase, int kext, int gshift,
+                                            f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int lc = lane & 15;
+    const int kq = lane >> 4;
+    const int kwords = p.K >> 3;
+    const int groups = p.K >> gshift;
+    const int zwords = (groups + 7) >> 3;
+    const int out_cols = FUSED ? p.N / 2 : p.N;
+
+    const uint32_t *wp[RS];
+    const uint16_t *sp[RS];
+    const uint32_t *zp[RS];
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        const long row = (long)r * out_cols + min(tile_local * 16 + lc, out_cols - 1);
+        wp[r] = p.qweight + row * kwords + (kbase >> 3) + 4 * kq;
+        sp[r] = p.scales + row * groups;
+        zp[r] = p.qzeros + row * zwords;
+    }
+    const int nch = kext >> 7;
+    const uint32_t bias = PAIR_BIAS;
+    Slot<RS> ring[STREAM_DEPTH];
+
+    auto issue = [&](Slot<RS> &s, int c) {
+        const int g = (kbase + c * KCHUNK + 32 * kq) >> gshift;
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            s.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(wp[r] + c * 16));
+            s.sbits[r] = sp[r][g];
+            s.zword[r] = zp[r][g >> 3];
         }
-        const DevProblem p = plan[lo];
-        if (t != blockIdx.x) __syncthreads();  // LDS of the previous tile is free again
-        tile_body<R, 1, WPB>(p, t - p.tile_begin, smem);
+    };
+    auto compute = [&](const Slot<RS> &s, int c) {
+        const int g = (kbase + c * KCHUNK + 32 * kq) >> gshift;
+        const int kloc = c * KCHUNK + 32 * kq;
+        bf16x8_t xa[4][MB];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const int m = min(16 * b + lc, p.M - 1);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * t);
+                xa[t][b] = __builtin_bit_cast(bf16x8_t, raw);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            const uint32_t z = (s.zword[r] >> (4 * (g & 7))) & 0xFu;
+            const GroupConst gc = make_group_const(s.sbits[r], z);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                uint32_t wb[4];
+                dequant_word(s.w[r][t], gc, bias, wb);
+                const u32x4_t wv = {wb[0], wb[1], wb[2], wb[3]};
+                const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+                    acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[t][b], bop, acc[r][b], 0, 0, 0);
+            }
+        }
+    };
+
+#pragma unroll
+    for (int d = 0; d < STREAM_DEPTH; ++d)
+        if (d < nch) issue(ring[d], d);
+    for (int c0 = 0; c0 < nch; c0 += STREAM_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < STREAM_DEPTH; ++d) {
+            if (c0 + d < nch) {
+                compute(ring[d], c0 + d);
+                if (c0 + d + STREAM_DEPTH < nch) issue(ring[d], c0 + d + STREAM_DEPTH);
+            }
+        }
+    }
+}
+
+template <int MB, bool FUSED>
+__device__ __forceinline__ void store_tile(const DevProblem &p, int tile_local,
+                                           const f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int out_cols = FUSED ? p.N / 2 : p.N;
+    const int col = tile_local * 16 + (lane & 15);
+    if (col >= out_cols) return;
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = 16 * b + 4 * (lane >> 4) + i;
+            if (m < p.M) {
+                float v = acc[0][b][i];
+                if (FUSED) v = (v / (1.0f + __expf(-v))) * acc[FUSED ? 1 : 0][b][i];
+                p.y[(long)m * out_cols + col] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+            }
+        }
+}
+
+// tiles [t0, t1) of problem p (local tile indices); all waves of the block call this together
+template <int MB, bool FUSED, int WPB>
+__device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int wave = threadIdx.x >> 6;
+    const int gshift = __builtin_ctz((unsigned)p.G);
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int xstride = p.kc + XPAD;
+    if (p.kc >= p.K) {
+        __syncthreads();  // readers of whatever was staged before are done
+        stage_x(p, 0, p.K, xs, xstride, WPB * WAVE);
+        __syncthreads();
+        for (int tile = t0 + wave; tile < t1; tile += WPB) {
+            f32x4_t acc[RS][MB];
+#pragma unroll
+            for (int r = 0; r < RS; ++r)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            stream_rows<MB, FUSED>(p, tile, xs, xstride, 0, p.K, gshift, acc);
+            store_tile<MB, FUSED>(p, tile, acc);
+        }
+    } else {
+        // activations do not fit: rounds of one tile per wave, K walked in staged passes
+        for (int round = t0; round < t1; round += WPB) {
+            const int tile = round + wave;
+            const bool active = tile < t1;
+            f32x4_t acc[RS][MB];
+#pragma unroll
+            for (int r = 0; r < RS; ++r)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int kbase = 0; kbase < p.K; kbase += p.kc) {
+                const int kext = min(p.kc, p.K - kbase);
+                __syncthreads();
+                stage_x(p, kbase, kext, xs, xstride, WPB * WAVE);
+                __syncthreads();
+                if (active) stream_rows<MB, FUSED>(p, tile, xs, xstride, kbase, kext, gshift, acc);
+            }
+            if (active) store_tile<MB, FUSED>(p, tile, acc);
+        }
+    }
+}
+
+template <int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
+                                                                const int32_t *__restrict__ block_begin,
+                                                                int n_problems) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    int t = block_begin[blockIdx.x];
+    const int t_end = block_begin[blockIdx.x + 1];
+    if (t >= t_end) return;  // block-uniform
+    // largest i with plan[i].tile_begin <= t
+    int lo = 0, hi = n_problems - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (plan[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
+    }
+    for (int pi = lo; t < t_end && pi < n_problems; ++pi) {
+        const DevProblem p = plan[pi];
+        const int out_cols = p.fused ? p.N / 2 : p.N;
+        const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
+        if (p.fused)
+            stream_segment<1, true, WPB>(p, t - p.tile_begin, seg_end - p.tile_begin, smem);
+        else
+            stream_segment<1, false, WPB>(p, t - p.tile_begin, seg_end - p.tile_begin, smem);
+        t = seg_end;
     }
 }
 
@@ -450,10 +637,12 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_grouped_kernel(const DevProble
 // host side
 // -------------------------------------------------------------------------
 constexpr int TILE_WPB = 8;
-constexpr int GROUPED_R = 4;
-constexpr int MAX_TILE_M = 16;                  // activation rows one tile-kernel launch takes
-constexpr size_t LDS_X_BUDGET = 40 * 1024;      // staged activations per workgroup
-constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // staged extents shorter than K are multiples of this
+constexpr int MAX_TILE_M = 16;                  // activation rows one record / launch takes
+constexpr size_t LDS_X_BUDGET = 40 * 1024;      // split kernel: staged activations per workgroup
+constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // split kernel: shorter staged extents are multiples of this
+constexpr size_t STREAM_X_SINGLE = 72 * 1024;   // stream kernel: all of K staged if it fits this
+constexpr size_t STREAM_X_PASS = 36 * 1024;     // stream kernel: staged bytes per pass otherwise
+constexpr size_t LDS_PER_CU = 160 * 1024;
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -468,17 +657,29 @@ int check_problem(const void *x, const void *qw, const void *sc, const void *qz,
     return VRL_INT4_OK;
 }
 
+bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+// shapes the MFMA kernels take; everything else goes to the generic kernel
 bool tile_path_ok(const DevProblem &p) {
-    return p.K % KCHUNK == 0 && p.G % 32 == 0 && p.M <= MAX_TILE_M;
+    return p.K % KCHUNK == 0 && p.G % 32 == 0 && pow2(p.G) && p.M <= MAX_TILE_M;
 }
 
-// k extent of x staged per pass: all of K when M rows of it fit the budget,
+// split kernel: k extent of x staged per pass, all of K when M rows of it fit the budget,
 // else the largest multiple of STAGE_STEP that does (M <= 16 always fits one step)
 int staged_k(int M, int K) {
     if ((size_t)M * (K + XPAD) * 2 <= LDS_X_BUDGET) return K;
     long kc = (long)(LDS_X_BUDGET / ((size_t)M * 2)) - XPAD;
     kc -= kc % STAGE_STEP;
     if (kc < STAGE_STEP) kc = STAGE_STEP;
+    return (int)(kc < K ? kc : K);
+}
+
+// stream kernel: all of K if it fits, else passes that are multiples of KCHUNK
+int stream_staged_k(int M, int K) {
+    if ((size_t)M * (K + XPAD) * 2 <= STREAM_X_SINGLE) return K;
+    long kc = (long)(STREAM_X_PASS / ((size_t)M * 2)) - XPAD;
+    kc -= kc % KCHUNK;
+    if (kc < KCHUNK) kc = KCHUNK;
     return (int)(kc < K ? kc : K);
 }
 
@@ -555,14 +756,21 @@ int run_rows(const void *x, const void *qw, const void *sc, const void *qz, void
     return VRL_INT4_OK;
 }
 
+// Plan blob: [PlanHeader][DevProblem x n_records][int32 block_begin x (grid + 1)]
 struct PlanHeader {
     uint32_t magic;
-    int32_t n_problems;
+    int32_t n_records;
     int32_t total_tiles;
-    int32_t max_smem;
+    int32_t grid;
 };
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
+constexpr int MAX_PLAN_GRID = 4096;
+
+size_t plan_bytes_for(int n_records) {
+    return sizeof(PlanHeader) + (size_t)n_records * sizeof(DevProblem) +
+           (size_t)(MAX_PLAN_GRID + 1) * sizeof(int32_t);
+}
 
 }  // namespace
 
@@ -612,19 +820,20 @@ int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *q
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {
     if (n_problems < 1) return 0;
-    return sizeof(PlanHeader) + (size_t)n_problems * sizeof(DevProblem);
+    return plan_bytes_for(n_problems);
 }
 
 int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems, void *plan_host,
-                                size_t plan_bytes, int *total_tiles) {
-    if (!problems || !plan_host || !total_tiles) return VRL_INT4_ENULL;
+                                size_t plan_bytes, vrl_int4_plan_info *info) {
+    if (!problems || !plan_host || !info) return VRL_INT4_ENULL;
     if (n_problems < 1 || plan_bytes < vrl_int4_grouped_plan_size(n_problems)) return VRL_INT4_EPLAN;
-    PlanHeader hdr;
-    hdr.magic = PLAN_MAGIC;
-    hdr.n_problems = n_problems;
-    hdr.max_smem = 0;
-    DevProblem *recs = reinterpret_cast<DevProblem *>(static_cast<uint8_t *>(plan_host) + sizeof hdr);
+    uint8_t *base = static_cast<uint8_t *>(plan_host);
+    DevProblem *recs = reinterpret_cast<DevProblem *>(base + sizeof(PlanHeader));
+    int32_t *block_begin = reinterpret_cast<int32_t *>(recs + n_problems);
+
     long tiles = 0;
+    double total_cost = 0.0;
+    size_t smem = 0;
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
         int rc = check_problem(q.x, q.qweight, q.scales, q.qzeros, q.y, q.M, q.N, q.K, q.G);
@@ -639,37 +848,85 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         p.y = static_cast<uint16_t *>(q.y);
         p.M = q.M; p.N = q.N; p.K = q.K; p.G = q.G;
         p.fused = q.fused_gate_up ? 1 : 0;
-        if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take tile-path shapes only
-        p.kc = staged_k(p.M, p.K);
+        if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take MFMA-path shapes only
+        p.kc = stream_staged_k(p.M, p.K);
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
-        const int cols_per_tile = p.fused ? 16 * (GROUPED_R / 2) : 16 * GROUPED_R;
-        tiles += (out_cols + cols_per_tile - 1) / cols_per_tile;
+        const long nt = (out_cols + 15) / 16;
+        tiles += nt;
         if (tiles >= (1L << 30)) return VRL_INT4_ESHAPE;
-        const size_t smem = tile_smem_bytes<GROUPED_R, 1>(p.M, p.kc);
-        if ((int)smem > hdr.max_smem) hdr.max_smem = (int)smem;
+        total_cost += (double)nt * ((double)p.K * (p.fused ? 2 : 1) + 512.0);
+        const size_t need = (size_t)p.M * (p.kc + XPAD) * 2;
+        if (need > smem) smem = need;
         recs[i] = p;
     }
+
+    // one contiguous tile range per workgroup, balanced by streamed bytes
+    int per_cu = (int)(LDS_PER_CU / (smem ? smem : 1));
+    if (per_cu > 4) per_cu = 4;
+    if (per_cu < 1) per_cu = 1;
+    long grid = (long)device_cu_count() * per_cu;
+    if (grid > MAX_PLAN_GRID) grid = MAX_PLAN_GRID;
+    const long max_useful = (tiles + STREAM_WPB - 1) / STREAM_WPB;
+    if (grid > max_useful) grid = max_useful;
+    {
+        int b = 0;
+        double acc_cost = 0.0;
+        block_begin[0] = 0;
+        for (int i = 0; i < n_problems; ++i) {
+            const DevProblem &p = recs[i];
+            const int out_cols = p.fused ? p.N / 2 : p.N;
+            const int nt = (out_cols + 15) / 16;
+            const double c = (double)p.K * (p.fused ? 2 : 1) + 512.0;
+            for (int t = 0; t < nt; ++t) {
+                // tile (p.tile_begin + t) starts block b+1 once the blocks so far hold their share
+                while (b + 1 < grid && acc_cost >= total_cost * (b + 1) / (double)grid) {
+                    ++b;
+                    block_begin[b] = p.tile_begin + t;
+                }
+                acc_cost += c;
+            }
+        }
+        while (b < grid) {
+            ++b;
+            block_begin[b] = (int)tiles;
+        }
+    }
+
+    PlanHeader hdr;
+    hdr.magic = PLAN_MAGIC;
+    hdr.n_records = n_problems;
     hdr.total_tiles = (int)tiles;
+    hdr.grid = (int)grid;
     memcpy(plan_host, &hdr, sizeof hdr);
-    *total_tiles = (int)tiles;
+    memset(info, 0, sizeof *info);
+    info->n_problems = n_problems;
+    info->total_tiles = (int)tiles;
+    info->grid = (int)grid;
+    info->block_threads = STREAM_WPB * WAVE;
+    info->lds_bytes = (int)smem;
     return VRL_INT4_OK;
 }
 
-int vrl_int4_gemv_grouped_bf16(const void *plan_dev, int n_problems, int total_tiles,
+int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *info,
                                void *hip_stream) {
-    if (!plan_dev) return VRL_INT4_ENULL;
-    if (n_problems < 1 || total_tiles < 1 || !aligned16(plan_dev)) return VRL_INT4_EPLAN;
-    const DevProblem *recs =
-        reinterpret_cast<const DevProblem *>(static_cast<const uint8_t *>(plan_dev) + sizeof(PlanHeader));
-    // LDS: the most any record can need (staged activations never exceed the budget)
-    size_t smem = tile_smem_bytes<GROUPED_R, 1>(1, 0);
-    if (LDS_X_BUDGET > smem) smem = LDS_X_BUDGET;
-    int blocks = device_cu_count() * 2;
-    if (blocks > total_tiles) blocks = total_tiles;
-    hipLaunchKernelGGL((gemv_grouped_kernel<GROUPED_R, TILE_WPB>), dim3(blocks),
-                       dim3(TILE_WPB * WAVE), smem, reinterpret_cast<hipStream_t>(hip_stream), recs,
-                       n_problems, total_tiles);
+    if (!plan_dev || !info) return VRL_INT4_ENULL;
+    if (info->n_problems < 1 || info->total_tiles < 1 || info->grid < 1 ||
+        info->grid > MAX_PLAN_GRID || info->block_threads != STREAM_WPB * WAVE ||
+        info->lds_bytes < 0 || (size_t)info->lds_bytes > LDS_PER_CU || !aligned16(plan_dev))
+        return VRL_INT4_EPLAN;
+    const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
+    const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + sizeof(PlanHeader));
+    const int32_t *block_begin = reinterpret_cast<const int32_t *>(recs + info->n_problems);
+    if (info->lds_bytes > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&gemv_stream_kernel<STREAM_WPB>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL((gemv_stream_kernel<STREAM_WPB>), dim3(info->grid), dim3(STREAM_WPB * WAVE),
+                       (size_t)info->lds_bytes, reinterpret_cast<hipStream_t>(hip_stream), recs,
+                       block_begin, info->n_problems);
     return (int)hipGetLastError();
 }
 

@@ -162,18 +162,18 @@ class GroupedGemv:
              rec.M, rec.N, rec.K, rec.G, rec.fused_gate_up) = vals
         size = lib.vrl_int4_grouped_plan_size(n)
         host = torch.empty(size, dtype=torch.uint8)
-        tiles = ctypes.c_int(0)
-        rc = lib.vrl_int4_grouped_plan_build(table, n, host.data_ptr(), size, ctypes.byref(tiles))
+        self.info = _lib.PlanInfo()
+        with torch.cuda.device(dev):  # the plan is sized for this device's CU count
+            rc = lib.vrl_int4_grouped_plan_build(table, n, host.data_ptr(), size,
+                                                 ctypes.byref(self.info))
         _lib.check(rc, "vrl_int4_grouped_plan_build")
         self.device = dev
-        self.n_problems = n
-        self.total_tiles = int(tiles.value)
         self.plan = host.to(dev)
 
     def launch(self):
         lib = _lib.load()
         with torch.cuda.device(self.device):
-            rc = lib.vrl_int4_gemv_grouped_bf16(self.plan.data_ptr(), self.n_problems,
-                                                self.total_tiles, _stream_handle(self.device))
+            rc = lib.vrl_int4_gemv_grouped_bf16(self.plan.data_ptr(), ctypes.byref(self.info),
+                                                _stream_handle(self.device))
         _lib.check(rc, "vrl_int4_gemv_grouped_bf16")
         return self.outputs
