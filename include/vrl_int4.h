@@ -81,6 +81,21 @@ int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void
                                void *hip_stream);
 
 /*
+ * One-time repack of a canonical operand triple (group size 128) into the
+ * MFMA-shaped blob the grouped launch streams fastest: every wave load is one
+ * contiguous KiB and the matrix cores do the scale/zero arithmetic.  Loader
+ * glue: runs once per weight after the policy is built (the reference builds
+ * its policy at vrl/models/families/janus_pro/builder.py:11-33).
+ * vrl_int4_prepacked_bytes() is the blob size (0 if the shape has no prepacked
+ * form: G != 128 or K % 128 != 0); the blob needs 16-byte alignment.  The
+ * arithmetic contract is unchanged: the weights a kernel rebuilds from the blob
+ * are bit for bit the canonical dequantised tile.
+ */
+size_t vrl_int4_prepacked_bytes(int N, int K, int G);
+int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros, void *packed,
+                     int N, int K, int G, void *hip_stream);
+
+/*
  * Grouped launch: several independent GEMVs (for example q/k/v of one layer, or
  * a whole decode step's weight set when the caller streams them back to back)
  * in ONE kernel launch, so small matrices share the machine instead of paying
@@ -90,7 +105,8 @@ int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void
  * device memory once, and reused for every launch while the pointers stay
  * valid.  vrl_int4_grouped_plan_size() gives its size; vrl_int4_grouped_plan_build()
  * validates every problem against the preconditions above (and, in addition,
- * requires K % 128 == 0, G a power of two >= 32 and M <= 16 per problem),
+ * requires K % 128 == 0, G a power of two >= 32 and M <= 16 per problem; a
+ * prepacked problem needs G == 128 and, if fused, N/2 a multiple of 16),
  * fills a host buffer and a small launch descriptor; vrl_int4_gemv_grouped_bf16()
  * takes the DEVICE copy of the blob plus that descriptor.  The plan is built for
  * the current device (its CU count sizes the launch).
@@ -103,7 +119,8 @@ typedef struct vrl_int4_problem {
     void *y;
     int32_t M, N, K, G;
     int32_t fused_gate_up; /* 0: y[M,N]; 1: rows are gate||up, y[M,N/2] with the SiLU epilogue */
-    int32_t reserved[3];
+    int32_t prepacked;     /* 1: qweight is a blob made by vrl_int4_prepack(); scales/qzeros unused */
+    int32_t reserved[2];
 } vrl_int4_problem;
 
 typedef struct vrl_int4_plan_info {
@@ -112,7 +129,8 @@ typedef struct vrl_int4_plan_info {
     int32_t grid;          /* workgroups of the launch */
     int32_t block_threads; /* threads per workgroup */
     int32_t lds_bytes;     /* dynamic LDS per workgroup */
-    int32_t reserved[3];
+    int32_t variant;       /* which record kinds the plan holds (selects the kernel build) */
+    int32_t reserved[2];
 } vrl_int4_plan_info;
 
 size_t vrl_int4_grouped_plan_size(int n_problems);

@@ -84,6 +84,19 @@ def test_null_and_alignment_are_reported(lib):
     assert lib.vrl_int4_gate_up_silu_bf16(p, p, p, None, p, 1, 8, 128, 128, None) == 1003
 
 
+def test_prepacked_size_and_validation(lib):
+    keep, p = buf(4096)
+    # per 16-row tile: ceil(nsc/4) KiB of scale/zero words + nsc * 4 KiB of weights, nsc = ceil(K/512)
+    assert lib.vrl_int4_prepacked_bytes(2048, 2048, 128) == 128 * (1024 + 4 * 4096)
+    assert lib.vrl_int4_prepacked_bytes(2048, 5632, 128) == 128 * (3 * 1024 + 11 * 4096)
+    assert lib.vrl_int4_prepacked_bytes(17, 128, 128) == 2 * (1024 + 4096)
+    assert lib.vrl_int4_prepacked_bytes(16, 256, 64) == 0
+    assert lib.vrl_int4_prepacked_bytes(16, 200, 128) == 0
+    assert lib.vrl_int4_prepack(p, p, p, None, 16, 128, 128, None) == 1003
+    assert lib.vrl_int4_prepack(p, p, p, p + 4, 16, 128, 128, None) == 1002
+    assert lib.vrl_int4_prepack(p, p, p, p, 16, 256, 64, None) == 1001
+
+
 def test_grouped_plan_validation(lib):
     keep, p = buf(4096)
     assert lib.vrl_int4_grouped_plan_size(0) == 0

@@ -274,6 +274,127 @@ def test_grouped_launch_matches_single_launches(ops_mod):
             assert (diff <= ulp).all()
 
 
+# ------------------------------------------------------------------ prepacked weights
+PP_SHAPES = [
+    # M, K, N, fused
+    (1, 2048, 2048, False), (1, 5632, 2048, False), (1, 2048, 5632, False),
+    (1, 128, 16, False),        # K padded from 128 to 512
+    (3, 640, 50, False),        # ragged N and K
+    (16, 2048, 256, False), (16, 5632, 64, False),   # the second needs staged passes
+    (7, 11008, 96, False),      # 21.5 super-chunks
+    (20, 1024, 48, False),      # two slabs of activation rows
+    (1, 2048, 2 * 5632, True), (8, 4096, 2 * 704, True), (16, 1024, 2 * 48, True),
+]
+
+
+def run_grouped(ops_mod, problems):
+    grouped = ops_mod.GroupedGemv(problems)
+    outs = grouped.launch()
+    torch.cuda.synchronize()
+    return grouped, outs
+
+
+@pytest.mark.parametrize("M,K,N,fused", PP_SHAPES)
+def test_prepacked_grouped_parity(ops_mod, M, K, N, fused):
+    say("prepacked", M, K, N, fused)
+    G = 128
+    ops = o.make_operands(6000 + M + K + N, M, K, N, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    _, (y,) = run_grouped(ops_mod, [(d["x"], pw, fused)])
+    if not fused:
+        assert_gemv_close(bf16_to_bits(y), ops, G, f"prepacked M{M} K{K} N{N}")
+        return
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    ref = o.gate_up_silu_f64(*args)
+    ref_op = o.bf16_bits_to_f32(o.gate_up_silu_bf16(*args)).astype(np.float64)
+    got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
+    assert got.shape == ref.shape
+    # against the float64 truth: bf16 tolerance plus two ulps for the fp32 epilogue of near-cancelling sums
+    tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
+    assert (np.abs(got - ref) <= tol).all()
+    assert (np.abs(got - ref_op) <= tol).all()
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 512, 32), (4, 1024, 48), (16, 640, 16)])
+def test_prepacked_one_hot_is_the_exact_weight_column(ops_mod, M, K, N):
+    """The matrix-core dequant of the prepacked path reproduces the canonical tile bit for bit."""
+    say("prepacked one-hot", M, K, N)
+    G = 128
+    ops = o.make_operands(7000 + K, M, K, N, G, "loguniform")
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    for k0 in sorted(set([0, 1, 3, 4, 7, 8, 31, 32, 127, 128, 129, K // 2 + 5, K - 9, K - 1])):
+        x = np.zeros((M, K), dtype=np.float32)
+        for m in range(M):
+            x[m, (k0 + 29 * m) % K] = 1.0
+        xd = bits_to_bf16(o.f32_to_bf16_bits(x), DEV)
+        _, (y,) = run_grouped(ops_mod, [(xd, pw, False)])
+        y = bf16_to_bits(y)
+        for m in range(M):
+            want = w[:, (k0 + 29 * m) % K]
+            same = (y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)
+            assert same.all(), (k0, m)
+
+
+def test_prepacked_every_q_z_pair(ops_mod):
+    """All 256 (q, z) pairs x every bf16 mantissa at three exponents through the 4x4x4 dequant."""
+    say("prepacked exhaustive one-hot")
+    G, K = 128, 128
+    mant = np.arange(128, dtype=np.uint16)
+    scales = np.concatenate([(e << 7) | mant for e in (0x60, 0x78, 0x7C)]).astype(np.uint16)
+    scales = np.concatenate([scales, scales[:128] | 0x8000])
+    rows = [(int(sb), z) for sb in scales for z in range(16)]
+    N = len(rows)
+    q = np.tile(np.arange(16, dtype=np.uint8), (N, K // 16))
+    z = np.array([r[1] for r in rows], dtype=np.uint8)[:, None]
+    sb = np.array([r[0] for r in rows], dtype=np.uint16)[:, None]
+    ops = {"qweight": o.pack_nibbles(q), "scales_bits": sb, "qzeros": o.pack_nibbles(z)}
+    w = o.dequant_bf16(ops["qweight"], sb, ops["qzeros"], G)
+    x = np.zeros((16, K), dtype=np.float32)
+    for m in range(16):
+        x[m, 16 * (m % 8) + m] = 1.0      # activation row m selects a k with q = m
+    pw = ops_mod.int4_prepack(torch.from_numpy(ops["qweight"]).to(DEV), bits_to_bf16(sb, DEV),
+                              torch.from_numpy(ops["qzeros"]).to(DEV), G)
+    _, (y,) = run_grouped(ops_mod, [(bits_to_bf16(o.f32_to_bf16_bits(x), DEV), pw, False)])
+    y = bf16_to_bits(y)
+    for m in range(16):
+        want = w[:, 16 * (m % 8) + m]
+        same = (y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)
+        assert same.all(), m
+
+
+def test_prepacked_and_canonical_records_in_one_plan(ops_mod):
+    say("prepacked mixed plan")
+    G = 128
+    problems, checks = [], []
+    for i, (M, K, N, pp) in enumerate([(1, 2048, 2048, True), (1, 2048, 2048, False), (2, 5632, 512, True),
+                                       (1, 2048, 100, False)]):
+        ops = o.make_operands(8000 + i, M, K, N, G)
+        d = to_device(ops, DEV)
+        if pp:
+            problems.append((d["x"], ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G), False))
+        else:
+            problems.append((d["x"], d["qweight"], d["scales"], d["qzeros"], G, False))
+        checks.append(ops)
+    grouped, outs = run_grouped(ops_mod, problems)
+    for y, ops in zip(outs, checks):
+        assert_gemv_close(bf16_to_bits(y), ops, G, "mixed plan")
+    first = [y.clone() for y in outs]
+    grouped.launch()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(first, grouped.outputs))
+
+
+def test_prepack_rejects_other_group_sizes(ops_mod):
+    ops = o.make_operands(11, 1, 256, 16, 64)
+    d = to_device(ops, DEV)
+    assert not ops_mod.PrepackedWeight.supported(16, 256, 64)
+    with pytest.raises(ValueError):
+        ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], 64)
+
+
 # ------------------------------------------------------------------ contract violations
 def test_operator_contract_errors(ops_mod):
     ops = o.make_operands(10, 2, 256, 16, 128)

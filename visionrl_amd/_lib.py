@@ -21,6 +21,8 @@ SYMBOLS = (
     "vrl_int4_gemv_bf16",
     "vrl_int4_dequant_bf16",
     "vrl_int4_gate_up_silu_bf16",
+    "vrl_int4_prepacked_bytes",
+    "vrl_int4_prepack",
     "vrl_int4_grouped_plan_size",
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
@@ -45,7 +47,8 @@ class Problem(ctypes.Structure):
         ("K", ctypes.c_int32),
         ("G", ctypes.c_int32),
         ("fused_gate_up", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 3),
+        ("prepacked", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 2),
     ]
 
 
@@ -58,7 +61,8 @@ class PlanInfo(ctypes.Structure):
         ("grid", ctypes.c_int32),
         ("block_threads", ctypes.c_int32),
         ("lds_bytes", ctypes.c_int32),
-        ("reserved", ctypes.c_int32 * 3),
+        ("variant", ctypes.c_int32),
+        ("reserved", ctypes.c_int32 * 2),
     ]
 
 
@@ -78,6 +82,10 @@ def _bind(lib):
     lib.vrl_int4_dequant_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     lib.vrl_int4_gate_up_silu_bf16.restype = ci
     lib.vrl_int4_gate_up_silu_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, vp]
+    lib.vrl_int4_prepacked_bytes.restype = ctypes.c_size_t
+    lib.vrl_int4_prepacked_bytes.argtypes = [ci, ci, ci]
+    lib.vrl_int4_prepack.restype = ci
+    lib.vrl_int4_prepack.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     lib.vrl_int4_grouped_plan_size.restype = ctypes.c_size_t
     lib.vrl_int4_grouped_plan_size.argtypes = [ci]
     lib.vrl_int4_grouped_plan_build.restype = ci

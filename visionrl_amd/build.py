@@ -24,6 +24,8 @@ HIPCC_FLAGS = [
     "-shared",
     "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go straight to VGPRs: the dequant path converts them at once
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

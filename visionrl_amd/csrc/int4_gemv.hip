@@ -56,7 +56,7 @@ struct DevProblem {
     int32_t fused;       // gate||up rows with SiLU epilogue
     int32_t tile_begin;  // first tile index of this problem inside a grouped launch
     int32_t kc;          // k extent of x staged in LDS per pass (multiple of KCHUNK)
-    int32_t pad;
+    int32_t prepacked;   // qweight points at a prepacked blob (scales/qzeros unused)
 };
 static_assert(sizeof(DevProblem) == 72, "plan record layout is part of the plan format");
 
@@ -436,7 +436,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_tile_kernel(DevProblem p) {
 // activations in LDS once, then each wave streams whole tiles - no K split, so
 // no partial sums to meet - keeping STREAM_DEPTH 128-k chunks of its 16 rows in
 // flight (non-temporal global_load_dwordx4: the weights are read exactly once).
-constexpr int STREAM_WPB = 4;
+constexpr int STREAM_WPB = 8;
 constexpr int STREAM_DEPTH = 4;
 
 template <int RS>
@@ -607,7 +607,275 @@ __device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int 
     }
 }
 
-template <int WPB>
+// -------------------------------------------------------------------------
+// prepacked weights: MFMA-shaped tiles, dequantised by the matrix cores
+// -------------------------------------------------------------------------
+// A one-time repack (prepack_kernel) turns the canonical operand triple into a
+// blob a wave can stream with fully contiguous 1 KB loads and dequantise almost
+// without VALU work.  Group size 128 only.  Per 16-row tile, K padded to 512:
+//
+//   [meta  : ceil(nsc/4) x 64 lanes x 16 B]   word e of lane l in block mb is
+//            (scale bits << 16) | zero  of row (l % 16), group 4*(4*mb+e) + l/16
+//   [words : nsc x 4 x 64 lanes x 16 B]       super-chunk sc, load j, lane l, dword d
+//
+// with l = 16*kq + 4*rq + i.  Nibble nu of a weight dword holds
+//   q[row 4*rq + kp][k = 512*sc + 128*kq + 32*j + 8*d + 4*c + i],
+//   c = (nu % 4) / 2,  kp = 2*(nu % 2) + (nu >= 4).
+// So ((v >> 4s) & 0x000F000F) | 0x43004300 is a bf16 pair (128+q) of two
+// neighbouring ROWS at one k, which is the A operand of v_mfma_f32_4x4x4_16b_bf16
+// (16 independent 4x4x4 products, one per lane quad): with B = diag(scale of the
+// lane's row) and C = -(128+z)*scale it returns the exact fp32 products
+// (q-z)*s for the lane's own row at four consecutive k.  v_cvt_pk_bf16_f32
+// rounds them (the one RNE of the contract), and two such results are the B
+// operand of v_mfma_f32_16x16x32_bf16 against the staged activations.
+// Per 8 weights and lane: 7 VALU unpack ops, 4 conversions, 3 MFMA issues.
+constexpr int PP_SC = 512;  // k per super-chunk: lane group kq owns one 128-k scale group
+
+__host__ __device__ inline int pp_nsc(int K) { return (K + PP_SC - 1) / PP_SC; }
+__host__ __device__ inline long pp_meta_u4(int K) { return (long)((pp_nsc(K) + 3) / 4) * 64; }
+__host__ __device__ inline long pp_tile_u4(int K) { return pp_meta_u4(K) + (long)pp_nsc(K) * 4 * 64; }
+
+__global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict__ qweight,
+                                                      const uint16_t *__restrict__ scales,
+                                                      const uint32_t *__restrict__ qzeros,
+                                                      u32x4_t *__restrict__ blob, int N, int K) {
+    const int kwords = K >> 3;
+    const int groups = K / 128;
+    const int zwords = (groups + 7) >> 3;
+    const long meta_u4 = pp_meta_u4(K);
+    const long tile_u4 = pp_tile_u4(K);
+    const long ntiles = (N + 15) / 16;
+    const long total = ntiles * tile_u4;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long tile = idx / tile_u4;
+        const long rem = idx - tile * tile_u4;
+        u32x4_t out = {0u, 0u, 0u, 0u};
+        if (rem < meta_u4) {
+            const int mb = (int)(rem >> 6);
+            const int lane = (int)(rem & 63);
+            const long row = tile * 16 + (lane & 15);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int g = 4 * (4 * mb + e) + (lane >> 4);
+                if (row < N && g < groups) {
+                    const uint32_t sb = scales[row * groups + g];
+                    const uint32_t z = (qzeros[row * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xFu;
+                    out[e] = (sb << 16) | z;
+                }
+            }
+        } else {
+            const long r2 = rem - meta_u4;
+            const int sc = (int)(r2 >> 8);
+            const int j = (int)((r2 >> 6) & 3);
+            const int lane = (int)(r2 & 63);
+            const int kq = lane >> 4, rq = (lane >> 2) & 3, i = lane & 3;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int nu = 0; nu < 8; ++nu) {
+                    const int c = (nu & 3) >> 1;
+                    const int kp = 2 * (nu & 1) + (nu >> 2);
+                    const long row = tile * 16 + 4 * rq + kp;
+                    const int k = sc * PP_SC + kq * 128 + j * 32 + d * 8 + 4 * c + i;
+                    if (row < N && k < K) {
+                        const uint32_t src = qweight[row * kwords + (k >> 3)];
+                        word |= ((src >> (4 * (k & 7))) & 0xFu) << (4 * nu);
+                    }
+                }
+                out[d] = word;
+            }
+        }
+        blob[idx] = out;
+    }
+}
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+// natural-order staging of x[:, k0:k1) (k beyond K reads as zero)
+__device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int k1, uint16_t *xs,
+                                                int xstride, int nthreads) {
+    const int words_per_row = (k1 - k0) >> 3;
+    const int total = p.M * words_per_row;
+    for (int idx = threadIdx.x; idx < total; idx += nthreads) {
+        const int m = idx / words_per_row;
+        const int j = idx - m * words_per_row;
+        const int k = k0 + (j << 3);
+        u32x4_t d = {0u, 0u, 0u, 0u};
+        if (k < p.K) d = *reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k);
+        *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = d;
+    }
+}
+
+struct PPGroup {
+    bf16x4_t bdiag;  // B operand of the 4x4x4 product: scale at k' = lane % 4, zero elsewhere
+    f32x4_t cq;      // C operand: -(128 + z) * scale in all four rows
+};
+
+__device__ __forceinline__ PPGroup pp_group(uint32_t meta_word, int j4) {
+    const uint32_t sb = meta_word >> 16;
+    const float s = __builtin_bit_cast(float, meta_word & 0xFFFF0000u);
+    const float c = -(128.0f + (float)(meta_word & 15u)) * s;
+    u32x2_t bd;
+    bd[0] = (j4 == 0) ? sb : (j4 == 1 ? (sb << 16) : 0u);
+    bd[1] = (j4 == 2) ? sb : (j4 == 3 ? (sb << 16) : 0u);
+    PPGroup g;
+    g.bdiag = __builtin_bit_cast(bf16x4_t, bd);
+    g.cq = f32x4_t{c, c, c, c};
+    return g;
+}
+
+// acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob;
+// xs holds x for exactly that k range
+template <int MB, bool FUSED>
+__device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_local, const uint16_t *xs,
+                                               int xstride, int sc0, int sc1,
+                                               f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int lc = lane & 15;
+    const int kq = lane >> 4;
+    const int j4 = lane & 3;
+    const long meta_u4 = pp_meta_u4(p.K);
+    const long tile_u4 = pp_tile_u4(p.K);
+    const int out_tiles = (FUSED ? p.N / 2 : p.N + 15) / 16;
+
+    // both must sit in registers for (v & mask) | bias to select v_and_or_b32
+    uint32_t mask = PAIR_MASK, bias = PAIR_BIAS;
+    asm volatile("" : "+s"(mask));
+    asm volatile("" : "+v"(bias));
+
+    const u32x4_t *mp[RS];
+    const u32x4_t *wp[RS];
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        mp[r] = reinterpret_cast<const u32x4_t *>(p.qweight) +
+                (long)(tile_local + r * out_tiles) * tile_u4 + lane;
+        wp[r] = mp[r] + meta_u4 + (long)sc0 * 256;
+    }
+    const int nld = (sc1 - sc0) * 4;
+    u32x4_t ring[STREAM_DEPTH][RS];
+    u32x4_t mt[RS];
+    PPGroup grp[RS];
+#pragma unroll
+    for (int d = 0; d < STREAM_DEPTH; ++d)
+        if (d < nld) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) ring[d][r] = __builtin_nontemporal_load(wp[r] + d * 64);
+        }
+#pragma unroll
+    for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc0 >> 2) * 64];
+
+    for (int l0 = 0; l0 < nld; l0 += STREAM_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < STREAM_DEPTH; ++d) {
+            const int ld = l0 + d;
+            if (ld < nld) {
+                const int sc = sc0 + (ld >> 2);
+                const int j = ld & 3;
+                if (j == 0) {
+                    if (ld != 0 && (sc & 3) == 0) {
+#pragma unroll
+                        for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
+                    }
+#pragma unroll
+                    for (int r = 0; r < RS; ++r) {
+                        const int e = sc & 3;
+                        const uint32_t mw = e == 0 ? mt[r][0] : (e == 1 ? mt[r][1] : (e == 2 ? mt[r][2] : mt[r][3]));
+                        grp[r] = pp_group(mw, j4);
+                    }
+                }
+                u32x4_t w[RS];
+#pragma unroll
+                for (int r = 0; r < RS; ++r) w[r] = ring[d][r];
+                if (ld + STREAM_DEPTH < nld) {
+#pragma unroll
+                    for (int r = 0; r < RS; ++r)
+                        ring[d][r] = __builtin_nontemporal_load(wp[r] + (ld + STREAM_DEPTH) * 64);
+                }
+                const int kloc = (sc - sc0) * PP_SC + kq * 128 + j * 32;
+#pragma unroll
+                for (int dd = 0; dd < 4; ++dd) {
+                    bf16x8_t xa[MB];
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) {
+                        const int m = min(16 * b + lc, p.M - 1);
+                        const u32x4_t raw =
+                            *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
+                        xa[b] = __builtin_bit_cast(bf16x8_t, raw);
+                    }
+#pragma unroll
+                    for (int r = 0; r < RS; ++r) {
+                        const uint32_t v = w[r][dd];
+                        u32x2_t a0, a1;
+                        a0[0] = (v & mask) | bias;
+                        a0[1] = ((v >> 4) & mask) | bias;
+                        a1[0] = ((v >> 8) & mask) | bias;
+                        a1[1] = ((v >> 12) & mask) | bias;
+                        const f32x4_t d0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                            __builtin_bit_cast(bf16x4_t, a0), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                        const f32x4_t d1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                            __builtin_bit_cast(bf16x4_t, a1), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                        const u32x4_t wv = {pack_bf16_rne(d0[0], d0[1]), pack_bf16_rne(d0[2], d0[3]),
+                                            pack_bf16_rne(d1[0], d1[1]), pack_bf16_rne(d1[2], d1[3])};
+                        const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+                        for (int b = 0; b < MB; ++b)
+                            acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int MB, bool FUSED, int WPB>
+__device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int wave = threadIdx.x >> 6;
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int xstride = p.kc + XPAD;
+    const int nsc = pp_nsc(p.K);
+    const int sc_pass = p.kc / PP_SC;
+    if (sc_pass >= nsc) {
+        __syncthreads();
+        stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+        __syncthreads();
+        for (int tile = t0 + wave; tile < t1; tile += WPB) {
+            f32x4_t acc[RS][MB];
+#pragma unroll
+            for (int r = 0; r < RS; ++r)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, 0, nsc, acc);
+            store_tile<MB, FUSED>(p, tile, acc);
+        }
+    } else {
+        for (int round = t0; round < t1; round += WPB) {
+            const int tile = round + wave;
+            const bool active = tile < t1;
+            f32x4_t acc[RS][MB];
+#pragma unroll
+            for (int r = 0; r < RS; ++r)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int sc0 = 0; sc0 < nsc; sc0 += sc_pass) {
+                const int sc1 = min(nsc, sc0 + sc_pass);
+                __syncthreads();
+                stage_x_natural(p, sc0 * PP_SC, sc1 * PP_SC, xs, xstride, WPB * WAVE);
+                __syncthreads();
+                if (active) stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, sc0, sc1, acc);
+            }
+            if (active) store_tile<MB, FUSED>(p, tile, acc);
+        }
+    }
+}
+
+// CANON / PP / FUSED say which kinds of record the plan holds, so that a plan of
+// plain prepacked GEMVs runs the variant with the smallest register footprint.
+template <int WPB, bool CANON, bool PP, bool FUSED>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
                                                                 const int32_t *__restrict__ block_begin,
                                                                 int n_problems) {
@@ -625,10 +893,14 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
         const DevProblem p = plan[pi];
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
-        if (p.fused)
-            stream_segment<1, true, WPB>(p, t - p.tile_begin, seg_end - p.tile_begin, smem);
-        else
-            stream_segment<1, false, WPB>(p, t - p.tile_begin, seg_end - p.tile_begin, smem);
+        const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
+        if (PP && (!CANON || p.prepacked)) {
+            if (FUSED && p.fused) stream_segment_pp<1, FUSED, WPB>(p, a, b, smem);
+            else stream_segment_pp<1, false, WPB>(p, a, b, smem);
+        } else if (CANON) {
+            if (FUSED && p.fused) stream_segment<1, FUSED, WPB>(p, a, b, smem);
+            else stream_segment<1, false, WPB>(p, a, b, smem);
+        }
         t = seg_end;
     }
 }
@@ -681,6 +953,19 @@ int stream_staged_k(int M, int K) {
     kc -= kc % KCHUNK;
     if (kc < KCHUNK) kc = KCHUNK;
     return (int)(kc < K ? kc : K);
+}
+
+// prepacked blobs exist for group size 128 only
+bool prepack_ok(long N, long K, long G) { return G == 128 && K % 128 == 0 && N >= 1 && N * K < (1L << 40); }
+
+// prepacked stream: all of the padded K if it fits, else whole super-chunks per pass
+int pp_staged_k(int M, int K) {
+    const int kpad = pp_nsc(K) * PP_SC;
+    if ((size_t)M * (kpad + XPAD) * 2 <= STREAM_X_SINGLE) return kpad;
+    long kc = (long)(STREAM_X_PASS / ((size_t)M * 2)) - XPAD;
+    kc -= kc % PP_SC;
+    if (kc < PP_SC) kc = PP_SC;
+    return (int)kc;
 }
 
 template <int R, int MB>
@@ -766,6 +1051,21 @@ struct PlanHeader {
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
+constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4;
+
+template <bool CANON, bool PP, bool FUSED>
+int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *block_begin,
+                  hipStream_t stream) {
+    auto kernel = &gemv_stream_kernel<STREAM_WPB, CANON, PP, FUSED>;
+    if (info->lds_bytes > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(STREAM_WPB * WAVE), (size_t)info->lds_bytes,
+                       stream, recs, block_begin, info->n_problems);
+    return (int)hipGetLastError();
+}
 
 size_t plan_bytes_for(int n_records) {
     return sizeof(PlanHeader) + (size_t)n_records * sizeof(DevProblem) +
@@ -818,6 +1118,27 @@ int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *q
     return (int)hipGetLastError();
 }
 
+size_t vrl_int4_prepacked_bytes(int N, int K, int G) {
+    if (!prepack_ok(N, K, G)) return 0;
+    return (size_t)((N + 15) / 16) * (size_t)pp_tile_u4(K) * 16;
+}
+
+int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros, void *packed,
+                     int N, int K, int G, void *hip_stream) {
+    int rc = check_problem(qweight, qweight, scales, qzeros, packed, 1, N, K, G);
+    if (rc != VRL_INT4_OK) return rc;
+    if (!prepack_ok(N, K, G)) return VRL_INT4_ESHAPE;
+    const long total = (long)((N + 15) / 16) * pp_tile_u4(K);
+    long blocks = (total + 255) / 256;
+    const long cap = (long)device_cu_count() * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(prepack_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(hip_stream),
+                       static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
+                       static_cast<const uint32_t *>(qzeros), static_cast<u32x4_t *>(packed), N, K);
+    return (int)hipGetLastError();
+}
+
 size_t vrl_int4_grouped_plan_size(int n_problems) {
     if (n_problems < 1) return 0;
     return plan_bytes_for(n_problems);
@@ -834,9 +1155,15 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     long tiles = 0;
     double total_cost = 0.0;
     size_t smem = 0;
+    int variant = 0;
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
-        int rc = check_problem(q.x, q.qweight, q.scales, q.qzeros, q.y, q.M, q.N, q.K, q.G);
+        variant |= (q.prepacked ? VARIANT_PP : VARIANT_CANON) | (q.fused_gate_up ? VARIANT_FUSED : 0);
+        int rc;
+        if (q.prepacked)
+            rc = check_problem(q.x, q.qweight, q.qweight, q.qweight, q.y, q.M, q.N, q.K, q.G);
+        else
+            rc = check_problem(q.x, q.qweight, q.scales, q.qzeros, q.y, q.M, q.N, q.K, q.G);
         if (rc != VRL_INT4_OK) return rc;
         if (q.fused_gate_up && q.N % 2 != 0) return VRL_INT4_ESHAPE;
         DevProblem p;
@@ -848,8 +1175,14 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         p.y = static_cast<uint16_t *>(q.y);
         p.M = q.M; p.N = q.N; p.K = q.K; p.G = q.G;
         p.fused = q.fused_gate_up ? 1 : 0;
+        p.prepacked = q.prepacked ? 1 : 0;
         if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take MFMA-path shapes only
-        p.kc = stream_staged_k(p.M, p.K);
+        if (p.prepacked) {
+            if (!prepack_ok(p.N, p.K, p.G) || (p.fused && (p.N / 2) % 16 != 0)) return VRL_INT4_ESHAPE;
+            p.kc = pp_staged_k(p.M, p.K);
+        } else {
+            p.kc = stream_staged_k(p.M, p.K);
+        }
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const long nt = (out_cols + 15) / 16;
@@ -905,6 +1238,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     info->grid = (int)grid;
     info->block_threads = STREAM_WPB * WAVE;
     info->lds_bytes = (int)smem;
+    info->variant = variant;
     return VRL_INT4_OK;
 }
 
@@ -918,16 +1252,16 @@ int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *i
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
     const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + sizeof(PlanHeader));
     const int32_t *block_begin = reinterpret_cast<const int32_t *>(recs + info->n_problems);
-    if (info->lds_bytes > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&gemv_stream_kernel<STREAM_WPB>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
-        if (e != hipSuccess) return (int)e;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    switch (info->variant) {
+        case VARIANT_PP: return launch_stream<false, true, false>(info, recs, block_begin, stream);
+        case VARIANT_PP | VARIANT_FUSED: return launch_stream<false, true, true>(info, recs, block_begin, stream);
+        case VARIANT_CANON: return launch_stream<true, false, false>(info, recs, block_begin, stream);
+        case VARIANT_CANON | VARIANT_FUSED: return launch_stream<true, false, true>(info, recs, block_begin, stream);
+        case VARIANT_CANON | VARIANT_PP: return launch_stream<true, true, false>(info, recs, block_begin, stream);
+        case VARIANT_CANON | VARIANT_PP | VARIANT_FUSED: return launch_stream<true, true, true>(info, recs, block_begin, stream);
+        default: return VRL_INT4_EPLAN;
     }
-    hipLaunchKernelGGL((gemv_stream_kernel<STREAM_WPB>), dim3(info->grid), dim3(STREAM_WPB * WAVE),
-                       (size_t)info->lds_bytes, reinterpret_cast<hipStream_t>(hip_stream), recs,
-                       block_begin, info->n_problems);
-    return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -22,7 +22,8 @@ import torch
 from . import _lib
 from .int4_format import check_packed
 
-__all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "GroupedGemv"]
+__all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_prepack", "PrepackedWeight",
+           "GroupedGemv"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -118,14 +119,53 @@ def _(x, qweight_gu, scales_gu, qzeros_gu, group_size):
     return x.new_empty((x.shape[0], qweight_gu.shape[0] // 2))
 
 
+class PrepackedWeight:
+    """A weight repacked once for the grouped launch (group size 128 only).
+
+    ``blob`` is an opaque ``uint8`` device tensor made by the library from the
+    canonical ``(qweight, scales, qzeros)`` triple; ``N``, ``K`` and
+    ``group_size`` describe the operand it stands for.  The weights the kernels
+    rebuild from it are bit for bit the canonical dequantised tile.
+    """
+
+    def __init__(self, blob: torch.Tensor, N: int, K: int, group_size: int):
+        self.blob, self.N, self.K, self.group_size = blob, int(N), int(K), int(group_size)
+
+    @staticmethod
+    def supported(N: int, K: int, group_size: int) -> bool:
+        return _lib.load().vrl_int4_prepacked_bytes(int(N), int(K), int(group_size)) > 0
+
+
+def int4_prepack(qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
+                 group_size: int) -> PrepackedWeight:
+    """Repack a canonical operand triple on its device; raises ``ValueError`` if the
+    shape has no prepacked form (group size other than 128)."""
+    N, K, _ = check_packed(qweight, scales, qzeros, group_size)
+    dev = _require_device("qweight", qweight)
+    _require_device("scales", scales, dev)
+    _require_device("qzeros", qzeros, dev)
+    lib = _lib.load()
+    nbytes = lib.vrl_int4_prepacked_bytes(N, K, int(group_size))
+    if nbytes == 0:
+        raise ValueError(f"no prepacked form for N={N}, K={K}, group_size={group_size} "
+                         "(needs group_size 128)")
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.vrl_int4_prepack(qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
+                                  blob.data_ptr(), N, K, int(group_size), _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_prepack")
+    return PrepackedWeight(blob, N, K, group_size)
+
+
 class GroupedGemv:
     """Several independent int4 GEMVs enqueued as one kernel launch.
 
     ``problems`` is a list of ``(x, qweight, scales, qzeros, group_size, fused)``
-    tuples; outputs are allocated once here and overwritten by every
-    :meth:`launch`.  The plan (pointer table) is validated and built on the host
-    by the library, copied to the device once, and stays valid while the tensors
-    captured here are alive and not reallocated.
+    tuples, or ``(x, prepacked_weight, fused)`` with a :class:`PrepackedWeight`;
+    outputs are allocated once here and overwritten by every :meth:`launch`.  The
+    plan (pointer table) is validated and built on the host by the library,
+    copied to the device once, and stays valid while the tensors captured here
+    are alive and not reallocated.
     """
 
     MAX_ROWS = 16  # activation rows one record of the plan may carry
@@ -138,8 +178,25 @@ class GroupedGemv:
         self.outputs = []
         dev = None
         records = []
-        for x, qweight, scales, qzeros, group_size, fused in problems:
-            M, N, K, d = _check_call(x, qweight, scales, qzeros, group_size)
+        for prob in problems:
+            if len(prob) == 3:
+                x, pw, fused = prob
+                if not isinstance(pw, PrepackedWeight):
+                    raise TypeError("(x, weight, fused) problems take a PrepackedWeight")
+                if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != pw.K or x.shape[0] < 1:
+                    raise ValueError(f"x must be bfloat16 [M, {pw.K}]")
+                d = _require_device("x", x)
+                _require_device("prepacked blob", pw.blob, d)
+                M, N, K, group_size = x.shape[0], pw.N, pw.K, pw.group_size
+                ptrs = (pw.blob.data_ptr(), 0, 0)
+                keep = (x, pw)
+                prepacked = 1
+            else:
+                x, qweight, scales, qzeros, group_size, fused = prob
+                M, N, K, d = _check_call(x, qweight, scales, qzeros, group_size)
+                ptrs = (qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr())
+                keep = (x, qweight, scales, qzeros)
+                prepacked = 0
             if dev is None:
                 dev = d
             elif d != dev:
@@ -147,19 +204,18 @@ class GroupedGemv:
             if fused and N % 2 != 0:
                 raise ValueError("gate||up operand needs an even number of rows")
             y = torch.empty((M, N // 2 if fused else N), dtype=torch.bfloat16, device=dev)
-            self._keep.append((x, qweight, scales, qzeros))
+            self._keep.append(keep)
             self.outputs.append(y)
             # one record per slab of MAX_ROWS activation rows (row slices stay contiguous)
             for m0 in range(0, M, self.MAX_ROWS):
                 m1 = min(M, m0 + self.MAX_ROWS)
-                records.append((x[m0:m1].data_ptr(), qweight.data_ptr(), scales.data_ptr(),
-                                qzeros.data_ptr(), y[m0:m1].data_ptr(), m1 - m0, N, K,
-                                int(group_size), 1 if fused else 0))
+                records.append((x[m0:m1].data_ptr(), *ptrs, y[m0:m1].data_ptr(), m1 - m0, N, K,
+                                int(group_size), 1 if fused else 0, prepacked))
         n = len(records)
         table = (_lib.Problem * n)()
         for rec, vals in zip(table, records):
             (rec.x, rec.qweight, rec.scales, rec.qzeros, rec.y,
-             rec.M, rec.N, rec.K, rec.G, rec.fused_gate_up) = vals
+             rec.M, rec.N, rec.K, rec.G, rec.fused_gate_up, rec.prepacked) = vals
         size = lib.vrl_int4_grouped_plan_size(n)
         host = torch.empty(size, dtype=torch.uint8)
         self.info = _lib.PlanInfo()
