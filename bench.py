@@ -78,6 +78,7 @@ def time_region(fn, steps: int, warmup: int):
 
 def build_set(cfg: int, M: int, device, with_head: bool):
     """All linears of one decode step: list of dicts with operands and byte counts."""
+    from visionrl_amd import ops
     from visionrl_amd.int4_format import algorithmic_bytes
 
     items = []
@@ -87,11 +88,13 @@ def build_set(cfg: int, M: int, device, with_head: bool):
             qw, sc, qz = make_weights(1000 * cfg + 10 * layer + proj, K, N, GROUP, device)
             items.append({"name": f"l{layer}.{name}", "layer": layer, "proj": name, "K": K, "N": N,
                           "x": xs[K], "qweight": qw, "scales": sc, "qzeros": qz,
+                          "prepacked": ops.int4_prepack(qw, sc, qz, GROUP),
                           "bytes": algorithmic_bytes(M, K, N, GROUP)})
     if with_head:
         qw, sc, qz = make_weights(1000 * cfg + 999, HIDDEN, HEAD, GROUP, device)
         items.append({"name": "gen_head", "layer": LAYERS, "proj": "head", "K": HIDDEN, "N": HEAD,
                       "x": xs[HIDDEN], "qweight": qw, "scales": sc, "qzeros": qz,
+                      "prepacked": ops.int4_prepack(qw, sc, qz, GROUP),
                       "bytes": algorithmic_bytes(M, HIDDEN, HEAD, GROUP)})
     return items
 
@@ -108,10 +111,15 @@ def measure_set(items, steps: int, warmup: int):
         out["GBps"][name] = total_bytes / (ms * 1e-3) / 1e9
         out["launches_per_step"][name] = launches
 
-    # one launch for the whole set
-    grouped = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
-                               for it in items])
+    # one launch for the whole set, weights in the prepacked (MFMA-shaped) layout
+    grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items])
     record("grouped_1_launch", time_region(grouped.launch, steps, warmup), 1)
+
+    # the same launch over the canonical layout (no load-time repack)
+    canon = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
+                             for it in items])
+    record("grouped_1_launch_canonical_layout", time_region(canon.launch, steps, warmup), 1)
+    del canon
 
     # one launch per linear, stream ordered
     def eager():
@@ -145,8 +153,7 @@ def measure_set(items, steps: int, warmup: int):
         for names in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",), ("head",)):
             sel = [its[n] for n in names if n in its]
             if sel:
-                plans.append(ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"],
-                                               GROUP, False) for it in sel]))
+                plans.append(ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in sel]))
 
     def layered():
         for plan in plans:
@@ -225,6 +232,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true",
                     help="run just the grouped decode-step launches (for profilers)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run plain 1 GiB device copies and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus 1 only)")
@@ -233,14 +242,21 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "copies": args.steps}))
+        return
     from visionrl_amd import ops
 
     items = build_set(2, 1, device, with_head=False)
     torch.cuda.synchronize()
 
     if args.only_headline:
-        grouped = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
-                                   for it in items])
+        grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items])
         ms = time_region(grouped.launch, args.steps, args.warmup)
         print(json.dumps({"ms_per_step": ms}))
         return
@@ -282,11 +298,12 @@ def main():
         "config": {"workload": "Janus-Pro-1B decoder linear set, M=1: 24 layers x (4x 2048->2048, "
                                "2x 2048->5632, 1x 5632->2048), int4 group 128, 168 GEMVs, distinct weights",
                    "algorithmic_bytes_per_step": total_bytes,
-                   "launch": "one grouped launch per step (all 168 GEMVs in one kernel)"},
+                   "launch": "one grouped launch per step (all 168 GEMVs in one kernel), weights "
+                             "repacked once at load into the MFMA-shaped layout"},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": load_traffic("gemv_grouped_kernel"),
-                     "kernel": "gemv_grouped_kernel", "bytes_per_launch": total_bytes,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": load_traffic("gemv_stream_kernel"),
+                     "kernel": "gemv_stream_kernel", "bytes_per_launch": total_bytes,
                      "avg_launch_ms": kernel_ms},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,

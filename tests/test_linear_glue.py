@@ -1,0 +1,220 @@
+"""``Int4Linear`` and the policy glue: structure on CPU, numerics on the GPU.
+
+The stand-in policy mirrors the accessors the reference exposes
+(``JanusProPolicy._lm_trunk`` / ``_base``, vrl/models/families/janus_pro/policy.py:226-266)
+around a real, randomly initialised Hugging Face ``LlamaModel`` built offline from a config,
+the way the reference's own tests stub the trunk (tests/models/test_janus_wrapper.py:30-87).
+"""
+
+import types
+
+import pytest
+import torch
+from torch import nn
+
+from visionrl_amd.linear import Int4GateUpSiLU, Int4Linear, Int4LlamaMLP
+from visionrl_amd.policy_glue import (apply_int4_to_policy, build_int4_runtime_bundle,
+                                      int4_options_from_spec)
+
+HIDDEN, INTER, HEADS, LAYERS, VOCAB_IMG = 256, 512, 4, 2, 1024
+
+
+def tiny_llama():
+    from transformers import LlamaConfig, LlamaModel
+
+    cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=LAYERS,
+                      num_attention_heads=HEADS, num_key_value_heads=HEADS, vocab_size=128,
+                      max_position_embeddings=64)
+    torch.manual_seed(0)
+    return LlamaModel(cfg).to(torch.bfloat16).eval()
+
+
+class StubMMGPT(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.language_model = types.SimpleNamespace(model=tiny_llama())
+        torch.manual_seed(1)
+        self.gen_head = nn.Linear(HIDDEN, VOCAB_IMG, bias=False).to(torch.bfloat16)
+
+
+class StubPolicy:
+    """Only the two accessors the glue uses."""
+
+    def __init__(self):
+        self.mmgpt = StubMMGPT()
+
+    def _base(self):
+        return self.mmgpt
+
+    def _lm_trunk(self):
+        return self.mmgpt.language_model.model
+
+
+def test_apply_swaps_every_decode_linear():
+    policy = StubPolicy()
+    summary = apply_int4_to_policy(policy, group_size=128)
+    assert summary == {"linears": 7 * LAYERS, "fused_mlps": LAYERS, "head_linears": 1, "group_size": 128}
+    for layer in policy._lm_trunk().layers:
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            mod = getattr(layer.self_attn, name)
+            assert isinstance(mod, Int4Linear)
+            assert (mod.in_features, mod.out_features) == (HIDDEN, HIDDEN)
+            assert mod.qweight.shape == (HIDDEN, HIDDEN // 8) and mod.qweight.dtype == torch.int32
+            assert mod.scales.shape == (HIDDEN, HIDDEN // 128) and mod.scales.dtype == torch.bfloat16
+        assert isinstance(layer.mlp, Int4LlamaMLP)
+        assert isinstance(layer.mlp.gate_up, Int4GateUpSiLU)
+        assert layer.mlp.gate_up.qweight.shape == (2 * INTER, HIDDEN // 8)
+        assert layer.mlp.down_proj.in_features == INTER
+    assert isinstance(policy._base().gen_head, Int4Linear)
+    # nothing left to do on a second pass
+    again = apply_int4_to_policy(policy, group_size=128)
+    assert again["linears"] == 0 and again["fused_mlps"] == 0 and again["head_linears"] == 0
+
+
+def test_targets_and_unfused_mlp():
+    policy = StubPolicy()
+    summary = apply_int4_to_policy(policy, group_size=64, targets=("q_proj", "v_proj", "down_proj"),
+                                   fuse_mlp=True, head=False)
+    assert summary["linears"] == 3 * LAYERS and summary["fused_mlps"] == 0 and summary["head_linears"] == 0
+    layer = policy._lm_trunk().layers[0]
+    assert isinstance(layer.self_attn.q_proj, Int4Linear) and layer.self_attn.q_proj.group_size == 64
+    assert isinstance(layer.self_attn.k_proj, nn.Linear)
+    assert isinstance(layer.mlp.down_proj, Int4Linear) and isinstance(layer.mlp.gate_proj, nn.Linear)
+    assert isinstance(policy._base().gen_head, nn.Linear)
+    with pytest.raises(ValueError):
+        apply_int4_to_policy(policy, targets=("lm_head",))
+
+
+def test_lora_wrapper_keeps_its_adapter():
+    """A PEFT-style wrapper (frozen weight in ``base_layer``) gets only its base quantised."""
+
+    class LoraLike(nn.Module):
+        def __init__(self, base):
+            super().__init__()
+            self.base_layer = base
+            self.lora_A = nn.Linear(base.in_features, 4, bias=False)
+            self.lora_B = nn.Linear(4, base.out_features, bias=False)
+
+        def forward(self, x):
+            return self.base_layer(x) + self.lora_B(self.lora_A(x))
+
+    policy = StubPolicy()
+    attn = policy._lm_trunk().layers[0].self_attn
+    attn.q_proj = LoraLike(attn.q_proj)
+    apply_int4_to_policy(policy, head=False)
+    assert isinstance(attn.q_proj, LoraLike)
+    assert isinstance(attn.q_proj.base_layer, Int4Linear)
+    assert isinstance(attn.q_proj.lora_A, nn.Linear)
+
+
+def test_state_dict_round_trip():
+    lin = nn.Linear(256, 48, bias=True).to(torch.bfloat16)
+    a = Int4Linear.from_linear(lin, 64)
+    b = Int4Linear(256, 48, 64, bias=True)
+    b.load_state_dict(a.state_dict())
+    for k, v in a.state_dict().items():
+        assert torch.equal(v, b.state_dict()[k]), k
+    assert set(a.state_dict()) == {"qweight", "scales", "qzeros", "bias"}
+    with pytest.raises(ValueError):
+        Int4Linear(250, 48, 128)
+
+
+def test_runtime_spec_options_and_builder_wrapper():
+    spec = types.SimpleNamespace(extra={})
+    assert int4_options_from_spec(spec) is None
+    spec.extra["int4"] = True
+    assert int4_options_from_spec(spec)["group_size"] == 128
+    spec.extra["int4"] = {"group_size": 64, "head": False}
+    opt = int4_options_from_spec(spec)
+    assert opt["group_size"] == 64 and opt["head"] is False and opt["fuse_mlp"] is True
+    spec.extra["int4"] = {"bits": 3}
+    with pytest.raises(ValueError):
+        int4_options_from_spec(spec)
+    spec.extra["int4"] = "yes"
+    with pytest.raises(TypeError):
+        int4_options_from_spec(spec)
+
+    spec.extra["int4"] = {"group_size": 128}
+    bundle = build_int4_runtime_bundle(
+        spec, lambda s: types.SimpleNamespace(policy=StubPolicy(), metadata={"model_path": "stub"}))
+    assert bundle.metadata["int4"]["linears"] == 7 * LAYERS
+    assert isinstance(bundle.policy._base().gen_head, Int4Linear)
+    plain = build_int4_runtime_bundle(types.SimpleNamespace(extra={}),
+                                      lambda s: types.SimpleNamespace(policy=StubPolicy(), metadata={}))
+    assert "int4" not in plain.metadata
+    assert isinstance(plain.policy._base().gen_head, nn.Linear)
+
+
+def test_cpu_forward_fails_loudly():
+    lin = Int4Linear.from_linear(nn.Linear(128, 8, bias=False).to(torch.bfloat16), 128)
+    with pytest.raises(ValueError, match="no CPU path"):
+        lin(torch.zeros(1, 128, dtype=torch.bfloat16))
+    with pytest.raises(TypeError):
+        lin(torch.zeros(1, 128, dtype=torch.float32))
+
+
+# ---------------------------------------------------------------------- GPU numerics
+@pytest.mark.gpu
+def test_int4_linear_matches_dequantised_linear():
+    dev = "cuda:0"
+    torch.manual_seed(2)
+    lin = nn.Linear(512, 96, bias=True).to(torch.bfloat16).to(dev)
+    q = Int4Linear.from_linear(lin, 128)
+    x = torch.randn(3, 5, 512, device=dev).to(torch.bfloat16)
+    w = q.dequantize()
+    assert w.shape == (96, 512) and w.dtype == torch.bfloat16
+    ref = (x.reshape(-1, 512).double() @ w.double().t()).reshape(3, 5, 96)
+    y = q(x)
+    assert y.shape == (3, 5, 96) and y.dtype == torch.bfloat16
+    err = (y.double() - (ref + q.bias.double())).abs()
+    assert (err <= 2.0 ** -7 * ref.abs() + 2.0 ** -6).all()
+    # the quantiser keeps the weights within one step
+    step = q.scales.float().repeat_interleave(128, dim=1)
+    assert ((w.float() - lin.weight.float()).abs() <= 1.01 * step).all()
+
+
+@pytest.mark.gpu
+def test_swapped_trunk_tracks_the_dequantised_trunk():
+    """int4 modules vs the same model running nn.Linear on the dequantised weights: one decode
+    step with a KV cache, as the reference drives the trunk (policy.py:673-678)."""
+    dev = "cuda:0"
+    policy = StubPolicy()
+    policy.mmgpt.to(dev)
+    policy.mmgpt.language_model.model.to(dev)
+    reference = StubPolicy()
+    reference.mmgpt.to(dev)
+    reference.mmgpt.language_model.model.to(dev)
+    reference._lm_trunk().load_state_dict(policy._lm_trunk().state_dict())
+    reference.mmgpt.gen_head.load_state_dict(policy.mmgpt.gen_head.state_dict())
+
+    apply_int4_to_policy(policy, group_size=128)
+    # give the reference copy the dequantised weights
+    for lq, lr in zip(policy._lm_trunk().layers, reference._lm_trunk().layers):
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            getattr(lr.self_attn, name).weight.data.copy_(getattr(lq.self_attn, name).dequantize())
+        gu = lq.mlp.gate_up
+        from visionrl_amd import ops
+        w = ops.int4_dequant(gu.qweight, gu.scales, gu.qzeros, gu.group_size)
+        lr.mlp.gate_proj.weight.data.copy_(w[:INTER])
+        lr.mlp.up_proj.weight.data.copy_(w[INTER:])
+        lr.mlp.down_proj.weight.data.copy_(lq.mlp.down_proj.dequantize())
+    reference.mmgpt.gen_head.weight.data.copy_(policy.mmgpt.gen_head.dequantize())
+
+    torch.manual_seed(3)
+    prompt = torch.randn(2, 6, HIDDEN, device=dev).to(torch.bfloat16) * 0.5
+    step = torch.randn(2, 1, HIDDEN, device=dev).to(torch.bfloat16) * 0.5
+    outs = []
+    with torch.no_grad():
+        for pol in (policy, reference):
+            trunk = pol._lm_trunk()
+            pre = trunk(inputs_embeds=prompt, use_cache=True)
+            dec = trunk(inputs_embeds=step, past_key_values=pre.past_key_values, use_cache=True)
+            logits = pol._base().gen_head(dec.last_hidden_state[:, -1:, :])
+            outs.append((pre.last_hidden_state.float(), dec.last_hidden_state.float(), logits.float()))
+    for a, b in zip(outs[0], outs[1]):
+        assert a.shape == b.shape
+        assert torch.isfinite(a).all()
+        # same weights, bf16 activations everywhere: only accumulation order and the fused
+        # fp32 SiLU epilogue differ
+        assert (a - b).abs().max() <= 0.05 * b.abs().max() + 1e-3
+    assert outs[0][2].shape == (2, 1, VOCAB_IMG)

@@ -436,7 +436,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_tile_kernel(DevProblem p) {
 // activations in LDS once, then each wave streams whole tiles - no K split, so
 // no partial sums to meet - keeping STREAM_DEPTH 128-k chunks of its 16 rows in
 // flight (non-temporal global_load_dwordx4: the weights are read exactly once).
-constexpr int STREAM_WPB = 8;
+constexpr int STREAM_WPB = 4;
 constexpr int STREAM_DEPTH = 4;
 
 template <int RS>
@@ -1196,7 +1196,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
 
     // one contiguous tile range per workgroup, balanced by streamed bytes
     int per_cu = (int)(LDS_PER_CU / (smem ? smem : 1));
-    if (per_cu > 4) per_cu = 4;
+    if (per_cu > 5) per_cu = 5;  // 20 waves per CU is what the register budget of the kernels allows
     if (per_cu < 1) per_cu = 1;
     long grid = (long)device_cu_count() * per_cu;
     if (grid > MAX_PLAN_GRID) grid = MAX_PLAN_GRID;
