@@ -31,6 +31,8 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "../../include/vrl_int4.h"
 
 namespace {
@@ -755,79 +757,85 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
                 (long)(tile_local + r * out_tiles) * tile_u4 + lane;
         wp[r] = mp[r] + meta_u4 + (long)sc0 * 256;
     }
-    const int nld = (sc1 - sc0) * 4;
-    u32x4_t ring[STREAM_DEPTH][RS];
+    static_assert(STREAM_DEPTH == 4, "the ring holds exactly one super-chunk (four loads per lane)");
+    u32x4_t ring[4][RS];
     u32x4_t mt[RS];
     PPGroup grp[RS];
 #pragma unroll
-    for (int d = 0; d < STREAM_DEPTH; ++d)
-        if (d < nld) {
+    for (int d = 0; d < 4; ++d)
 #pragma unroll
-            for (int r = 0; r < RS; ++r) ring[d][r] = __builtin_nontemporal_load(wp[r] + d * 64);
-        }
+        for (int r = 0; r < RS; ++r) ring[d][r] = __builtin_nontemporal_load(wp[r] + d * 64);
 #pragma unroll
     for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc0 >> 2) * 64];
 
-    for (int l0 = 0; l0 < nld; l0 += STREAM_DEPTH) {
+    // one super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside;
+    // REFILL says whether the ring is topped up from the following super-chunk
+    auto super_chunk = [&](int sc, auto refill) {
+        constexpr bool REFILL = decltype(refill)::value;
 #pragma unroll
-        for (int d = 0; d < STREAM_DEPTH; ++d) {
-            const int ld = l0 + d;
-            if (ld < nld) {
-                const int sc = sc0 + (ld >> 2);
-                const int j = ld & 3;
-                if (j == 0) {
-                    if (ld != 0 && (sc & 3) == 0) {
+        for (int r = 0; r < RS; ++r) {
+            const int e = sc & 3;
+            const uint32_t mw = e == 0 ? mt[r][0] : (e == 1 ? mt[r][1] : (e == 2 ? mt[r][2] : mt[r][3]));
+            grp[r] = pp_group(mw, j4);
+        }
+        const long nxt = (long)(sc + 1 - sc0) * 256;
 #pragma unroll
-                        for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
-                    }
+        for (int d = 0; d < 4; ++d) {
+            u32x4_t w[RS];
 #pragma unroll
-                    for (int r = 0; r < RS; ++r) {
-                        const int e = sc & 3;
-                        const uint32_t mw = e == 0 ? mt[r][0] : (e == 1 ? mt[r][1] : (e == 2 ? mt[r][2] : mt[r][3]));
-                        grp[r] = pp_group(mw, j4);
-                    }
+            for (int r = 0; r < RS; ++r) w[r] = ring[d][r];
+            if (REFILL) {
+#pragma unroll
+                for (int r = 0; r < RS; ++r)
+                    ring[d][r] = __builtin_nontemporal_load(wp[r] + nxt + d * 64);
+            }
+            const int kloc = (sc - sc0) * PP_SC + kq * 128 + d * 32;
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                bf16x8_t xa[MB];
+#pragma unroll
+                for (int b = 0; b < MB; ++b) {
+                    const int m = min(16 * b + lc, p.M - 1);
+                    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
+                    xa[b] = __builtin_bit_cast(bf16x8_t, raw);
                 }
-                u32x4_t w[RS];
 #pragma unroll
-                for (int r = 0; r < RS; ++r) w[r] = ring[d][r];
-                if (ld + STREAM_DEPTH < nld) {
+                for (int r = 0; r < RS; ++r) {
+                    const uint32_t v = w[r][dd];
+                    u32x2_t a0, a1;
+                    a0[0] = (v & mask) | bias;
+                    a0[1] = ((v >> 4) & mask) | bias;
+                    a1[0] = ((v >> 8) & mask) | bias;
+                    a1[1] = ((v >> 12) & mask) | bias;
+                    const f32x4_t d0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                        __builtin_bit_cast(bf16x4_t, a0), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                    const f32x4_t d1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                        __builtin_bit_cast(bf16x4_t, a1), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                    const u32x4_t wv = {pack_bf16_rne(d0[0], d0[1]), pack_bf16_rne(d0[2], d0[3]),
+                                        pack_bf16_rne(d1[0], d1[1]), pack_bf16_rne(d1[2], d1[3])};
+                    const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
 #pragma unroll
-                    for (int r = 0; r < RS; ++r)
-                        ring[d][r] = __builtin_nontemporal_load(wp[r] + (ld + STREAM_DEPTH) * 64);
-                }
-                const int kloc = (sc - sc0) * PP_SC + kq * 128 + j * 32;
-#pragma unroll
-                for (int dd = 0; dd < 4; ++dd) {
-                    bf16x8_t xa[MB];
-#pragma unroll
-                    for (int b = 0; b < MB; ++b) {
-                        const int m = min(16 * b + lc, p.M - 1);
-                        const u32x4_t raw =
-                            *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
-                        xa[b] = __builtin_bit_cast(bf16x8_t, raw);
-                    }
-#pragma unroll
-                    for (int r = 0; r < RS; ++r) {
-                        const uint32_t v = w[r][dd];
-                        u32x2_t a0, a1;
-                        a0[0] = (v & mask) | bias;
-                        a0[1] = ((v >> 4) & mask) | bias;
-                        a1[0] = ((v >> 8) & mask) | bias;
-                        a1[1] = ((v >> 12) & mask) | bias;
-                        const f32x4_t d0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
-                            __builtin_bit_cast(bf16x4_t, a0), grp[r].bdiag, grp[r].cq, 0, 0, 0);
-                        const f32x4_t d1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
-                            __builtin_bit_cast(bf16x4_t, a1), grp[r].bdiag, grp[r].cq, 0, 0, 0);
-                        const u32x4_t wv = {pack_bf16_rne(d0[0], d0[1]), pack_bf16_rne(d0[2], d0[3]),
-                                            pack_bf16_rne(d1[0], d1[1]), pack_bf16_rne(d1[2], d1[3])};
-                        const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
-#pragma unroll
-                        for (int b = 0; b < MB; ++b)
-                            acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
-                    }
+                    for (int b = 0; b < MB; ++b)
+                        acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
                 }
             }
         }
+    };
+
+    for (int sc = sc0; sc < sc1 - 1; ++sc) {
+        if (sc != sc0 && (sc & 3) == 0) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
+        }
+        super_chunk(sc, std::true_type{});
+    }
+    {
+        const int sc = sc1 - 1;
+        if (sc != sc0 && (sc & 3) == 0) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
+        }
+        super_chunk(sc, std::false_type{});
     }
 }
 
