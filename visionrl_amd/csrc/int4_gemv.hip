@@ -42,6 +42,14 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
+// Pointers read out of a plan record lose their address space; loads through these
+// typedefs are global_load (vmcnt only) instead of flat_load (vmcnt and lgkmcnt).
+typedef const __attribute__((address_space(1))) u32x4_t *gptr_u4;
+
+__device__ __forceinline__ gptr_u4 as_global(const u32x4_t *p) {
+    return (gptr_u4)(uintptr_t)p;
+}
+
 constexpr int WAVE = 64;
 constexpr int KCHUNK = 128;          // k covered by one wave step (4 lanes x 32 k per row)
 constexpr uint32_t PAIR_MASK = 0x000F000Fu;
@@ -749,11 +757,11 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
     asm volatile("" : "+s"(mask));
     asm volatile("" : "+v"(bias));
 
-    const u32x4_t *mp[RS];
-    const u32x4_t *wp[RS];
+    gptr_u4 mp[RS];
+    gptr_u4 wp[RS];
 #pragma unroll
     for (int r = 0; r < RS; ++r) {
-        mp[r] = reinterpret_cast<const u32x4_t *>(p.qweight) +
+        mp[r] = as_global(reinterpret_cast<const u32x4_t *>(p.qweight)) +
                 (long)(tile_local + r * out_tiles) * tile_u4 + lane;
         wp[r] = mp[r] + meta_u4 + (long)sc0 * 256;
     }
