@@ -282,8 +282,13 @@ PP_SHAPES = [
     (3, 640, 50, False),        # ragged N and K
     (16, 2048, 256, False), (16, 5632, 64, False),   # the second needs staged passes
     (7, 11008, 96, False),      # 21.5 super-chunks
-    (20, 1024, 48, False),      # two slabs of activation rows
+    (20, 1024, 48, False),      # 17..32 rows: two MFMA row blocks per weight tile
+    (32, 2048, 512, False),     # rollout batch, x staged whole in a 16-wave workgroup
+    (32, 5632, 96, False),      # rollout batch with staged passes over K
+    (40, 512, 32, False),       # more than 32 rows: two records
+    (12, 4096, 64, False),      # 8-wave workgroups
     (1, 2048, 2 * 5632, True), (8, 4096, 2 * 704, True), (16, 1024, 2 * 48, True),
+    (32, 2048, 2 * 64, True),
 ]
 
 

@@ -446,7 +446,6 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_tile_kernel(DevProblem p) {
 // activations in LDS once, then each wave streams whole tiles - no K split, so
 // no partial sums to meet - keeping STREAM_DEPTH 128-k chunks of its 16 rows in
 // flight (non-temporal global_load_dwordx4: the weights are read exactly once).
-constexpr int STREAM_WPB = 4;
 constexpr int STREAM_DEPTH = 4;
 
 template <int RS>
@@ -891,7 +890,10 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 
 // CANON / PP / FUSED say which kinds of record the plan holds, so that a plan of
 // plain prepacked GEMVs runs the variant with the smallest register footprint.
-template <int WPB, bool CANON, bool PP, bool FUSED>
+// WPB (waves per workgroup) grows with the LDS the staged activations need, so that
+// about 16 waves stay resident per CU; MB = 2 carries up to 32 activation rows per
+// record with two A operands per weight tile (weights streamed once).
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
                                                                 const int32_t *__restrict__ block_begin,
                                                                 int n_problems) {
@@ -911,11 +913,11 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
         if (PP && (!CANON || p.prepacked)) {
-            if (FUSED && p.fused) stream_segment_pp<1, FUSED, WPB>(p, a, b, smem);
-            else stream_segment_pp<1, false, WPB>(p, a, b, smem);
+            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB>(p, a, b, smem);
+            else stream_segment_pp<MB, false, WPB>(p, a, b, smem);
         } else if (CANON) {
-            if (FUSED && p.fused) stream_segment<1, FUSED, WPB>(p, a, b, smem);
-            else stream_segment<1, false, WPB>(p, a, b, smem);
+            if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
+            else stream_segment<MB, false, WPB>(p, a, b, smem);
         }
         t = seg_end;
     }
@@ -925,11 +927,13 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
 // host side
 // -------------------------------------------------------------------------
 constexpr int TILE_WPB = 8;
-constexpr int MAX_TILE_M = 16;                  // activation rows one record / launch takes
+constexpr int MAX_TILE_M = 16;                  // activation rows one single-launch slab / canonical record takes
+constexpr int MAX_PP_M = 32;                    // activation rows a prepacked record of a grouped plan takes
 constexpr size_t LDS_X_BUDGET = 40 * 1024;      // split kernel: staged activations per workgroup
 constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // split kernel: shorter staged extents are multiples of this
-constexpr size_t STREAM_X_SINGLE = 72 * 1024;   // stream kernel: all of K staged if it fits this
-constexpr size_t STREAM_X_PASS = 36 * 1024;     // stream kernel: staged bytes per pass otherwise
+// stream kernel: workgroup shapes by the LDS the staged activations need
+struct StreamShape { int wpb; int per_cu; size_t lds; };
+constexpr StreamShape STREAM_SHAPES[3] = {{4, 5, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -949,7 +953,7 @@ bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 // shapes the MFMA kernels take; everything else goes to the generic kernel
 bool tile_path_ok(const DevProblem &p) {
-    return p.K % KCHUNK == 0 && p.G % 32 == 0 && pow2(p.G) && p.M <= MAX_TILE_M;
+    return p.K % KCHUNK == 0 && p.G % 32 == 0 && pow2(p.G) && p.M <= (p.prepacked ? MAX_PP_M : MAX_TILE_M);
 }
 
 // split kernel: k extent of x staged per pass, all of K when M rows of it fit the budget,
@@ -962,10 +966,10 @@ int staged_k(int M, int K) {
     return (int)(kc < K ? kc : K);
 }
 
-// stream kernel: all of K if it fits, else passes that are multiples of KCHUNK
-int stream_staged_k(int M, int K) {
-    if ((size_t)M * (K + XPAD) * 2 <= STREAM_X_SINGLE) return K;
-    long kc = (long)(STREAM_X_PASS / ((size_t)M * 2)) - XPAD;
+// stream kernel, canonical records: all of K if it fits `lds`, else passes that are multiples of KCHUNK
+int stream_staged_k(int M, int K, size_t lds) {
+    if ((size_t)M * (K + XPAD) * 2 <= lds) return K;
+    long kc = (long)(lds / ((size_t)M * 2)) - XPAD;
     kc -= kc % KCHUNK;
     if (kc < KCHUNK) kc = KCHUNK;
     return (int)(kc < K ? kc : K);
@@ -974,11 +978,11 @@ int stream_staged_k(int M, int K) {
 // prepacked blobs exist for group size 128 only
 bool prepack_ok(long N, long K, long G) { return G == 128 && K % 128 == 0 && N >= 1 && N * K < (1L << 40); }
 
-// prepacked stream: all of the padded K if it fits, else whole super-chunks per pass
-int pp_staged_k(int M, int K) {
+// stream kernel, prepacked records: all of the padded K if it fits, else whole super-chunks per pass
+int pp_staged_k(int M, int K, size_t lds) {
     const int kpad = pp_nsc(K) * PP_SC;
-    if ((size_t)M * (kpad + XPAD) * 2 <= STREAM_X_SINGLE) return kpad;
-    long kc = (long)(STREAM_X_PASS / ((size_t)M * 2)) - XPAD;
+    if ((size_t)M * (kpad + XPAD) * 2 <= lds) return kpad;
+    long kc = (long)(lds / ((size_t)M * 2)) - XPAD;
     kc -= kc % PP_SC;
     if (kc < PP_SC) kc = PP_SC;
     return (int)kc;
@@ -1067,21 +1071,36 @@ struct PlanHeader {
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
-constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4;
+constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8;
 
-template <bool CANON, bool PP, bool FUSED>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED>
 int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *block_begin,
                   hipStream_t stream) {
-    auto kernel = &gemv_stream_kernel<STREAM_WPB, CANON, PP, FUSED>;
+    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED>;
     if (info->lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(STREAM_WPB * WAVE), (size_t)info->lds_bytes,
+    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes,
                        stream, recs, block_begin, info->n_problems);
     return (int)hipGetLastError();
 }
+
+// which record kinds a kernel build must handle, for a given workgroup shape
+template <int WPB, int MB>
+int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *bb,
+                          hipStream_t stream) {
+    const int v = info->variant & (VARIANT_CANON | VARIANT_PP | VARIANT_FUSED);
+    if (v == VARIANT_PP) return launch_stream<WPB, MB, false, true, false>(info, recs, bb, stream);
+    if (v == (VARIANT_PP | VARIANT_FUSED)) return launch_stream<WPB, MB, false, true, true>(info, recs, bb, stream);
+    if constexpr (MB == 1 && WPB != 8) {  // canonical records: narrow and widest workgroups only
+        if (v & VARIANT_FUSED) return launch_stream<WPB, 1, true, true, true>(info, recs, bb, stream);
+        return launch_stream<WPB, 1, true, true, false>(info, recs, bb, stream);
+    }
+    return VRL_INT4_EPLAN;
+}
+
 
 size_t plan_bytes_for(int n_records) {
     return sizeof(PlanHeader) + (size_t)n_records * sizeof(DevProblem) +
@@ -1170,8 +1189,8 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
 
     long tiles = 0;
     double total_cost = 0.0;
-    size_t smem = 0;
     int variant = 0;
+    size_t x_need = 0;  // bytes the largest activation matrix needs if staged whole
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
         variant |= (q.prepacked ? VARIANT_PP : VARIANT_CANON) | (q.fused_gate_up ? VARIANT_FUSED : 0);
@@ -1193,30 +1212,47 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         p.fused = q.fused_gate_up ? 1 : 0;
         p.prepacked = q.prepacked ? 1 : 0;
         if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take MFMA-path shapes only
-        if (p.prepacked) {
-            if (!prepack_ok(p.N, p.K, p.G) || (p.fused && (p.N / 2) % 16 != 0)) return VRL_INT4_ESHAPE;
-            p.kc = pp_staged_k(p.M, p.K);
-        } else {
-            p.kc = stream_staged_k(p.M, p.K);
-        }
+        if (p.prepacked && (!prepack_ok(p.N, p.K, p.G) || (p.fused && (p.N / 2) % 16 != 0)))
+            return VRL_INT4_ESHAPE;
+        if (p.M > MAX_TILE_M) variant |= VARIANT_MB2;
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const long nt = (out_cols + 15) / 16;
         tiles += nt;
         if (tiles >= (1L << 30)) return VRL_INT4_ESHAPE;
         total_cost += (double)nt * ((double)p.K * (p.fused ? 2 : 1) + 512.0);
+        const int kfull = p.prepacked ? pp_nsc(p.K) * PP_SC : p.K;
+        const size_t need = (size_t)p.M * (kfull + XPAD) * 2;
+        if (need > x_need) x_need = need;
+        recs[i] = p;
+    }
+    // more than 16 activation rows per record: prepacked-only plans (two A operands per tile)
+    if ((variant & VARIANT_MB2) && (variant & VARIANT_CANON)) return VRL_INT4_ESHAPE;
+
+    // workgroup shape: the narrowest whose LDS holds the largest activation matrix whole
+    // (plans with canonical or 32-row records have no 8-wave build); the widest one otherwise,
+    // walking K in staged passes
+    int shape = 2;
+    for (int i = 0; i < 3; ++i) {
+        if (x_need > STREAM_SHAPES[i].lds) continue;
+        if (i == 1 && (variant & VARIANT_CANON)) continue;
+        shape = i;
+        break;
+    }
+    if (variant & VARIANT_MB2) shape = 2;
+    const StreamShape sh = STREAM_SHAPES[shape];
+    size_t smem = 0;
+    for (int i = 0; i < n_problems; ++i) {
+        DevProblem &p = recs[i];
+        p.kc = p.prepacked ? pp_staged_k(p.M, p.K, sh.lds) : stream_staged_k(p.M, p.K, sh.lds);
         const size_t need = (size_t)p.M * (p.kc + XPAD) * 2;
         if (need > smem) smem = need;
-        recs[i] = p;
     }
 
     // one contiguous tile range per workgroup, balanced by streamed bytes
-    int per_cu = (int)(LDS_PER_CU / (smem ? smem : 1));
-    if (per_cu > 5) per_cu = 5;  // 20 waves per CU is what the register budget of the kernels allows
-    if (per_cu < 1) per_cu = 1;
-    long grid = (long)device_cu_count() * per_cu;
+    long grid = (long)device_cu_count() * sh.per_cu;
     if (grid > MAX_PLAN_GRID) grid = MAX_PLAN_GRID;
-    const long max_useful = (tiles + STREAM_WPB - 1) / STREAM_WPB;
+    const long max_useful = (tiles + sh.wpb - 1) / sh.wpb;
     if (grid > max_useful) grid = max_useful;
     {
         int b = 0;
@@ -1252,7 +1288,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     info->n_problems = n_problems;
     info->total_tiles = (int)tiles;
     info->grid = (int)grid;
-    info->block_threads = STREAM_WPB * WAVE;
+    info->block_threads = sh.wpb * WAVE;
     info->lds_bytes = (int)smem;
     info->variant = variant;
     return VRL_INT4_OK;
@@ -1262,20 +1298,20 @@ int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *i
                                void *hip_stream) {
     if (!plan_dev || !info) return VRL_INT4_ENULL;
     if (info->n_problems < 1 || info->total_tiles < 1 || info->grid < 1 ||
-        info->grid > MAX_PLAN_GRID || info->block_threads != STREAM_WPB * WAVE ||
-        info->lds_bytes < 0 || (size_t)info->lds_bytes > LDS_PER_CU || !aligned16(plan_dev))
+        info->grid > MAX_PLAN_GRID || info->lds_bytes < 0 || (size_t)info->lds_bytes > LDS_PER_CU ||
+        !aligned16(plan_dev))
         return VRL_INT4_EPLAN;
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
     const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + sizeof(PlanHeader));
     const int32_t *block_begin = reinterpret_cast<const int32_t *>(recs + info->n_problems);
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    switch (info->variant) {
-        case VARIANT_PP: return launch_stream<false, true, false>(info, recs, block_begin, stream);
-        case VARIANT_PP | VARIANT_FUSED: return launch_stream<false, true, true>(info, recs, block_begin, stream);
-        case VARIANT_CANON: return launch_stream<true, false, false>(info, recs, block_begin, stream);
-        case VARIANT_CANON | VARIANT_FUSED: return launch_stream<true, false, true>(info, recs, block_begin, stream);
-        case VARIANT_CANON | VARIANT_PP: return launch_stream<true, true, false>(info, recs, block_begin, stream);
-        case VARIANT_CANON | VARIANT_PP | VARIANT_FUSED: return launch_stream<true, true, true>(info, recs, block_begin, stream);
+    const bool mb2 = (info->variant & VARIANT_MB2) != 0;
+    switch (info->block_threads) {
+        case 4 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<4, 1>(info, recs, block_begin, stream);
+        case 8 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<8, 1>(info, recs, block_begin, stream);
+        case 16 * WAVE:
+            return mb2 ? launch_stream_variant<16, 2>(info, recs, block_begin, stream)
+                       : launch_stream_variant<16, 1>(info, recs, block_begin, stream);
         default: return VRL_INT4_EPLAN;
     }
 }

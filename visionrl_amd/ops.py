@@ -168,7 +168,8 @@ class GroupedGemv:
     are alive and not reallocated.
     """
 
-    MAX_ROWS = 16  # activation rows one record of the plan may carry
+    MAX_ROWS = 16            # activation rows one canonical record of the plan may carry
+    MAX_ROWS_PREPACKED = 32  # ... and one prepacked record (two MFMA row blocks per weight tile)
 
     def __init__(self, problems):
         if not problems:
@@ -206,9 +207,10 @@ class GroupedGemv:
             y = torch.empty((M, N // 2 if fused else N), dtype=torch.bfloat16, device=dev)
             self._keep.append(keep)
             self.outputs.append(y)
-            # one record per slab of MAX_ROWS activation rows (row slices stay contiguous)
-            for m0 in range(0, M, self.MAX_ROWS):
-                m1 = min(M, m0 + self.MAX_ROWS)
+            # one record per slab of activation rows (row slices stay contiguous)
+            rows = self.MAX_ROWS_PREPACKED if prepacked else self.MAX_ROWS
+            for m0 in range(0, M, rows):
+                m1 = min(M, m0 + rows)
                 records.append((x[m0:m1].data_ptr(), *ptrs, y[m0:m1].data_ptr(), m1 - m0, N, K,
                                 int(group_size), 1 if fused else 0, prepacked))
         n = len(records)
