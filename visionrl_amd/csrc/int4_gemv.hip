@@ -855,10 +855,16 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
     const int nsc = pp_nsc(p.K);
     const int sc_pass = p.kc / PP_SC;
     if (sc_pass >= nsc) {
+        // Tiles of the segment are handed out through a counter in LDS: waves on one SIMD do
+        // not progress at equal rates (older waves win the issue arbitration), and with a
+        // fixed deal the workgroup would wait at the next barrier for its slowest wave.
+        __shared__ int next_tile;
         __syncthreads();
+        if (threadIdx.x == 0) next_tile = t0 + WPB;
         stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
         __syncthreads();
-        for (int tile = t0 + wave; tile < t1; tile += WPB) {
+        int tile = t0 + wave;
+        while (tile < t1) {
             f32x4_t acc[RS][MB];
 #pragma unroll
             for (int r = 0; r < RS; ++r)
@@ -866,6 +872,9 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
                 for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, 0, nsc, acc);
             store_tile<MB, FUSED>(p, tile, acc);
+            int nt = 0;
+            if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
+            tile = __builtin_amdgcn_readfirstlane(nt);
         }
     } else {
         for (int round = t0; round < t1; round += WPB) {
@@ -933,7 +942,9 @@ constexpr size_t LDS_X_BUDGET = 40 * 1024;      // split kernel: staged activati
 constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // split kernel: shorter staged extents are multiples of this
 // stream kernel: workgroup shapes by the LDS the staged activations need
 struct StreamShape { int wpb; int per_cu; size_t lds; };
-constexpr StreamShape STREAM_SHAPES[3] = {{4, 5, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
+// {waves per workgroup, workgroups per CU, LDS it may use}; the narrow shape is launched with twice
+// the resident number of workgroups so that the hardware dispatcher evens out the tail
+constexpr StreamShape STREAM_SHAPES[3] = {{4, 10, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
