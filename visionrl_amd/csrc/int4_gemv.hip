@@ -942,9 +942,9 @@ constexpr size_t LDS_X_BUDGET = 40 * 1024;      // split kernel: staged activati
 constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // split kernel: shorter staged extents are multiples of this
 // stream kernel: workgroup shapes by the LDS the staged activations need
 struct StreamShape { int wpb; int per_cu; size_t lds; };
-// {waves per workgroup, workgroups per CU, LDS it may use}; the narrow shape is launched with twice
-// the resident number of workgroups so that the hardware dispatcher evens out the tail
-constexpr StreamShape STREAM_SHAPES[3] = {{4, 10, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
+// {waves per workgroup, workgroups per CU, LDS it may use}; the narrow shape is launched with three
+// times the resident number of workgroups (5 per CU) so that the hardware dispatcher evens out the tail
+constexpr StreamShape STREAM_SHAPES[3] = {{4, 15, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
