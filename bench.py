@@ -172,11 +172,30 @@ def per_call_latency(items, steps: int):
     for it in items:
         shapes.setdefault((it["K"], it["N"]), []).append(it)
     for (K, N), group in shapes.items():
-        def rotate():
+        outs = [torch.empty((it["x"].shape[0], N), dtype=torch.bfloat16, device=it["x"].device)
+                for it in group]
+
+        def rotate_op():
             for it in group:
                 ops.int4_gemv(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP)
-        ms = time_region(rotate, max(2, steps // 50), 1) / len(group)
-        res[f"{K}x{N}"] = {"us_per_call": ms * 1e3, "GBps": group[0]["bytes"] / (ms * 1e-3) / 1e9,
+
+        def rotate_direct():
+            for it, y in zip(group, outs):
+                ops.int4_gemv_into(y, it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP)
+
+        graph = torch.cuda.CUDAGraph()
+        rotate_direct()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            rotate_direct()
+        reps = max(2, steps // 50)
+        ms_op = time_region(rotate_op, reps, 1) / len(group)
+        ms_direct = time_region(rotate_direct, reps, 1) / len(group)
+        ms_graph = time_region(graph.replay, max(5, steps // 10), 2) / len(group)
+        res[f"{K}x{N}"] = {"us_per_call_torch_op": ms_op * 1e3,
+                           "us_per_call_direct": ms_direct * 1e3,
+                           "us_per_call_hip_graph": ms_graph * 1e3,
+                           "GBps_hip_graph": group[0]["bytes"] / (ms_graph * 1e-3) / 1e9,
                            "distinct_weights": len(group)}
     return res
 

@@ -324,6 +324,12 @@ __device__ __forceinline__ void tile_body(const DevProblem &p, int tile, uint8_t
         return g;
     };
 
+    // the first chunk of weights does not depend on x: request it before staging, so that a
+    // small matrix costs one memory round trip instead of two
+    Prefetch<R> cur, nxt;
+    int g_cur = 0, g_nxt = 0;
+    if (wave * KCHUNK < min(kc, K)) g_cur = issue(wave, cur);
+
     for (int kbase = 0; kbase < K; kbase += kc) {
         const int kext = min(kc, K - kbase);
         // ---- stage x[:, kbase : kbase+kext] into LDS, pair-interleaved per 8 k ----
@@ -349,9 +355,7 @@ __device__ __forceinline__ void tile_body(const DevProblem &p, int tile, uint8_t
         const int c_begin = kbase / KCHUNK;
         const int c_end = (kbase + kext) / KCHUNK;
         int chunk = c_begin + wave;
-        Prefetch<R> cur, nxt;
-        int g_cur = 0, g_nxt = 0;
-        if (chunk < c_end) g_cur = issue(chunk, cur);
+        if (kbase != 0 && chunk < c_end) g_cur = issue(chunk, cur);
         for (; chunk < c_end; chunk += WPB) {
             const bool more = chunk + WPB < c_end;
             if (more) g_nxt = issue(chunk + WPB, nxt);

@@ -79,7 +79,11 @@ class Int4Linear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
-        y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        if torch.compiler.is_compiling():
+            y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
+            y = torch.empty((rows.shape[0], self.out_features), dtype=torch.bfloat16, device=rows.device)
+            ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*x.shape[:-1], self.out_features)

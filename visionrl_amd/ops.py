@@ -22,8 +22,8 @@ import torch
 from . import _lib
 from .int4_format import check_packed
 
-__all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_prepack", "PrepackedWeight",
-           "GroupedGemv"]
+__all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
+           "PrepackedWeight", "GroupedGemv"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -74,6 +74,40 @@ def int4_gemv(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
 @int4_gemv.register_fake
 def _(x, qweight, scales, qzeros, group_size):
     return x.new_empty((x.shape[0], qweight.shape[0]))
+
+
+def int4_gemv_into(y: torch.Tensor, x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+                   qzeros: torch.Tensor, group_size: int) -> torch.Tensor:
+    """Lean eager form of ``int4_gemv``: writes into a caller-provided ``y[M,N]``.
+
+    No allocation and no operator dispatch, for decode loops that call the same
+    layer thousands of times; shapes and dtypes are still checked (by the
+    library for the shape rules, here for the rest).
+    """
+    if x.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or scales.dtype != torch.bfloat16:
+        raise TypeError("x, y and scales must be bfloat16")
+    if qweight.dtype != torch.int32 or qzeros.dtype != torch.int32:
+        raise TypeError("qweight and qzeros must be int32")
+    if x.dim() != 2 or y.dim() != 2 or qweight.dim() != 2:
+        raise ValueError("x, y and qweight must be 2-D")
+    M, K = x.shape
+    N = qweight.shape[0]
+    if qweight.shape[1] * 8 != K or tuple(y.shape) != (M, N):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, qweight {tuple(qweight.shape)}, y {tuple(y.shape)}")
+    groups = K // int(group_size) if group_size else 0
+    if tuple(scales.shape) != (N, groups) or tuple(qzeros.shape) != (N, (groups + 7) // 8):
+        raise ValueError("scales / qzeros do not match qweight and group_size")
+    dev = x.device
+    for name, t in (("x", x), ("y", y), ("qweight", qweight), ("scales", scales), ("qzeros", qzeros)):
+        if t.device != dev or dev.type != "cuda":
+            raise ValueError(f"{name} must live on the same ROCm device; the int4 operators have no CPU path")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+    rc = _lib.load().vrl_int4_gemv_bf16(x.data_ptr(), qweight.data_ptr(), scales.data_ptr(),
+                                        qzeros.data_ptr(), y.data_ptr(), M, N, K, int(group_size),
+                                        _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_gemv_bf16")
+    return y
 
 
 @torch.library.custom_op("vrl_hip::int4_dequant", mutates_args=())
