@@ -251,6 +251,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true",
                     help="run just the grouped decode-step launches (for profilers)")
+    ap.add_argument("--single-calls", action="store_true",
+                    help="loop single-GEMV launches over distinct weights per shape and exit (for profilers)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run plain 1 GiB device copies and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -270,6 +272,19 @@ def main():
         print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "copies": args.steps}))
         return
     from visionrl_amd import ops
+
+    if args.single_calls:
+        for M in (1, 32):
+            for K, N in ((HIDDEN, HIDDEN), (HIDDEN, INTER), (INTER, HIDDEN), (HIDDEN, HEAD)):
+                ws = [make_weights(100 + i, K, N, GROUP, device) for i in range(40)]
+                x = make_x(1, M, K, device)
+                y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+                for _ in range(3):
+                    for qw, sc, qz in ws:
+                        ops.int4_gemv_into(y, x, qw, sc, qz, GROUP)
+                torch.cuda.synchronize()
+        print(json.dumps({"single_calls": "done"}))
+        return
 
     items = build_set(2, 1, device, with_head=False)
     torch.cuda.synchronize()
