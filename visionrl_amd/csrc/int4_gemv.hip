@@ -850,7 +850,7 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
     }
 }
 
-template <int MB, bool FUSED, int WPB>
+template <int MB, bool FUSED, int WPB, bool PASSES>
 __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = threadIdx.x >> 6;
@@ -858,7 +858,7 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
     const int xstride = p.kc + XPAD;
     const int nsc = pp_nsc(p.K);
     const int sc_pass = p.kc / PP_SC;
-    if (sc_pass >= nsc) {
+    if (!PASSES || sc_pass >= nsc) {
         // Tiles of the segment are handed out through a counter in LDS: waves on one SIMD do
         // not progress at equal rates (older waves win the issue arbitration), and with a
         // fixed deal the workgroup would wait at the next barrier for its slowest wave.
@@ -880,23 +880,34 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
             if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
             tile = __builtin_amdgcn_readfirstlane(nt);
         }
-    } else {
-        for (int round = t0; round < t1; round += WPB) {
-            const int tile = round + wave;
-            const bool active = tile < t1;
-            f32x4_t acc[RS][MB];
+    } else if constexpr (PASSES) {
+        // activations do not fit: K is walked in staged passes, and every wave carries T tiles
+        // through a pass so that one staging serves T * WPB tiles
+        constexpr int T = FUSED ? 1 : (MB == 2 ? 2 : 4);
+        for (int round = t0; round < t1; round += WPB * T) {
+            f32x4_t acc[T][RS][MB];
 #pragma unroll
-            for (int r = 0; r < RS; ++r)
+            for (int i = 0; i < T; ++i)
 #pragma unroll
-                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                for (int r = 0; r < RS; ++r)
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) acc[i][r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             for (int sc0 = 0; sc0 < nsc; sc0 += sc_pass) {
                 const int sc1 = min(nsc, sc0 + sc_pass);
                 __syncthreads();
                 stage_x_natural(p, sc0 * PP_SC, sc1 * PP_SC, xs, xstride, WPB * WAVE);
                 __syncthreads();
-                if (active) stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, sc0, sc1, acc);
+#pragma unroll
+                for (int i = 0; i < T; ++i) {
+                    const int tile = round + i * WPB + wave;  // neighbouring waves, neighbouring tiles
+                    if (tile < t1) stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, sc0, sc1, acc[i]);
+                }
             }
-            if (active) store_tile<MB, FUSED>(p, tile, acc);
+#pragma unroll
+            for (int i = 0; i < T; ++i) {
+                const int tile = round + i * WPB + wave;
+                if (tile < t1) store_tile<MB, FUSED>(p, tile, acc[i]);
+            }
         }
     }
 }
@@ -905,8 +916,10 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // plain prepacked GEMVs runs the variant with the smallest register footprint.
 // WPB (waves per workgroup) grows with the LDS the staged activations need, so that
 // about 16 waves stay resident per CU; MB = 2 carries up to 32 activation rows per
-// record with two A operands per weight tile (weights streamed once).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED>
+// record with two A operands per weight tile (weights streamed once); PASSES adds the
+// path for prepacked records whose activations do not fit LDS whole (it carries several
+// accumulator tiles, so plans that do not need it run a build without it).
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
                                                                 const int32_t *__restrict__ block_begin,
                                                                 int n_problems) {
@@ -926,8 +939,8 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
         if (PP && (!CANON || p.prepacked)) {
-            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB>(p, a, b, smem);
-            else stream_segment_pp<MB, false, WPB>(p, a, b, smem);
+            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES>(p, a, b, smem);
+            else stream_segment_pp<MB, false, WPB, PASSES>(p, a, b, smem);
         } else if (CANON) {
             if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
             else stream_segment<MB, false, WPB>(p, a, b, smem);
@@ -1086,12 +1099,12 @@ struct PlanHeader {
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
-constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8;
+constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16;
 
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
 int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *block_begin,
                   hipStream_t stream) {
-    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED>;
+    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES>;
     if (info->lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
@@ -1107,11 +1120,23 @@ template <int WPB, int MB>
 int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *bb,
                           hipStream_t stream) {
     const int v = info->variant & (VARIANT_CANON | VARIANT_PP | VARIANT_FUSED);
-    if (v == VARIANT_PP) return launch_stream<WPB, MB, false, true, false>(info, recs, bb, stream);
-    if (v == (VARIANT_PP | VARIANT_FUSED)) return launch_stream<WPB, MB, false, true, true>(info, recs, bb, stream);
+    const bool passes = (info->variant & VARIANT_PASSES) != 0;
+    if (v == VARIANT_PP) {
+        // only the widest workgroups ever need passes: narrower shapes are chosen because x fits
+        if constexpr (WPB == 16) {
+            if (passes) return launch_stream<WPB, MB, false, true, false, true>(info, recs, bb, stream);
+        }
+        return launch_stream<WPB, MB, false, true, false, false>(info, recs, bb, stream);
+    }
+    if (v == (VARIANT_PP | VARIANT_FUSED)) {
+        if constexpr (WPB == 16) {
+            if (passes) return launch_stream<WPB, MB, false, true, true, true>(info, recs, bb, stream);
+        }
+        return launch_stream<WPB, MB, false, true, true, false>(info, recs, bb, stream);
+    }
     if constexpr (MB == 1 && WPB != 8) {  // canonical records: narrow and widest workgroups only
-        if (v & VARIANT_FUSED) return launch_stream<WPB, 1, true, true, true>(info, recs, bb, stream);
-        return launch_stream<WPB, 1, true, true, false>(info, recs, bb, stream);
+        if (v & VARIANT_FUSED) return launch_stream<WPB, 1, true, true, true, WPB == 16>(info, recs, bb, stream);
+        return launch_stream<WPB, 1, true, true, false, WPB == 16>(info, recs, bb, stream);
     }
     return VRL_INT4_EPLAN;
 }
@@ -1262,6 +1287,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         p.kc = p.prepacked ? pp_staged_k(p.M, p.K, sh.lds) : stream_staged_k(p.M, p.K, sh.lds);
         const size_t need = (size_t)p.M * (p.kc + XPAD) * 2;
         if (need > smem) smem = need;
+        if (p.prepacked && p.kc < pp_nsc(p.K) * PP_SC) variant |= VARIANT_PASSES;
     }
 
     // one contiguous tile range per workgroup, balanced by streamed bytes
