@@ -46,9 +46,16 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 // typedefs are global_load (vmcnt only) instead of flat_load (vmcnt and lgkmcnt).
 typedef const __attribute__((address_space(1))) u32x4_t *gptr_u4;
 
+typedef __attribute__((address_space(1))) uint16_t *gptr_u16;
+typedef const __attribute__((address_space(1))) uint16_t *gptr_cu16;
+typedef const __attribute__((address_space(1))) uint32_t *gptr_cu32;
+
 __device__ __forceinline__ gptr_u4 as_global(const u32x4_t *p) {
     return (gptr_u4)(uintptr_t)p;
 }
+__device__ __forceinline__ gptr_u16 as_global(uint16_t *p) { return (gptr_u16)(uintptr_t)p; }
+__device__ __forceinline__ gptr_cu16 as_global(const uint16_t *p) { return (gptr_cu16)(uintptr_t)p; }
+__device__ __forceinline__ gptr_cu32 as_global(const uint32_t *p) { return (gptr_cu32)(uintptr_t)p; }
 
 constexpr int WAVE = 64;
 constexpr int KCHUNK = 128;          // k covered by one wave step (4 lanes x 32 k per row)
@@ -466,7 +473,7 @@ __device__ __forceinline__ void stage_x(const DevProblem &p, int kbase, int kext
     for (int idx = threadIdx.x; idx < total; idx += nthreads) {
         const int m = idx / words_per_row;
         const int j = idx - m * words_per_row;
-        const u32x4_t d = *reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + kbase + (j << 3));
+        const u32x4_t d = *as_global(reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + kbase + (j << 3)));
         u32x4_t o;
         o[0] = (d[0] & 0xFFFFu) | (d[2] << 16);      // x0, x4
         o[1] = (d[0] >> 16) | (d[2] & 0xFFFF0000u);  // x1, x5
@@ -490,15 +497,15 @@ __device__ __forceinline__ void stream_rows(const DevProblem &p, int tile_local,
     const int zwords = (groups + 7) >> 3;
     const int out_cols = FUSED ? p.N / 2 : p.N;
 
-    const uint32_t *wp[RS];
-    const uint16_t *sp[RS];
-    const uint32_t *zp[RS];
+    gptr_cu32 wp[RS];
+    gptr_cu16 sp[RS];
+    gptr_cu32 zp[RS];
 #pragma unroll
     for (int r = 0; r < RS; ++r) {
         const long row = (long)r * out_cols + min(tile_local * 16 + lc, out_cols - 1);
-        wp[r] = p.qweight + row * kwords + (kbase >> 3) + 4 * kq;
-        sp[r] = p.scales + row * groups;
-        zp[r] = p.qzeros + row * zwords;
+        wp[r] = as_global(p.qweight) + row * kwords + (kbase >> 3) + 4 * kq;
+        sp[r] = as_global(p.scales) + row * groups;
+        zp[r] = as_global(p.qzeros) + row * zwords;
     }
     const int nch = kext >> 7;
     const uint32_t bias = PAIR_BIAS;
@@ -508,7 +515,7 @@ __device__ __forceinline__ void stream_rows(const DevProblem &p, int tile_local,
         const int g = (kbase + c * KCHUNK + 32 * kq) >> gshift;
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
-            s.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(wp[r] + c * 16));
+            s.w[r] = __builtin_nontemporal_load((gptr_u4)(wp[r] + c * 16));
             s.sbits[r] = sp[r][g];
             s.zword[r] = zp[r][g >> 3];
         }
@@ -572,7 +579,9 @@ __device__ __forceinline__ void store_tile(const DevProblem &p, int tile_local,
             if (m < p.M) {
                 float v = acc[0][b][i];
                 if (FUSED) v = (v / (1.0f + __expf(-v))) * acc[FUSED ? 1 : 0][b][i];
-                p.y[(long)m * out_cols + col] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+                // a global (not flat) store: a pending flat access makes every later wait on
+                // the load counter a wait for zero
+                as_global(p.y)[(long)m * out_cols + col] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
             }
         }
 }
@@ -717,7 +726,7 @@ __device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int
         const int j = idx - m * words_per_row;
         const int k = k0 + (j << 3);
         u32x4_t d = {0u, 0u, 0u, 0u};
-        if (k < p.K) d = *reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k);
+        if (k < p.K) d = *as_global(reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k));
         *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = d;
     }
 }
@@ -769,37 +778,30 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
         wp[r] = mp[r] + meta_u4 + (long)sc0 * 256;
     }
     static_assert(STREAM_DEPTH == 4, "the ring holds exactly one super-chunk (four loads per lane)");
+    // meta word of this lane for super-chunk sc: dword (sc % 4) of the lane's 16 bytes in block sc / 4
+    auto meta_ptr = [&](int r, int sc) { return (gptr_cu32)mp[r] + (long)(sc >> 2) * 256 + (sc & 3); };
     u32x4_t ring[4][RS];
-    u32x4_t mt[RS];
+    uint32_t mnext[RS];
     PPGroup grp[RS];
+#pragma unroll
+    for (int r = 0; r < RS; ++r) mnext[r] = *meta_ptr(r, sc0);
 #pragma unroll
     for (int d = 0; d < 4; ++d)
 #pragma unroll
         for (int r = 0; r < RS; ++r) ring[d][r] = __builtin_nontemporal_load(wp[r] + d * 64);
-#pragma unroll
-    for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc0 >> 2) * 64];
 
-    // one super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside;
-    // REFILL says whether the ring is topped up from the following super-chunk
+    // One super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside.
+    // REFILL: each ring slot is reloaded from the following super-chunk as soon as its last
+    // word is consumed, and the next meta word rides with slot 0.  The scheduling barriers
+    // pin the loads there: left alone, the scheduler gathers them at the end of the body and
+    // the wave then waits out a whole memory latency per super-chunk.
     auto super_chunk = [&](int sc, auto refill) {
         constexpr bool REFILL = decltype(refill)::value;
 #pragma unroll
-        for (int r = 0; r < RS; ++r) {
-            const int e = sc & 3;
-            const uint32_t mw = e == 0 ? mt[r][0] : (e == 1 ? mt[r][1] : (e == 2 ? mt[r][2] : mt[r][3]));
-            grp[r] = pp_group(mw, j4);
-        }
+        for (int r = 0; r < RS; ++r) grp[r] = pp_group(mnext[r], j4);
         const long nxt = (long)(sc + 1 - sc0) * 256;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            u32x4_t w[RS];
-#pragma unroll
-            for (int r = 0; r < RS; ++r) w[r] = ring[d][r];
-            if (REFILL) {
-#pragma unroll
-                for (int r = 0; r < RS; ++r)
-                    ring[d][r] = __builtin_nontemporal_load(wp[r] + nxt + d * 64);
-            }
             const int kloc = (sc - sc0) * PP_SC + kq * 128 + d * 32;
 #pragma unroll
             for (int dd = 0; dd < 4; ++dd) {
@@ -812,7 +814,7 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
                 }
 #pragma unroll
                 for (int r = 0; r < RS; ++r) {
-                    const uint32_t v = w[r][dd];
+                    const uint32_t v = ring[d][r][dd];
                     u32x2_t a0, a1;
                     a0[0] = (v & mask) | bias;
                     a0[1] = ((v >> 4) & mask) | bias;
@@ -830,24 +832,20 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
                         acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
                 }
             }
+            if (REFILL) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < RS; ++r) {
+                    if (d == 0) mnext[r] = *meta_ptr(r, sc + 1);
+                    ring[d][r] = __builtin_nontemporal_load(wp[r] + nxt + d * 64);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
-    for (int sc = sc0; sc < sc1 - 1; ++sc) {
-        if (sc != sc0 && (sc & 3) == 0) {
-#pragma unroll
-            for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
-        }
-        super_chunk(sc, std::true_type{});
-    }
-    {
-        const int sc = sc1 - 1;
-        if (sc != sc0 && (sc & 3) == 0) {
-#pragma unroll
-            for (int r = 0; r < RS; ++r) mt[r] = mp[r][(long)(sc >> 2) * 64];
-        }
-        super_chunk(sc, std::false_type{});
-    }
+    for (int sc = sc0; sc < sc1 - 1; ++sc) super_chunk(sc, std::true_type{});
+    super_chunk(sc1 - 1, std::false_type{});
 }
 
 template <int MB, bool FUSED, int WPB, bool PASSES>
