@@ -87,7 +87,8 @@ int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void
  * glue: runs once per weight after the policy is built (the reference builds
  * its policy at vrl/models/families/janus_pro/builder.py:11-33).
  * vrl_int4_prepacked_bytes() is the blob size (0 if the shape has no prepacked
- * form: G != 128 or K % 128 != 0); the blob needs 16-byte alignment.  The
+ * form: G != 128, K % 128 != 0, or a blob of 2 GiB or more); the blob needs
+ * 16-byte alignment.  The
  * arithmetic contract is unchanged: the weights a kernel rebuilds from the blob
  * are bit for bit the canonical dequantised tile.
  */

@@ -749,57 +749,102 @@ __device__ __forceinline__ PPGroup pp_group(uint32_t meta_word, int j4) {
     return g;
 }
 
-// acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob;
-// xs holds x for exactly that k range
+// Per-wave stream state of the prepacked path: four 16-byte loads per lane in flight (one
+// super-chunk) and the meta word that goes with them.
+template <int RS>
+struct PPRing {
+    u32x4_t slot[4][RS];
+    uint32_t meta[RS];
+};
+
+// The prepacked blob is read through a buffer resource: uniform base and size in SGPRs, one
+// VGPR (16 * lane) as the per-lane offset for every load, the tile / super-chunk position as
+// a scalar offset.  Reads past the blob return zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int BUFFER_NT = 2;  // cache-policy bit: non-temporal (streamed once)
+
+__device__ __forceinline__ rsrc_t pp_blob_rsrc(const DevProblem &p) {
+    const uint32_t bytes = (uint32_t)((p.N + 15) / 16) * (uint32_t)(pp_tile_u4(p.K) * 16);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.qweight), 0, (int)bytes, 0x00020000);
+}
+
+template <bool FUSED>
+struct PPTilePtr {
+    uint32_t words[FUSED ? 2 : 1];  // byte offset of the tile's super-chunk sc0 (16 bytes per lane follow)
+    uint32_t meta[FUSED ? 2 : 1];   // byte offset of lane 0's meta word of super-chunk sc0
+};
+
+// where tile `tile_local` of the blob starts, at super-chunk sc0
+template <bool FUSED>
+__device__ __forceinline__ PPTilePtr<FUSED> pp_tile_ptr(const DevProblem &p, int tile_local, int sc0) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const uint32_t meta_bytes = (uint32_t)pp_meta_u4(p.K) * 16u;
+    const uint32_t tile_bytes = (uint32_t)pp_tile_u4(p.K) * 16u;
+    const int out_tiles = (FUSED ? p.N / 2 : p.N + 15) / 16;
+    PPTilePtr<FUSED> t;
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        const uint32_t base = (uint32_t)(tile_local + r * out_tiles) * tile_bytes;
+        t.words[r] = base + meta_bytes + (uint32_t)sc0 * 4096u;
+        // meta word of super-chunk sc: dword (sc % 4) of the lane's 16 bytes in block sc / 4
+        t.meta[r] = base + (uint32_t)(sc0 >> 2) * 1024u + (uint32_t)(sc0 & 3) * 4u;
+    }
+    return t;
+}
+
+// the five loads of one super-chunk: meta word, then four 16-byte slots; slot d alone when
+// called with that d, so that a refill can follow each slot's last use
+template <bool FUSED>
+__device__ __forceinline__ void pp_load_slot(rsrc_t rsrc, uint32_t voff, const uint32_t (&words)[FUSED ? 2 : 1],
+                                             const uint32_t (&meta)[FUSED ? 2 : 1], int d,
+                                             PPRing<FUSED ? 2 : 1> &ring) {
+    constexpr int RS = FUSED ? 2 : 1;
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        if (d == 0) ring.meta[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, meta[r], 0);
+        ring.slot[d][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + d * 1024, words[r], BUFFER_NT);
+    }
+}
+
+// issue the loads of a tile's first super-chunk
+template <bool FUSED>
+__device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t, PPRing<FUSED ? 2 : 1> &ring) {
+    const uint32_t voff = (threadIdx.x & (WAVE - 1)) * 16u;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED>(rsrc, voff, t.words, t.meta, d, ring);
+}
+
+// acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob; xs holds x
+// for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
+// if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
+// never runs dry between tiles.
 template <int MB, bool FUSED>
-__device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_local, const uint16_t *xs,
-                                               int xstride, int sc0, int sc1,
+__device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
+                                               int next_tile, const uint16_t *xs, int xstride,
+                                               int sc0, int sc1, PPRing<FUSED ? 2 : 1> &ring,
                                                f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
     constexpr int RS = FUSED ? 2 : 1;
     const int lane = threadIdx.x & (WAVE - 1);
     const int lc = lane & 15;
     const int kq = lane >> 4;
     const int j4 = lane & 3;
-    const long meta_u4 = pp_meta_u4(p.K);
-    const long tile_u4 = pp_tile_u4(p.K);
-    const int out_tiles = (FUSED ? p.N / 2 : p.N + 15) / 16;
 
     // both must sit in registers for (v & mask) | bias to select v_and_or_b32
     uint32_t mask = PAIR_MASK, bias = PAIR_BIAS;
     asm volatile("" : "+s"(mask));
     asm volatile("" : "+v"(bias));
 
-    gptr_u4 mp[RS];
-    gptr_u4 wp[RS];
-#pragma unroll
-    for (int r = 0; r < RS; ++r) {
-        mp[r] = as_global(reinterpret_cast<const u32x4_t *>(p.qweight)) +
-                (long)(tile_local + r * out_tiles) * tile_u4 + lane;
-        wp[r] = mp[r] + meta_u4 + (long)sc0 * 256;
-    }
     static_assert(STREAM_DEPTH == 4, "the ring holds exactly one super-chunk (four loads per lane)");
-    // meta word of this lane for super-chunk sc: dword (sc % 4) of the lane's 16 bytes in block sc / 4
-    auto meta_ptr = [&](int r, int sc) { return (gptr_cu32)mp[r] + (long)(sc >> 2) * 256 + (sc & 3); };
-    u32x4_t ring[4][RS];
-    uint32_t mnext[RS];
     PPGroup grp[RS];
-#pragma unroll
-    for (int r = 0; r < RS; ++r) mnext[r] = *meta_ptr(r, sc0);
-#pragma unroll
-    for (int d = 0; d < 4; ++d)
-#pragma unroll
-        for (int r = 0; r < RS; ++r) ring[d][r] = __builtin_nontemporal_load(wp[r] + d * 64);
 
     // One super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside.
-    // REFILL: each ring slot is reloaded from the following super-chunk as soon as its last
-    // word is consumed, and the next meta word rides with slot 0.  The scheduling barriers
-    // pin the loads there: left alone, the scheduler gathers them at the end of the body and
-    // the wave then waits out a whole memory latency per super-chunk.
-    auto super_chunk = [&](int sc, auto refill) {
-        constexpr bool REFILL = decltype(refill)::value;
+    // Each ring slot is reloaded from offset rw (and the meta word from rm, with slot 0) as
+    // soon as its last word is consumed.  The scheduling barriers pin the loads there: left alone,
+    // the scheduler gathers them at the end of the body and the wave then waits out a whole
+    // memory latency per super-chunk.
+    auto super_chunk = [&](int sc, uint32_t rv, const uint32_t (&rw)[RS], const uint32_t (&rm)[RS]) {
 #pragma unroll
-        for (int r = 0; r < RS; ++r) grp[r] = pp_group(mnext[r], j4);
-        const long nxt = (long)(sc + 1 - sc0) * 256;
+        for (int r = 0; r < RS; ++r) grp[r] = pp_group(ring.meta[r], j4);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             const int kloc = (sc - sc0) * PP_SC + kq * 128 + d * 32;
@@ -814,7 +859,7 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
                 }
 #pragma unroll
                 for (int r = 0; r < RS; ++r) {
-                    const uint32_t v = ring[d][r][dd];
+                    const uint32_t v = ring.slot[d][r][dd];
                     u32x2_t a0, a1;
                     a0[0] = (v & mask) | bias;
                     a0[1] = ((v >> 4) & mask) | bias;
@@ -832,26 +877,38 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, int tile_loc
                         acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
                 }
             }
-            if (REFILL) {
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int r = 0; r < RS; ++r) {
-                    if (d == 0) mnext[r] = *meta_ptr(r, sc + 1);
-                    ring[d][r] = __builtin_nontemporal_load(wp[r] + nxt + d * 64);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            __builtin_amdgcn_sched_barrier(0);
+            pp_load_slot<FUSED>(rsrc, rv, rw, rm, d, ring);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    for (int sc = sc0; sc < sc1 - 1; ++sc) super_chunk(sc, std::true_type{});
-    super_chunk(sc1 - 1, std::false_type{});
+    // After the last super-chunk the ring is refilled from the next tile's first one.  With no
+    // next tile it is refilled all the same, every lane from the 16 bytes of lane 0 in this
+    // tile (a single cache line per load, contents unused), so that the loop body exists once
+    // and has no branch.
+    const bool has_next = next_tile >= 0;
+    const PPTilePtr<FUSED> nxt = pp_tile_ptr<FUSED>(p, has_next ? next_tile : 0, sc0);
+    const uint32_t voff = lane * 16u;
+    for (int sc = sc0; sc < sc1; ++sc) {
+        const bool last = sc + 1 == sc1;
+        uint32_t rw[RS], rm[RS];
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            const uint32_t w_same = cur.words[r] + (uint32_t)(sc + 1 - sc0) * 4096u;
+            const uint32_t m_same = cur.meta[r] + (uint32_t)((((sc + 1) >> 2) - (sc0 >> 2)) * 1024 +
+                                                             (((sc + 1) & 3) - (sc0 & 3)) * 4);
+            rw[r] = last ? (has_next ? nxt.words[r] : cur.words[r]) : w_same;
+            rm[r] = last ? (has_next ? nxt.meta[r] : cur.meta[r]) : m_same;
+        }
+        super_chunk(sc, (last && !has_next) ? 0u : voff, rw, rm);
+    }
 }
 
 template <int MB, bool FUSED, int WPB, bool PASSES>
 __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     constexpr int RS = FUSED ? 2 : 1;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile offsets stay scalar
     uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
     const int xstride = p.kc + XPAD;
     const int nsc = pp_nsc(p.K);
@@ -860,28 +917,37 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
         // Tiles of the segment are handed out through a counter in LDS: waves on one SIMD do
         // not progress at equal rates (older waves win the issue arbitration), and with a
         // fixed deal the workgroup would wait at the next barrier for its slowest wave.
+        // A wave draws its next tile before it starts the current one, so that the last
+        // super-chunk of a tile already pulls in the first of the next.
         __shared__ int next_tile;
+        int tile = t0 + wave;
+        PPRing<RS> ring;
+        const rsrc_t rsrc = pp_blob_rsrc(p);
+        PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile < t1 ? tile : t0, 0);
+        if (tile < t1) pp_prime<FUSED>(rsrc, cur, ring);  // weights are on their way while x is staged
         __syncthreads();
         if (threadIdx.x == 0) next_tile = t0 + WPB;
         stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
         __syncthreads();
-        int tile = t0 + wave;
         while (tile < t1) {
+            int nt = 0;
+            if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
+            nt = __builtin_amdgcn_readfirstlane(nt);
             f32x4_t acc[RS][MB];
 #pragma unroll
             for (int r = 0; r < RS; ++r)
 #pragma unroll
                 for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, 0, nsc, acc);
+            stream_rows_pp<MB, FUSED>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
             store_tile<MB, FUSED>(p, tile, acc);
-            int nt = 0;
-            if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
-            tile = __builtin_amdgcn_readfirstlane(nt);
+            tile = nt;
+            if (tile < t1) cur = pp_tile_ptr<FUSED>(p, tile, 0);
         }
     } else if constexpr (PASSES) {
         // activations do not fit: K is walked in staged passes, and every wave carries T tiles
         // through a pass so that one staging serves T * WPB tiles
         constexpr int T = FUSED ? 1 : (MB == 2 ? 2 : 4);
+        const rsrc_t rsrc = pp_blob_rsrc(p);
         for (int round = t0; round < t1; round += WPB * T) {
             f32x4_t acc[T][RS][MB];
 #pragma unroll
@@ -898,7 +964,12 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 #pragma unroll
                 for (int i = 0; i < T; ++i) {
                     const int tile = round + i * WPB + wave;  // neighbouring waves, neighbouring tiles
-                    if (tile < t1) stream_rows_pp<MB, FUSED>(p, tile, xs, xstride, sc0, sc1, acc[i]);
+                    if (tile < t1) {
+                        PPRing<RS> ring;
+                        const PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile, sc0);
+                        pp_prime<FUSED>(rsrc, cur, ring);
+                        stream_rows_pp<MB, FUSED>(p, rsrc, cur, -1, xs, xstride, sc0, sc1, ring, acc[i]);
+                    }
                 }
             }
 #pragma unroll
@@ -1002,7 +1073,11 @@ int stream_staged_k(int M, int K, size_t lds) {
 }
 
 // prepacked blobs exist for group size 128 only
-bool prepack_ok(long N, long K, long G) { return G == 128 && K % 128 == 0 && N >= 1 && N * K < (1L << 40); }
+// the stream kernel addresses a blob with 32-bit byte offsets, so a blob stays below 2 GiB
+bool prepack_ok(long N, long K, long G) {
+    if (G != 128 || K % 128 != 0 || N < 1 || K < 128 || N * K >= (1L << 40)) return false;
+    return ((N + 15) / 16) * pp_tile_u4((int)K) * 16 < (1L << 31);
+}
 
 // stream kernel, prepacked records: all of the padded K if it fits, else whole super-chunks per pass
 int pp_staged_k(int M, int K, size_t lds) {
