@@ -113,12 +113,16 @@ def test_grouped_plan_validation(lib):
     assert info.total_tiles == 4 + 7        # 16-column tiles: 64/16 and ceil(100/16)
     assert 1 <= info.grid <= info.total_tiles and info.block_threads % 64 == 0
     assert info.lds_bytes >= 1 * (256 + 8) * 2
-    # the per-workgroup tile ranges stored after the records cover every tile exactly once
+    # the per-workgroup table stored after the records ({first tile, its record} per workgroup)
+    # covers every tile exactly once, and names the record each range starts in
     import struct
     rec_bytes = 72   # 5 pointers + 8 int32 per record
-    begins = struct.unpack_from(f"{info.grid + 1}i", plan.raw, 16 + 2 * rec_bytes)
+    table = struct.unpack_from(f"{2 * (info.grid + 1)}i", plan.raw, 16 + 2 * rec_bytes)
+    begins, first_rec = table[0::2], table[1::2]
     assert begins[0] == 0 and begins[-1] == info.total_tiles
     assert all(a <= b for a, b in zip(begins, begins[1:]))
+    # records are laid out longest tiles first (equal K here: caller order kept), record 1 starts at tile 4
+    assert all(r == (1 if b >= 4 else 0) for b, r in zip(begins, first_rec))
     # undersized buffer, bad shape inside the list, shapes only the generic kernel takes, nulls
     assert lib.vrl_int4_grouped_plan_build(probs, 2, plan, size - 1, ctypes.byref(info)) == 1004
     probs[1].K = 100

@@ -31,7 +31,9 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <algorithm>
 #include <type_traits>
+#include <vector>
 
 #include "../../include/vrl_int4.h"
 
@@ -990,18 +992,15 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // accumulator tiles, so plans that do not need it run a build without it).
 template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
-                                                                const int32_t *__restrict__ block_begin,
+                                                                const int2 *__restrict__ block_tab,
                                                                 int n_problems) {
     extern __shared__ __align__(16) uint8_t smem[];
-    int t = block_begin[blockIdx.x];
-    const int t_end = block_begin[blockIdx.x + 1];
+    // block_tab[b] = {first tile of workgroup b, record that tile belongs to}
+    const int2 entry = block_tab[blockIdx.x];
+    int t = entry.x;
+    const int t_end = block_tab[blockIdx.x + 1].x;
     if (t >= t_end) return;  // block-uniform
-    // largest i with plan[i].tile_begin <= t
-    int lo = 0, hi = n_problems - 1;
-    while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (plan[mid].tile_begin <= t) lo = mid; else hi = mid - 1;
-    }
+    const int lo = entry.y;
     for (int pi = lo; t < t_end && pi < n_problems; ++pi) {
         const DevProblem p = plan[pi];
         const int out_cols = p.fused ? p.N / 2 : p.N;
@@ -1162,7 +1161,7 @@ int run_rows(const void *x, const void *qw, const void *sc, const void *qz, void
     return VRL_INT4_OK;
 }
 
-// Plan blob: [PlanHeader][DevProblem x n_records][int32 block_begin x (grid + 1)]
+// Plan blob: [PlanHeader][DevProblem x n_records][int2 {first tile, its record} x (MAX_PLAN_GRID + 1)]
 struct PlanHeader {
     uint32_t magic;
     int32_t n_records;
@@ -1175,7 +1174,7 @@ constexpr int MAX_PLAN_GRID = 4096;
 constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16;
 
 template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
-int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *block_begin,
+int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
                   hipStream_t stream) {
     auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES>;
     if (info->lds_bytes > 64 * 1024) {
@@ -1190,7 +1189,7 @@ int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const 
 
 // which record kinds a kernel build must handle, for a given workgroup shape
 template <int WPB, int MB>
-int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs, const int32_t *bb,
+int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb,
                           hipStream_t stream) {
     const int v = info->variant & (VARIANT_CANON | VARIANT_PP | VARIANT_FUSED);
     const bool passes = (info->variant & VARIANT_PASSES) != 0;
@@ -1217,7 +1216,7 @@ int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs
 
 size_t plan_bytes_for(int n_records) {
     return sizeof(PlanHeader) + (size_t)n_records * sizeof(DevProblem) +
-           (size_t)(MAX_PLAN_GRID + 1) * sizeof(int32_t);
+           (size_t)(MAX_PLAN_GRID + 1) * sizeof(int2);
 }
 
 }  // namespace
@@ -1298,7 +1297,8 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     if (n_problems < 1 || plan_bytes < vrl_int4_grouped_plan_size(n_problems)) return VRL_INT4_EPLAN;
     uint8_t *base = static_cast<uint8_t *>(plan_host);
     DevProblem *recs = reinterpret_cast<DevProblem *>(base + sizeof(PlanHeader));
-    int32_t *block_begin = reinterpret_cast<int32_t *>(recs + n_problems);
+    int2 *block_tab = reinterpret_cast<int2 *>(recs + n_problems);
+    std::vector<int32_t> block_begin((size_t)MAX_PLAN_GRID + 1, 0);
 
     long tiles = 0;
     double total_cost = 0.0;
@@ -1338,6 +1338,18 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         const size_t need = (size_t)p.M * (kfull + XPAD) * 2;
         if (need > x_need) x_need = need;
         recs[i] = p;
+    }
+    // Records go into the blob longest tiles first (the kernel only needs tile_begin to ascend
+    // with the record index): the ranges that start last then hold the shortest tiles.
+    {
+        std::stable_sort(recs, recs + n_problems, [](const DevProblem &a, const DevProblem &b) {
+            return (long)a.K * (a.fused ? 2 : 1) > (long)b.K * (b.fused ? 2 : 1);
+        });
+        long t = 0;
+        for (int i = 0; i < n_problems; ++i) {
+            recs[i].tile_begin = (int)t;
+            t += ((recs[i].fused ? recs[i].N / 2 : recs[i].N) + 15) / 16;
+        }
     }
     // more than 16 activation rows per record: prepacked-only plans (two A operands per tile)
     if ((variant & VARIANT_MB2) && (variant & VARIANT_CANON)) return VRL_INT4_ESHAPE;
@@ -1390,6 +1402,11 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             ++b;
             block_begin[b] = (int)tiles;
         }
+        int rec = 0;
+        for (long k = 0; k <= grid; ++k) {
+            while (rec + 1 < n_problems && recs[rec + 1].tile_begin <= block_begin[(size_t)k]) ++rec;
+            block_tab[k] = make_int2(block_begin[(size_t)k], rec);
+        }
     }
 
     PlanHeader hdr;
@@ -1417,7 +1434,7 @@ int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *i
         return VRL_INT4_EPLAN;
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
     const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + sizeof(PlanHeader));
-    const int32_t *block_begin = reinterpret_cast<const int32_t *>(recs + info->n_problems);
+    const int2 *block_begin = reinterpret_cast<const int2 *>(recs + info->n_problems);
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const bool mb2 = (info->variant & VARIANT_MB2) != 0;
     switch (info->block_threads) {
