@@ -87,9 +87,9 @@ def test_null_and_alignment_are_reported(lib):
 def test_prepacked_size_and_validation(lib):
     keep, p = buf(4096)
     # per 16-row tile: ceil(nsc/4) KiB of scale/zero words + nsc * 4 KiB of weights, nsc = ceil(K/512)
-    assert lib.vrl_int4_prepacked_bytes(2048, 2048, 128) == 128 * (1024 + 4 * 4096)
-    assert lib.vrl_int4_prepacked_bytes(2048, 5632, 128) == 128 * (3 * 1024 + 11 * 4096)
-    assert lib.vrl_int4_prepacked_bytes(17, 128, 128) == 2 * (1024 + 4096)
+    assert lib.vrl_int4_prepacked_bytes(2048, 2048, 128) == 128 * (4 * 256 + 4 * 4096)
+    assert lib.vrl_int4_prepacked_bytes(2048, 5632, 128) == 128 * (11 * 256 + 11 * 4096)
+    assert lib.vrl_int4_prepacked_bytes(17, 128, 128) == 2 * (256 + 4096)
     assert lib.vrl_int4_prepacked_bytes(16, 256, 64) == 0
     assert lib.vrl_int4_prepacked_bytes(16, 200, 128) == 0
     assert lib.vrl_int4_prepack(p, p, p, None, 16, 128, 128, None) == 1003

@@ -638,8 +638,8 @@ __device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int 
 // blob a wave can stream with fully contiguous 1 KB loads and dequantise almost
 // without VALU work.  Group size 128 only.  Per 16-row tile, K padded to 512:
 //
-//   [meta  : ceil(nsc/4) x 64 lanes x 16 B]   word e of lane l in block mb is
-//            (scale bits << 16) | zero  of row (l % 16), group 4*(4*mb+e) + l/16
+//   [meta  : nsc x 64 lanes x 4 B]            the word of super-chunk sc and lane l is
+//            (scale bits << 16) | zero  of row (l % 16), group 4*sc + l/16
 //   [words : nsc x 4 x 64 lanes x 16 B]       super-chunk sc, load j, lane l, dword d
 //
 // with l = 16*kq + 4*rq + i.  Nibble nu of a weight dword holds
@@ -656,7 +656,7 @@ __device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int 
 constexpr int PP_SC = 512;  // k per super-chunk: lane group kq owns one 128-k scale group
 
 __host__ __device__ inline int pp_nsc(int K) { return (K + PP_SC - 1) / PP_SC; }
-__host__ __device__ inline long pp_meta_u4(int K) { return (long)((pp_nsc(K) + 3) / 4) * 64; }
+__host__ __device__ inline long pp_meta_u4(int K) { return (long)pp_nsc(K) * 16; }  // 64 words per super-chunk
 __host__ __device__ inline long pp_tile_u4(int K) { return pp_meta_u4(K) + (long)pp_nsc(K) * 4 * 64; }
 
 __global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict__ qweight,
@@ -676,12 +676,13 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict
         const long rem = idx - tile * tile_u4;
         u32x4_t out = {0u, 0u, 0u, 0u};
         if (rem < meta_u4) {
-            const int mb = (int)(rem >> 6);
-            const int lane = (int)(rem & 63);
-            const long row = tile * 16 + (lane & 15);
+            // meta word of (super-chunk sc, lane): row lane % 16 of the tile, group 4 * sc + lane / 16
+            const int sc = (int)(rem >> 4);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int g = 4 * (4 * mb + e) + (lane >> 4);
+                const int lane = 4 * (int)(rem & 15) + e;
+                const long row = tile * 16 + (lane & 15);
+                const int g = 4 * sc + (lane >> 4);
                 if (row < N && g < groups) {
                     const uint32_t sb = scales[row * groups + g];
                     const uint32_t z = (qzeros[row * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xFu;
@@ -764,6 +765,7 @@ struct PPRing {
 // a scalar offset.  Reads past the blob return zero instead of faulting.
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int BUFFER_NT = 2;  // cache-policy bit: non-temporal (streamed once)
+constexpr uint32_t PP_OUT_OF_RANGE = 0x7FFF0000u;  // a per-lane offset no blob reaches (blobs stay below this)
 
 __device__ __forceinline__ rsrc_t pp_blob_rsrc(const DevProblem &p) {
     const uint32_t bytes = (uint32_t)((p.N + 15) / 16) * (uint32_t)(pp_tile_u4(p.K) * 16);
@@ -773,7 +775,7 @@ __device__ __forceinline__ rsrc_t pp_blob_rsrc(const DevProblem &p) {
 template <bool FUSED>
 struct PPTilePtr {
     uint32_t words[FUSED ? 2 : 1];  // byte offset of the tile's super-chunk sc0 (16 bytes per lane follow)
-    uint32_t meta[FUSED ? 2 : 1];   // byte offset of lane 0's meta word of super-chunk sc0
+    uint32_t meta[FUSED ? 2 : 1];   // byte offset of super-chunk sc0's 64 meta words (4 bytes per lane follow)
 };
 
 // where tile `tile_local` of the blob starts, at super-chunk sc0
@@ -788,8 +790,7 @@ __device__ __forceinline__ PPTilePtr<FUSED> pp_tile_ptr(const DevProblem &p, int
     for (int r = 0; r < RS; ++r) {
         const uint32_t base = (uint32_t)(tile_local + r * out_tiles) * tile_bytes;
         t.words[r] = base + meta_bytes + (uint32_t)sc0 * 4096u;
-        // meta word of super-chunk sc: dword (sc % 4) of the lane's 16 bytes in block sc / 4
-        t.meta[r] = base + (uint32_t)(sc0 >> 2) * 1024u + (uint32_t)(sc0 & 3) * 4u;
+        t.meta[r] = base + (uint32_t)sc0 * 256u;
     }
     return t;
 }
@@ -797,13 +798,14 @@ __device__ __forceinline__ PPTilePtr<FUSED> pp_tile_ptr(const DevProblem &p, int
 // the five loads of one super-chunk: meta word, then four 16-byte slots; slot d alone when
 // called with that d, so that a refill can follow each slot's last use
 template <bool FUSED>
-__device__ __forceinline__ void pp_load_slot(rsrc_t rsrc, uint32_t voff, const uint32_t (&words)[FUSED ? 2 : 1],
+__device__ __forceinline__ void pp_load_slot(rsrc_t rsrc, uint32_t voff, uint32_t mvoff,
+                                             const uint32_t (&words)[FUSED ? 2 : 1],
                                              const uint32_t (&meta)[FUSED ? 2 : 1], int d,
                                              PPRing<FUSED ? 2 : 1> &ring) {
     constexpr int RS = FUSED ? 2 : 1;
 #pragma unroll
     for (int r = 0; r < RS; ++r) {
-        if (d == 0) ring.meta[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, meta[r], 0);
+        if (d == 0) ring.meta[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, mvoff, meta[r], 0);
         ring.slot[d][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + d * 1024, words[r], BUFFER_NT);
     }
 }
@@ -813,7 +815,7 @@ template <bool FUSED>
 __device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t, PPRing<FUSED ? 2 : 1> &ring) {
     const uint32_t voff = (threadIdx.x & (WAVE - 1)) * 16u;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED>(rsrc, voff, t.words, t.meta, d, ring);
+    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED>(rsrc, voff, voff >> 2, t.words, t.meta, d, ring);
 }
 
 // acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob; xs holds x
@@ -844,7 +846,8 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
     // soon as its last word is consumed.  The scheduling barriers pin the loads there: left alone,
     // the scheduler gathers them at the end of the body and the wave then waits out a whole
     // memory latency per super-chunk.
-    auto super_chunk = [&](int sc, uint32_t rv, const uint32_t (&rw)[RS], const uint32_t (&rm)[RS]) {
+    auto super_chunk = [&](int sc, uint32_t rv, uint32_t rmv, const uint32_t (&rw)[RS],
+                           const uint32_t (&rm)[RS]) {
 #pragma unroll
         for (int r = 0; r < RS; ++r) grp[r] = pp_group(ring.meta[r], j4);
 #pragma unroll
@@ -880,15 +883,15 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            pp_load_slot<FUSED>(rsrc, rv, rw, rm, d, ring);
+            pp_load_slot<FUSED>(rsrc, rv, rmv, rw, rm, d, ring);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
     // After the last super-chunk the ring is refilled from the next tile's first one.  With no
-    // next tile it is refilled all the same, every lane from the 16 bytes of lane 0 in this
-    // tile (a single cache line per load, contents unused), so that the loop body exists once
-    // and has no branch.
+    // next tile the refill is issued all the same, with a per-lane offset beyond the end of
+    // the blob: the buffer range check answers such a load with zeros without touching
+    // memory, and the loop body exists once and has no branch.
     const bool has_next = next_tile >= 0;
     const PPTilePtr<FUSED> nxt = pp_tile_ptr<FUSED>(p, has_next ? next_tile : 0, sc0);
     const uint32_t voff = lane * 16u;
@@ -898,12 +901,12 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
             const uint32_t w_same = cur.words[r] + (uint32_t)(sc + 1 - sc0) * 4096u;
-            const uint32_t m_same = cur.meta[r] + (uint32_t)((((sc + 1) >> 2) - (sc0 >> 2)) * 1024 +
-                                                             (((sc + 1) & 3) - (sc0 & 3)) * 4);
+            const uint32_t m_same = cur.meta[r] + (uint32_t)(sc + 1 - sc0) * 256u;
             rw[r] = last ? (has_next ? nxt.words[r] : cur.words[r]) : w_same;
             rm[r] = last ? (has_next ? nxt.meta[r] : cur.meta[r]) : m_same;
         }
-        super_chunk(sc, (last && !has_next) ? 0u : voff, rw, rm);
+        const bool dry = last && !has_next;
+        super_chunk(sc, dry ? PP_OUT_OF_RANGE : voff, dry ? PP_OUT_OF_RANGE : voff >> 2, rw, rm);
     }
 }
 
@@ -1075,7 +1078,7 @@ int stream_staged_k(int M, int K, size_t lds) {
 // the stream kernel addresses a blob with 32-bit byte offsets, so a blob stays below 2 GiB
 bool prepack_ok(long N, long K, long G) {
     if (G != 128 || K % 128 != 0 || N < 1 || K < 128 || N * K >= (1L << 40)) return false;
-    return ((N + 15) / 16) * pp_tile_u4((int)K) * 16 < (1L << 31);
+    return ((N + 15) / 16) * pp_tile_u4((int)K) * 16 < (long)PP_OUT_OF_RANGE;
 }
 
 // stream kernel, prepacked records: all of the padded K if it fits, else whole super-chunks per pass
