@@ -75,7 +75,8 @@ struct DevProblem {
     int32_t fused;       // gate||up rows with SiLU epilogue
     int32_t tile_begin;  // first tile index of this problem inside a grouped launch
     int32_t kc;          // k extent of x staged in LDS per pass (multiple of KCHUNK)
-    int32_t prepacked;   // qweight points at a prepacked blob (scales/qzeros unused)
+    int32_t prepacked;   // bit 0: qweight points at a prepacked blob (scales/qzeros unused);
+                         // bit 1: a row of zeros is staged behind the activation rows (PP_ZERO_ROW)
 };
 static_assert(sizeof(DevProblem) == 72, "plan record layout is part of the plan format");
 
@@ -719,17 +720,20 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
-// natural-order staging of x[:, k0:k1) (k beyond K reads as zero)
+constexpr int PP_ZERO_ROW = 2;  // DevProblem::prepacked bit
+
+// natural-order staging of x[:, k0:k1) (k beyond K reads as zero), plus a row of zeros at
+// row M if the record asks for one
 __device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int k1, uint16_t *xs,
                                                 int xstride, int nthreads) {
     const int words_per_row = (k1 - k0) >> 3;
-    const int total = p.M * words_per_row;
+    const int total = (p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0)) * words_per_row;
     for (int idx = threadIdx.x; idx < total; idx += nthreads) {
         const int m = idx / words_per_row;
         const int j = idx - m * words_per_row;
         const int k = k0 + (j << 3);
         u32x4_t d = {0u, 0u, 0u, 0u};
-        if (k < p.K) d = *as_global(reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k));
+        if (k < p.K && m < p.M) d = *as_global(reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k));
         *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = d;
     }
 }
@@ -840,6 +844,10 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
 
     static_assert(STREAM_DEPTH == 4, "the ring holds exactly one super-chunk (four loads per lane)");
     PPGroup grp[RS];
+    // A-operand rows beyond M are padding: they read the staged row of zeros if there is one
+    // (quiet multipliers; the chip runs this kernel at its power limit, so that shows up as
+    // clock), else a copy of the last row
+    const int pad_row = (p.prepacked & PP_ZERO_ROW) ? p.M : p.M - 1;
 
     // One super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside.
     // Each ring slot is reloaded from offset rw (and the meta word from rm, with slot 0) as
@@ -858,7 +866,7 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                 bf16x8_t xa[MB];
 #pragma unroll
                 for (int b = 0; b < MB; ++b) {
-                    const int m = min(16 * b + lc, p.M - 1);
+                    const int m = min(16 * b + lc, pad_row);
                     const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
                     xa[b] = __builtin_bit_cast(bf16x8_t, raw);
                 }
@@ -1030,8 +1038,8 @@ constexpr size_t LDS_X_BUDGET = 40 * 1024;      // split kernel: staged activati
 constexpr int STAGE_STEP = KCHUNK * TILE_WPB;   // split kernel: shorter staged extents are multiples of this
 // stream kernel: workgroup shapes by the LDS the staged activations need
 struct StreamShape { int wpb; int per_cu; size_t lds; };
-// {waves per workgroup, workgroups per CU, LDS it may use}; the narrow shape is launched with three
-// times the resident number of workgroups (5 per CU) so that the hardware dispatcher evens out the tail
+// {waves per workgroup, workgroups per CU to launch when the runtime cannot say how many are
+// resident, LDS the shape may use}
 constexpr StreamShape STREAM_SHAPES[3] = {{4, 15, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
 
@@ -1176,14 +1184,24 @@ constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
 constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16;
 
+// With recs == nullptr nothing is launched: info->grid receives the number of workgroups of
+// this build that one CU holds at info->lds_bytes (the plan builder sizes the grid with it).
 template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
-int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
+int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
                   hipStream_t stream) {
     auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES>;
     if (info->lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
         if (e != hipSuccess) return (int)e;
+    }
+    if (!recs) {
+        int per_cu = 0;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &per_cu, reinterpret_cast<const void *>(kernel), WPB * WAVE, (size_t)info->lds_bytes);
+        if (e != hipSuccess) return (int)e;
+        info->grid = per_cu;
+        return VRL_INT4_OK;
     }
     hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes,
                        stream, recs, block_begin, info->n_problems);
@@ -1192,7 +1210,7 @@ int launch_stream(const vrl_int4_plan_info *info, const DevProblem *recs, const 
 
 // which record kinds a kernel build must handle, for a given workgroup shape
 template <int WPB, int MB>
-int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb,
+int launch_stream_variant(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb,
                           hipStream_t stream) {
     const int v = info->variant & (VARIANT_CANON | VARIANT_PP | VARIANT_FUSED);
     const bool passes = (info->variant & VARIANT_PASSES) != 0;
@@ -1216,6 +1234,19 @@ int launch_stream_variant(const vrl_int4_plan_info *info, const DevProblem *recs
     return VRL_INT4_EPLAN;
 }
 
+
+int dispatch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab,
+                    hipStream_t stream) {
+    const bool mb2 = (info->variant & VARIANT_MB2) != 0;
+    switch (info->block_threads) {
+        case 4 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<4, 1>(info, recs, block_tab, stream);
+        case 8 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<8, 1>(info, recs, block_tab, stream);
+        case 16 * WAVE:
+            return mb2 ? launch_stream_variant<16, 2>(info, recs, block_tab, stream)
+                       : launch_stream_variant<16, 1>(info, recs, block_tab, stream);
+        default: return VRL_INT4_EPLAN;
+    }
+}
 
 size_t plan_bytes_for(int n_records) {
     return sizeof(PlanHeader) + (size_t)n_records * sizeof(DevProblem) +
@@ -1377,9 +1408,43 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         if (need > smem) smem = need;
         if (p.prepacked && p.kc < pp_nsc(p.K) * PP_SC) variant |= VARIANT_PASSES;
     }
-
-    // one contiguous tile range per workgroup, balanced by streamed bytes
-    long grid = (long)device_cu_count() * sh.per_cu;
+    // How many workgroups of this build a CU holds at a given LDS size (0: the runtime cannot say).
+    auto resident_per_cu = [&](size_t lds_bytes) {
+        vrl_int4_plan_info probe;
+        memset(&probe, 0, sizeof probe);
+        probe.block_threads = sh.wpb * WAVE;
+        probe.lds_bytes = (int)lds_bytes;
+        probe.variant = variant;
+        if (dispatch_stream(&probe, nullptr, nullptr, nullptr) != VRL_INT4_OK) return 0;
+        return probe.grid;
+    };
+    // One contiguous tile range per workgroup, balanced by streamed bytes.  The grid is what the
+    // device holds at once (every workgroup runs from start to end, no second round of
+    // prologues: measured 1 % faster than a grid twice as deep); if the runtime cannot say how
+    // many fit, the table's deeper grid is used and the dispatcher evens out the tail.
+    long per_cu = sh.per_cu;
+    const int resident = resident_per_cu(smem);
+    if (resident >= 1) per_cu = resident;
+    // Prepacked records with unused A-operand rows stage one more row, of zeros, for those
+    // rows to read, if that costs no residency.
+    if (resident >= 1) {
+        const int rows_per_record = (variant & VARIANT_MB2) ? 32 : 16;
+        size_t smem_z = smem;
+        for (int i = 0; i < n_problems; ++i) {
+            const DevProblem &p = recs[i];
+            const size_t need = (size_t)(p.M + 1) * (p.kc + XPAD) * 2;
+            if (p.prepacked && p.M < rows_per_record && need <= sh.lds && need > smem_z) smem_z = need;
+        }
+        if (smem_z == smem || resident_per_cu(smem_z) == resident) {
+            for (int i = 0; i < n_problems; ++i) {
+                DevProblem &p = recs[i];
+                if (p.prepacked && p.M < rows_per_record && (size_t)(p.M + 1) * (p.kc + XPAD) * 2 <= smem_z)
+                    p.prepacked |= PP_ZERO_ROW;
+            }
+            smem = smem_z;
+        }
+    }
+    long grid = (long)device_cu_count() * per_cu;
     if (grid > MAX_PLAN_GRID) grid = MAX_PLAN_GRID;
     const long max_useful = (tiles + sh.wpb - 1) / sh.wpb;
     if (grid > max_useful) grid = max_useful;
@@ -1438,16 +1503,8 @@ int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *i
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
     const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + sizeof(PlanHeader));
     const int2 *block_begin = reinterpret_cast<const int2 *>(recs + info->n_problems);
-    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const bool mb2 = (info->variant & VARIANT_MB2) != 0;
-    switch (info->block_threads) {
-        case 4 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<4, 1>(info, recs, block_begin, stream);
-        case 8 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<8, 1>(info, recs, block_begin, stream);
-        case 16 * WAVE:
-            return mb2 ? launch_stream_variant<16, 2>(info, recs, block_begin, stream)
-                       : launch_stream_variant<16, 1>(info, recs, block_begin, stream);
-        default: return VRL_INT4_EPLAN;
-    }
+    vrl_int4_plan_info launch = *info;
+    return dispatch_stream(&launch, recs, block_begin, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
 }  // extern "C"
