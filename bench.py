@@ -76,13 +76,32 @@ def time_region(fn, steps: int, warmup: int):
     return start.elapsed_time(end) / steps
 
 
-def build_set(cfg: int, M: int, device, with_head: bool):
+def build_set(cfg: int, M: int, device, with_head: bool, hidden: int = HIDDEN, inter: int = INTER,
+              layers: int = LAYERS, head: int = HEAD, canonical: bool = True):
     """All linears of one decode step: list of dicts with operands and byte counts."""
     from visionrl_amd import ops
     from visionrl_amd.int4_format import algorithmic_bytes
 
     items = []
-    xs = {K: make_x(1000 * cfg + 7, M, K, device) for K in (HIDDEN, INTER)}
+    xs = {K: make_x(1000 * cfg + 7, M, K, device) for K in (hidden, inter)}
+    linears = [("q", hidden, hidden), ("k", hidden, hidden), ("v", hidden, hidden), ("o", hidden, hidden),
+               ("gate", hidden, inter), ("up", hidden, inter), ("down", inter, hidden)]
+    if (hidden, inter, layers, head) != (HIDDEN, INTER, LAYERS, HEAD):
+        for layer in range(layers):
+            for proj, (name, K, N) in enumerate(linears):
+                qw, sc, qz = make_weights(1000 * cfg + 10 * layer + proj, K, N, GROUP, device)
+                it = {"name": f"l{layer}.{name}", "layer": layer, "proj": name, "K": K, "N": N, "x": xs[K],
+                      "prepacked": ops.int4_prepack(qw, sc, qz, GROUP),
+                      "bytes": algorithmic_bytes(M, K, N, GROUP)}
+                if canonical:
+                    it.update({"qweight": qw, "scales": sc, "qzeros": qz})
+                items.append(it)
+        if with_head:
+            qw, sc, qz = make_weights(1000 * cfg + 999, hidden, head, GROUP, device)
+            items.append({"name": "gen_head", "layer": layers, "proj": "head", "K": hidden, "N": head,
+                          "x": xs[hidden], "prepacked": ops.int4_prepack(qw, sc, qz, GROUP),
+                          "bytes": algorithmic_bytes(M, hidden, head, GROUP)})
+        return items
     for layer in range(LAYERS):
         for proj, (name, K, N) in enumerate(LAYER_LINEARS):
             qw, sc, qz = make_weights(1000 * cfg + 10 * layer + proj, K, N, GROUP, device)
@@ -153,14 +172,83 @@ def measure_set(items, steps: int, warmup: int):
         for names in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",), ("head",)):
             sel = [its[n] for n in names if n in its]
             if sel:
-                plans.append(ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in sel]))
+                probs = [(it["x"], it["prepacked"], False) for it in sel]
+                direct = all(it["x"].shape[0] <= ops.DirectGemv.MAX_ROWS for it in sel)
+                plans.append(ops.DirectGemv(probs) if direct else ops.GroupedGemv(probs))
 
     def layered():
         for plan in plans:
             plan.launch()
 
     record("per_layer_4_launches", time_region(layered, max(5, steps // 5), max(2, warmup // 5)), len(plans))
+    try:
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            layered()
+        record("per_layer_4_launches_hip_graph",
+               time_region(graph.replay, max(5, steps // 5), max(2, warmup // 5)), len(plans))
+    except Exception as exc:
+        out["layered_hip_graph_error"] = repr(exc)[:200]
     return out, total_bytes, grouped
+
+
+def other_configs(device, steps: int, warmup: int):
+    """The remaining benchmark configurations, one grouped launch each (prepacked layout)."""
+    from visionrl_amd import ops
+    from visionrl_amd.int4_format import algorithmic_bytes
+
+    res = {}
+    # 7B-class shapes: hidden 4096, intermediate 11008, 30 layers, head 4096 -> 16384
+    for M in (1, 8, 16):
+        items = build_set(4, M, device, with_head=True, hidden=4096, inter=11008, layers=30,
+                          head=16384, canonical=False)
+        nbytes = sum(it["bytes"] for it in items)
+        grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items])
+        ms = time_region(grouped.launch, max(10, steps // 10), max(2, warmup // 10))
+        res[f"7b_class_m{M}"] = {"ms_per_step": ms, "GBps": nbytes / (ms * 1e-3) / 1e9,
+                                 "algorithmic_bytes_per_step": nbytes, "gemvs": len(items)}
+        del items, grouped
+        torch.cuda.empty_cache()
+    # fused gate||up with the SiLU epilogue, K=4096, N=2x11008, M=8, over 24 distinct weight sets
+    K, I, M = 4096, 11008, 8
+    sets = []
+    for i in range(24):
+        qw, sc, qz = make_weights(5000 + i, K, 2 * I, GROUP, device)
+        sets.append(ops.int4_prepack(qw, sc, qz, GROUP))
+        del qw, sc, qz
+    x = make_x(5007, M, K, device)
+    nbytes = 24 * algorithmic_bytes(M, K, 2 * I, GROUP, fused_gate_up=True)
+    grouped = ops.GroupedGemv([(x, pw, True) for pw in sets])
+    ms = time_region(grouped.launch, max(10, steps // 10), max(2, warmup // 10))
+    res["fused_gate_up_silu_k4096_i11008_m8"] = {"ms_per_24_weight_sets": ms, "us_per_weight_set": ms * 1e3 / 24,
+                                                  "GBps": nbytes / (ms * 1e-3) / 1e9}
+    del sets, grouped
+    torch.cuda.empty_cache()
+    # group-size sweep, K=5632, N=2048, M=1: single launches over 48 distinct weight sets in a HIP graph
+    sweep = {}
+    for G in (32, 64, 128):
+        K, N = 5632, 2048
+        ws = [make_weights(5100 + i, K, N, G, device) for i in range(48)]
+        x = make_x(5107, 1, K, device)
+        ys = [torch.empty((1, N), dtype=torch.bfloat16, device=device) for _ in ws]
+
+        def rotate():
+            for (qw, sc, qz), y in zip(ws, ys):
+                ops.int4_gemv_into(y, x, qw, sc, qz, G)
+
+        rotate()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rotate()
+        ms = time_region(graph.replay, max(5, steps // 20), 2) / len(ws)
+        sweep[f"G{G}"] = {"us_per_call_hip_graph": ms * 1e3,
+                          "GBps": algorithmic_bytes(1, K, N, G) / (ms * 1e-3) / 1e9}
+        del ws, ys, graph
+        torch.cuda.empty_cache()
+    res["group_size_sweep_k5632_n2048_m1"] = sweep
+    return res
 
 
 def per_call_latency(items, steps: int):
@@ -188,6 +276,20 @@ def per_call_latency(items, steps: int):
         torch.cuda.synchronize()
         with torch.cuda.graph(graph):
             rotate_direct()
+        # the same matrices through the plan-free launch over the prepacked layout (records as
+        # kernel arguments, waves of a workgroup split K), replayed from a HIP graph
+        plans = [ops.DirectGemv([(it["x"], it["prepacked"], False)]) for it in group]
+
+        def rotate_plans():
+            for plan in plans:
+                plan.launch()
+
+        graph_p = torch.cuda.CUDAGraph()
+        rotate_plans()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph_p):
+            rotate_plans()
+        ms_plan = time_region(graph_p.replay, max(5, steps // 10), 2) / len(group)
         reps = max(2, steps // 50)
         ms_op = time_region(rotate_op, reps, 1) / len(group)
         ms_direct = time_region(rotate_direct, reps, 1) / len(group)
@@ -195,7 +297,8 @@ def per_call_latency(items, steps: int):
         res[f"{K}x{N}"] = {"us_per_call_torch_op": ms_op * 1e3,
                            "us_per_call_direct": ms_direct * 1e3,
                            "us_per_call_hip_graph": ms_graph * 1e3,
-                           "GBps_hip_graph": group[0]["bytes"] / (ms_graph * 1e-3) / 1e9,
+                           "us_per_call_prepacked_hip_graph": ms_plan * 1e3,
+                           "GBps_hip_graph": group[0]["bytes"] / (min(ms_graph, ms_plan) * 1e-3) / 1e9,
                            "distinct_weights": len(group)}
     return res
 
@@ -316,6 +419,11 @@ def main():
     del items32
     torch.cuda.empty_cache()
 
+    try:
+        others = other_configs(device, args.steps, args.warmup)
+    except Exception as exc:  # the other configurations are detail, never the headline
+        others = {"error": repr(exc)[:300]}
+
     result = {
         "metric": "int4 GEMV GB/s (% of HBM peak) + us/call, Janus-1B shapes at M=1 and M=32",
         "value": value,
@@ -341,7 +449,8 @@ def main():
                      "avg_launch_ms": kernel_ms},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,
-                   "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32},
+                   "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
+                   "other_configs": others},
     }
     print(json.dumps(result))
 

@@ -134,6 +134,17 @@ typedef struct vrl_int4_plan_info {
     int32_t reserved[2];
 } vrl_int4_plan_info;
 
+/*
+ * Plan-free launch of one to four prepacked GEMVs that share a kernel (one nn.Linear.forward
+ * over a prepacked weight, or the q|k|v / gate|up linears of one decoder layer,
+ * policy.py:673-678): the records travel as kernel arguments, one workgroup per 16-column
+ * tile with its waves splitting K.  Meant for decode (the launch is one memory round trip);
+ * every problem must have prepacked = 1, M <= 16 and activations of at most ~60 KB
+ * (M * K * 2 bytes), else VRL_INT4_ESHAPE and the caller uses a grouped plan or
+ * vrl_int4_gemv_bf16.  scales and qzeros of the records are ignored.
+ */
+int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream);
+
 size_t vrl_int4_grouped_plan_size(int n_problems);
 
 /* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems)) and *info. */

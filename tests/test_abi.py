@@ -140,3 +140,24 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.Int4LibraryError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_direct_prepacked_validation(lib):
+    keep, p = buf(4096)
+    probs = (_lib.Problem * 2)()
+    for rec in probs:
+        rec.x = rec.qweight = rec.y = p
+        rec.M, rec.N, rec.K, rec.G, rec.prepacked = 1, 64, 256, 128, 1
+    assert lib.vrl_int4_gemv_prepacked_bf16(None, 1, None) == 1003
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 0, None) == 1001
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 5, None) == 1001
+    probs[1].prepacked = 0                       # canonical records are not taken here
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
+    probs[1].prepacked, probs[1].M = 1, 17       # more than 16 activation rows
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
+    probs[1].M, probs[1].G = 1, 64               # no prepacked form for this group size
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
+    probs[1].G, probs[1].y = 128, p + 2          # misaligned output
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002
+    probs[1].y, probs[1].M, probs[1].K = p, 16, 4096   # activations beyond the LDS this path uses
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001

@@ -414,3 +414,87 @@ def test_operator_contract_errors(ops_mod):
         ops_mod.int4_gemv(d["x"], d["qweight"], d["scales"], d["qzeros"], 96)
     with pytest.raises(ValueError):
         ops_mod.int4_gemv(d["x"].t().contiguous().t(), d["qweight"], d["scales"], d["qzeros"], 128)
+
+
+# ------------------------------------------------------------------ plan-free launches of prepacked weights
+DIRECT_SHAPES = [
+    # M, K, N, fused
+    (1, 2048, 2048, False), (1, 5632, 2048, False), (1, 2048, 5632, False), (1, 11008, 96, False),
+    (1, 128, 16, False), (3, 640, 50, False), (16, 1536, 64, False), (7, 4096, 80, False),
+    (1, 2048, 2 * 5632, True), (8, 2048, 2 * 704, True), (5, 4096, 2 * 48, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,fused", DIRECT_SHAPES)
+def test_direct_prepacked_parity(ops_mod, M, K, N, fused):
+    say("direct prepacked", M, K, N, fused)
+    G = 128
+    ops = o.make_operands(9000 + M + K + N, M, K, N, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    (y,) = ops_mod.DirectGemv([(d["x"], pw, fused)]).launch()
+    torch.cuda.synchronize()
+    if not fused:
+        assert_gemv_close(bf16_to_bits(y), ops, G, f"direct M{M} K{K} N{N}")
+        return
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    ref = o.gate_up_silu_f64(*args)
+    got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
+    tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
+    assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all()
+
+
+def test_direct_group_matches_single_launches_and_plan(ops_mod):
+    """q|k|v-like group of three in one plan-free launch: same bits as one launch each and as a plan."""
+    say("direct group")
+    G = 128
+    probs, checks = [], []
+    for i, (M, K, N) in enumerate([(1, 2048, 2048), (1, 2048, 512), (1, 2048, 100)]):
+        ops = o.make_operands(9100 + i, M, K, N, G)
+        d = to_device(ops, DEV)
+        probs.append((d["x"], ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G), False))
+        checks.append(ops)
+    outs = [y.clone() for y in ops_mod.DirectGemv(probs).launch()]
+    torch.cuda.synchronize()
+    for y, ops in zip(outs, checks):
+        assert_gemv_close(bf16_to_bits(y), ops, G, "direct group")
+    singles = [ops_mod.DirectGemv([p]).launch()[0] for p in probs]
+    planned = ops_mod.GroupedGemv(probs).launch()
+    torch.cuda.synchronize()
+    for a, b, c in zip(outs, singles, planned):
+        assert torch.equal(a, b) and torch.equal(a, c)   # same kernel body, same summation order
+
+
+def test_direct_one_hot_is_the_exact_weight_column(ops_mod):
+    say("direct one-hot")
+    G, M, K, N = 128, 2, 1024, 48
+    ops = o.make_operands(9200, M, K, N, G, "loguniform")
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    for k0 in (0, 5, 127, 128, 511, 512, 777, K - 1):
+        x = np.zeros((M, K), dtype=np.float32)
+        for m in range(M):
+            x[m, (k0 + 300 * m) % K] = 1.0
+        (y,) = ops_mod.DirectGemv([(bits_to_bf16(o.f32_to_bf16_bits(x), DEV), pw, False)]).launch()
+        torch.cuda.synchronize()
+        y = bf16_to_bits(y)
+        for m in range(M):
+            want = w[:, (k0 + 300 * m) % K]
+            assert ((y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)).all(), (k0, m)
+
+
+def test_direct_rejects_what_it_cannot_take(ops_mod):
+    G = 128
+    ops = o.make_operands(9300, 17, 256, 32, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(d["x"], pw, False)])            # 17 rows
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(d["x"][:1], pw, False)] * 5)    # five problems
+    big = o.make_operands(9301, 16, 4096, 16, G)             # 16 x 4096 activations do not fit this path
+    db = to_device(big, DEV)
+    pwb = ops_mod.int4_prepack(db["qweight"], db["scales"], db["qzeros"], G)
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(db["x"], pwb, False)]).launch()

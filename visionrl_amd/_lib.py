@@ -23,6 +23,7 @@ SYMBOLS = (
     "vrl_int4_gate_up_silu_bf16",
     "vrl_int4_prepacked_bytes",
     "vrl_int4_prepack",
+    "vrl_int4_gemv_prepacked_bf16",
     "vrl_int4_grouped_plan_size",
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
@@ -86,6 +87,8 @@ def _bind(lib):
     lib.vrl_int4_prepacked_bytes.argtypes = [ci, ci, ci]
     lib.vrl_int4_prepack.restype = ci
     lib.vrl_int4_prepack.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
+    lib.vrl_int4_gemv_prepacked_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_bf16.argtypes = [ctypes.POINTER(Problem), ci, vp]
     lib.vrl_int4_grouped_plan_size.restype = ctypes.c_size_t
     lib.vrl_int4_grouped_plan_size.argtypes = [ci]
     lib.vrl_int4_grouped_plan_build.restype = ci

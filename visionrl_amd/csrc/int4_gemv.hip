@@ -994,6 +994,99 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
     }
 }
 
+// Small plans (fewer tiles than the device has workgroup slots): the waves of a workgroup
+// share one tile, each taking a contiguous quarter of its super-chunks, and the partial
+// tiles meet in LDS.  A tile is then one or two memory round trips instead of a serial walk
+// over K by a single wave; this is the latency mode for launches of a few matrices
+// (q|k|v of one layer, one o_proj, ...).  LDS: staged activations, then WPB x RS partial tiles.
+template <bool FUSED, int WPB>
+__device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (WAVE - 1);
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int xstride = p.kc + XPAD;
+    const int xrows = p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0);
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + (size_t)xrows * xstride * 2);
+    const int nsc = pp_nsc(p.K);
+    const int per = (nsc + WPB - 1) / WPB;
+    const int sc0 = min(nsc, wave * per), sc1 = min(nsc, sc0 + per);
+    const bool work = sc0 < sc1;  // wave-uniform
+    const rsrc_t rsrc = pp_blob_rsrc(p);
+    PPRing<RS> ring;
+    PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, t0, sc0);
+    if (work) pp_prime<FUSED>(rsrc, cur, ring);  // weights are on their way while x is staged
+    __syncthreads();
+    stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+    __syncthreads();
+    for (int tile = t0; tile < t1; ++tile) {
+        const int next = tile + 1 < t1 ? tile + 1 : -1;
+        f32x4_t acc[RS][1];
+#pragma unroll
+        for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (work) {
+            stream_rows_pp<1, FUSED>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
+            if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
+        }
+        if (wave != 0) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) red[((wave - 1) * RS + r) * WAVE + lane] = acc[r][0];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int w = 1; w < WPB; ++w)
+#pragma unroll
+                for (int r = 0; r < RS; ++r) acc[r][0] += red[((w - 1) * RS + r) * WAVE + lane];
+            store_tile<1, FUSED>(p, tile, acc);
+        }
+        if (next >= 0) __syncthreads();  // the partial tiles are read before they are rewritten
+    }
+}
+
+template <bool FUSED, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem *__restrict__ plan,
+                                                               const int2 *__restrict__ block_tab,
+                                                               int n_problems) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int2 entry = block_tab[blockIdx.x];
+    int t = entry.x;
+    const int t_end = block_tab[blockIdx.x + 1].x;
+    if (t >= t_end) return;  // block-uniform
+    for (int pi = entry.y; t < t_end && pi < n_problems; ++pi) {
+        const DevProblem p = plan[pi];
+        const int out_cols = p.fused ? p.N / 2 : p.N;
+        const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
+        const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
+        if (FUSED && p.fused) split_segment_pp<FUSED, WPB>(p, a, b, smem);
+        else split_segment_pp<false, WPB>(p, a, b, smem);
+        t = seg_end;
+    }
+}
+
+// The same latency mode without a plan in device memory: up to DIRECT_MAX records travel
+// as kernel arguments (no dependent loads before the first weight request), one workgroup per
+// tile.  This is the single-call path of a prepacked weight (and of q|k|v, gate|up groups).
+constexpr int DIRECT_MAX = 4;
+struct DirectArgs {
+    int32_t n;
+    int32_t pad;
+    DevProblem recs[DIRECT_MAX];
+};
+
+template <bool FUSED, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int t = blockIdx.x;
+    DevProblem p = a.recs[0];
+#pragma unroll
+    for (int k = 1; k < DIRECT_MAX; ++k)
+        if (k < a.n && a.recs[k].tile_begin <= t) p = a.recs[k];  // scalar selects, no indexing
+    const int local = t - p.tile_begin;
+    if (FUSED && p.fused) split_segment_pp<FUSED, WPB>(p, local, local + 1, smem);
+    else split_segment_pp<false, WPB>(p, local, local + 1, smem);
+}
+
 // CANON / PP / FUSED say which kinds of record the plan holds, so that a plan of
 // plain prepacked GEMVs runs the variant with the smallest register footprint.
 // WPB (waves per workgroup) grows with the LDS the staged activations need, so that
@@ -1182,7 +1275,8 @@ struct PlanHeader {
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
-constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16;
+constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16,
+              VARIANT_SPLIT = 32;
 
 // With recs == nullptr nothing is launched: info->grid receives the number of workgroups of
 // this build that one CU holds at info->lds_bytes (the plan builder sizes the grid with it).
@@ -1235,9 +1329,48 @@ int launch_stream_variant(vrl_int4_plan_info *info, const DevProblem *recs, cons
 }
 
 
+template <bool FUSED, int WPB>
+int launch_split(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab, hipStream_t stream) {
+    auto kernel = &gemv_split_kernel<FUSED, WPB>;
+    if (!recs) {
+        int per_cu = 0;
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &per_cu, reinterpret_cast<const void *>(kernel), WPB * WAVE, (size_t)info->lds_bytes);
+        if (e != hipSuccess) return (int)e;
+        info->grid = per_cu;
+        return VRL_INT4_OK;
+    }
+    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes, stream, recs,
+                       block_tab, info->n_problems);
+    return (int)hipGetLastError();
+}
+
+template <int WPB>
+int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab,
+                         hipStream_t stream) {
+    return (info->variant & VARIANT_FUSED) ? launch_split<true, WPB>(info, recs, block_tab, stream)
+                                           : launch_split<false, WPB>(info, recs, block_tab, stream);
+}
+
+template <bool FUSED, int WPB>
+int launch_direct(const DirectArgs &args, int tiles, size_t lds, hipStream_t stream) {
+    hipLaunchKernelGGL((gemv_split_direct_kernel<FUSED, WPB>), dim3(tiles), dim3(WPB * WAVE), lds, stream, args);
+    return (int)hipGetLastError();
+}
+
 int dispatch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab,
                     hipStream_t stream) {
     const bool mb2 = (info->variant & VARIANT_MB2) != 0;
+    if (info->variant & VARIANT_SPLIT) {
+        if (mb2 || (size_t)info->lds_bytes > 64 * 1024 || (info->variant & (VARIANT_CANON | VARIANT_PASSES)))
+            return VRL_INT4_EPLAN;
+        switch (info->block_threads) {
+            case 4 * WAVE: return launch_split_variant<4>(info, recs, block_tab, stream);
+            case 8 * WAVE: return launch_split_variant<8>(info, recs, block_tab, stream);
+            case 16 * WAVE: return launch_split_variant<16>(info, recs, block_tab, stream);
+            default: return VRL_INT4_EPLAN;
+        }
+    }
     switch (info->block_threads) {
         case 4 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<4, 1>(info, recs, block_tab, stream);
         case 8 * WAVE: return mb2 ? VRL_INT4_EPLAN : launch_stream_variant<8, 1>(info, recs, block_tab, stream);
@@ -1318,6 +1451,67 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
                        static_cast<const uint32_t *>(qzeros), static_cast<u32x4_t *>(packed), N, K);
     return (int)hipGetLastError();
+}
+
+int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {
+    if (!problems) return VRL_INT4_ENULL;
+    if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
+    DirectArgs args;
+    memset(&args, 0, sizeof args);
+    args.n = n_problems;
+    long tiles = 0;
+    bool fused_any = false;
+    int max_nsc = 1;
+    size_t x_bytes = 0;
+    for (int i = 0; i < n_problems; ++i) {
+        const vrl_int4_problem &q = problems[i];
+        if (!q.prepacked) return VRL_INT4_ESHAPE;
+        int rc = check_problem(q.x, q.qweight, q.qweight, q.qweight, q.y, q.M, q.N, q.K, q.G);
+        if (rc != VRL_INT4_OK) return rc;
+        if (q.M > MAX_TILE_M || !prepack_ok(q.N, q.K, q.G)) return VRL_INT4_ESHAPE;
+        if (q.fused_gate_up && (q.N % 2 != 0 || (q.N / 2) % 16 != 0)) return VRL_INT4_ESHAPE;
+        DevProblem &p = args.recs[i];
+        p.x = static_cast<const uint16_t *>(q.x);
+        p.qweight = static_cast<const uint32_t *>(q.qweight);
+        p.y = static_cast<uint16_t *>(q.y);
+        p.M = q.M; p.N = q.N; p.K = q.K; p.G = q.G;
+        p.fused = q.fused_gate_up ? 1 : 0;
+        p.prepacked = 1;
+        p.kc = pp_nsc(q.K) * PP_SC;
+        p.tile_begin = (int)tiles;
+        tiles += ((p.fused ? p.N / 2 : p.N) + 15) / 16;
+        fused_any |= p.fused != 0;
+        max_nsc = std::max(max_nsc, pp_nsc(q.K));
+        x_bytes = std::max(x_bytes, (size_t)p.M * (p.kc + XPAD) * 2);
+    }
+    if (tiles > MAX_PLAN_GRID) return VRL_INT4_ESHAPE;
+    const int wpb = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
+    const size_t red = (size_t)(wpb - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
+    // padding rows of the A operand read a staged row of zeros where LDS is plentiful
+    size_t xz_bytes = x_bytes;
+    for (int i = 0; i < n_problems; ++i) {
+        DevProblem &p = args.recs[i];
+        const size_t need = (size_t)(p.M + 1) * (p.kc + XPAD) * 2;
+        if (p.M < MAX_TILE_M && need + red <= 32 * 1024) {
+            p.prepacked |= PP_ZERO_ROW;
+            xz_bytes = std::max(xz_bytes, need);
+        }
+    }
+    const size_t lds = xz_bytes + red;
+    if (lds > 64 * 1024) return VRL_INT4_ESHAPE;  // activations too large for this path: use a plan
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    if (fused_any) {
+        switch (wpb) {
+            case 4: return launch_direct<true, 4>(args, (int)tiles, lds, stream);
+            case 8: return launch_direct<true, 8>(args, (int)tiles, lds, stream);
+            default: return launch_direct<true, 16>(args, (int)tiles, lds, stream);
+        }
+    }
+    switch (wpb) {
+        case 4: return launch_direct<false, 4>(args, (int)tiles, lds, stream);
+        case 8: return launch_direct<false, 8>(args, (int)tiles, lds, stream);
+        default: return launch_direct<false, 16>(args, (int)tiles, lds, stream);
+    }
 }
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {
@@ -1408,11 +1602,12 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         if (need > smem) smem = need;
         if (p.prepacked && p.kc < pp_nsc(p.K) * PP_SC) variant |= VARIANT_PASSES;
     }
+    int wpb = sh.wpb;  // waves per workgroup of the launch
     // How many workgroups of this build a CU holds at a given LDS size (0: the runtime cannot say).
     auto resident_per_cu = [&](size_t lds_bytes) {
         vrl_int4_plan_info probe;
         memset(&probe, 0, sizeof probe);
-        probe.block_threads = sh.wpb * WAVE;
+        probe.block_threads = wpb * WAVE;
         probe.lds_bytes = (int)lds_bytes;
         probe.variant = variant;
         if (dispatch_stream(&probe, nullptr, nullptr, nullptr) != VRL_INT4_OK) return 0;
@@ -1422,8 +1617,32 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     // device holds at once (every workgroup runs from start to end, no second round of
     // prologues: measured 1 % faster than a grid twice as deep); if the runtime cannot say how
     // many fit, the table's deeper grid is used and the dispatcher evens out the tail.
+    // Plans with fewer tiles than the device has workgroup slots take the latency mode: one
+    // workgroup per tile, its waves splitting K (gemv_split_kernel); the partial tiles need LDS
+    // behind the staged activations.
+    // As many waves share a tile as it has super-chunks (4, 8 or 16), fewer if the plan would
+    // not fit the device at that width.
+    size_t red_bytes = 0;
+    if (shape == 0 && !(variant & (VARIANT_CANON | VARIANT_MB2 | VARIANT_PASSES))) {
+        int max_nsc = 1;
+        for (int i = 0; i < n_problems; ++i) max_nsc = std::max(max_nsc, pp_nsc(recs[i].K));
+        variant |= VARIANT_SPLIT;
+        for (int w = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4); w >= 4; w /= 2) {
+            const size_t rb = (size_t)(w - 1) * ((variant & VARIANT_FUSED) ? 2 : 1) * WAVE * sizeof(f32x4_t);
+            wpb = w;
+            const int slots = resident_per_cu(smem + rb);
+            if (slots >= 1 && tiles <= (long)device_cu_count() * slots && tiles <= MAX_PLAN_GRID) {
+                red_bytes = rb;
+                break;
+            }
+        }
+        if (red_bytes == 0) {
+            variant &= ~VARIANT_SPLIT;
+            wpb = sh.wpb;
+        }
+    }
     long per_cu = sh.per_cu;
-    const int resident = resident_per_cu(smem);
+    const int resident = resident_per_cu(smem + red_bytes);
     if (resident >= 1) per_cu = resident;
     // Prepacked records with unused A-operand rows stage one more row, of zeros, for those
     // rows to read, if that costs no residency.
@@ -1435,7 +1654,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             const size_t need = (size_t)(p.M + 1) * (p.kc + XPAD) * 2;
             if (p.prepacked && p.M < rows_per_record && need <= sh.lds && need > smem_z) smem_z = need;
         }
-        if (smem_z == smem || resident_per_cu(smem_z) == resident) {
+        if (smem_z == smem || resident_per_cu(smem_z + red_bytes) == resident) {
             for (int i = 0; i < n_problems; ++i) {
                 DevProblem &p = recs[i];
                 if (p.prepacked && p.M < rows_per_record && (size_t)(p.M + 1) * (p.kc + XPAD) * 2 <= smem_z)
@@ -1444,10 +1663,20 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             smem = smem_z;
         }
     }
+    smem += red_bytes;
     long grid = (long)device_cu_count() * per_cu;
     if (grid > MAX_PLAN_GRID) grid = MAX_PLAN_GRID;
     const long max_useful = (tiles + sh.wpb - 1) / sh.wpb;
     if (grid > max_useful) grid = max_useful;
+    if (variant & VARIANT_SPLIT) {
+        grid = tiles;
+        for (long k = 0; k <= grid; ++k) block_begin[(size_t)k] = (int)k;
+        int rec = 0;
+        for (long k = 0; k <= grid; ++k) {
+            while (rec + 1 < n_problems && recs[rec + 1].tile_begin <= block_begin[(size_t)k]) ++rec;
+            block_tab[k] = make_int2(block_begin[(size_t)k], rec);
+        }
+    } else
     {
         int b = 0;
         double acc_cost = 0.0;
@@ -1487,7 +1716,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     info->n_problems = n_problems;
     info->total_tiles = (int)tiles;
     info->grid = (int)grid;
-    info->block_threads = sh.wpb * WAVE;
+    info->block_threads = wpb * WAVE;
     info->lds_bytes = (int)smem;
     info->variant = variant;
     return VRL_INT4_OK;

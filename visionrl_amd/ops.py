@@ -269,3 +269,69 @@ class GroupedGemv:
                                                 _stream_handle(self.device))
         _lib.check(rc, "vrl_int4_gemv_grouped_bf16")
         return self.outputs
+
+
+class DirectGemv:
+    """One to four prepacked GEMVs launched together without a plan in device memory.
+
+    The decode-time form of a linear (or of the q|k|v / gate|up linears of one decoder
+    layer, ``vrl/models/families/janus_pro/policy.py:673-678``): the problem records
+    travel as kernel arguments, so a launch is one memory round trip.  ``problems`` is a
+    list of ``(x, prepacked_weight, fused)``; every x has at most 16 rows.  Outputs are
+    allocated here once and overwritten by every :meth:`launch`; the record table is
+    built once, the tensors captured here must stay alive and in place.
+    """
+
+    MAX_PROBLEMS = 4
+    MAX_ROWS = 16
+
+    def __init__(self, problems, outputs=None):
+        if not 1 <= len(problems) <= self.MAX_PROBLEMS:
+            raise ValueError(f"DirectGemv takes 1 to {self.MAX_PROBLEMS} problems")
+        self._keep = []
+        self.outputs = []
+        self.table = (_lib.Problem * len(problems))()
+        dev = None
+        for i, (rec, (x, pw, fused)) in enumerate(zip(self.table, problems)):
+            if not isinstance(pw, PrepackedWeight):
+                raise TypeError("DirectGemv problems take a PrepackedWeight")
+            if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != pw.K or not 1 <= x.shape[0] <= self.MAX_ROWS:
+                raise ValueError(f"x must be bfloat16 [1..{self.MAX_ROWS}, {pw.K}]")
+            if not x.is_contiguous():
+                raise ValueError("x must be contiguous")
+            d = _require_device("x", x)
+            _require_device("prepacked blob", pw.blob, d)
+            if dev is None:
+                dev = d
+            elif d != dev:
+                raise ValueError("all problems of one launch must share one device")
+            if fused and pw.N % 2 != 0:
+                raise ValueError("gate||up operand needs an even number of rows")
+            cols = pw.N // 2 if fused else pw.N
+            if outputs is None:
+                y = torch.empty((x.shape[0], cols), dtype=torch.bfloat16, device=dev)
+            else:
+                y = outputs[i]
+                if y.dtype != torch.bfloat16 or tuple(y.shape) != (x.shape[0], cols) or not y.is_contiguous():
+                    raise ValueError(f"output {i} must be contiguous bfloat16 [{x.shape[0]}, {cols}]")
+                _require_device("y", y, dev)
+            self._keep.append((x, pw))
+            self.outputs.append(y)
+            rec.x, rec.qweight, rec.scales, rec.qzeros, rec.y = x.data_ptr(), pw.blob.data_ptr(), 0, 0, y.data_ptr()
+            rec.M, rec.N, rec.K, rec.G = x.shape[0], pw.N, pw.K, pw.group_size
+            rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
+        self.device = dev
+
+    def launch(self):
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            rc = lib.vrl_int4_gemv_prepacked_bf16(self.table, len(self.table), _stream_handle(self.device))
+        _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
+        return self.outputs
+
+
+def int4_gemv_prepacked_into(y: torch.Tensor, x: torch.Tensor, weight: PrepackedWeight,
+                             fused: bool = False) -> torch.Tensor:
+    """``y = x . dequant(weight)^T`` over a prepacked weight, one plan-free launch (M <= 16)."""
+    DirectGemv([(x, weight, fused)], outputs=[y]).launch()
+    return y
