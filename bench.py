@@ -303,6 +303,17 @@ def per_call_latency(items, steps: int):
     return res
 
 
+def launch_floor_us(device, nodes: int = 96, reps: int = 50):
+    """us per node of a HIP graph of tiny dependent kernels: what a launch costs with no work in it."""
+    t = torch.zeros(64, device=device)
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        for _ in range(nodes):
+            t.add_(1.0)
+    return time_region(graph.replay, reps, 3) / nodes * 1e3
+
+
 def cpu_baseline(seconds: float = 12.0):
     """PyTorch dequant + matmul on the host cores over one decoder layer's seven linears."""
     from oracle import int4_oracle as oracle  # the checker, used here as the reported CPU baseline
@@ -400,6 +411,10 @@ def main():
 
     strat, total_bytes, grouped = measure_set(items, args.steps, args.warmup)
     latency = per_call_latency(items, args.steps)
+    try:
+        latency["empty_kernel_hip_graph_node_us"] = launch_floor_us(device)
+    except Exception as exc:
+        latency["empty_kernel_error"] = repr(exc)[:200]
 
     best = max(strat["GBps"], key=lambda k: strat["GBps"][k])
     headline = "grouped_1_launch"

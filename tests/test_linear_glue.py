@@ -53,7 +53,9 @@ class StubPolicy:
 def test_apply_swaps_every_decode_linear():
     policy = StubPolicy()
     summary = apply_int4_to_policy(policy, group_size=128)
-    assert summary == {"linears": 7 * LAYERS, "fused_mlps": LAYERS, "head_linears": 1, "group_size": 128}
+    # nothing is prepacked on the CPU: the MFMA-shaped copies are made only for weights on a GPU
+    assert summary == {"linears": 7 * LAYERS, "fused_mlps": LAYERS, "head_linears": 1, "group_size": 128,
+                       "prepacked": 0}
     for layer in policy._lm_trunk().layers:
         for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
             mod = getattr(layer.self_attn, name)
@@ -187,7 +189,9 @@ def test_swapped_trunk_tracks_the_dequantised_trunk():
     reference._lm_trunk().load_state_dict(policy._lm_trunk().state_dict())
     reference.mmgpt.gen_head.load_state_dict(policy.mmgpt.gen_head.state_dict())
 
-    apply_int4_to_policy(policy, group_size=128)
+    summary = apply_int4_to_policy(policy, group_size=128)
+    # every quantised module got its prepacked copy: q/k/v/o + gate||up + down per layer, and the head
+    assert summary["prepacked"] == 6 * LAYERS + 1
     # give the reference copy the dequantised weights
     for lq, lr in zip(policy._lm_trunk().layers, reference._lm_trunk().layers):
         for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
@@ -218,3 +222,26 @@ def test_swapped_trunk_tracks_the_dequantised_trunk():
         # fp32 SiLU epilogue differ
         assert (a - b).abs().max() <= 0.05 * b.abs().max() + 1e-3
     assert outs[0][2].shape == (2, 1, VOCAB_IMG)
+
+
+@pytest.mark.gpu
+def test_prepacked_module_path_agrees_with_the_canonical_one():
+    """Decode-sized calls go through the plan-free launch once a module is prepacked; larger ones
+    keep the canonical kernels.  Both are the same arithmetic up to fp32 summation order."""
+    dev = "cuda:0"
+    torch.manual_seed(4)
+    lin = nn.Linear(1024, 160, bias=False).to(torch.bfloat16).to(dev)
+    q = Int4Linear.from_linear(lin, 128)
+    w = q.dequantize().double()
+    for rows in (1, 5, 16, 40):
+        x = torch.randn(rows, 1024, device=dev).to(torch.bfloat16)
+        plain = q(x)
+        q.prepack_()
+        assert q._packed is not None and q._direct_rows == 16
+        fast = q(x)
+        del q._packed
+        ref = x.double() @ w.t()
+        for y in (plain, fast):
+            assert (y.double() - ref).abs().le(2.0 ** -7 * ref.abs() + 2.0 ** -6).all()
+        if rows > 16:
+            assert torch.equal(plain, fast)      # same kernel: beyond 16 rows the prepacked copy is not used

@@ -73,6 +73,20 @@ class Int4Linear(nn.Module):
         """Accepts zero-points as an unpacked ``uint8 [N, K/G]`` tensor and packs them."""
         return cls.from_packed(qweight, scales, pack_nibbles(zeros_u8.to(torch.int32)), group_size, bias)
 
+    def prepack_(self) -> "Int4Linear":
+        """Keep a prepacked copy of the weight for decode-sized calls (a second copy in HBM).
+
+        Calls with few activation rows then go through the plan-free launch over the
+        MFMA-shaped blob; larger ones, and ``torch.compile``, keep using the canonical
+        buffers, which stay the module's ``state_dict``.  No-op if the shape has no prepacked form.
+        """
+        self._packed = None
+        if self.qweight.is_cuda and ops.PrepackedWeight.supported(self.out_features, self.in_features,
+                                                                  self.group_size):
+            self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
+            self._direct_rows = self._packed.direct_rows()
+        return self
+
     def dequantize(self) -> torch.Tensor:
         """The canonical bf16 weight ``[N, K]`` (bit-exact tile), e.g. for the train-time replay."""
         return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
@@ -83,7 +97,11 @@ class Int4Linear(nn.Module):
             y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
             y = torch.empty((rows.shape[0], self.out_features), dtype=torch.bfloat16, device=rows.device)
-            ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
+            packed = getattr(self, "_packed", None)
+            if packed is not None and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
+                ops.int4_gemv_prepacked_into(y, rows, packed)
+            else:
+                ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*x.shape[:-1], self.out_features)
@@ -110,9 +128,24 @@ class Int4GateUpSiLU(nn.Module):
         self.register_buffer("scales", torch.cat([gate.scales, up.scales], dim=0).contiguous())
         self.register_buffer("qzeros", torch.cat([gate.qzeros, up.qzeros], dim=0).contiguous())
 
+    def prepack_(self) -> "Int4GateUpSiLU":
+        """Keep a prepacked copy of gate||up for decode-sized calls (see ``Int4Linear.prepack_``)."""
+        self._packed = None
+        if self.qweight.is_cuda and self.intermediate_size % 16 == 0 and \
+                ops.PrepackedWeight.supported(2 * self.intermediate_size, self.in_features, self.group_size):
+            self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
+            self._direct_rows = self._packed.direct_rows(fused=True)
+        return self
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
-        y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        packed = getattr(self, "_packed", None)
+        if packed is not None and not torch.compiler.is_compiling() and rows.shape[0] <= self._direct_rows \
+                and packed.blob.device == rows.device:
+            y = torch.empty((rows.shape[0], self.intermediate_size), dtype=torch.bfloat16, device=rows.device)
+            ops.int4_gemv_prepacked_into(y, rows, packed, fused=True)
+        else:
+            y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         return y.reshape(*x.shape[:-1], self.intermediate_size)
 
 
@@ -132,6 +165,11 @@ class Int4LlamaMLP(nn.Module):
         as_int4 = lambda m: m if isinstance(m, Int4Linear) else Int4Linear.from_linear(m, group_size)
         self.gate_up = Int4GateUpSiLU(as_int4(mlp.gate_proj), as_int4(mlp.up_proj))
         self.down_proj = as_int4(mlp.down_proj)
+
+    def prepack_(self) -> "Int4LlamaMLP":
+        self.gate_up.prepack_()
+        self.down_proj.prepack_()
+        return self
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.down_proj(self.gate_up(x))

@@ -169,6 +169,17 @@ class PrepackedWeight:
     def supported(N: int, K: int, group_size: int) -> bool:
         return _lib.load().vrl_int4_prepacked_bytes(int(N), int(K), int(group_size)) > 0
 
+    def direct_rows(self, fused: bool = False) -> int:
+        """Most activation rows a plan-free launch (:class:`DirectGemv`) takes for this weight.
+
+        Mirrors the library's rule: the staged activations (K padded to 512, 8 elements of
+        row padding) plus the partial tiles of the K-split must fit 64 KiB of LDS.
+        """
+        nsc = (self.K + 511) // 512
+        waves = 16 if nsc > 8 else (8 if nsc > 4 else 4)
+        spare = 64 * 1024 - (waves - 1) * (2 if fused else 1) * 1024
+        return max(0, min(16, spare // ((nsc * 512 + 8) * 2)))
+
 
 def int4_prepack(qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
                  group_size: int) -> PrepackedWeight:
@@ -332,6 +343,23 @@ class DirectGemv:
 
 def int4_gemv_prepacked_into(y: torch.Tensor, x: torch.Tensor, weight: PrepackedWeight,
                              fused: bool = False) -> torch.Tensor:
-    """``y = x . dequant(weight)^T`` over a prepacked weight, one plan-free launch (M <= 16)."""
-    DirectGemv([(x, weight, fused)], outputs=[y]).launch()
+    """``y = x . dequant(weight)^T`` over a prepacked weight, one plan-free launch.
+
+    Lean eager path (module forward): bf16 contiguous ``x [M <= weight.direct_rows(), K]``
+    and ``y`` on the weight's device; shape preconditions are checked by the library.
+    """
+    if x.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or not x.is_contiguous() or not y.is_contiguous():
+        raise ValueError("x and y must be contiguous bfloat16")
+    if x.dim() != 2 or x.shape[1] != weight.K or tuple(y.shape) != (x.shape[0], weight.N // 2 if fused else weight.N):
+        raise ValueError("x must be [M, K] and y [M, N] for this weight")
+    dev = _require_device("x", x)
+    _require_device("y", y, dev)
+    _require_device("prepacked blob", weight.blob, dev)
+    rec = _lib.Problem()
+    rec.x, rec.qweight, rec.y = x.data_ptr(), weight.blob.data_ptr(), y.data_ptr()
+    rec.M, rec.N, rec.K, rec.G = x.shape[0], weight.N, weight.K, weight.group_size
+    rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
+    with torch.cuda.device(dev):
+        rc = _lib.load().vrl_int4_gemv_prepacked_bf16(ctypes.byref(rec), 1, _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
     return y

@@ -13,7 +13,7 @@ Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
 * ``builder.py:11-33``, ``:77-113`` and ``vrl/distributed/ray/rollout/worker.py:143-163``:
   rollout workers build the policy from a ``RuntimeBuildSpec`` whose ``extra``
   dict is the only channel for new scalar options; ``extra["int4"]`` carries
-  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true}``.
+  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true}``.
 
 Nothing here imports the reference; the policy is duck-typed.
 """
@@ -24,7 +24,7 @@ from typing import Any, Callable, Iterable
 
 from torch import nn
 
-from .linear import Int4Linear, Int4LlamaMLP
+from .linear import Int4GateUpSiLU, Int4Linear, Int4LlamaMLP
 
 ATTN_TARGETS = ("q_proj", "k_proj", "v_proj", "o_proj")
 MLP_TARGETS = ("gate_proj", "up_proj", "down_proj")
@@ -80,12 +80,14 @@ def _swap_all_linears(module: nn.Module, group_size: int) -> int:
 
 def apply_int4_to_policy(policy: Any, group_size: int = 128,
                          targets: Iterable[str] = DEFAULT_TARGETS, fuse_mlp: bool = True,
-                         head: bool = True) -> dict:
+                         head: bool = True, prepack: bool = True) -> dict:
     """Quantise the decode linears of ``policy`` in place; returns a count summary.
 
     ``fuse_mlp`` replaces a whole MLP block by :class:`Int4LlamaMLP` (gate||up with
     the SiLU epilogue in one launch) when all three projections are targeted and
-    none of them carries a LoRA adapter.
+    none of them carries a LoRA adapter.  ``prepack`` keeps a second, MFMA-shaped copy
+    of every quantised weight that lives on a GPU, which decode-sized calls (up to 16
+    activation rows) stream through the plan-free launch.
     """
     targets = tuple(targets)
     unknown = set(targets) - set(DEFAULT_TARGETS)
@@ -119,6 +121,14 @@ def apply_int4_to_policy(policy: Any, group_size: int = 128,
             summary["head_linears"] += int(_swap_linear(owner, "gen_head", group_size))
         else:
             summary["head_linears"] += _swap_all_linears(owner.gen_head, group_size)
+    summary["prepacked"] = 0
+    if prepack:
+        roots = [trunk] + ([owner.gen_head] if head and owner is not None else [])
+        for root in roots:
+            for mod in root.modules():
+                if isinstance(mod, (Int4Linear, Int4GateUpSiLU)):
+                    mod.prepack_()
+                    summary["prepacked"] += int(getattr(mod, "_packed", None) is not None)
     return summary
 
 
@@ -136,14 +146,15 @@ def int4_options_from_spec(spec: Any) -> dict | None:
         opt = {}
     if not isinstance(opt, dict):
         raise TypeError('RuntimeBuildSpec.extra["int4"] must be true or a dict of options')
-    allowed = {"group_size", "targets", "fuse_mlp", "head"}
+    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack"}
     unknown = set(opt) - allowed
     if unknown:
         raise ValueError(f'unknown keys in extra["int4"]: {sorted(unknown)}')
     return {"group_size": int(opt.get("group_size", 128)),
             "targets": tuple(opt.get("targets", DEFAULT_TARGETS)),
             "fuse_mlp": bool(opt.get("fuse_mlp", True)),
-            "head": bool(opt.get("head", True))}
+            "head": bool(opt.get("head", True)),
+            "prepack": bool(opt.get("prepack", True))}
 
 
 def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
