@@ -232,20 +232,29 @@ def other_configs(device, steps: int, warmup: int):
         ws = [make_weights(5100 + i, K, N, G, device) for i in range(48)]
         x = make_x(5107, 1, K, device)
         ys = [torch.empty((1, N), dtype=torch.bfloat16, device=device) for _ in ws]
+        direct = [ops.DirectGemv([(x, ops.int4_prepack(qw, sc, qz, G), False)]) for qw, sc, qz in ws]
 
         def rotate():
             for (qw, sc, qz), y in zip(ws, ys):
                 ops.int4_gemv_into(y, x, qw, sc, qz, G)
 
-        rotate()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            rotate()
-        ms = time_region(graph.replay, max(5, steps // 20), 2) / len(ws)
-        sweep[f"G{G}"] = {"us_per_call_hip_graph": ms * 1e3,
-                          "GBps": algorithmic_bytes(1, K, N, G) / (ms * 1e-3) / 1e9}
-        del ws, ys, graph
+        def rotate_direct():
+            for launch in direct:
+                launch.launch()
+
+        entry = {}
+        for name, fn in (("canonical", rotate), ("prepacked", rotate_direct)):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            ms = time_region(graph.replay, max(5, steps // 20), 2) / len(ws)
+            entry[f"us_per_call_{name}_hip_graph"] = ms * 1e3
+            entry[f"GBps_{name}"] = algorithmic_bytes(1, K, N, G) / (ms * 1e-3) / 1e9
+            del graph
+        sweep[f"G{G}"] = entry
+        del ws, ys, direct
         torch.cuda.empty_cache()
     res["group_size_sweep_k5632_n2048_m1"] = sweep
     return res

@@ -81,14 +81,14 @@ int vrl_int4_gate_up_silu_bf16(const void *x, const void *qweight_gu, const void
                                void *hip_stream);
 
 /*
- * One-time repack of a canonical operand triple (group size 128) into the
+ * One-time repack of a canonical operand triple (group size 32, 64 or 128) into the
  * MFMA-shaped blob the grouped launch streams fastest: every wave load is one
  * contiguous KiB and the matrix cores do the scale/zero arithmetic.  Loader
  * glue: runs once per weight after the policy is built (the reference builds
  * its policy at vrl/models/families/janus_pro/builder.py:11-33).
  * vrl_int4_prepacked_bytes() is the blob size (0 if the shape has no prepacked
- * form: G != 128, K % 128 != 0, or a blob of 2 GiB or more); the blob needs
- * 16-byte alignment.  The
+ * form: G not in {32, 64, 128}, K % 128 != 0, or a blob of 2 GiB or more); the
+ * blob needs 16-byte alignment.  The
  * arithmetic contract is unchanged: the weights a kernel rebuilds from the blob
  * are bit for bit the canonical dequantised tile.
  */
@@ -107,7 +107,10 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
  * valid.  vrl_int4_grouped_plan_size() gives its size; vrl_int4_grouped_plan_build()
  * validates every problem against the preconditions above (and, in addition,
  * requires K % 128 == 0, G a power of two >= 32 and M <= 16 per problem; a
- * prepacked problem needs G == 128 and, if fused, N/2 a multiple of 16),
+ * prepacked problem takes M <= 32, needs G in {32, 64, 128} and, if fused, N/2 a
+ * multiple of 16; the prepacked problems of a plan with more tiles than the
+ * device has workgroup slots share one group size, which is 128 if the plan
+ * also holds canonical problems),
  * fills a host buffer and a small launch descriptor; vrl_int4_gemv_grouped_bf16()
  * takes the DEVICE copy of the blob plus that descriptor.  The plan is built for
  * the current device (its CU count sizes the launch).

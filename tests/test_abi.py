@@ -90,11 +90,14 @@ def test_prepacked_size_and_validation(lib):
     assert lib.vrl_int4_prepacked_bytes(2048, 2048, 128) == 128 * (4 * 256 + 4 * 4096)
     assert lib.vrl_int4_prepacked_bytes(2048, 5632, 128) == 128 * (11 * 256 + 11 * 4096)
     assert lib.vrl_int4_prepacked_bytes(17, 128, 128) == 2 * (256 + 4096)
-    assert lib.vrl_int4_prepacked_bytes(16, 256, 64) == 0
+    assert lib.vrl_int4_prepacked_bytes(16, 256, 64) == 2 * 256 + 4096    # two meta words per lane
+    assert lib.vrl_int4_prepacked_bytes(16, 256, 32) == 4 * 256 + 4096
+    assert lib.vrl_int4_prepacked_bytes(16, 256, 16) == 0
+    assert lib.vrl_int4_prepacked_bytes(16, 256, 256) == 0
     assert lib.vrl_int4_prepacked_bytes(16, 200, 128) == 0
     assert lib.vrl_int4_prepack(p, p, p, None, 16, 128, 128, None) == 1003
     assert lib.vrl_int4_prepack(p, p, p, p + 4, 16, 128, 128, None) == 1002
-    assert lib.vrl_int4_prepack(p, p, p, p, 16, 256, 64, None) == 1001
+    assert lib.vrl_int4_prepack(p, p, p, p, 16, 256, 16, None) == 1001
 
 
 def test_grouped_plan_validation(lib):
@@ -155,7 +158,7 @@ def test_direct_prepacked_validation(lib):
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
     probs[1].prepacked, probs[1].M = 1, 17       # more than 16 activation rows
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
-    probs[1].M, probs[1].G = 1, 64               # no prepacked form for this group size
+    probs[1].M, probs[1].G = 1, 16               # no prepacked form for this group size
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
     probs[1].G, probs[1].y = 128, p + 2          # misaligned output
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002

@@ -393,11 +393,82 @@ def test_prepacked_and_canonical_records_in_one_plan(ops_mod):
 
 
 def test_prepack_rejects_other_group_sizes(ops_mod):
-    ops = o.make_operands(11, 1, 256, 16, 64)
+    ops = o.make_operands(11, 1, 256, 16, 16)
     d = to_device(ops, DEV)
-    assert not ops_mod.PrepackedWeight.supported(16, 256, 64)
+    assert not ops_mod.PrepackedWeight.supported(16, 256, 16)
+    assert not ops_mod.PrepackedWeight.supported(16, 256, 256)
     with pytest.raises(ValueError):
-        ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], 64)
+        ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], 16)
+
+
+PP_GROUP_SHAPES = [
+    # M, K, N, G, fused
+    (1, 5632, 2048, 32, False), (1, 5632, 2048, 64, False),     # the group-size sweep configuration
+    (1, 128, 16, 32, False), (3, 640, 50, 64, False), (16, 2048, 256, 32, False),
+    (32, 2048, 128, 64, False), (32, 5632, 96, 32, False), (12, 4096, 64, 64, False),
+    (1, 2048, 2 * 704, 64, True), (8, 1024, 2 * 48, 32, True),
+]
+
+
+@pytest.mark.parametrize("M,K,N,G,fused", PP_GROUP_SHAPES)
+def test_prepacked_small_groups_parity(ops_mod, M, K, N, G, fused):
+    """Group sizes 32 and 64 through the prepacked layout: grouped plan, and plan-free launch where it applies.
+    Scales log-uniform over 1e-4..1e-1 with asymmetric zero-points, as in the sweep configuration."""
+    say("prepacked groups", M, K, N, G, fused)
+    ops = o.make_operands(9500 + M + K + N + G, M, K, N, G, "loguniform")
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    results = [run_grouped(ops_mod, [(d["x"], pw, fused)])[1][0]]
+    if M <= pw.direct_rows(fused):
+        results.append(ops_mod.DirectGemv([(d["x"], pw, fused)]).launch()[0])
+        torch.cuda.synchronize()
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    for y in results:
+        if not fused:
+            assert_gemv_close(bf16_to_bits(y), ops, G, f"prepacked G{G} M{M} K{K} N{N}")
+            continue
+        ref = o.gate_up_silu_f64(*args)
+        got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
+        tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
+        assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all()
+
+
+@pytest.mark.parametrize("G", [32, 64])
+def test_prepacked_small_groups_one_hot_exact(ops_mod, G):
+    """Every group boundary of the lane's 128-k span picks the right scale and zero-point, bit for bit."""
+    say("prepacked groups one-hot", G)
+    M, K, N = 4, 1024, 48
+    ops = o.make_operands(9600 + G, M, K, N, G, "loguniform")
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    for k0 in sorted(set([0, 31, 32, 33, 63, 64, 65, 95, 96, 127, 128, 160, 511, 512, 544, K - 33, K - 1])):
+        x = np.zeros((M, K), dtype=np.float32)
+        for m in range(M):
+            x[m, (k0 + 37 * m) % K] = 1.0
+        xd = bits_to_bf16(o.f32_to_bf16_bits(x), DEV)
+        outs = [run_grouped(ops_mod, [(xd, pw, False)])[1][0], ops_mod.DirectGemv([(xd, pw, False)]).launch()[0]]
+        torch.cuda.synchronize()
+        for y in outs:
+            y = bf16_to_bits(y)
+            for m in range(M):
+                want = w[:, (k0 + 37 * m) % K]
+                assert ((y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)).all(), (G, k0, m)
+
+
+def test_grouped_plan_takes_one_prepacked_group_size(ops_mod):
+    """A throughput plan (more tiles than the latency kernel takes) holds prepacked records of one group size."""
+    say("mixed group sizes")
+    probs = []
+    for i, G in enumerate((128, 64)):
+        ops = o.make_operands(9700 + i, 1, 256, 16 * 2100, G)     # 2100 tiles each: beyond the latency mode
+        d = to_device(ops, DEV)
+        probs.append((d["x"], ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G), False))
+    with pytest.raises(ValueError):
+        ops_mod.GroupedGemv(probs)
+    for p in probs:                                              # each alone is fine
+        ops_mod.GroupedGemv([p]).launch()
+    torch.cuda.synchronize()
 
 
 # ------------------------------------------------------------------ contract violations

@@ -637,10 +637,11 @@ __device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int 
 // -------------------------------------------------------------------------
 // A one-time repack (prepack_kernel) turns the canonical operand triple into a
 // blob a wave can stream with fully contiguous 1 KB loads and dequantise almost
-// without VALU work.  Group size 128 only.  Per 16-row tile, K padded to 512:
+// without VALU work.  Group sizes 32, 64 and 128.  Per 16-row tile, K padded to 512:
 //
-//   [meta  : nsc x 64 lanes x 4 B]            the word of super-chunk sc and lane l is
-//            (scale bits << 16) | zero  of row (l % 16), group 4*sc + l/16
+//   [meta  : nsc x 64 lanes x gq x 4 B]       word e of super-chunk sc and lane l is
+//            (scale bits << 16) | zero  of row (l % 16), group (4*sc + l/16)*gq + e;
+//            gq = 128 / G groups lie in the 128 k a lane owns per super-chunk
 //   [words : nsc x 4 x 64 lanes x 16 B]       super-chunk sc, load j, lane l, dword d
 //
 // with l = 16*kq + 4*rq + i.  Nibble nu of a weight dword holds
@@ -657,18 +658,22 @@ __device__ __forceinline__ void stream_segment(const DevProblem &p, int t0, int 
 constexpr int PP_SC = 512;  // k per super-chunk: lane group kq owns one 128-k scale group
 
 __host__ __device__ inline int pp_nsc(int K) { return (K + PP_SC - 1) / PP_SC; }
-__host__ __device__ inline long pp_meta_u4(int K) { return (long)pp_nsc(K) * 16; }  // 64 words per super-chunk
-__host__ __device__ inline long pp_tile_u4(int K) { return pp_meta_u4(K) + (long)pp_nsc(K) * 4 * 64; }
+// groups per lane and super-chunk: a lane owns 128 consecutive k of one row
+__host__ __device__ inline int pp_gq(int G) { return 128 / G; }
+// 64 lanes x gq words per super-chunk
+__host__ __device__ inline long pp_meta_u4(int K, int G) { return (long)pp_nsc(K) * 16 * pp_gq(G); }
+__host__ __device__ inline long pp_tile_u4(int K, int G) { return pp_meta_u4(K, G) + (long)pp_nsc(K) * 4 * 64; }
 
 __global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict__ qweight,
                                                       const uint16_t *__restrict__ scales,
                                                       const uint32_t *__restrict__ qzeros,
-                                                      u32x4_t *__restrict__ blob, int N, int K) {
+                                                      u32x4_t *__restrict__ blob, int N, int K, int G) {
     const int kwords = K >> 3;
-    const int groups = K / 128;
+    const int groups = K / G;
     const int zwords = (groups + 7) >> 3;
-    const long meta_u4 = pp_meta_u4(K);
-    const long tile_u4 = pp_tile_u4(K);
+    const int gq = pp_gq(G);
+    const long meta_u4 = pp_meta_u4(K, G);
+    const long tile_u4 = pp_tile_u4(K, G);
     const long ntiles = (N + 15) / 16;
     const long total = ntiles * tile_u4;
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -677,13 +682,14 @@ __global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict
         const long rem = idx - tile * tile_u4;
         u32x4_t out = {0u, 0u, 0u, 0u};
         if (rem < meta_u4) {
-            // meta word of (super-chunk sc, lane): row lane % 16 of the tile, group 4 * sc + lane / 16
-            const int sc = (int)(rem >> 4);
+            // meta word w of the tile: super-chunk w / (64 gq), lane (w / gq) % 64, sub-group w % gq
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int lane = 4 * (int)(rem & 15) + e;
+                const long w = 4 * rem + e;
+                const int sc = (int)(w / (64 * gq));
+                const int lane = (int)(w / gq) & 63;
                 const long row = tile * 16 + (lane & 15);
-                const int g = 4 * sc + (lane >> 4);
+                const int g = (4 * sc + (lane >> 4)) * gq + (int)(w % gq);
                 if (row < N && g < groups) {
                     const uint32_t sb = scales[row * groups + g];
                     const uint32_t z = (qzeros[row * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xFu;
@@ -758,10 +764,10 @@ __device__ __forceinline__ PPGroup pp_group(uint32_t meta_word, int j4) {
 
 // Per-wave stream state of the prepacked path: four 16-byte loads per lane in flight (one
 // super-chunk) and the meta word that goes with them.
-template <int RS>
+template <int RS, int GQ>
 struct PPRing {
     u32x4_t slot[4][RS];
-    uint32_t meta[RS];
+    uint32_t meta[RS][GQ];  // one word per group the lane's 128 k span (GQ = 128 / G)
 };
 
 // The prepacked blob is read through a buffer resource: uniform base and size in SGPRs, one
@@ -772,64 +778,80 @@ constexpr int BUFFER_NT = 2;  // cache-policy bit: non-temporal (streamed once)
 constexpr uint32_t PP_OUT_OF_RANGE = 0x7FFF0000u;  // a per-lane offset no blob reaches (blobs stay below this)
 
 __device__ __forceinline__ rsrc_t pp_blob_rsrc(const DevProblem &p) {
-    const uint32_t bytes = (uint32_t)((p.N + 15) / 16) * (uint32_t)(pp_tile_u4(p.K) * 16);
+    const uint32_t bytes = (uint32_t)((p.N + 15) / 16) * (uint32_t)(pp_tile_u4(p.K, p.G) * 16);
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.qweight), 0, (int)bytes, 0x00020000);
 }
 
 template <bool FUSED>
 struct PPTilePtr {
     uint32_t words[FUSED ? 2 : 1];  // byte offset of the tile's super-chunk sc0 (16 bytes per lane follow)
-    uint32_t meta[FUSED ? 2 : 1];   // byte offset of super-chunk sc0's 64 meta words (4 bytes per lane follow)
+    uint32_t meta[FUSED ? 2 : 1];   // byte offset of super-chunk sc0's meta words (4 * GQ bytes per lane follow)
 };
 
 // where tile `tile_local` of the blob starts, at super-chunk sc0
 template <bool FUSED>
 __device__ __forceinline__ PPTilePtr<FUSED> pp_tile_ptr(const DevProblem &p, int tile_local, int sc0) {
     constexpr int RS = FUSED ? 2 : 1;
-    const uint32_t meta_bytes = (uint32_t)pp_meta_u4(p.K) * 16u;
-    const uint32_t tile_bytes = (uint32_t)pp_tile_u4(p.K) * 16u;
+    const uint32_t meta_bytes = (uint32_t)pp_meta_u4(p.K, p.G) * 16u;
+    const uint32_t tile_bytes = (uint32_t)pp_tile_u4(p.K, p.G) * 16u;
     const int out_tiles = (FUSED ? p.N / 2 : p.N + 15) / 16;
     PPTilePtr<FUSED> t;
 #pragma unroll
     for (int r = 0; r < RS; ++r) {
         const uint32_t base = (uint32_t)(tile_local + r * out_tiles) * tile_bytes;
         t.words[r] = base + meta_bytes + (uint32_t)sc0 * 4096u;
-        t.meta[r] = base + (uint32_t)sc0 * 256u;
+        t.meta[r] = base + (uint32_t)sc0 * 256u * (uint32_t)pp_gq(p.G);
     }
     return t;
 }
 
-// the five loads of one super-chunk: meta word, then four 16-byte slots; slot d alone when
+// the five loads of one super-chunk: meta words, then four 16-byte slots; slot d alone when
 // called with that d, so that a refill can follow each slot's last use
-template <bool FUSED>
+template <bool FUSED, int GQ>
 __device__ __forceinline__ void pp_load_slot(rsrc_t rsrc, uint32_t voff, uint32_t mvoff,
                                              const uint32_t (&words)[FUSED ? 2 : 1],
                                              const uint32_t (&meta)[FUSED ? 2 : 1], int d,
-                                             PPRing<FUSED ? 2 : 1> &ring) {
+                                             PPRing<FUSED ? 2 : 1, GQ> &ring) {
     constexpr int RS = FUSED ? 2 : 1;
 #pragma unroll
     for (int r = 0; r < RS; ++r) {
-        if (d == 0) ring.meta[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, mvoff, meta[r], 0);
+        if (d == 0) {
+            if constexpr (GQ == 1) {
+                ring.meta[r][0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, mvoff, meta[r], 0);
+            } else if constexpr (GQ == 2) {
+                const u32x2_t m = __builtin_amdgcn_raw_buffer_load_b64(rsrc, mvoff, meta[r], 0);
+                ring.meta[r][0] = m[0];
+                ring.meta[r][1] = m[1];
+            } else {
+                const u32x4_t m = __builtin_amdgcn_raw_buffer_load_b128(rsrc, mvoff, meta[r], 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ring.meta[r][e] = m[e];
+            }
+        }
         ring.slot[d][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + d * 1024, words[r], BUFFER_NT);
     }
 }
 
+// per-lane byte offset of the meta words: 4 * GQ bytes per lane
+template <int GQ>
+__device__ __forceinline__ uint32_t pp_meta_voff(uint32_t voff) { return (voff >> 2) * GQ; }
+
 // issue the loads of a tile's first super-chunk
-template <bool FUSED>
-__device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t, PPRing<FUSED ? 2 : 1> &ring) {
+template <bool FUSED, int GQ>
+__device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t, PPRing<FUSED ? 2 : 1, GQ> &ring) {
     const uint32_t voff = (threadIdx.x & (WAVE - 1)) * 16u;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED>(rsrc, voff, voff >> 2, t.words, t.meta, d, ring);
+    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED, GQ>(rsrc, voff, pp_meta_voff<GQ>(voff), t.words, t.meta, d, ring);
 }
 
 // acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob; xs holds x
 // for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
 // if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
 // never runs dry between tiles.
-template <int MB, bool FUSED>
+template <int MB, bool FUSED, int GQ>
 __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
                                                int next_tile, const uint16_t *xs, int xstride,
-                                               int sc0, int sc1, PPRing<FUSED ? 2 : 1> &ring,
+                                               int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
                                                f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
     constexpr int RS = FUSED ? 2 : 1;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -856,10 +878,19 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
     // memory latency per super-chunk.
     auto super_chunk = [&](int sc, uint32_t rv, uint32_t rmv, const uint32_t (&rw)[RS],
                            const uint32_t (&rm)[RS]) {
+        // this super-chunk's meta words: the ring's copy is overwritten by the refill that rides
+        // with slot 0, the later groups of the lane's span are needed after that
+        uint32_t mcur[RS][GQ];
 #pragma unroll
-        for (int r = 0; r < RS; ++r) grp[r] = pp_group(ring.meta[r], j4);
+        for (int r = 0; r < RS; ++r)
+#pragma unroll
+            for (int e = 0; e < GQ; ++e) mcur[r][e] = ring.meta[r][e];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
+            if (d % (4 / GQ) == 0) {  // load d covers 32 k: a new group every 4 / GQ loads
+#pragma unroll
+                for (int r = 0; r < RS; ++r) grp[r] = pp_group(mcur[r][d * GQ / 4], j4);
+            }
             const int kloc = (sc - sc0) * PP_SC + kq * 128 + d * 32;
 #pragma unroll
             for (int dd = 0; dd < 4; ++dd) {
@@ -891,7 +922,7 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            pp_load_slot<FUSED>(rsrc, rv, rmv, rw, rm, d, ring);
+            pp_load_slot<FUSED, GQ>(rsrc, rv, rmv, rw, rm, d, ring);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -909,16 +940,16 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
             const uint32_t w_same = cur.words[r] + (uint32_t)(sc + 1 - sc0) * 4096u;
-            const uint32_t m_same = cur.meta[r] + (uint32_t)(sc + 1 - sc0) * 256u;
+            const uint32_t m_same = cur.meta[r] + (uint32_t)(sc + 1 - sc0) * 256u * GQ;
             rw[r] = last ? (has_next ? nxt.words[r] : cur.words[r]) : w_same;
             rm[r] = last ? (has_next ? nxt.meta[r] : cur.meta[r]) : m_same;
         }
         const bool dry = last && !has_next;
-        super_chunk(sc, dry ? PP_OUT_OF_RANGE : voff, dry ? PP_OUT_OF_RANGE : voff >> 2, rw, rm);
+        super_chunk(sc, dry ? PP_OUT_OF_RANGE : voff, dry ? PP_OUT_OF_RANGE : pp_meta_voff<GQ>(voff), rw, rm);
     }
 }
 
-template <int MB, bool FUSED, int WPB, bool PASSES>
+template <int MB, bool FUSED, int WPB, bool PASSES, int GQ>
 __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile offsets stay scalar
@@ -934,10 +965,10 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
         // super-chunk of a tile already pulls in the first of the next.
         __shared__ int next_tile;
         int tile = t0 + wave;
-        PPRing<RS> ring;
+        PPRing<RS, GQ> ring;
         const rsrc_t rsrc = pp_blob_rsrc(p);
         PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile < t1 ? tile : t0, 0);
-        if (tile < t1) pp_prime<FUSED>(rsrc, cur, ring);  // weights are on their way while x is staged
+        if (tile < t1) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
         __syncthreads();
         if (threadIdx.x == 0) next_tile = t0 + WPB;
         stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
@@ -951,7 +982,7 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
             for (int r = 0; r < RS; ++r)
 #pragma unroll
                 for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            stream_rows_pp<MB, FUSED>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
+            stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
             store_tile<MB, FUSED>(p, tile, acc);
             tile = nt;
             if (tile < t1) cur = pp_tile_ptr<FUSED>(p, tile, 0);
@@ -978,10 +1009,10 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
                 for (int i = 0; i < T; ++i) {
                     const int tile = round + i * WPB + wave;  // neighbouring waves, neighbouring tiles
                     if (tile < t1) {
-                        PPRing<RS> ring;
+                        PPRing<RS, GQ> ring;
                         const PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile, sc0);
-                        pp_prime<FUSED>(rsrc, cur, ring);
-                        stream_rows_pp<MB, FUSED>(p, rsrc, cur, -1, xs, xstride, sc0, sc1, ring, acc[i]);
+                        pp_prime<FUSED, GQ>(rsrc, cur, ring);
+                        stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, -1, xs, xstride, sc0, sc1, ring, acc[i]);
                     }
                 }
             }
@@ -999,7 +1030,7 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // tiles meet in LDS.  A tile is then one or two memory round trips instead of a serial walk
 // over K by a single wave; this is the latency mode for launches of a few matrices
 // (q|k|v of one layer, one o_proj, ...).  LDS: staged activations, then WPB x RS partial tiles.
-template <bool FUSED, int WPB>
+template <bool FUSED, int WPB, int GQ>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1013,9 +1044,9 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     const int sc0 = min(nsc, wave * per), sc1 = min(nsc, sc0 + per);
     const bool work = sc0 < sc1;  // wave-uniform
     const rsrc_t rsrc = pp_blob_rsrc(p);
-    PPRing<RS> ring;
+    PPRing<RS, GQ> ring;
     PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, t0, sc0);
-    if (work) pp_prime<FUSED>(rsrc, cur, ring);  // weights are on their way while x is staged
+    if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
     __syncthreads();
     stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
     __syncthreads();
@@ -1025,7 +1056,7 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 #pragma unroll
         for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if (work) {
-            stream_rows_pp<1, FUSED>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
+            stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
             if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
         }
         if (wave != 0) {
@@ -1044,6 +1075,20 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     }
 }
 
+// the latency kernels take any of the three group sizes in one build (they are not register-critical)
+template <bool FUSED, int WPB>
+__device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    if (FUSED && p.fused) {
+        if (p.G == 128) split_segment_pp<FUSED, WPB, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<FUSED, WPB, 2>(p, t0, t1, smem);
+        else split_segment_pp<FUSED, WPB, 4>(p, t0, t1, smem);
+    } else {
+        if (p.G == 128) split_segment_pp<false, WPB, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<false, WPB, 2>(p, t0, t1, smem);
+        else split_segment_pp<false, WPB, 4>(p, t0, t1, smem);
+    }
+}
+
 template <bool FUSED, int WPB>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem *__restrict__ plan,
                                                                const int2 *__restrict__ block_tab,
@@ -1058,8 +1103,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
-        if (FUSED && p.fused) split_segment_pp<FUSED, WPB>(p, a, b, smem);
-        else split_segment_pp<false, WPB>(p, a, b, smem);
+        split_by_group<FUSED, WPB>(p, a, b, smem);
         t = seg_end;
     }
 }
@@ -1083,8 +1127,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_direct_kernel(DirectArgs
     for (int k = 1; k < DIRECT_MAX; ++k)
         if (k < a.n && a.recs[k].tile_begin <= t) p = a.recs[k];  // scalar selects, no indexing
     const int local = t - p.tile_begin;
-    if (FUSED && p.fused) split_segment_pp<FUSED, WPB>(p, local, local + 1, smem);
-    else split_segment_pp<false, WPB>(p, local, local + 1, smem);
+    split_by_group<FUSED, WPB>(p, local, local + 1, smem);
 }
 
 // CANON / PP / FUSED say which kinds of record the plan holds, so that a plan of
@@ -1094,7 +1137,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_direct_kernel(DirectArgs
 // record with two A operands per weight tile (weights streamed once); PASSES adds the
 // path for prepacked records whose activations do not fit LDS whole (it carries several
 // accumulator tiles, so plans that do not need it run a build without it).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
                                                                 const int2 *__restrict__ block_tab,
                                                                 int n_problems) {
@@ -1111,8 +1154,8 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
         if (PP && (!CANON || p.prepacked)) {
-            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES>(p, a, b, smem);
-            else stream_segment_pp<MB, false, WPB, PASSES>(p, a, b, smem);
+            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES, GQ>(p, a, b, smem);
+            else stream_segment_pp<MB, false, WPB, PASSES, GQ>(p, a, b, smem);
         } else if (CANON) {
             if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
             else stream_segment<MB, false, WPB>(p, a, b, smem);
@@ -1175,11 +1218,11 @@ int stream_staged_k(int M, int K, size_t lds) {
     return (int)(kc < K ? kc : K);
 }
 
-// prepacked blobs exist for group size 128 only
+// prepacked blobs exist for group sizes 32, 64 and 128
 // the stream kernel addresses a blob with 32-bit byte offsets, so a blob stays below 2 GiB
 bool prepack_ok(long N, long K, long G) {
-    if (G != 128 || K % 128 != 0 || N < 1 || K < 128 || N * K >= (1L << 40)) return false;
-    return ((N + 15) / 16) * pp_tile_u4((int)K) * 16 < (long)PP_OUT_OF_RANGE;
+    if ((G != 128 && G != 64 && G != 32) || K % 128 != 0 || N < 1 || K < 128 || N * K >= (1L << 40)) return false;
+    return ((N + 15) / 16) * pp_tile_u4((int)K, (int)G) * 16 < (long)PP_OUT_OF_RANGE;
 }
 
 // stream kernel, prepacked records: all of the padded K if it fits, else whole super-chunks per pass
@@ -1276,14 +1319,14 @@ static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
 constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16,
-              VARIANT_SPLIT = 32;
+              VARIANT_SPLIT = 32, VARIANT_G64 = 64, VARIANT_G32 = 128;
 
 // With recs == nullptr nothing is launched: info->grid receives the number of workgroups of
 // this build that one CU holds at info->lds_bytes (the plan builder sizes the grid with it).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ = 1>
 int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
                   hipStream_t stream) {
-    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES>;
+    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ>;
     if (info->lds_bytes > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
@@ -1302,25 +1345,42 @@ int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *
     return (int)hipGetLastError();
 }
 
+// prepacked-only plans: fused or not, staged passes or not (only the widest workgroups ever
+// need passes: narrower shapes are chosen because x fits), group size
+template <int WPB, int MB, bool FUSED, int GQ>
+int launch_stream_pp_g(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb, hipStream_t stream,
+                       bool passes) {
+    if constexpr (WPB == 16) {
+        if (passes) return launch_stream<WPB, MB, false, true, FUSED, true, GQ>(info, recs, bb, stream);
+    }
+    return launch_stream<WPB, MB, false, true, FUSED, false, GQ>(info, recs, bb, stream);
+}
+
+template <int WPB, int MB>
+int launch_stream_pp(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb, hipStream_t stream,
+                     bool fused, bool passes, int gq) {
+    if (fused) {
+        if (gq == 1) return launch_stream_pp_g<WPB, MB, true, 1>(info, recs, bb, stream, passes);
+        if (gq == 2) return launch_stream_pp_g<WPB, MB, true, 2>(info, recs, bb, stream, passes);
+        return launch_stream_pp_g<WPB, MB, true, 4>(info, recs, bb, stream, passes);
+    }
+    if (gq == 1) return launch_stream_pp_g<WPB, MB, false, 1>(info, recs, bb, stream, passes);
+    if (gq == 2) return launch_stream_pp_g<WPB, MB, false, 2>(info, recs, bb, stream, passes);
+    return launch_stream_pp_g<WPB, MB, false, 4>(info, recs, bb, stream, passes);
+}
+
 // which record kinds a kernel build must handle, for a given workgroup shape
 template <int WPB, int MB>
 int launch_stream_variant(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *bb,
                           hipStream_t stream) {
     const int v = info->variant & (VARIANT_CANON | VARIANT_PP | VARIANT_FUSED);
     const bool passes = (info->variant & VARIANT_PASSES) != 0;
-    if (v == VARIANT_PP) {
-        // only the widest workgroups ever need passes: narrower shapes are chosen because x fits
-        if constexpr (WPB == 16) {
-            if (passes) return launch_stream<WPB, MB, false, true, false, true>(info, recs, bb, stream);
-        }
-        return launch_stream<WPB, MB, false, true, false, false>(info, recs, bb, stream);
+    // prepacked-only plans hold one group size (the kernel build is specialised for it)
+    const int gq = (info->variant & VARIANT_G32) ? 4 : ((info->variant & VARIANT_G64) ? 2 : 1);
+    if (v == VARIANT_PP || v == (VARIANT_PP | VARIANT_FUSED)) {
+        return launch_stream_pp<WPB, MB>(info, recs, bb, stream, (v & VARIANT_FUSED) != 0, passes, gq);
     }
-    if (v == (VARIANT_PP | VARIANT_FUSED)) {
-        if constexpr (WPB == 16) {
-            if (passes) return launch_stream<WPB, MB, false, true, true, true>(info, recs, bb, stream);
-        }
-        return launch_stream<WPB, MB, false, true, true, false>(info, recs, bb, stream);
-    }
+    if (gq != 1) return VRL_INT4_EPLAN;
     if constexpr (MB == 1 && WPB != 8) {  // canonical records: narrow and widest workgroups only
         if (v & VARIANT_FUSED) return launch_stream<WPB, 1, true, true, true, WPB == 16>(info, recs, bb, stream);
         return launch_stream<WPB, 1, true, true, false, WPB == 16>(info, recs, bb, stream);
@@ -1434,7 +1494,7 @@ int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *q
 
 size_t vrl_int4_prepacked_bytes(int N, int K, int G) {
     if (!prepack_ok(N, K, G)) return 0;
-    return (size_t)((N + 15) / 16) * (size_t)pp_tile_u4(K) * 16;
+    return (size_t)((N + 15) / 16) * (size_t)pp_tile_u4(K, G) * 16;
 }
 
 int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros, void *packed,
@@ -1442,14 +1502,14 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     int rc = check_problem(qweight, qweight, scales, qzeros, packed, 1, N, K, G);
     if (rc != VRL_INT4_OK) return rc;
     if (!prepack_ok(N, K, G)) return VRL_INT4_ESHAPE;
-    const long total = (long)((N + 15) / 16) * pp_tile_u4(K);
+    const long total = (long)((N + 15) / 16) * pp_tile_u4(K, G);
     long blocks = (total + 255) / 256;
     const long cap = (long)device_cu_count() * 32;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(prepack_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
-                       static_cast<const uint32_t *>(qzeros), static_cast<u32x4_t *>(packed), N, K);
+                       static_cast<const uint32_t *>(qzeros), static_cast<u32x4_t *>(packed), N, K, G);
     return (int)hipGetLastError();
 }
 
@@ -1531,6 +1591,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     long tiles = 0;
     double total_cost = 0.0;
     int variant = 0;
+    int pp_group_size = 0;      // group size of the prepacked records, -1 if they differ
     size_t x_need = 0;  // bytes the largest activation matrix needs if staged whole
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
@@ -1555,6 +1616,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         if (!tile_path_ok(p)) return VRL_INT4_ESHAPE;  // grouped launches take MFMA-path shapes only
         if (p.prepacked && (!prepack_ok(p.N, p.K, p.G) || (p.fused && (p.N / 2) % 16 != 0)))
             return VRL_INT4_ESHAPE;
+        if (p.prepacked) pp_group_size = (pp_group_size == 0 || pp_group_size == p.G) ? p.G : -1;
         if (p.M > MAX_TILE_M) variant |= VARIANT_MB2;
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
@@ -1640,6 +1702,12 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             variant &= ~VARIANT_SPLIT;
             wpb = sh.wpb;
         }
+    }
+    // The throughput kernel is built per group size: its prepacked records share one, and only
+    // 128 goes together with canonical records.  (The latency kernel takes them mixed.)
+    if (!(variant & VARIANT_SPLIT) && pp_group_size != 0) {
+        if (pp_group_size < 0 || ((variant & VARIANT_CANON) && pp_group_size != 128)) return VRL_INT4_ESHAPE;
+        variant |= pp_group_size == 64 ? VARIANT_G64 : (pp_group_size == 32 ? VARIANT_G32 : 0);
     }
     long per_cu = sh.per_cu;
     const int resident = resident_per_cu(smem + red_bytes);

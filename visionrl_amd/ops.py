@@ -154,7 +154,7 @@ def _(x, qweight_gu, scales_gu, qzeros_gu, group_size):
 
 
 class PrepackedWeight:
-    """A weight repacked once for the grouped launch (group size 128 only).
+    """A weight repacked once for the grouped and plan-free launches (group sizes 32, 64, 128).
 
     ``blob`` is an opaque ``uint8`` device tensor made by the library from the
     canonical ``(qweight, scales, qzeros)`` triple; ``N``, ``K`` and
