@@ -312,6 +312,51 @@ def per_call_latency(items, steps: int):
     return res
 
 
+def module_path(items, steps: int):
+    """The drop-in modules as a decode step calls them: q, k, v, o, gate||up, down per layer, M=1."""
+    from visionrl_amd.linear import Int4GateUpSiLU, Int4Linear
+
+    layers = {}
+    for it in items:
+        if it["proj"] != "head":
+            layers.setdefault(it["layer"], {})[it["proj"]] = Int4Linear.from_packed(
+                it["qweight"], it["scales"], it["qzeros"], GROUP)
+    x_h = items[0]["x"].reshape(1, 1, HIDDEN)
+    out = {}
+    for mode in ("canonical", "prepacked", "prepacked_qkv_grouped"):
+        stack = []
+        for mods in layers.values():
+            q, k, v, o = mods["q"], mods["k"], mods["v"], mods["o"]
+            gate_up, down = Int4GateUpSiLU(mods["gate"], mods["up"]), mods["down"]
+            for m in (q, k, v, o, gate_up, down):
+                m._packed = None
+                m._group = None
+                if mode != "canonical":
+                    m.prepack_()
+            if mode == "prepacked_qkv_grouped":
+                q.group_with(k, v)
+            stack.append((q, k, v, o, gate_up, down))
+
+        def step():
+            for q, k, v, o, gate_up, down in stack:
+                q(x_h), k(x_h), v(x_h)
+                o(x_h)
+                down(gate_up(x_h))
+
+        with torch.no_grad():
+            eager_ms = time_region(step, max(3, steps // 50), 1)
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph):
+                step()
+            graph_ms = time_region(graph.replay, max(5, steps // 10), 2)
+        out[mode] = {"eager_ms_per_step": eager_ms, "hip_graph_ms_per_step": graph_ms,
+                     "launches_per_step": len(stack) * (4 if mode == "prepacked_qkv_grouped" else 6)}
+        del graph, stack
+        torch.cuda.empty_cache()
+    return out
+
+
 def launch_floor_us(device, nodes: int = 96, reps: int = 50):
     """us per node of a HIP graph of tiny dependent kernels: what a launch costs with no work in it."""
     t = torch.zeros(64, device=device)
@@ -424,6 +469,10 @@ def main():
         latency["empty_kernel_hip_graph_node_us"] = launch_floor_us(device)
     except Exception as exc:
         latency["empty_kernel_error"] = repr(exc)[:200]
+    try:
+        modules = module_path(items, args.steps)
+    except Exception as exc:
+        modules = {"error": repr(exc)[:300]}
 
     best = max(strat["GBps"], key=lambda k: strat["GBps"][k])
     headline = "grouped_1_launch"
@@ -474,7 +523,7 @@ def main():
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,
                    "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
-                   "other_configs": others},
+                   "m1_through_modules": modules, "other_configs": others},
     }
     print(json.dumps(result))
 

@@ -55,7 +55,7 @@ def test_apply_swaps_every_decode_linear():
     summary = apply_int4_to_policy(policy, group_size=128)
     # nothing is prepacked on the CPU: the MFMA-shaped copies are made only for weights on a GPU
     assert summary == {"linears": 7 * LAYERS, "fused_mlps": LAYERS, "head_linears": 1, "group_size": 128,
-                       "prepacked": 0}
+                       "prepacked": 0, "qkv_groups": 0}
     for layer in policy._lm_trunk().layers:
         for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
             mod = getattr(layer.self_attn, name)
@@ -192,6 +192,7 @@ def test_swapped_trunk_tracks_the_dequantised_trunk():
     summary = apply_int4_to_policy(policy, group_size=128)
     # every quantised module got its prepacked copy: q/k/v/o + gate||up + down per layer, and the head
     assert summary["prepacked"] == 6 * LAYERS + 1
+    assert summary["qkv_groups"] == LAYERS       # q|k|v of every layer share one launch per decode step
     # give the reference copy the dequantised weights
     for lq, lr in zip(policy._lm_trunk().layers, reference._lm_trunk().layers):
         for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
@@ -245,3 +246,32 @@ def test_prepacked_module_path_agrees_with_the_canonical_one():
             assert (y.double() - ref).abs().le(2.0 ** -7 * ref.abs() + 2.0 ** -6).all()
         if rows > 16:
             assert torch.equal(plain, fast)      # same kernel: beyond 16 rows the prepacked copy is not used
+
+
+@pytest.mark.gpu
+def test_grouped_siblings_hand_results_over_by_tensor_identity():
+    """q|k|v grouped: the leader's launch computes all three; a sibling returns the handed result only
+    for the very same input object, and computes on its own otherwise."""
+    dev = "cuda:0"
+    torch.manual_seed(6)
+    mods = [Int4Linear.from_linear(nn.Linear(512, n, bias=(n == 96)).to(torch.bfloat16).to(dev), 128).prepack_()
+            for n in (128, 96, 64)]
+    alone = [Int4Linear.from_packed(m.qweight, m.scales, m.qzeros, 128, bias=m.bias).prepack_() for m in mods]
+    q, k, v = mods
+    q.group_with(k, v)
+    x = torch.randn(2, 1, 512, device=dev).to(torch.bfloat16)
+    want = [m(x) for m in alone]
+    got_q = q(x)
+    assert k._handed is not None and v._handed is not None
+    got_k, got_v = k(x), v(x)
+    assert k._handed is None and v._handed is None
+    for a, b in zip(want, (got_q, got_k, got_v)):
+        assert torch.equal(a, b)                         # same kernel body, one tile per workgroup either way
+    # another tensor with equal contents is not the same input: the sibling computes it itself
+    q(x)
+    other = x.clone() * 2
+    assert torch.equal(k(other), alone[1](other))
+    assert torch.equal(v(x), want[2])                    # v still takes what q handed it for x
+    # more rows than the plan-free launch takes: every module on its own
+    big = torch.randn(40, 512, device=dev).to(torch.bfloat16)
+    assert torch.equal(q(big), alone[0](big)) and k._handed is None

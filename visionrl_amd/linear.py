@@ -87,18 +87,57 @@ class Int4Linear(nn.Module):
             self._direct_rows = self._packed.direct_rows()
         return self
 
+    def group_with(self, *others: "Int4Linear") -> "Int4Linear":
+        """Launch ``others`` together with this module whenever it is called (q|k|v of one layer).
+
+        Modules that are applied to the same input one after the other, as
+        ``LlamaAttention`` applies ``q_proj``, ``k_proj``, ``v_proj`` to ``hidden_states``
+        (reached from ``vrl/models/families/janus_pro/policy.py:673-678``): a decode-sized call
+        of this module computes all of them in one plan-free launch and hands each sibling its
+        result, which the sibling returns when it is called with the very same tensor object
+        next.  Needs ``prepack_()`` on every member; anything else falls back to one launch each.
+        """
+        if len(others) + 1 > ops.DirectGemv.MAX_PROBLEMS:
+            raise ValueError(f"at most {ops.DirectGemv.MAX_PROBLEMS} modules per group")
+        if any(o.in_features != self.in_features for o in others):
+            raise ValueError("grouped modules take the same input")
+        self._group = (self, *others)
+        return self
+
     def dequantize(self) -> torch.Tensor:
         """The canonical bf16 weight ``[N, K]`` (bit-exact tile), e.g. for the train-time replay."""
         return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
 
+    def _group_ready(self, rows: torch.Tensor):
+        group = getattr(self, "_group", None)
+        if group is None:
+            return None
+        for m in group:
+            packed = getattr(m, "_packed", None)
+            if packed is None or rows.shape[0] > m._direct_rows or packed.blob.device != rows.device:
+                return None
+        return group
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
+        handed = getattr(self, "_handed", None)
+        if handed is not None:
+            self._handed = None
         if torch.compiler.is_compiling():
             y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        elif handed is not None and handed[0] is x:  # computed by the group leader's launch
+            y = handed[1]
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
             y = torch.empty((rows.shape[0], self.out_features), dtype=torch.bfloat16, device=rows.device)
             packed = getattr(self, "_packed", None)
-            if packed is not None and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
+            group = self._group_ready(rows)
+            if group is not None:
+                ys = [y] + [torch.empty((rows.shape[0], m.out_features), dtype=torch.bfloat16,
+                                        device=rows.device) for m in group[1:]]
+                ops.int4_gemv_prepacked_multi_into(ys, rows, [m._packed for m in group])
+                for m, ym in zip(group[1:], ys[1:]):
+                    m._handed = (x, ym)
+            elif packed is not None and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
                 ops.int4_gemv_prepacked_into(y, rows, packed)
             else:
                 ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)

@@ -15,6 +15,7 @@ missing library raises ``Int4LibraryError``.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 
 import torch
@@ -23,11 +24,22 @@ from . import _lib
 from .int4_format import check_packed
 
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
-           "PrepackedWeight", "GroupedGemv"]
+           "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
+           "int4_gemv_prepacked_multi_into"]
 
 
 def _stream_handle(device: torch.device) -> int:
     return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+_NULL = contextlib.nullcontext()
+
+
+def _on(device: torch.device):
+    """Context that makes ``device`` current; free when it already is (the decode-loop case)."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _NULL
+    return torch.cuda.device(device)
 
 
 def _require_device(name: str, t: torch.Tensor, device: torch.device | None = None) -> torch.device:
@@ -275,7 +287,7 @@ class GroupedGemv:
 
     def launch(self):
         lib = _lib.load()
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             rc = lib.vrl_int4_gemv_grouped_bf16(self.plan.data_ptr(), ctypes.byref(self.info),
                                                 _stream_handle(self.device))
         _lib.check(rc, "vrl_int4_gemv_grouped_bf16")
@@ -335,7 +347,7 @@ class DirectGemv:
 
     def launch(self):
         lib = _lib.load()
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             rc = lib.vrl_int4_gemv_prepacked_bf16(self.table, len(self.table), _stream_handle(self.device))
         _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
         return self.outputs
@@ -359,7 +371,33 @@ def int4_gemv_prepacked_into(y: torch.Tensor, x: torch.Tensor, weight: Prepacked
     rec.x, rec.qweight, rec.y = x.data_ptr(), weight.blob.data_ptr(), y.data_ptr()
     rec.M, rec.N, rec.K, rec.G = x.shape[0], weight.N, weight.K, weight.group_size
     rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = _lib.load().vrl_int4_gemv_prepacked_bf16(ctypes.byref(rec), 1, _stream_handle(dev))
     _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
     return y
+
+
+def int4_gemv_prepacked_multi_into(ys, x: torch.Tensor, weights) -> None:
+    """One plan-free launch for up to four prepacked weights applied to the same ``x`` (q|k|v).
+
+    Lean eager path like :func:`int4_gemv_prepacked_into`: ``x`` bf16 contiguous ``[M, K]``,
+    ``ys[i]`` bf16 contiguous ``[M, weights[i].N]``, all on one device.
+    """
+    n = len(weights)
+    if not 1 <= n <= DirectGemv.MAX_PROBLEMS or len(ys) != n:
+        raise ValueError(f"1 to {DirectGemv.MAX_PROBLEMS} weights, one output each")
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("x must be contiguous bfloat16 [M, K]")
+    dev = _require_device("x", x)
+    table = (_lib.Problem * n)()
+    for rec, w, y in zip(table, weights, ys):
+        if w.K != x.shape[1] or y.dtype != torch.bfloat16 or tuple(y.shape) != (x.shape[0], w.N) or \
+                not y.is_contiguous():
+            raise ValueError("every weight must take x's K and every output be contiguous bfloat16 [M, N]")
+        _require_device("y", y, dev)
+        _require_device("prepacked blob", w.blob, dev)
+        rec.x, rec.qweight, rec.y = x.data_ptr(), w.blob.data_ptr(), y.data_ptr()
+        rec.M, rec.N, rec.K, rec.G, rec.prepacked = x.shape[0], w.N, w.K, w.group_size, 1
+    with _on(dev):
+        rc = _lib.load().vrl_int4_gemv_prepacked_bf16(table, n, _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")

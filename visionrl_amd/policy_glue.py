@@ -13,7 +13,7 @@ Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
 * ``builder.py:11-33``, ``:77-113`` and ``vrl/distributed/ray/rollout/worker.py:143-163``:
   rollout workers build the policy from a ``RuntimeBuildSpec`` whose ``extra``
   dict is the only channel for new scalar options; ``extra["int4"]`` carries
-  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true}``.
+  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true}``.
 
 Nothing here imports the reference; the policy is duck-typed.
 """
@@ -68,6 +68,14 @@ def _swap_linear(parent: nn.Module, name: str, group_size: int) -> bool:
     return False
 
 
+def _int4_of(module):
+    """The ``Int4Linear`` behind ``module``: itself, or the ``base_layer`` of a PEFT wrapper."""
+    if isinstance(module, Int4Linear):
+        return module
+    inner = getattr(module, "base_layer", None)
+    return inner if isinstance(inner, Int4Linear) else None
+
+
 def _swap_all_linears(module: nn.Module, group_size: int) -> int:
     n = 0
     for name, child in list(module.named_children()):
@@ -80,14 +88,15 @@ def _swap_all_linears(module: nn.Module, group_size: int) -> int:
 
 def apply_int4_to_policy(policy: Any, group_size: int = 128,
                          targets: Iterable[str] = DEFAULT_TARGETS, fuse_mlp: bool = True,
-                         head: bool = True, prepack: bool = True) -> dict:
+                         head: bool = True, prepack: bool = True, group_qkv: bool = True) -> dict:
     """Quantise the decode linears of ``policy`` in place; returns a count summary.
 
     ``fuse_mlp`` replaces a whole MLP block by :class:`Int4LlamaMLP` (gate||up with
     the SiLU epilogue in one launch) when all three projections are targeted and
     none of them carries a LoRA adapter.  ``prepack`` keeps a second, MFMA-shaped copy
     of every quantised weight that lives on a GPU, which decode-sized calls (up to 16
-    activation rows) stream through the plan-free launch.
+    activation rows) stream through the plan-free launch; with ``group_qkv`` the three
+    projections of an attention block then share one launch per decode step.
     """
     targets = tuple(targets)
     unknown = set(targets) - set(DEFAULT_TARGETS)
@@ -129,6 +138,14 @@ def apply_int4_to_policy(policy: Any, group_size: int = 128,
                 if isinstance(mod, (Int4Linear, Int4GateUpSiLU)):
                     mod.prepack_()
                     summary["prepacked"] += int(getattr(mod, "_packed", None) is not None)
+    summary["qkv_groups"] = 0
+    if prepack and group_qkv:
+        for layer in trunk.layers:
+            attn = getattr(layer, "self_attn", None)
+            members = [_int4_of(getattr(attn, n, None)) for n in ("q_proj", "k_proj", "v_proj")] if attn else []
+            if members and all(m is not None and getattr(m, "_packed", None) is not None for m in members):
+                members[0].group_with(*members[1:])
+                summary["qkv_groups"] += 1
     return summary
 
 
@@ -146,7 +163,7 @@ def int4_options_from_spec(spec: Any) -> dict | None:
         opt = {}
     if not isinstance(opt, dict):
         raise TypeError('RuntimeBuildSpec.extra["int4"] must be true or a dict of options')
-    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack"}
+    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack", "group_qkv"}
     unknown = set(opt) - allowed
     if unknown:
         raise ValueError(f'unknown keys in extra["int4"]: {sorted(unknown)}')
@@ -154,7 +171,8 @@ def int4_options_from_spec(spec: Any) -> dict | None:
             "targets": tuple(opt.get("targets", DEFAULT_TARGETS)),
             "fuse_mlp": bool(opt.get("fuse_mlp", True)),
             "head": bool(opt.get("head", True)),
-            "prepack": bool(opt.get("prepack", True))}
+            "prepack": bool(opt.get("prepack", True)),
+            "group_qkv": bool(opt.get("group_qkv", True))}
 
 
 def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
