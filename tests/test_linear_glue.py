@@ -109,6 +109,59 @@ def test_lora_wrapper_keeps_its_adapter():
     assert isinstance(attn.q_proj.lora_A, nn.Linear)
 
 
+def test_lora_only_weight_sync_leaves_the_int4_base_alone():
+    """The rollout worker's update path (worker.py:55-71) on an int4 policy: adapter tensors are copied
+    in place, base weights of the trainer's state dict are skipped, misfits are refused."""
+    from visionrl_amd.policy_glue import install_lora_weight_sync
+
+    class LoraLike(nn.Module):
+        def __init__(self, base):
+            super().__init__()
+            self.base_layer = base
+            self.lora_A = nn.ModuleDict({"default": nn.Linear(base.in_features, 4, bias=False)})
+            self.lora_B = nn.ModuleDict({"default": nn.Linear(4, base.out_features, bias=False)})
+
+        def forward(self, x):
+            return self.base_layer(x) + self.lora_B["default"](self.lora_A["default"](x))
+
+    class ModulePolicy(nn.Module):       # the reference's policy is an nn.Module holding the network
+        def __init__(self):
+            super().__init__()
+            self.trunk = tiny_llama()
+            for layer in self.trunk.layers:
+                layer.self_attn.q_proj = LoraLike(layer.self_attn.q_proj)
+
+        def _lm_trunk(self):
+            return self.trunk
+
+    trainer, rollout = ModulePolicy(), ModulePolicy()
+    apply_int4_to_policy(rollout, group_size=128, head=False)
+    install_lora_weight_sync(rollout)
+    state = trainer.state_dict()                             # what the trainer exports: everything
+    for key in state:
+        if "lora_" in key:
+            state[key] = torch.randn_like(state[key])
+    before = {k: v.clone() for k, v in rollout.state_dict().items()}
+    ptrs = {k: v.data_ptr() for k, v in rollout.state_dict().items()}
+    summary = rollout.load_trainable_state(state)
+    assert summary["loaded"] == 2 * LAYERS and summary["skipped"] == len(state) - 2 * LAYERS
+    after = rollout.state_dict()
+    for key, value in after.items():
+        assert value.data_ptr() == ptrs[key]                  # in place: plans and graphs stay valid
+        if "lora_" in key:
+            assert torch.equal(value, state[key].to(value.dtype))
+        else:
+            assert torch.equal(value, before[key])            # qweight / scales / qzeros untouched
+    with pytest.raises(ValueError, match="no adapter"):
+        rollout.load_trainable_state({k: v for k, v in state.items() if "lora_" not in k})
+    bad = {k: (v[:1] if "lora_A" in k else v) for k, v in state.items()}
+    with pytest.raises(ValueError, match="shape"):
+        rollout.load_trainable_state(bad)
+    with pytest.raises(ValueError, match="no such adapter"):
+        rollout.load_trainable_state({"trunk.layers.9.self_attn.q_proj.lora_A.default.weight":
+                                      torch.zeros(4, HIDDEN)})
+
+
 def test_state_dict_round_trip():
     lin = nn.Linear(256, 48, bias=True).to(torch.bfloat16)
     a = Int4Linear.from_linear(lin, 64)

@@ -15,13 +15,21 @@ Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
   dict is the only channel for new scalar options; ``extra["int4"]`` carries
   ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true}``.
 
+* ``vrl/distributed/ray/rollout/worker.py:55-71``: a rollout worker applies synced trainer
+  weights through ``policy.load_trainable_state(state)``, which the Janus-Pro policy does not
+  define (the diffusion policies do, ``vrl/models/diffusion.py:233-256``);
+  :func:`install_lora_weight_sync` gives an int4 policy that method for the
+  ``sync_trainable_state: "lora_only"`` mode (``vrl/rollouts/runtime/config.py:20-37``).
+
 Nothing here imports the reference; the policy is duck-typed.
 """
 
 from __future__ import annotations
 
-from typing import Any, Callable, Iterable
+import types
+from typing import Any, Callable, Iterable, Mapping
 
+import torch
 from torch import nn
 
 from .linear import Int4GateUpSiLU, Int4Linear, Int4LlamaMLP
@@ -189,3 +197,62 @@ def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
         if isinstance(meta, dict):
             meta["int4"] = summary
     return bundle
+
+
+# ---------------------------------------------------------------------- weight sync (LoRA only)
+def _policy_root(policy: Any) -> nn.Module:
+    """The module whose ``state_dict`` keys the trainer's copy of the policy uses."""
+    if isinstance(policy, nn.Module):
+        return policy
+    for name in ("mmgpt", "model"):
+        root = getattr(policy, name, None)
+        if isinstance(root, nn.Module):
+            return root
+    raise TypeError("expected an nn.Module policy or one holding its network in .mmgpt / .model")
+
+
+def load_lora_state(policy: Any, state_dict: Mapping[str, Any], prefix: str = "") -> dict:
+    """Copy the adapter tensors of ``state_dict`` into ``policy``; the int4 base stays as it is.
+
+    ``state_dict`` is what the trainer exports for the policy
+    (``vrl/trainers/checkpointing.py:217-227``: a full ``state_dict()``) or just its adapter
+    part.  Keys with ``lora_`` in them must name a tensor of the same shape in the rollout
+    policy and are copied in place (no re-quantisation, no reallocation: captured HIP graphs
+    and grouped plans stay valid).  Every other key is a frozen base weight the rollout copy
+    holds in int4 and is skipped.  Returns ``{"loaded": n, "skipped": m}``; raises
+    ``ValueError`` if there is nothing to load or an adapter key does not fit.
+    """
+    root = _policy_root(policy)
+    own = dict(root.named_parameters())
+    own.update(dict(root.named_buffers()))
+    loaded = skipped = 0
+    problems = []
+    with torch.no_grad():
+        for key, value in state_dict.items():
+            name = key[len(prefix):] if prefix and key.startswith(prefix) else key
+            if "lora_" not in name:
+                skipped += 1
+                continue
+            target = own.get(name)
+            if target is None:
+                problems.append(f"{key}: no such adapter tensor in the rollout policy")
+            elif tuple(target.shape) != tuple(value.shape):
+                problems.append(f"{key}: shape {tuple(value.shape)} != {tuple(target.shape)}")
+            else:
+                target.copy_(value.to(device=target.device, dtype=target.dtype))
+                loaded += 1
+    if problems:
+        raise ValueError("adapter state does not fit the rollout policy: " + "; ".join(problems[:5]))
+    if loaded == 0:
+        raise ValueError("load_trainable_state received no adapter (lora_*) tensors")
+    return {"loaded": loaded, "skipped": skipped}
+
+
+def install_lora_weight_sync(policy: Any, prefix: str = "") -> Any:
+    """Give ``policy`` the ``load_trainable_state(state)`` method rollout workers call."""
+
+    def load_trainable_state(self, state_dict: Mapping[str, Any]) -> dict:
+        return load_lora_state(self, state_dict, prefix=prefix)
+
+    policy.load_trainable_state = types.MethodType(load_trainable_state, policy)
+    return policy
