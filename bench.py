@@ -357,6 +357,41 @@ def module_path(items, steps: int):
     return out
 
 
+def decode_tail(device, steps: int):
+    """CFG + softmax + draw + log-probability over [2B, 16384] logits: fused launch vs the tensor ops."""
+    import torch.nn.functional as F
+    from visionrl_amd import ops
+
+    out = {}
+    for B in (1, 16):
+        gen = torch.Generator(device=device).manual_seed(6000 + B)
+        logits = (torch.randn((2 * B, HEAD), generator=gen, device=device) * 3).to(torch.bfloat16)
+        w, T = 5.0, 1.0
+
+        def torch_ops():
+            cond, uncond = logits.chunk(2, dim=0)
+            guided = uncond + w * (cond - uncond)
+            probs = F.softmax(guided / T, dim=-1)
+            sampled = torch.multinomial(probs, num_samples=1).squeeze(-1)
+            lp = F.log_softmax(cond / T, dim=-1).gather(-1, sampled.unsqueeze(-1)).squeeze(-1)
+            return sampled, lp
+
+        def fused():
+            return ops.cfg_sample(logits, w, T)
+
+        entry = {}
+        for name, fn in (("torch_ops", torch_ops), ("fused", fused)):
+            entry[f"{name}_eager_us"] = time_region(fn, max(20, steps // 5), 5) * 1e3
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph):
+                fn()
+            entry[f"{name}_hip_graph_us"] = time_region(graph.replay, max(20, steps // 5), 5) * 1e3
+            del graph
+        out[f"B{B}"] = entry
+    return out
+
+
 def launch_floor_us(device, nodes: int = 96, reps: int = 50):
     """us per node of a HIP graph of tiny dependent kernels: what a launch costs with no work in it."""
     t = torch.zeros(64, device=device)
@@ -473,6 +508,10 @@ def main():
         modules = module_path(items, args.steps)
     except Exception as exc:
         modules = {"error": repr(exc)[:300]}
+    try:
+        tail = decode_tail(device, args.steps)
+    except Exception as exc:
+        tail = {"error": repr(exc)[:300]}
 
     best = max(strat["GBps"], key=lambda k: strat["GBps"][k])
     headline = "grouped_1_launch"
@@ -523,7 +562,7 @@ def main():
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,
                    "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
-                   "m1_through_modules": modules, "other_configs": others},
+                   "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "other_configs": others},
     }
     print(json.dumps(result))
 

@@ -157,6 +157,23 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
 int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *info,
                                void *hip_stream);
 
+/*
+ * Tail of a decode step after the image-token head, one launch (replaces the tensor ops of
+ * vrl/models/families/janus_pro/policy.py:686-693):
+ *   guided  = uncond + cfg_weight * (cond - uncond)
+ *   probs   = softmax(guided / temperature)
+ *   sampled = argmax(probs / noise)                  (torch.multinomial(probs, 1) for noise ~ Exp(1))
+ *   logprob = log_softmax(cond / temperature)[sampled]
+ * logits is bf16 [2B, V] with the conditional rows first (policy.py:685 chunks it that way), noise
+ * bf16 [B, V] of strictly positive draws, sampled int64 [B], logprob float [B].  Every step is
+ * computed in fp32 and rounded to bf16 where the reference's bf16 tensors are (the division by
+ * the temperature is the product with fl(1/temperature), as torch divides by a host scalar);
+ * the sums of the two softmaxes are fp32 in a fixed order.  Equal maxima resolve to the lowest index.
+ * Preconditions: B >= 1, V >= 1, temperature > 0, non-NULL naturally aligned pointers.
+ */
+int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_t *sampled, float *logprob,
+                        int B, int V, float cfg_weight, float temperature, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -311,3 +311,42 @@ def torch_cpu_linear(x, qweight, scales, qzeros, group_size):
     import torch
 
     return torch.nn.functional.linear(x, torch_dequant(qweight, scales, qzeros, group_size))
+
+
+# ---------------------------------------------------------------------------
+# decode-step tail: CFG combine, softmax, one multinomial draw, log-probability
+# Follows vrl/models/families/janus_pro/policy.py:686-693 with the arithmetic torch applies
+# to bf16 tensors (fp32 per op, result rounded to bf16; tensor / host scalar is a product
+# with fl(1/scalar); multinomial(probs, 1) is argmax(probs / q), q ~ Exp(1)).
+# ---------------------------------------------------------------------------
+def _round_bf16_f32(v: np.ndarray) -> np.ndarray:
+    return bf16_bits_to_f32(f32_to_bf16_bits(np.asarray(v, dtype=np.float32)))
+
+
+def cfg_sample(logits_bits: np.ndarray, noise_bits: np.ndarray, cfg_weight: float, temperature: float):
+    """Returns ``(sampled [B] int64, logprob [B] float32, probs [B,V] float32, ratio [B,V] float32)``.
+
+    ``logits_bits`` uint16 ``[2B, V]`` (conditional rows first), ``noise_bits`` uint16 ``[B, V]``.
+    ``probs`` and ``ratio`` (= probs / noise, the quantity whose argmax is the draw) are
+    returned so that a test can judge near-ties.
+    """
+    f32 = np.float32
+    B = logits_bits.shape[0] // 2
+    c = bf16_bits_to_f32(logits_bits[:B])
+    u = bf16_bits_to_f32(logits_bits[B:])
+    q = bf16_bits_to_f32(noise_bits)
+    w, inv_t = f32(cfg_weight), f32(1.0) / f32(temperature)
+    d = _round_bf16_f32(c - u)
+    g = _round_bf16_f32(u + _round_bf16_f32(w * d))
+    gt = _round_bf16_f32(g * inv_t)
+    ct = _round_bf16_f32(c * inv_t)
+    eg = np.exp((gt - gt.max(axis=1, keepdims=True)).astype(f32)).astype(f32)
+    probs = _round_bf16_f32(eg / eg.sum(axis=1, keepdims=True, dtype=f32))
+    with np.errstate(divide="ignore", invalid="ignore"):
+        ratio = _round_bf16_f32(probs / q)
+    sampled = np.argmax(ratio, axis=1).astype(np.int64)          # first index among equal maxima
+    mc = ct.max(axis=1, keepdims=True)
+    lse = np.log(np.exp((ct - mc).astype(f32)).astype(f32).sum(axis=1, keepdims=True, dtype=f32)).astype(f32)
+    lp_all = _round_bf16_f32(ct - mc - lse)
+    logprob = lp_all[np.arange(B), sampled].astype(f32)
+    return sampled, logprob, probs, ratio

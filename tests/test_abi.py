@@ -24,7 +24,7 @@ def lib():
 def declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(vrl_int4_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(vrl_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -164,3 +164,16 @@ def test_direct_prepacked_validation(lib):
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002
     probs[1].y, probs[1].M, probs[1].K = p, 16, 4096   # activations beyond the LDS this path uses
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
+
+
+def test_cfg_sample_validation(lib):
+    keep, p = buf(4096)
+    f = lib.vrl_cfg_sample_bf16
+    assert f(None, p, p, p, 1, 16, 1.0, 1.0, None) == 1003
+    assert f(p, p, p, None, 1, 16, 1.0, 1.0, None) == 1003
+    assert f(p, p, p, p, 0, 16, 1.0, 1.0, None) == 1001
+    assert f(p, p, p, p, 1, 0, 1.0, 1.0, None) == 1001
+    assert f(p, p, p, p, 1, 16, 1.0, 0.0, None) == 1001          # temperature must be positive
+    assert f(p, p, p, p, 1, 16, 1.0, float("nan"), None) == 1001
+    assert f(p + 1, p, p, p, 1, 16, 1.0, 1.0, None) == 1002
+    assert f(p, p, p + 4, p, 1, 16, 1.0, 1.0, None) == 1002      # int64 output

@@ -27,6 +27,7 @@ SYMBOLS = (
     "vrl_int4_grouped_plan_size",
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
+    "vrl_cfg_sample_bf16",
 )
 
 
@@ -96,6 +97,8 @@ def _bind(lib):
         ctypes.POINTER(Problem), ci, vp, ctypes.c_size_t, ctypes.POINTER(PlanInfo)]
     lib.vrl_int4_gemv_grouped_bf16.restype = ci
     lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
+    lib.vrl_cfg_sample_bf16.restype = ci
+    lib.vrl_cfg_sample_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_float, ctypes.c_float, vp]
 
 
 def load():

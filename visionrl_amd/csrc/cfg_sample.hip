@@ -1,0 +1,179 @@
+// Tail of an autoregressive decode step after the image-token head, as one kernel:
+// classifier-free-guidance combine, softmax, one multinomial draw, log-probability of the draw.
+//
+// Restates vrl/models/families/janus_pro/policy.py:686-693 with the arithmetic torch applies to
+// bf16 tensors there (every tensor op computes in fp32 and rounds its result to bf16):
+//   guided  = uncond + w * (cond - uncond)            three roundings
+//   probs   = softmax(guided / T)                     division by a host scalar = product with fl(1/T)
+//   sampled = multinomial(probs, 1)                   = argmax(probs / q), q ~ Exp(1) drawn by the caller
+//                                                       with the call torch.multinomial makes itself
+//   lp      = log_softmax(cond / T)[sampled]
+// One workgroup per batch row walks the row three times (maxima, sums, draw); the row
+// (6 bytes per vocabulary entry) stays in cache between the walks.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/vrl_int4.h"
+
+namespace {
+
+constexpr int THREADS = 1024;
+constexpr int WAVE = 64;
+constexpr int WAVES = THREADS / WAVE;
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+// round to nearest even, NaN kept quiet: what a torch bf16 kernel stores
+__device__ __forceinline__ float round_bf16(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return __builtin_bit_cast(float, u | 0x00400000u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return __builtin_bit_cast(float, u & 0xFFFF0000u);
+}
+
+struct Row {
+    const uint16_t *cond;
+    const uint16_t *uncond;
+    const uint16_t *noise;
+};
+
+// guided / T and cond / T of one vocabulary entry, as bf16 values held in floats
+__device__ __forceinline__ void scaled_logits(const Row &r, int i, float w, float inv_t, float &gt, float &ct) {
+    const float c = bf16_to_f32(r.cond[i]);
+    const float u = bf16_to_f32(r.uncond[i]);
+    const float d = round_bf16(c - u);
+    const float g = round_bf16(u + round_bf16(w * d));
+    gt = round_bf16(g * inv_t);
+    ct = round_bf16(c * inv_t);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+template <bool MAX>
+__device__ __forceinline__ void block_reduce2(float &a, float &b, float (*lds)[WAVES]) {
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    a = MAX ? wave_max(a) : wave_sum(a);
+    b = MAX ? wave_max(b) : wave_sum(b);
+    __syncthreads();  // the buffer may still be read from the previous reduction
+    if (lane == 0) {
+        lds[0][wave] = a;
+        lds[1][wave] = b;
+    }
+    __syncthreads();
+    a = lds[0][0];
+    b = lds[1][0];
+#pragma unroll
+    for (int k = 1; k < WAVES; ++k) {  // same order in every thread: every thread holds the same result
+        a = MAX ? fmaxf(a, lds[0][k]) : a + lds[0][k];
+        b = MAX ? fmaxf(b, lds[1][k]) : b + lds[1][k];
+    }
+}
+
+__global__ __launch_bounds__(THREADS) void cfg_sample_kernel(const uint16_t *__restrict__ logits,
+                                                             const uint16_t *__restrict__ noise,
+                                                             long long *__restrict__ sampled,
+                                                             float *__restrict__ logprob, int B, int V,
+                                                             float w, float inv_t) {
+    __shared__ float red[2][WAVES];
+    __shared__ float best_v[WAVES];
+    __shared__ int best_i[WAVES];
+    const int b = blockIdx.x;
+    Row r;
+    r.cond = logits + (long)b * V;
+    r.uncond = logits + (long)(B + b) * V;
+    r.noise = noise + (long)b * V;
+
+    // walk 1: maxima of guided / T and of cond / T
+    float mg = -INFINITY, mc = -INFINITY;
+    for (int i = threadIdx.x; i < V; i += THREADS) {
+        float gt, ct;
+        scaled_logits(r, i, w, inv_t, gt, ct);
+        mg = fmaxf(mg, gt);
+        mc = fmaxf(mc, ct);
+    }
+    block_reduce2<true>(mg, mc, red);
+
+    // walk 2: the two softmax denominators
+    float sg = 0.0f, sc = 0.0f;
+    for (int i = threadIdx.x; i < V; i += THREADS) {
+        float gt, ct;
+        scaled_logits(r, i, w, inv_t, gt, ct);
+        sg += expf(gt - mg);
+        sc += expf(ct - mc);
+    }
+    block_reduce2<false>(sg, sc, red);
+
+    // walk 3: argmax of probs / q, lowest index among equal maxima
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < V; i += THREADS) {
+        float gt, ct;
+        scaled_logits(r, i, w, inv_t, gt, ct);
+        const float p = round_bf16(expf(gt - mg) / sg);
+        const float ratio = round_bf16(p / bf16_to_f32(r.noise[i]));
+        if (ratio > bv || (ratio == bv && i < bi) || (ratio != ratio && bv == bv)) {
+            bv = ratio;   // a NaN ratio wins over numbers, as in torch's argmax
+            bi = i;
+        }
+    }
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, WAVE);
+        const int oi = __shfl_xor(bi, off, WAVE);
+        const bool other_nan = ov != ov, mine_nan = bv != bv;
+        const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
+        if (take) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) {
+        best_v[wave] = bv;
+        best_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < WAVES; ++k) {
+            const float ov = best_v[k];
+            const int oi = best_i[k];
+            const bool other_nan = ov != ov, mine_nan = bv != bv;
+            const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
+            if (take) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (bi >= V) bi = 0;  // V >= 1, so only if every ratio compared false: cannot happen for finite input
+        float gt, ct;
+        scaled_logits(r, bi, w, inv_t, gt, ct);
+        sampled[b] = bi;
+        logprob[b] = round_bf16(ct - mc - logf(sc));
+    }
+}
+
+}  // namespace
+
+extern "C" int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_t *sampled, float *logprob,
+                                   int B, int V, float cfg_weight, float temperature, void *hip_stream) {
+    if (!logits || !noise || !sampled || !logprob) return VRL_INT4_ENULL;
+    if (B < 1 || V < 1 || B > (1 << 20) || (long)B * V >= (1L << 40) || !(temperature > 0.0f)) return VRL_INT4_ESHAPE;
+    if ((reinterpret_cast<uintptr_t>(logits) & 1u) || (reinterpret_cast<uintptr_t>(noise) & 1u) ||
+        (reinterpret_cast<uintptr_t>(sampled) & 7u) || (reinterpret_cast<uintptr_t>(logprob) & 3u))
+        return VRL_INT4_EALIGN;
+    hipLaunchKernelGGL(cfg_sample_kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
+                       static_cast<const uint16_t *>(logits), static_cast<const uint16_t *>(noise),
+                       reinterpret_cast<long long *>(sampled), logprob, B, V, cfg_weight, 1.0f / temperature);
+    return (int)hipGetLastError();
+}

@@ -25,7 +25,7 @@ from .int4_format import check_packed
 
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
-           "int4_gemv_prepacked_multi_into"]
+           "int4_gemv_prepacked_multi_into", "cfg_sample"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -401,3 +401,35 @@ def int4_gemv_prepacked_multi_into(ys, x: torch.Tensor, weights) -> None:
     with _on(dev):
         rc = _lib.load().vrl_int4_gemv_prepacked_bf16(table, n, _stream_handle(dev))
     _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
+
+
+def cfg_sample(logits: torch.Tensor, cfg_weight: float, temperature: float, *,
+               generator: torch.Generator | None = None, noise: torch.Tensor | None = None):
+    """CFG combine, softmax, one multinomial draw and its log-probability, in one launch.
+
+    Stands for ``vrl/models/families/janus_pro/policy.py:686-693``: ``logits`` is the head's
+    bf16 ``[2B, V]`` output with the conditional rows first; returns ``(sampled int64 [B],
+    logprob float32 [B])``.  The draw consumes the random stream exactly as
+    ``torch.multinomial(probs, 1)`` does (one ``exponential_(1)`` over a bf16 ``[B, V]``
+    tensor), so a seeded rollout samples the same tokens; pass ``noise`` to supply the
+    exponential draws yourself.
+    """
+    if logits.dtype != torch.bfloat16 or logits.dim() != 2 or logits.shape[0] % 2 != 0 or logits.shape[0] < 2:
+        raise ValueError("logits must be bfloat16 [2B, V]: conditional rows, then unconditional rows")
+    if not temperature > 0:
+        raise ValueError("temperature must be positive")
+    dev = _require_device("logits", logits)
+    B, V = logits.shape[0] // 2, logits.shape[1]
+    if noise is None:
+        noise = torch.empty((B, V), dtype=torch.bfloat16, device=dev).exponential_(1.0, generator=generator)
+    elif noise.dtype != torch.bfloat16 or tuple(noise.shape) != (B, V):
+        raise ValueError(f"noise must be bfloat16 [{B}, {V}]")
+    _require_device("noise", noise, dev)
+    sampled = torch.empty(B, dtype=torch.int64, device=dev)
+    logprob = torch.empty(B, dtype=torch.float32, device=dev)
+    with _on(dev):
+        rc = _lib.load().vrl_cfg_sample_bf16(logits.data_ptr(), noise.data_ptr(), sampled.data_ptr(),
+                                             logprob.data_ptr(), B, V, float(cfg_weight), float(temperature),
+                                             _stream_handle(dev))
+    _lib.check(rc, "vrl_cfg_sample_bf16")
+    return sampled, logprob
