@@ -26,6 +26,16 @@ by mathematics in ``tests/test_oracle.py``: known-answer words, exhaustive
 that reduce the GEMV to an integer matmul or to a column of the dequant tile,
 and the independent C restatement in ``int4_oracle.c``.
 
+``cfg_sample`` restates the tensor ops that follow the image-token head in a decode step
+(``policy.py:686-693``).  Their arithmetic lives in torch, not in the reference; the function is
+pinned (``tests/test_cfg_sample.py``) by closed forms (constant noise samples the mode of the
+guided logits evaluated independently in float64, zero guidance weight ignores the conditional
+rows, the log-probability against a float64 log-softmax, a tiny draw wins), and by running the
+very same torch ops in bfloat16: on the CPU for temperatures where dividing and multiplying by
+the reciprocal coincide, and on the device (GPU tests) under one seed for the rest.  The
+reference's tests hold no numeric vector for it (``tests/models/test_janus_wrapper.py:142-175``
+checks shapes, dtypes and ranges only): PARITY UNPINNED against the reference here too.
+
 bf16 values travel as ``uint16`` bit patterns (numpy has no bf16 dtype).
 """
 
