@@ -1,0 +1,507 @@
+// The prepacked (MFMA-shaped) weight layout: repack kernel, the throughput stream over it and the
+// latency kernels whose waves split K.
+#pragma once
+
+#include "canonical.hpp"
+
+namespace {
+
+// -------------------------------------------------------------------------
+// prepacked weights: MFMA-shaped tiles, dequantised by the matrix cores
+// -------------------------------------------------------------------------
+// A one-time repack (prepack_kernel) turns the canonical operand triple into a
+// blob a wave can stream with fully contiguous 1 KB loads and dequantise almost
+// without VALU work.  Group sizes 32, 64 and 128.  Per 16-row tile, K padded to 512:
+//
+//   [meta  : nsc x 64 lanes x gq x 4 B]       word e of super-chunk sc and lane l is
+//            (scale bits << 16) | zero  of row (l % 16), group (4*sc + l/16)*gq + e;
+//            gq = 128 / G groups lie in the 128 k a lane owns per super-chunk
+//   [words : nsc x 4 x 64 lanes x 16 B]       super-chunk sc, load j, lane l, dword d
+//
+// with l = 16*kq + 4*rq + i.  Nibble nu of a weight dword holds
+//   q[row 4*rq + kp][k = 512*sc + 128*kq + 32*j + 8*d + 4*c + i],
+//   c = (nu % 4) / 2,  kp = 2*(nu % 2) + (nu >= 4).
+// So ((v >> 4s) & 0x000F000F) | 0x43004300 is a bf16 pair (128+q) of two
+// neighbouring ROWS at one k, which is the A operand of v_mfma_f32_4x4x4_16b_bf16
+// (16 independent 4x4x4 products, one per lane quad): with B = diag(scale of the
+// lane's row) and C = -(128+z)*scale it returns the exact fp32 products
+// (q-z)*s for the lane's own row at four consecutive k.  v_cvt_pk_bf16_f32
+// rounds them (the one RNE of the contract), and two such results are the B
+// operand of v_mfma_f32_16x16x32_bf16 against the staged activations.
+// Per 8 weights and lane: 7 VALU unpack ops, 4 conversions, 3 MFMA issues.
+constexpr int PP_SC = 512;  // k per super-chunk: lane group kq owns one 128-k scale group
+
+__host__ __device__ inline int pp_nsc(int K) { return (K + PP_SC - 1) / PP_SC; }
+// groups per lane and super-chunk: a lane owns 128 consecutive k of one row
+__host__ __device__ inline int pp_gq(int G) { return 128 / G; }
+// 64 lanes x gq words per super-chunk
+__host__ __device__ inline long pp_meta_u4(int K, int G) { return (long)pp_nsc(K) * 16 * pp_gq(G); }
+__host__ __device__ inline long pp_tile_u4(int K, int G) { return pp_meta_u4(K, G) + (long)pp_nsc(K) * 4 * 64; }
+
+__global__ __launch_bounds__(256) void prepack_kernel(const uint32_t *__restrict__ qweight,
+                                                      const uint16_t *__restrict__ scales,
+                                                      const uint32_t *__restrict__ qzeros,
+                                                      u32x4_t *__restrict__ blob, int N, int K, int G) {
+    const int kwords = K >> 3;
+    const int groups = K / G;
+    const int zwords = (groups + 7) >> 3;
+    const int gq = pp_gq(G);
+    const long meta_u4 = pp_meta_u4(K, G);
+    const long tile_u4 = pp_tile_u4(K, G);
+    const long ntiles = (N + 15) / 16;
+    const long total = ntiles * tile_u4;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long tile = idx / tile_u4;
+        const long rem = idx - tile * tile_u4;
+        u32x4_t out = {0u, 0u, 0u, 0u};
+        if (rem < meta_u4) {
+            // meta word w of the tile: super-chunk w / (64 gq), lane (w / gq) % 64, sub-group w % gq
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const long w = 4 * rem + e;
+                const int sc = (int)(w / (64 * gq));
+                const int lane = (int)(w / gq) & 63;
+                const long row = tile * 16 + (lane & 15);
+                const int g = (4 * sc + (lane >> 4)) * gq + (int)(w % gq);
+                if (row < N && g < groups) {
+                    const uint32_t sb = scales[row * groups + g];
+                    const uint32_t z = (qzeros[row * zwords + (g >> 3)] >> (4 * (g & 7))) & 0xFu;
+                    out[e] = (sb << 16) | z;
+                }
+            }
+        } else {
+            const long r2 = rem - meta_u4;
+            const int sc = (int)(r2 >> 8);
+            const int j = (int)((r2 >> 6) & 3);
+            const int lane = (int)(r2 & 63);
+            const int kq = lane >> 4, rq = (lane >> 2) & 3, i = lane & 3;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int nu = 0; nu < 8; ++nu) {
+                    const int c = (nu & 3) >> 1;
+                    const int kp = 2 * (nu & 1) + (nu >> 2);
+                    const long row = tile * 16 + 4 * rq + kp;
+                    const int k = sc * PP_SC + kq * 128 + j * 32 + d * 8 + 4 * c + i;
+                    if (row < N && k < K) {
+                        const uint32_t src = qweight[row * kwords + (k >> 3)];
+                        word |= ((src >> (4 * (k & 7))) & 0xFu) << (4 * nu);
+                    }
+                }
+                out[d] = word;
+            }
+        }
+        blob[idx] = out;
+    }
+}
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+constexpr int PP_ZERO_ROW = 2;  // DevProblem::prepacked bit
+
+// natural-order staging of x[:, k0:k1) (k beyond K reads as zero), plus a row of zeros at
+// row M if the record asks for one
+__device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int k1, uint16_t *xs,
+                                                int xstride, int nthreads) {
+    const int words_per_row = (k1 - k0) >> 3;
+    const int total = (p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0)) * words_per_row;
+    for (int idx = threadIdx.x; idx < total; idx += nthreads) {
+        const int m = idx / words_per_row;
+        const int j = idx - m * words_per_row;
+        const int k = k0 + (j << 3);
+        u32x4_t d = {0u, 0u, 0u, 0u};
+        if (k < p.K && m < p.M) d = *as_global(reinterpret_cast<const u32x4_t *>(p.x + (long)m * p.K + k));
+        *reinterpret_cast<u32x4_t *>(xs + m * xstride + (j << 3)) = d;
+    }
+}
+
+struct PPGroup {
+    bf16x4_t bdiag;  // B operand of the 4x4x4 product: scale at k' = lane % 4, zero elsewhere
+    f32x4_t cq;      // C operand: -(128 + z) * scale in all four rows
+};
+
+__device__ __forceinline__ PPGroup pp_group(uint32_t meta_word, int j4) {
+    const uint32_t sb = meta_word >> 16;
+    const float s = __builtin_bit_cast(float, meta_word & 0xFFFF0000u);
+    const float c = -(128.0f + (float)(meta_word & 15u)) * s;
+    u32x2_t bd;
+    bd[0] = (j4 == 0) ? sb : (j4 == 1 ? (sb << 16) : 0u);
+    bd[1] = (j4 == 2) ? sb : (j4 == 3 ? (sb << 16) : 0u);
+    PPGroup g;
+    g.bdiag = __builtin_bit_cast(bf16x4_t, bd);
+    g.cq = f32x4_t{c, c, c, c};
+    return g;
+}
+
+// Per-wave stream state of the prepacked path: four 16-byte loads per lane in flight (one
+// super-chunk) and the meta word that goes with them.
+template <int RS, int GQ>
+struct PPRing {
+    u32x4_t slot[4][RS];
+    uint32_t meta[RS][GQ];  // one word per group the lane's 128 k span (GQ = 128 / G)
+};
+
+// The prepacked blob is read through a buffer resource: uniform base and size in SGPRs, one
+// VGPR (16 * lane) as the per-lane offset for every load, the tile / super-chunk position as
+// a scalar offset.  Reads past the blob return zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int BUFFER_NT = 2;  // cache-policy bit: non-temporal (streamed once)
+constexpr uint32_t PP_OUT_OF_RANGE = 0x7FFF0000u;  // a per-lane offset no blob reaches (blobs stay below this)
+
+__device__ __forceinline__ rsrc_t pp_blob_rsrc(const DevProblem &p) {
+    const uint32_t bytes = (uint32_t)((p.N + 15) / 16) * (uint32_t)(pp_tile_u4(p.K, p.G) * 16);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(p.qweight), 0, (int)bytes, 0x00020000);
+}
+
+template <bool FUSED>
+struct PPTilePtr {
+    uint32_t words[FUSED ? 2 : 1];  // byte offset of the tile's super-chunk sc0 (16 bytes per lane follow)
+    uint32_t meta[FUSED ? 2 : 1];   // byte offset of super-chunk sc0's meta words (4 * GQ bytes per lane follow)
+};
+
+// where tile `tile_local` of the blob starts, at super-chunk sc0
+template <bool FUSED>
+__device__ __forceinline__ PPTilePtr<FUSED> pp_tile_ptr(const DevProblem &p, int tile_local, int sc0) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const uint32_t meta_bytes = (uint32_t)pp_meta_u4(p.K, p.G) * 16u;
+    const uint32_t tile_bytes = (uint32_t)pp_tile_u4(p.K, p.G) * 16u;
+    const int out_tiles = (FUSED ? p.N / 2 : p.N + 15) / 16;
+    PPTilePtr<FUSED> t;
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        const uint32_t base = (uint32_t)(tile_local + r * out_tiles) * tile_bytes;
+        t.words[r] = base + meta_bytes + (uint32_t)sc0 * 4096u;
+        t.meta[r] = base + (uint32_t)sc0 * 256u * (uint32_t)pp_gq(p.G);
+    }
+    return t;
+}
+
+// the five loads of one super-chunk: meta words, then four 16-byte slots; slot d alone when
+// called with that d, so that a refill can follow each slot's last use
+template <bool FUSED, int GQ>
+__device__ __forceinline__ void pp_load_slot(rsrc_t rsrc, uint32_t voff, uint32_t mvoff,
+                                             const uint32_t (&words)[FUSED ? 2 : 1],
+                                             const uint32_t (&meta)[FUSED ? 2 : 1], int d,
+                                             PPRing<FUSED ? 2 : 1, GQ> &ring) {
+    constexpr int RS = FUSED ? 2 : 1;
+#pragma unroll
+    for (int r = 0; r < RS; ++r) {
+        if (d == 0) {
+            if constexpr (GQ == 1) {
+                ring.meta[r][0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, mvoff, meta[r], 0);
+            } else if constexpr (GQ == 2) {
+                const u32x2_t m = __builtin_amdgcn_raw_buffer_load_b64(rsrc, mvoff, meta[r], 0);
+                ring.meta[r][0] = m[0];
+                ring.meta[r][1] = m[1];
+            } else {
+                const u32x4_t m = __builtin_amdgcn_raw_buffer_load_b128(rsrc, mvoff, meta[r], 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ring.meta[r][e] = m[e];
+            }
+        }
+        ring.slot[d][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + d * 1024, words[r], BUFFER_NT);
+    }
+}
+
+// per-lane byte offset of the meta words: 4 * GQ bytes per lane
+template <int GQ>
+__device__ __forceinline__ uint32_t pp_meta_voff(uint32_t voff) { return (voff >> 2) * GQ; }
+
+// issue the loads of a tile's first super-chunk
+template <bool FUSED, int GQ>
+__device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t, PPRing<FUSED ? 2 : 1, GQ> &ring) {
+    const uint32_t voff = (threadIdx.x & (WAVE - 1)) * 16u;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) pp_load_slot<FUSED, GQ>(rsrc, voff, pp_meta_voff<GQ>(voff), t.words, t.meta, d, ring);
+}
+
+// acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob; xs holds x
+// for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
+// if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
+// never runs dry between tiles.
+template <int MB, bool FUSED, int GQ>
+__device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
+                                               int next_tile, const uint16_t *xs, int xstride,
+                                               int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
+                                               f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int lc = lane & 15;
+    const int kq = lane >> 4;
+    const int j4 = lane & 3;
+
+    // both must sit in registers for (v & mask) | bias to select v_and_or_b32
+    uint32_t mask = PAIR_MASK, bias = PAIR_BIAS;
+    asm volatile("" : "+s"(mask));
+    asm volatile("" : "+v"(bias));
+
+    static_assert(STREAM_DEPTH == 4, "the ring holds exactly one super-chunk (four loads per lane)");
+    PPGroup grp[RS];
+    // A-operand rows beyond M are padding: they read the staged row of zeros if there is one
+    // (quiet multipliers; the chip runs this kernel at its power limit, so that shows up as
+    // clock), else a copy of the last row
+    const int pad_row = (p.prepacked & PP_ZERO_ROW) ? p.M : p.M - 1;
+
+    // One super-chunk: 4 loads x 4 words per lane = 16 dequant + dot steps, no branch inside.
+    // Each ring slot is reloaded from offset rw (and the meta word from rm, with slot 0) as
+    // soon as its last word is consumed.  The scheduling barriers pin the loads there: left alone,
+    // the scheduler gathers them at the end of the body and the wave then waits out a whole
+    // memory latency per super-chunk.
+    auto super_chunk = [&](int sc, uint32_t rv, uint32_t rmv, const uint32_t (&rw)[RS],
+                           const uint32_t (&rm)[RS]) {
+        // this super-chunk's meta words: the ring's copy is overwritten by the refill that rides
+        // with slot 0, the later groups of the lane's span are needed after that
+        uint32_t mcur[RS][GQ];
+#pragma unroll
+        for (int r = 0; r < RS; ++r)
+#pragma unroll
+            for (int e = 0; e < GQ; ++e) mcur[r][e] = ring.meta[r][e];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            if (d % (4 / GQ) == 0) {  // load d covers 32 k: a new group every 4 / GQ loads
+#pragma unroll
+                for (int r = 0; r < RS; ++r) grp[r] = pp_group(mcur[r][d * GQ / 4], j4);
+            }
+            const int kloc = (sc - sc0) * PP_SC + kq * 128 + d * 32;
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                bf16x8_t xa[MB];
+#pragma unroll
+                for (int b = 0; b < MB; ++b) {
+                    const int m = min(16 * b + lc, pad_row);
+                    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
+                    xa[b] = __builtin_bit_cast(bf16x8_t, raw);
+                }
+#pragma unroll
+                for (int r = 0; r < RS; ++r) {
+                    const uint32_t v = ring.slot[d][r][dd];
+                    u32x2_t a0, a1;
+                    a0[0] = (v & mask) | bias;
+                    a0[1] = ((v >> 4) & mask) | bias;
+                    a1[0] = ((v >> 8) & mask) | bias;
+                    a1[1] = ((v >> 12) & mask) | bias;
+                    const f32x4_t d0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                        __builtin_bit_cast(bf16x4_t, a0), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                    const f32x4_t d1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                        __builtin_bit_cast(bf16x4_t, a1), grp[r].bdiag, grp[r].cq, 0, 0, 0);
+                    const u32x4_t wv = {pack_bf16_rne(d0[0], d0[1]), pack_bf16_rne(d0[2], d0[3]),
+                                        pack_bf16_rne(d1[0], d1[1]), pack_bf16_rne(d1[2], d1[3])};
+                    const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+                    for (int b = 0; b < MB; ++b)
+                        acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            pp_load_slot<FUSED, GQ>(rsrc, rv, rmv, rw, rm, d, ring);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // After the last super-chunk the ring is refilled from the next tile's first one.  With no
+    // next tile the refill is issued all the same, with a per-lane offset beyond the end of
+    // the blob: the buffer range check answers such a load with zeros without touching
+    // memory, and the loop body exists once and has no branch.
+    const bool has_next = next_tile >= 0;
+    const PPTilePtr<FUSED> nxt = pp_tile_ptr<FUSED>(p, has_next ? next_tile : 0, sc0);
+    const uint32_t voff = lane * 16u;
+    for (int sc = sc0; sc < sc1; ++sc) {
+        const bool last = sc + 1 == sc1;
+        uint32_t rw[RS], rm[RS];
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+            const uint32_t w_same = cur.words[r] + (uint32_t)(sc + 1 - sc0) * 4096u;
+            const uint32_t m_same = cur.meta[r] + (uint32_t)(sc + 1 - sc0) * 256u * GQ;
+            rw[r] = last ? (has_next ? nxt.words[r] : cur.words[r]) : w_same;
+            rm[r] = last ? (has_next ? nxt.meta[r] : cur.meta[r]) : m_same;
+        }
+        const bool dry = last && !has_next;
+        super_chunk(sc, dry ? PP_OUT_OF_RANGE : voff, dry ? PP_OUT_OF_RANGE : pp_meta_voff<GQ>(voff), rw, rm);
+    }
+}
+
+template <int MB, bool FUSED, int WPB, bool PASSES, int GQ>
+__device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile offsets stay scalar
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int xstride = p.kc + XPAD;
+    const int nsc = pp_nsc(p.K);
+    const int sc_pass = p.kc / PP_SC;
+    if (!PASSES || sc_pass >= nsc) {
+        // Tiles of the segment are handed out through a counter in LDS: waves on one SIMD do
+        // not progress at equal rates (older waves win the issue arbitration), and with a
+        // fixed deal the workgroup would wait at the next barrier for its slowest wave.
+        // A wave draws its next tile before it starts the current one, so that the last
+        // super-chunk of a tile already pulls in the first of the next.
+        __shared__ int next_tile;
+        int tile = t0 + wave;
+        PPRing<RS, GQ> ring;
+        const rsrc_t rsrc = pp_blob_rsrc(p);
+        PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile < t1 ? tile : t0, 0);
+        if (tile < t1) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
+        __syncthreads();
+        if (threadIdx.x == 0) next_tile = t0 + WPB;
+        stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+        __syncthreads();
+        while (tile < t1) {
+            int nt = 0;
+            if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
+            nt = __builtin_amdgcn_readfirstlane(nt);
+            f32x4_t acc[RS][MB];
+#pragma unroll
+            for (int r = 0; r < RS; ++r)
+#pragma unroll
+                for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
+            store_tile<MB, FUSED>(p, tile, acc);
+            tile = nt;
+            if (tile < t1) cur = pp_tile_ptr<FUSED>(p, tile, 0);
+        }
+    } else if constexpr (PASSES) {
+        // activations do not fit: K is walked in staged passes, and every wave carries T tiles
+        // through a pass so that one staging serves T * WPB tiles
+        constexpr int T = FUSED ? 1 : (MB == 2 ? 2 : 4);
+        const rsrc_t rsrc = pp_blob_rsrc(p);
+        for (int round = t0; round < t1; round += WPB * T) {
+            f32x4_t acc[T][RS][MB];
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+#pragma unroll
+                for (int r = 0; r < RS; ++r)
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) acc[i][r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int sc0 = 0; sc0 < nsc; sc0 += sc_pass) {
+                const int sc1 = min(nsc, sc0 + sc_pass);
+                __syncthreads();
+                stage_x_natural(p, sc0 * PP_SC, sc1 * PP_SC, xs, xstride, WPB * WAVE);
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < T; ++i) {
+                    const int tile = round + i * WPB + wave;  // neighbouring waves, neighbouring tiles
+                    if (tile < t1) {
+                        PPRing<RS, GQ> ring;
+                        const PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile, sc0);
+                        pp_prime<FUSED, GQ>(rsrc, cur, ring);
+                        stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, -1, xs, xstride, sc0, sc1, ring, acc[i]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < T; ++i) {
+                const int tile = round + i * WPB + wave;
+                if (tile < t1) store_tile<MB, FUSED>(p, tile, acc[i]);
+            }
+        }
+    }
+}
+
+// Small plans (fewer tiles than the device has workgroup slots): the waves of a workgroup
+// share one tile, each taking a contiguous quarter of its super-chunks, and the partial
+// tiles meet in LDS.  A tile is then one or two memory round trips instead of a serial walk
+// over K by a single wave; this is the latency mode for launches of a few matrices
+// (q|k|v of one layer, one o_proj, ...).  LDS: staged activations, then WPB x RS partial tiles.
+template <bool FUSED, int WPB, int GQ>
+__device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    constexpr int RS = FUSED ? 2 : 1;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (WAVE - 1);
+    uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
+    const int xstride = p.kc + XPAD;
+    const int xrows = p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0);
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + (size_t)xrows * xstride * 2);
+    const int nsc = pp_nsc(p.K);
+    const int per = (nsc + WPB - 1) / WPB;
+    const int sc0 = min(nsc, wave * per), sc1 = min(nsc, sc0 + per);
+    const bool work = sc0 < sc1;  // wave-uniform
+    const rsrc_t rsrc = pp_blob_rsrc(p);
+    PPRing<RS, GQ> ring;
+    PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, t0, sc0);
+    if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
+    __syncthreads();
+    stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+    __syncthreads();
+    for (int tile = t0; tile < t1; ++tile) {
+        const int next = tile + 1 < t1 ? tile + 1 : -1;
+        f32x4_t acc[RS][1];
+#pragma unroll
+        for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (work) {
+            stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
+            if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
+        }
+        if (wave != 0) {
+#pragma unroll
+            for (int r = 0; r < RS; ++r) red[((wave - 1) * RS + r) * WAVE + lane] = acc[r][0];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int w = 1; w < WPB; ++w)
+#pragma unroll
+                for (int r = 0; r < RS; ++r) acc[r][0] += red[((w - 1) * RS + r) * WAVE + lane];
+            store_tile<1, FUSED>(p, tile, acc);
+        }
+        if (next >= 0) __syncthreads();  // the partial tiles are read before they are rewritten
+    }
+}
+
+// the latency kernels take any of the three group sizes in one build (they are not register-critical)
+template <bool FUSED, int WPB>
+__device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+    if (FUSED && p.fused) {
+        if (p.G == 128) split_segment_pp<FUSED, WPB, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<FUSED, WPB, 2>(p, t0, t1, smem);
+        else split_segment_pp<FUSED, WPB, 4>(p, t0, t1, smem);
+    } else {
+        if (p.G == 128) split_segment_pp<false, WPB, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<false, WPB, 2>(p, t0, t1, smem);
+        else split_segment_pp<false, WPB, 4>(p, t0, t1, smem);
+    }
+}
+
+template <bool FUSED, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem *__restrict__ plan,
+                                                               const int2 *__restrict__ block_tab,
+                                                               int n_problems) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int2 entry = block_tab[blockIdx.x];
+    int t = entry.x;
+    const int t_end = block_tab[blockIdx.x + 1].x;
+    if (t >= t_end) return;  // block-uniform
+    for (int pi = entry.y; t < t_end && pi < n_problems; ++pi) {
+        const DevProblem p = plan[pi];
+        const int out_cols = p.fused ? p.N / 2 : p.N;
+        const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
+        const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
+        split_by_group<FUSED, WPB>(p, a, b, smem);
+        t = seg_end;
+    }
+}
+
+// The same latency mode without a plan in device memory: up to DIRECT_MAX records travel
+// as kernel arguments (no dependent loads before the first weight request), one workgroup per
+// tile.  This is the single-call path of a prepacked weight (and of q|k|v, gate|up groups).
+constexpr int DIRECT_MAX = 4;
+struct DirectArgs {
+    int32_t n;
+    int32_t pad;
+    DevProblem recs[DIRECT_MAX];
+};
+
+template <bool FUSED, int WPB>
+__global__ __launch_bounds__(WPB *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int t = blockIdx.x;
+    DevProblem p = a.recs[0];
+#pragma unroll
+    for (int k = 1; k < DIRECT_MAX; ++k)
+        if (k < a.n && a.recs[k].tile_begin <= t) p = a.recs[k];  // scalar selects, no indexing
+    const int local = t - p.tile_begin;
+    split_by_group<FUSED, WPB>(p, local, local + 1, smem);
+}
+
+}  // namespace
