@@ -482,9 +482,14 @@ def main():
                 ws = [make_weights(100 + i, K, N, GROUP, device) for i in range(40)]
                 x = make_x(1, M, K, device)
                 y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+                direct = []
+                if M <= ops.DirectGemv.MAX_ROWS:   # the plan-free launch over the prepacked layout
+                    direct = [ops.DirectGemv([(x, ops.int4_prepack(qw, sc, qz, GROUP), False)]) for qw, sc, qz in ws]
                 for _ in range(3):
                     for qw, sc, qz in ws:
                         ops.int4_gemv_into(y, x, qw, sc, qz, GROUP)
+                    for launch in direct:
+                        launch.launch()
                 torch.cuda.synchronize()
         print(json.dumps({"single_calls": "done"}))
         return
