@@ -85,6 +85,10 @@ class Int4Linear(nn.Module):
                                                                   self.group_size):
             self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
             self._direct_rows = self._packed.direct_rows()
+            self._call = ops.DirectCall([self._packed])
+        group = getattr(self, "_group", None)
+        if group is not None:  # rebuild the group's launch over the new copies
+            self.group_with(*group[1:])
         return self
 
     def group_with(self, *others: "Int4Linear") -> "Int4Linear":
@@ -102,21 +106,14 @@ class Int4Linear(nn.Module):
         if any(o.in_features != self.in_features for o in others):
             raise ValueError("grouped modules take the same input")
         self._group = (self, *others)
+        self._group_call = None
+        if all(getattr(m, "_packed", None) is not None for m in self._group):
+            self._group_call = ops.DirectCall([m._packed for m in self._group])
         return self
 
     def dequantize(self) -> torch.Tensor:
         """The canonical bf16 weight ``[N, K]`` (bit-exact tile), e.g. for the train-time replay."""
         return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
-
-    def _group_ready(self, rows: torch.Tensor):
-        group = getattr(self, "_group", None)
-        if group is None:
-            return None
-        for m in group:
-            packed = getattr(m, "_packed", None)
-            if packed is None or rows.shape[0] > m._direct_rows or packed.blob.device != rows.device:
-                return None
-        return group
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
@@ -128,18 +125,23 @@ class Int4Linear(nn.Module):
         elif handed is not None and handed[0] is x:  # computed by the group leader's launch
             y = handed[1]
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
-            y = torch.empty((rows.shape[0], self.out_features), dtype=torch.bfloat16, device=rows.device)
             packed = getattr(self, "_packed", None)
-            group = self._group_ready(rows)
-            if group is not None:
-                ys = [y] + [torch.empty((rows.shape[0], m.out_features), dtype=torch.bfloat16,
-                                        device=rows.device) for m in group[1:]]
-                ops.int4_gemv_prepacked_multi_into(ys, rows, [m._packed for m in group])
-                for m, ym in zip(group[1:], ys[1:]):
-                    m._handed = (x, ym)
-            elif packed is not None and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
-                ops.int4_gemv_prepacked_into(y, rows, packed)
+            M = rows.shape[0]
+            if packed is not None and packed.blob.device == rows.device:
+                call = getattr(self, "_group_call", None)
+                if call is not None and M <= call.max_rows:
+                    ys = call(rows)
+                    for m, ym in zip(self._group[1:], ys[1:]):
+                        m._handed = (x, ym)
+                    y = ys[0]
+                elif M <= self._direct_rows:
+                    y = self._call(rows)[0]
+                else:
+                    packed = None
             else:
+                packed = None
+            if packed is None:
+                y = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=rows.device)
                 ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
         if self.bias is not None:
             y = y + self.bias
@@ -174,6 +176,7 @@ class Int4GateUpSiLU(nn.Module):
                 ops.PrepackedWeight.supported(2 * self.intermediate_size, self.in_features, self.group_size):
             self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
             self._direct_rows = self._packed.direct_rows(fused=True)
+            self._call = ops.DirectCall([self._packed], fused=True)
         return self
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -181,8 +184,7 @@ class Int4GateUpSiLU(nn.Module):
         packed = getattr(self, "_packed", None)
         if packed is not None and not torch.compiler.is_compiling() and rows.shape[0] <= self._direct_rows \
                 and packed.blob.device == rows.device:
-            y = torch.empty((rows.shape[0], self.intermediate_size), dtype=torch.bfloat16, device=rows.device)
-            ops.int4_gemv_prepacked_into(y, rows, packed, fused=True)
+            y = self._call(rows)[0]
         else:
             y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         return y.reshape(*x.shape[:-1], self.intermediate_size)

@@ -25,7 +25,7 @@ from .int4_format import check_packed
 
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
-           "int4_gemv_prepacked_multi_into", "cfg_sample"]
+           "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -433,3 +433,57 @@ def cfg_sample(logits: torch.Tensor, cfg_weight: float, temperature: float, *,
                                              _stream_handle(dev))
     _lib.check(rc, "vrl_cfg_sample_bf16")
     return sampled, logprob
+
+
+class DirectCall:
+    """Reusable plan-free launch for one module's weight, or a q|k|v group: the eager decode path.
+
+    Everything that does not change between calls (blob pointers, shapes) sits in a record
+    table built once; a call fills in the activation pointer, the row count and the output
+    pointers, allocates all outputs as one buffer, and launches.  The Python side of a decode
+    step is host-bound, so this path validates only what can change (the caller, a module,
+    owns the rest): ``x2d`` must be a contiguous bf16 ``[M, K]`` tensor on the weights' device.
+    """
+
+    def __init__(self, weights, fused: bool = False):
+        if not 1 <= len(weights) <= DirectGemv.MAX_PROBLEMS:
+            raise ValueError(f"1 to {DirectGemv.MAX_PROBLEMS} weights")
+        self.table = (_lib.Problem * len(weights))()
+        self.cols = []
+        self.device = weights[0].blob.device
+        self.K = weights[0].K
+        for rec, w in zip(self.table, weights):
+            if w.K != self.K or w.blob.device != self.device:
+                raise ValueError("grouped weights take the same input on one device")
+            rec.qweight, rec.N, rec.K, rec.G = w.blob.data_ptr(), w.N, w.K, w.group_size
+            rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
+            self.cols.append(w.N // 2 if fused else w.N)
+        self._keep = list(weights)
+        self.max_rows = min(w.direct_rows(fused) for w in weights)
+        self._fn = _lib.load().vrl_int4_gemv_prepacked_bf16
+        self._n = len(weights)
+
+    def __call__(self, x2d: torch.Tensor):
+        M = x2d.shape[0]
+        if self._n == 1:
+            y = torch.empty((M, self.cols[0]), dtype=torch.bfloat16, device=x2d.device)
+            rec = self.table[0]
+            rec.x, rec.y, rec.M = x2d.data_ptr(), y.data_ptr(), M
+            with _on(self.device):
+                rc = self._fn(self.table, 1, torch.cuda.current_stream(self.device).cuda_stream)
+            if rc:
+                _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
+            return [y]
+        # every output starts on a 16-byte boundary of the one buffer
+        sizes = [(M * c + 7) & ~7 for c in self.cols]
+        buf = torch.empty(sum(sizes), dtype=torch.bfloat16, device=x2d.device)
+        xp, base, off, outs = x2d.data_ptr(), buf.data_ptr(), 0, []
+        for rec, c, size in zip(self.table, self.cols, sizes):
+            rec.x, rec.y, rec.M = xp, base + 2 * off, M
+            outs.append(buf[off:off + M * c].view(M, c))
+            off += size
+        with _on(self.device):
+            rc = self._fn(self.table, self._n, torch.cuda.current_stream(self.device).cuda_stream)
+        if rc:
+            _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
+        return outs
