@@ -138,13 +138,14 @@ typedef struct vrl_int4_plan_info {
 } vrl_int4_plan_info;
 
 /*
- * Plan-free launch of one to four prepacked GEMVs that share a kernel (one nn.Linear.forward
- * over a prepacked weight, or the q|k|v / gate|up linears of one decoder layer,
- * policy.py:673-678): the records travel as kernel arguments, one workgroup per 16-column
- * tile with its waves splitting K.  Meant for decode (the launch is one memory round trip);
- * every problem must have prepacked = 1, M <= 16 and activations of at most ~60 KB
- * (M * K * 2 bytes), else VRL_INT4_ESHAPE and the caller uses a grouped plan or
- * vrl_int4_gemv_bf16.  scales and qzeros of the records are ignored.
+ * Plan-free launch of a few prepacked GEMVs that share a kernel (one nn.Linear.forward over a
+ * prepacked weight, or the q|k|v / gate|up linears of one decoder layer, policy.py:673-678):
+ * the records travel as kernel arguments, the waves of a workgroup split K of a 16-column
+ * tile.  Meant for decode and rollout batches (the launch is one memory round trip).  Every
+ * problem must have prepacked = 1; activations are taken in slabs of at most 16 rows that
+ * fit LDS (fewer rows per slab for long K), and all slabs of a call together may number at
+ * most 8 (for K = 2048: three problems of 32 rows), else VRL_INT4_ESHAPE and the caller uses
+ * a grouped plan or vrl_int4_gemv_bf16.  scales and qzeros of the records are ignored.
  */
 int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream);
 

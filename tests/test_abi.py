@@ -153,16 +153,16 @@ def test_direct_prepacked_validation(lib):
         rec.M, rec.N, rec.K, rec.G, rec.prepacked = 1, 64, 256, 128, 1
     assert lib.vrl_int4_gemv_prepacked_bf16(None, 1, None) == 1003
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 0, None) == 1001
-    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 5, None) == 1001
+    assert lib.vrl_int4_gemv_prepacked_bf16(probs, 9, None) == 1001
     probs[1].prepacked = 0                       # canonical records are not taken here
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
-    probs[1].prepacked, probs[1].M = 1, 17       # more than 16 activation rows
+    probs[1].prepacked, probs[1].M = 1, 16 * 7 + 1   # eight slabs of 16 rows beside the first problem's one
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
     probs[1].M, probs[1].G = 1, 16               # no prepacked form for this group size
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
     probs[1].G, probs[1].y = 128, p + 2          # misaligned output
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002
-    probs[1].y, probs[1].M, probs[1].K = p, 16, 4096   # activations beyond the LDS this path uses
+    probs[1].y, probs[1].M, probs[1].K = p, 32, 16384  # LDS holds 4 such rows: 8 slabs, 9 with the first problem
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
 
 

@@ -493,6 +493,9 @@ DIRECT_SHAPES = [
     (1, 2048, 2048, False), (1, 5632, 2048, False), (1, 2048, 5632, False), (1, 11008, 96, False),
     (1, 128, 16, False), (3, 640, 50, False), (16, 1536, 64, False), (7, 4096, 80, False),
     (1, 2048, 2 * 5632, True), (8, 2048, 2 * 704, True), (5, 4096, 2 * 48, True),
+    # more than one slab of rows, several tiles per workgroup, a ragged last workgroup
+    (32, 2048, 2048, False), (17, 2048, 100, False), (32, 5632, 208, False), (9, 1024, 80, False),
+    (32, 11008, 48, False), (32, 2048, 2 * 720, True), (20, 4096, 2 * 112, True), (16, 2048, 2064, False),
 ]
 
 
@@ -557,15 +560,16 @@ def test_direct_one_hot_is_the_exact_weight_column(ops_mod):
 
 def test_direct_rejects_what_it_cannot_take(ops_mod):
     G = 128
-    ops = o.make_operands(9300, 17, 256, 32, G)
+    ops = o.make_operands(9300, 33, 256, 32, G)
     d = to_device(ops, DEV)
     pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
     with pytest.raises(ValueError):
-        ops_mod.DirectGemv([(d["x"], pw, False)])            # 17 rows
+        ops_mod.DirectGemv([(d["x"], pw, False)])            # 33 rows
     with pytest.raises(ValueError):
-        ops_mod.DirectGemv([(d["x"][:1], pw, False)] * 5)    # five problems
-    big = o.make_operands(9301, 16, 4096, 16, G)             # 16 x 4096 activations do not fit this path
+        ops_mod.DirectGemv([(d["x"][:1], pw, False)] * 9)    # nine problems
+    big = o.make_operands(9301, 32, 11008, 16, G)            # LDS holds 6 such rows: 6 slabs per problem
     db = to_device(big, DEV)
     pwb = ops_mod.int4_prepack(db["qweight"], db["scales"], db["qzeros"], G)
+    assert pwb.direct_slab_rows() == 6
     with pytest.raises(ValueError):
-        ops_mod.DirectGemv([(db["x"], pwb, False)]).launch()
+        ops_mod.DirectGemv([(db["x"], pwb, False)] * 2).launch()

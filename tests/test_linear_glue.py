@@ -291,7 +291,7 @@ def test_prepacked_module_path_agrees_with_the_canonical_one():
         x = torch.randn(rows, 1024, device=dev).to(torch.bfloat16)
         plain = q(x)
         q.prepack_()
-        assert q._packed is not None and q._direct_rows == 16
+        assert q._packed is not None and q._direct_rows == 32
         fast = q(x)
         del q._packed
         ref = x.double() @ w.t()

@@ -83,6 +83,7 @@ struct StreamShape { int wpb; int per_cu; size_t lds; };
 // resident, LDS the shape may use}
 constexpr StreamShape STREAM_SHAPES[3] = {{4, 15, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
+constexpr size_t DIRECT_LDS_CAP = 150 * 1024;   // plan-free launches: staged activations + partial tiles
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -317,10 +318,30 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int WPB>
-int launch_direct(const DirectArgs &args, int tiles, size_t lds, hipStream_t stream) {
-    hipLaunchKernelGGL((gemv_split_direct_kernel<FUSED, WPB>), dim3(tiles), dim3(WPB * WAVE), lds, stream, args);
+template <bool FUSED, int KS, int TW>
+int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW>;
+    if (lds > 64 * 1024) {
+        static bool raised = false;  // per instantiation; the attribute is a property of the function
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)DIRECT_LDS_CAP);
+            if (e != hipSuccess) return (int)e;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
     return (int)hipGetLastError();
+}
+
+template <bool FUSED>
+int launch_direct_shape(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
+    if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2>(args, workgroups, lds, stream);
+    if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1>(args, workgroups, lds, stream);
+    return VRL_INT4_EPLAN;
 }
 
 int dispatch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab,
@@ -421,40 +442,58 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
 int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {
     if (!problems) return VRL_INT4_ENULL;
     if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
-    DirectArgs args;
-    memset(&args, 0, sizeof args);
-    args.n = n_problems;
-    long tiles = 0;
     bool fused_any = false;
-    int max_nsc = 1;
-    size_t x_bytes = 0;
+    int max_nsc = 1, max_m = 1;
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
         if (!q.prepacked) return VRL_INT4_ESHAPE;
         int rc = check_problem(q.x, q.qweight, q.qweight, q.qweight, q.y, q.M, q.N, q.K, q.G);
         if (rc != VRL_INT4_OK) return rc;
-        if (q.M > MAX_TILE_M || !prepack_ok(q.N, q.K, q.G)) return VRL_INT4_ESHAPE;
+        if (!prepack_ok(q.N, q.K, q.G)) return VRL_INT4_ESHAPE;
         if (q.fused_gate_up && (q.N % 2 != 0 || (q.N / 2) % 16 != 0)) return VRL_INT4_ESHAPE;
-        DevProblem &p = args.recs[i];
-        p.x = static_cast<const uint16_t *>(q.x);
-        p.qweight = static_cast<const uint32_t *>(q.qweight);
-        p.y = static_cast<uint16_t *>(q.y);
-        p.M = q.M; p.N = q.N; p.K = q.K; p.G = q.G;
-        p.fused = q.fused_gate_up ? 1 : 0;
-        p.prepacked = 1;
-        p.kc = pp_nsc(q.K) * PP_SC;
-        p.tile_begin = (int)tiles;
-        tiles += ((p.fused ? p.N / 2 : p.N) + 15) / 16;
-        fused_any |= p.fused != 0;
+        fused_any |= q.fused_gate_up != 0;
         max_nsc = std::max(max_nsc, pp_nsc(q.K));
-        x_bytes = std::max(x_bytes, (size_t)p.M * (p.kc + XPAD) * 2);
+        max_m = std::max(max_m, q.M);
     }
-    if (tiles > MAX_PLAN_GRID) return VRL_INT4_ESHAPE;
-    const int wpb = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
-    const size_t red = (size_t)(wpb - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
+    // KS waves split K of a tile (one super-chunk each where K allows); with 8 or more
+    // activation rows a workgroup carries several tiles so that one staging of x serves them
+    const int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
+    const int tw = max_m >= 8 ? 16 / ks : 1;
+    const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
+    // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
+    DirectArgs args;
+    memset(&args, 0, sizeof args);
+    long workgroups = 0;
+    size_t x_bytes = 0;
+    for (int i = 0; i < n_problems; ++i) {
+        const vrl_int4_problem &q = problems[i];
+        const int kc = pp_nsc(q.K) * PP_SC;
+        const size_t row_bytes = (size_t)(kc + XPAD) * 2;
+        long rows = (long)((DIRECT_LDS_CAP - red) / row_bytes);
+        if (rows > MAX_TILE_M) rows = MAX_TILE_M;
+        if (rows < 1) return VRL_INT4_ESHAPE;
+        const int out_cols = q.fused_gate_up ? q.N / 2 : q.N;
+        const int tiles = (out_cols + 15) / 16;
+        for (int m0 = 0; m0 < q.M; m0 += (int)rows) {
+            if (args.n == DIRECT_MAX) return VRL_INT4_ESHAPE;  // too many slabs for one launch: use a plan
+            DevProblem &p = args.recs[args.n++];
+            p.x = static_cast<const uint16_t *>(q.x) + (long)m0 * q.K;
+            p.qweight = static_cast<const uint32_t *>(q.qweight);
+            p.y = static_cast<uint16_t *>(q.y) + (long)m0 * out_cols;
+            p.M = std::min<int>((int)rows, q.M - m0);
+            p.N = q.N; p.K = q.K; p.G = q.G;
+            p.fused = q.fused_gate_up ? 1 : 0;
+            p.prepacked = 1;
+            p.kc = kc;
+            p.tile_begin = (int)workgroups;  // first workgroup of the record
+            workgroups += (tiles + tw - 1) / tw;
+            x_bytes = std::max(x_bytes, (size_t)p.M * row_bytes);
+        }
+    }
+    if (workgroups > (1L << 20)) return VRL_INT4_ESHAPE;
     // padding rows of the A operand read a staged row of zeros where LDS is plentiful
     size_t xz_bytes = x_bytes;
-    for (int i = 0; i < n_problems; ++i) {
+    for (int i = 0; i < args.n; ++i) {
         DevProblem &p = args.recs[i];
         const size_t need = (size_t)(p.M + 1) * (p.kc + XPAD) * 2;
         if (p.M < MAX_TILE_M && need + red <= 32 * 1024) {
@@ -463,20 +502,9 @@ int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problem
         }
     }
     const size_t lds = xz_bytes + red;
-    if (lds > 64 * 1024) return VRL_INT4_ESHAPE;  // activations too large for this path: use a plan
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    if (fused_any) {
-        switch (wpb) {
-            case 4: return launch_direct<true, 4>(args, (int)tiles, lds, stream);
-            case 8: return launch_direct<true, 8>(args, (int)tiles, lds, stream);
-            default: return launch_direct<true, 16>(args, (int)tiles, lds, stream);
-        }
-    }
-    switch (wpb) {
-        case 4: return launch_direct<false, 4>(args, (int)tiles, lds, stream);
-        case 8: return launch_direct<false, 8>(args, (int)tiles, lds, stream);
-        default: return launch_direct<false, 16>(args, (int)tiles, lds, stream);
-    }
+    return fused_any ? launch_direct_shape<true>(args, ks, tw, (int)workgroups, lds, stream)
+                     : launch_direct_shape<false>(args, ks, tw, (int)workgroups, lds, stream);
 }
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {

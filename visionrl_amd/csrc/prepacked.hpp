@@ -399,33 +399,38 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
     }
 }
 
-// Small plans (fewer tiles than the device has workgroup slots): the waves of a workgroup
-// share one tile, each taking a contiguous quarter of its super-chunks, and the partial
-// tiles meet in LDS.  A tile is then one or two memory round trips instead of a serial walk
-// over K by a single wave; this is the latency mode for launches of a few matrices
-// (q|k|v of one layer, one o_proj, ...).  LDS: staged activations, then WPB x RS partial tiles.
-template <bool FUSED, int WPB, int GQ>
+// Small launches (fewer tiles than the device has workgroup slots): KS waves share one tile,
+// each taking a contiguous share of its super-chunks, and the partial tiles meet in LDS.  A
+// tile is then one or two memory round trips instead of a serial walk over K by a single
+// wave; this is the latency mode for launches of a few matrices (q|k|v of one layer, one
+// o_proj, ...).  A workgroup carries TW such tiles at once (KS * TW waves), so that one
+// staging of the activations serves TW tiles: that matters once x is tens of KB (8+ rows).
+// LDS: staged activations, then TW x (KS - 1) x RS partial tiles.
+template <bool FUSED, int KS, int TW, int GQ>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tw = wave / KS, kw = wave % KS;  // tile of the round, share of K
     const int lane = threadIdx.x & (WAVE - 1);
     uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
     const int xstride = p.kc + XPAD;
     const int xrows = p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0);
-    f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + (size_t)xrows * xstride * 2);
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + (size_t)xrows * xstride * 2) + tw * (KS - 1) * RS * WAVE;
     const int nsc = pp_nsc(p.K);
-    const int per = (nsc + WPB - 1) / WPB;
-    const int sc0 = min(nsc, wave * per), sc1 = min(nsc, sc0 + per);
-    const bool work = sc0 < sc1;  // wave-uniform
+    const int per = (nsc + KS - 1) / KS;
+    const int sc0 = min(nsc, kw * per), sc1 = min(nsc, sc0 + per);
     const rsrc_t rsrc = pp_blob_rsrc(p);
     PPRing<RS, GQ> ring;
-    PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, t0, sc0);
+    int tile = t0 + tw;
+    bool work = sc0 < sc1 && tile < t1;  // wave-uniform
+    PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, work ? tile : t0, sc0);
     if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
     __syncthreads();
-    stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+    stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
     __syncthreads();
-    for (int tile = t0; tile < t1; ++tile) {
-        const int next = tile + 1 < t1 ? tile + 1 : -1;
+    for (int base = t0; base < t1; base += TW) {
+        tile = base + tw;
+        const int next = tile + TW < t1 ? tile + TW : -1;
         f32x4_t acc[RS][1];
 #pragma unroll
         for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -433,33 +438,34 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
             stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
             if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
         }
-        if (wave != 0) {
+        if (kw != 0) {
 #pragma unroll
-            for (int r = 0; r < RS; ++r) red[((wave - 1) * RS + r) * WAVE + lane] = acc[r][0];
+            for (int r = 0; r < RS; ++r) red[((kw - 1) * RS + r) * WAVE + lane] = acc[r][0];
         }
         __syncthreads();
-        if (wave == 0) {
+        if (kw == 0 && tile < t1) {
 #pragma unroll
-            for (int w = 1; w < WPB; ++w)
+            for (int w = 1; w < KS; ++w)
 #pragma unroll
                 for (int r = 0; r < RS; ++r) acc[r][0] += red[((w - 1) * RS + r) * WAVE + lane];
             store_tile<1, FUSED>(p, tile, acc);
         }
-        if (next >= 0) __syncthreads();  // the partial tiles are read before they are rewritten
+        work = work && next >= 0;
+        if (base + TW < t1) __syncthreads();  // the partial tiles are read before they are rewritten
     }
 }
 
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
-template <bool FUSED, int WPB>
+template <bool FUSED, int KS, int TW>
 __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem) {
     if (FUSED && p.fused) {
-        if (p.G == 128) split_segment_pp<FUSED, WPB, 1>(p, t0, t1, smem);
-        else if (p.G == 64) split_segment_pp<FUSED, WPB, 2>(p, t0, t1, smem);
-        else split_segment_pp<FUSED, WPB, 4>(p, t0, t1, smem);
+        if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2>(p, t0, t1, smem);
+        else split_segment_pp<FUSED, KS, TW, 4>(p, t0, t1, smem);
     } else {
-        if (p.G == 128) split_segment_pp<false, WPB, 1>(p, t0, t1, smem);
-        else if (p.G == 64) split_segment_pp<false, WPB, 2>(p, t0, t1, smem);
-        else split_segment_pp<false, WPB, 4>(p, t0, t1, smem);
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1>(p, t0, t1, smem);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2>(p, t0, t1, smem);
+        else split_segment_pp<false, KS, TW, 4>(p, t0, t1, smem);
     }
 }
 
@@ -477,31 +483,34 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
-        split_by_group<FUSED, WPB>(p, a, b, smem);
+        split_by_group<FUSED, WPB, 1>(p, a, b, smem);
         t = seg_end;
     }
 }
 
 // The same latency mode without a plan in device memory: up to DIRECT_MAX records travel
-// as kernel arguments (no dependent loads before the first weight request), one workgroup per
-// tile.  This is the single-call path of a prepacked weight (and of q|k|v, gate|up groups).
-constexpr int DIRECT_MAX = 4;
+// as kernel arguments (no dependent loads before the first weight request).  Workgroup g of
+// the launch takes the TW tiles (g - first workgroup of its record) * TW ... of that record.
+// This is the single-call path of a prepacked weight (and of q|k|v, gate|up groups); the host
+// cuts activations of more than 16 rows, or too large for LDS, into row slabs, one record each.
+constexpr int DIRECT_MAX = 8;
 struct DirectArgs {
     int32_t n;
     int32_t pad;
-    DevProblem recs[DIRECT_MAX];
+    DevProblem recs[DIRECT_MAX];  // tile_begin holds the record's first workgroup here
 };
 
-template <bool FUSED, int WPB>
-__global__ __launch_bounds__(WPB *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
+template <bool FUSED, int KS, int TW>
+__global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    const int t = blockIdx.x;
+    const int g = blockIdx.x;
     DevProblem p = a.recs[0];
 #pragma unroll
     for (int k = 1; k < DIRECT_MAX; ++k)
-        if (k < a.n && a.recs[k].tile_begin <= t) p = a.recs[k];  // scalar selects, no indexing
-    const int local = t - p.tile_begin;
-    split_by_group<FUSED, WPB>(p, local, local + 1, smem);
+        if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
+    const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
+    const int t0 = (g - p.tile_begin) * TW;
+    split_by_group<FUSED, KS, TW>(p, t0, min(tiles, t0 + TW), smem);
 }
 
 }  // namespace

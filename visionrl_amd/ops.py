@@ -181,16 +181,24 @@ class PrepackedWeight:
     def supported(N: int, K: int, group_size: int) -> bool:
         return _lib.load().vrl_int4_prepacked_bytes(int(N), int(K), int(group_size)) > 0
 
-    def direct_rows(self, fused: bool = False) -> int:
-        """Most activation rows a plan-free launch (:class:`DirectGemv`) takes for this weight.
+    def direct_slab_rows(self, fused: bool = False) -> int:
+        """Activation rows one record of a plan-free launch carries for this weight.
 
-        Mirrors the library's rule: the staged activations (K padded to 512, 8 elements of
-        row padding) plus the partial tiles of the K-split must fit 64 KiB of LDS.
+        A lower bound of the library's rule: the staged rows (K padded to 512, 8 elements
+        of row padding) and the partial tiles of the K-split (at most 15 KiB, twice that for
+        gate||up) fit 150 KiB of LDS, 16 rows at most.
         """
         nsc = (self.K + 511) // 512
-        waves = 16 if nsc > 8 else (8 if nsc > 4 else 4)
-        spare = 64 * 1024 - (waves - 1) * (2 if fused else 1) * 1024
+        spare = 150 * 1024 - 15 * 1024 * (2 if fused else 1)
         return max(0, min(16, spare // ((nsc * 512 + 8) * 2)))
+
+    def direct_rows(self, fused: bool = False, weights: int = 1) -> int:
+        """Most activation rows a plan-free launch (:class:`DirectGemv`) takes for this weight
+        when ``weights`` such problems share the launch: the library cuts the rows into slabs
+        and a launch holds at most eight of them.  Capped at 32 rows: beyond that every slab
+        streams the weight again and a plan (:class:`GroupedGemv`) is the better launch."""
+        slab = self.direct_slab_rows(fused)
+        return min(32, slab * (DirectGemv.MAX_RECORDS // max(1, int(weights))))
 
 
 def int4_prepack(qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
@@ -295,18 +303,20 @@ class GroupedGemv:
 
 
 class DirectGemv:
-    """One to four prepacked GEMVs launched together without a plan in device memory.
+    """One to eight prepacked GEMVs launched together without a plan in device memory.
 
     The decode-time form of a linear (or of the q|k|v / gate|up linears of one decoder
     layer, ``vrl/models/families/janus_pro/policy.py:673-678``): the problem records
     travel as kernel arguments, so a launch is one memory round trip.  ``problems`` is a
-    list of ``(x, prepacked_weight, fused)``; every x has at most 16 rows.  Outputs are
-    allocated here once and overwritten by every :meth:`launch`; the record table is
+    list of ``(x, prepacked_weight, fused)``; every x has at most 32 rows, which the library
+    takes in slabs of up to 16 (fewer for long K), eight slabs per launch at most.  Outputs
+    are allocated here once and overwritten by every :meth:`launch`; the record table is
     built once, the tensors captured here must stay alive and in place.
     """
 
-    MAX_PROBLEMS = 4
-    MAX_ROWS = 16
+    MAX_PROBLEMS = 8
+    MAX_ROWS = 32
+    MAX_RECORDS = 8   # row slabs of all problems of one launch
 
     def __init__(self, problems, outputs=None):
         if not 1 <= len(problems) <= self.MAX_PROBLEMS:
@@ -378,7 +388,7 @@ def int4_gemv_prepacked_into(y: torch.Tensor, x: torch.Tensor, weight: Prepacked
 
 
 def int4_gemv_prepacked_multi_into(ys, x: torch.Tensor, weights) -> None:
-    """One plan-free launch for up to four prepacked weights applied to the same ``x`` (q|k|v).
+    """One plan-free launch for up to eight prepacked weights applied to the same ``x`` (q|k|v).
 
     Lean eager path like :func:`int4_gemv_prepacked_into`: ``x`` bf16 contiguous ``[M, K]``,
     ``ys[i]`` bf16 contiguous ``[M, weights[i].N]``, all on one device.
@@ -459,7 +469,7 @@ class DirectCall:
             rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
             self.cols.append(w.N // 2 if fused else w.N)
         self._keep = list(weights)
-        self.max_rows = min(w.direct_rows(fused) for w in weights)
+        self.max_rows = min(w.direct_rows(fused, len(weights)) for w in weights)
         self._fn = _lib.load().vrl_int4_gemv_prepacked_bf16
         self._n = len(weights)
 

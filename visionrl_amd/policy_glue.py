@@ -102,7 +102,7 @@ def apply_int4_to_policy(policy: Any, group_size: int = 128,
     ``fuse_mlp`` replaces a whole MLP block by :class:`Int4LlamaMLP` (gate||up with
     the SiLU epilogue in one launch) when all three projections are targeted and
     none of them carries a LoRA adapter.  ``prepack`` keeps a second, MFMA-shaped copy
-    of every quantised weight that lives on a GPU, which decode-sized calls (up to 16
+    of every quantised weight that lives on a GPU, which decode-sized calls (up to 32
     activation rows) stream through the plan-free launch; with ``group_qkv`` the three
     projections of an attention block then share one launch per decode step.
     """
