@@ -392,6 +392,116 @@ def decode_tail(device, steps: int):
     return out
 
 
+def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16)):
+    """ms per image token of the whole decode loop on a Janus-Pro-1B shaped policy (random weights).
+
+    ``reference_style`` is the loop of vrl/models/families/janus_pro/policy.py:624-731 with the trunk's
+    dynamic cache and the torch formulas for the tail, without its per-row cache copies and host
+    read-backs (so a lower bound for the reference); ``static_*`` is visionrl_amd.ar_decode.
+    """
+    import types
+
+    import torch.nn.functional as F
+    from torch import nn
+    from transformers import LlamaConfig, LlamaModel
+
+    from visionrl_amd.ar_decode import StaticARSampler
+    from visionrl_amd.policy_glue import apply_int4_to_policy
+
+    cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=LAYERS,
+                      num_attention_heads=16, num_key_value_heads=16, vocab_size=128,
+                      max_position_embeddings=1024)
+
+    class MMGPT(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.language_model = types.SimpleNamespace(model=LlamaModel(cfg).to(torch.bfloat16).eval())
+            self.gen_head = nn.Linear(HIDDEN, HEAD, bias=False).to(torch.bfloat16)
+            self.gen_embed = nn.Embedding(HEAD, HIDDEN).to(torch.bfloat16)
+
+        def prepare_gen_img_embeds(self, ids):
+            return self.gen_embed(ids)
+
+    class Policy:
+        def __init__(self):
+            self.mmgpt = MMGPT()
+            self.config = types.SimpleNamespace(cfg_weight=5.0, temperature=1.0, image_token_num=tokens)
+
+        def _base(self):
+            return self.mmgpt
+
+        def _lm_trunk(self):
+            return self.mmgpt.language_model.model
+
+    @torch.no_grad()
+    def reference_style(policy, cond, uncond, cmask, umask, n_img):
+        trunk, base = policy._lm_trunk(), policy._base()
+        B = cond.shape[0]
+        toks = torch.empty(B, n_img, dtype=torch.long, device=device)
+        lps = torch.empty(B, n_img, dtype=torch.float32, device=device)
+        embeds, attn, past = torch.cat([cond, uncond]), torch.cat([cmask, umask]), None
+        for pos in range(n_img):
+            out = trunk(inputs_embeds=embeds, attention_mask=attn, use_cache=True, past_key_values=past)
+            past = out.past_key_values
+            logits = base.gen_head(out.last_hidden_state[:, -1:, :]).squeeze(1)
+            c, u = logits.chunk(2, dim=0)
+            probs = F.softmax((u + 5.0 * (c - u)) / 1.0, dim=-1)
+            sampled = torch.multinomial(probs, num_samples=1).squeeze(-1)
+            lp = F.log_softmax(c / 1.0, dim=-1).gather(-1, sampled.unsqueeze(-1)).squeeze(-1)
+            toks[:, pos], lps[:, pos] = sampled, lp
+            embeds = base.prepare_gen_img_embeds(torch.cat([sampled, sampled]).unsqueeze(-1))
+            attn = torch.cat([attn, torch.ones(2 * B, 1, dtype=attn.dtype, device=device)], dim=1)
+        return toks, lps
+
+    def per_token_ms(fn):
+        fn()   # warm-up (and graph capture where there is one)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / tokens
+
+    out = {"tokens_per_call": tokens, "prompt_tokens": 16,
+           "model": "LlamaModel 24 x (2048, 5632), 16 heads, head 2048->16384, random weights"}
+    with torch.device(device):
+        torch.manual_seed(0)
+        policy = Policy()
+    policy.mmgpt.to(device)
+    policy._lm_trunk().to(device)
+    inputs = {}
+    for B in batches:
+        g = torch.Generator(device=device).manual_seed(7000 + B)
+        inputs[B] = (torch.randn((B, 16, HIDDEN), generator=g, device=device).to(torch.bfloat16),
+                     torch.randn((B, 16, HIDDEN), generator=g, device=device).to(torch.bfloat16),
+                     torch.ones((B, 16), dtype=torch.long, device=device),
+                     torch.ones((B, 16), dtype=torch.long, device=device))
+    for B in batches if only is None else ():
+        entry = out.setdefault(f"B{B}", {})
+        entry["bf16_reference_style_ms_per_token"] = per_token_ms(
+            lambda: reference_style(policy, *inputs[B], tokens))
+        sampler = StaticARSampler(policy, graph=True, fused_tail=False)
+        entry["bf16_static_hip_graph_ms_per_token"] = per_token_ms(
+            lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
+        del sampler
+        torch.cuda.empty_cache()
+    apply_int4_to_policy(policy, group_size=GROUP)
+    torch.cuda.empty_cache()
+    for B in batches:
+        entry = out.setdefault(f"B{B}", {})
+        if only is None:
+            entry["int4_reference_style_ms_per_token"] = per_token_ms(
+                lambda: reference_style(policy, *inputs[B], tokens))
+        for name, graph in (("int4_static_eager", False), ("int4_static_hip_graph", True)):
+            if only is not None and name != only:
+                continue
+            sampler = StaticARSampler(policy, graph=graph)
+            entry[f"{name}_ms_per_token"] = per_token_ms(
+                lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
+            del sampler
+            torch.cuda.empty_cache()
+    return out
+
+
 def launch_floor_us(device, nodes: int = 96, reps: int = 50):
     """us per node of a HIP graph of tiny dependent kernels: what a launch costs with no work in it."""
     t = torch.zeros(64, device=device)
@@ -456,6 +566,8 @@ def main():
                     help="run just the grouped decode-step launches (for profilers)")
     ap.add_argument("--single-calls", action="store_true",
                     help="loop single-GEMV launches over distinct weights per shape and exit (for profilers)")
+    ap.add_argument("--ar-decode", type=int, default=0, metavar="B",
+                    help="run only the recorded decode loop at batch B on the int4 policy and exit (for profilers)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run plain 1 GiB device copies and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -476,6 +588,9 @@ def main():
         return
     from visionrl_amd import ops
 
+    if args.ar_decode:
+        print(json.dumps(ar_decode_loop(device, only="int4_static_hip_graph", batches=(args.ar_decode,))))
+        return
     if args.single_calls:
         for M in (1, 32):
             for K, N in ((HIDDEN, HIDDEN), (HIDDEN, INTER), (INTER, HIDDEN), (HIDDEN, HEAD)):
@@ -537,6 +652,12 @@ def main():
     torch.cuda.empty_cache()
 
     try:
+        ar_loop = ar_decode_loop(device)
+    except Exception as exc:
+        ar_loop = {"error": repr(exc)[:300]}
+    torch.cuda.empty_cache()
+
+    try:
         others = other_configs(device, args.steps, args.warmup)
     except Exception as exc:  # the other configurations are detail, never the headline
         others = {"error": repr(exc)[:300]}
@@ -567,7 +688,8 @@ def main():
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency,
                    "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
-                   "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "other_configs": others},
+                   "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "ar_decode_loop_1b": ar_loop,
+                   "other_configs": others},
     }
     print(json.dumps(result))
 

@@ -1,0 +1,208 @@
+"""Static-cache / HIP-graph image-token sampling against the reference's decode loop.
+
+``reference_loop`` restates ``JanusProPolicy.sample_image_tokens`` + ``_sample_ar_step``
+(vrl/models/families/janus_pro/policy.py:476-525, :624-731) with plain torch and the trunk's own
+dynamic cache: concatenate the rows' caches, call the trunk on ``[cond; uncond]``, head, CFG
+combine, softmax -> multinomial, log_softmax -> gather, embed the sampled token for both halves,
+append a one to both masks.  The per-row split/concat of the cache (``vrl/models/ar.py:42-110``)
+is the identity when all rows advance together and is left out.  The policy stand-in wraps a
+real, randomly initialised Hugging Face ``LlamaModel`` like the reference's own stub
+(tests/models/test_janus_wrapper.py:30-87).
+"""
+
+import types
+
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from visionrl_amd.ar_decode import StaticARSampler, install_static_ar_sampler
+
+HIDDEN, INTER, HEADS, LAYERS, VOCAB_IMG = 256, 512, 4, 2, 1024
+
+
+class StubMMGPT(nn.Module):
+    def __init__(self, dtype):
+        super().__init__()
+        from transformers import LlamaConfig, LlamaModel
+
+        cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=LAYERS,
+                          num_attention_heads=HEADS, num_key_value_heads=HEADS, vocab_size=128,
+                          max_position_embeddings=256)
+        torch.manual_seed(0)
+        self.language_model = types.SimpleNamespace(model=LlamaModel(cfg).to(dtype).eval())
+        self.gen_head = nn.Linear(HIDDEN, VOCAB_IMG, bias=False).to(dtype)
+        self.gen_embed = nn.Embedding(VOCAB_IMG, HIDDEN).to(dtype)
+        with torch.no_grad():   # spread the logits so that draws are not all near-ties
+            self.gen_head.weight.mul_(8.0)
+
+    def prepare_gen_img_embeds(self, ids):
+        return self.gen_embed(ids)
+
+
+class StubPolicy:
+    def __init__(self, dtype=torch.float32, device="cpu"):
+        self.mmgpt = StubMMGPT(dtype)
+        self.mmgpt.language_model.model.to(device)
+        self.mmgpt.to(device)
+        self.config = types.SimpleNamespace(cfg_weight=5.0, temperature=1.0, image_token_num=12)
+
+    def _base(self):
+        return self.mmgpt
+
+    def _lm_trunk(self):
+        return self.mmgpt.language_model.model
+
+
+def make_inputs(B, n_text, dtype, device, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    cond = torch.randn(B, n_text, HIDDEN, generator=g).to(dtype).to(device)
+    uncond = torch.randn(B, n_text, HIDDEN, generator=g).to(dtype).to(device)
+    cmask = torch.ones(B, n_text, dtype=torch.long)
+    umask = torch.ones(B, n_text, dtype=torch.long)
+    for b in range(B):   # left padding of different lengths, as the tokenizer produces
+        cmask[b, :b % 3] = 0
+        umask[b, :(b + 2) % 4] = 0
+    return cond, uncond, cmask.to(device), umask.to(device)
+
+
+@torch.no_grad()
+def reference_loop(policy, cond, uncond, cmask, umask, cfg_weight, temperature, n_img):
+    trunk, base = policy._lm_trunk(), policy._base()
+    B = cond.shape[0]
+    tokens = torch.empty(B, n_img, dtype=torch.long, device=cond.device)
+    logprobs = torch.empty(B, n_img, dtype=torch.float32, device=cond.device)
+    embeds, attn, past = torch.cat([cond, uncond]), torch.cat([cmask, umask]), None
+    for pos in range(n_img):
+        out = trunk(inputs_embeds=embeds, attention_mask=attn, use_cache=True, past_key_values=past)
+        past = out.past_key_values
+        logits = base.gen_head(out.last_hidden_state[:, -1:, :]).squeeze(1)
+        c, u = logits.chunk(2, dim=0)
+        guided = u + cfg_weight * (c - u)
+        probs = F.softmax(guided / temperature, dim=-1)
+        sampled = torch.multinomial(probs, num_samples=1).squeeze(-1)
+        lp = F.log_softmax(c / temperature, dim=-1).gather(-1, sampled.unsqueeze(-1)).squeeze(-1)
+        tokens[:, pos], logprobs[:, pos] = sampled, lp
+        embeds = base.prepare_gen_img_embeds(torch.cat([sampled, sampled]).unsqueeze(-1))
+        attn = torch.cat([attn, torch.ones(2 * B, 1, dtype=attn.dtype, device=attn.device)], dim=1)
+    return tokens, logprobs
+
+
+# ------------------------------------------------------------------ CPU: the static-cache logic
+def test_static_cache_loop_samples_what_the_reference_loop_samples():
+    policy = StubPolicy()
+    cond, uncond, cmask, umask = make_inputs(3, 7, torch.float32, "cpu")
+    torch.manual_seed(11)
+    want_t, want_lp = reference_loop(policy, cond, uncond, cmask, umask, 5.0, 1.0, 12)
+    sampler = StaticARSampler(policy, graph=False, fused_tail=False)
+    torch.manual_seed(11)
+    got_t, got_lp = sampler.sample_image_tokens(cond, uncond, cmask, umask)   # defaults from policy.config
+    assert got_t.dtype == torch.long and got_lp.dtype == torch.float32 and got_t.shape == (3, 12)
+    assert torch.equal(got_t, want_t)
+    torch.testing.assert_close(got_lp, want_lp, rtol=1e-5, atol=1e-5)
+    assert len(want_t.unique()) > 6   # the draw is not degenerate
+
+    # a second call reuses the buffers (other prompts, other length inside the same bucket, other seed)
+    cond2, uncond2, cmask2, umask2 = make_inputs(3, 9, torch.float32, "cpu", seed=4)
+    torch.manual_seed(12)
+    want_t2, want_lp2 = reference_loop(policy, cond2, uncond2, cmask2, umask2, 5.0, 1.0, 10)
+    torch.manual_seed(12)
+    got_t2, got_lp2 = sampler.sample_image_tokens(cond2, uncond2, cmask2, umask2, image_token_num=10)
+    assert len(sampler._sessions) == 1
+    assert torch.equal(got_t2, want_t2)
+    torch.testing.assert_close(got_lp2, want_lp2, rtol=1e-5, atol=1e-5)
+    assert torch.equal(got_t, want_t)   # results of the first call are copies, not views of the buffers
+
+
+def test_guidance_and_temperature_reach_the_draw():
+    policy = StubPolicy()
+    cond, uncond, cmask, umask = make_inputs(2, 5, torch.float32, "cpu")
+    sampler = StaticARSampler(policy, graph=False, fused_tail=False)
+    for cfg, temp in ((1.0, 1.0), (7.5, 0.7)):
+        torch.manual_seed(5)
+        want = reference_loop(policy, cond, uncond, cmask, umask, cfg, temp, 6)
+        torch.manual_seed(5)
+        got = sampler.sample_image_tokens(cond, uncond, cmask, umask, cfg_weight=cfg, temperature=temp,
+                                          image_token_num=6)
+        assert torch.equal(got[0], want[0])
+        torch.testing.assert_close(got[1], want[1], rtol=1e-5, atol=1e-5)
+    assert len(sampler._sessions) == 2   # one per (guidance, temperature): they are baked into a recorded step
+
+
+def test_contract_violations_raise():
+    policy = StubPolicy()
+    cond, uncond, cmask, umask = make_inputs(2, 5, torch.float32, "cpu")
+    sampler = StaticARSampler(policy, graph=False, fused_tail=False)
+    with pytest.raises(ValueError):
+        sampler.sample_image_tokens(cond, uncond[:1], cmask, umask)
+    with pytest.raises(ValueError):
+        sampler.sample_image_tokens(cond, uncond, cmask[:, :4], umask)
+    with pytest.raises(ValueError):
+        sampler.sample_image_tokens(cond, uncond, cmask, umask, temperature=0.0)
+    policy.config = None
+    with pytest.raises(ValueError):
+        sampler.sample_image_tokens(cond, uncond, cmask, umask)
+    with pytest.raises(TypeError):
+        StaticARSampler(types.SimpleNamespace(_lm_trunk=policy._lm_trunk, _base=lambda: nn.Identity()))
+
+
+def test_install_replaces_the_policy_method():
+    policy = StubPolicy()
+    sampler = install_static_ar_sampler(policy, graph=False, fused_tail=False)
+    cond, uncond, cmask, umask = make_inputs(1, 4, torch.float32, "cpu")
+    torch.manual_seed(2)
+    want = reference_loop(policy, cond, uncond, cmask, umask, 3.0, 1.0, 5)
+    torch.manual_seed(2)
+    got = policy.sample_image_tokens(cond, uncond, cmask, umask, cfg_weight=3.0, temperature=1.0, image_token_num=5)
+    assert torch.equal(got[0], want[0]) and policy._static_ar_sampler is sampler
+
+
+# ------------------------------------------------------------------ GPU: int4 modules, fused tail, HIP graph
+@pytest.fixture(scope="module")
+def int4_policy():
+    from visionrl_amd.policy_glue import apply_int4_to_policy
+
+    policy = StubPolicy(torch.bfloat16, "cuda:0")
+    summary = apply_int4_to_policy(policy, group_size=128)
+    assert summary["prepacked"] > 0 and summary["qkv_groups"] == LAYERS
+    return policy
+
+
+@pytest.mark.gpu
+def test_graph_replays_equal_eager_steps(int4_policy):
+    """Every replayed step against the same step run eagerly: tokens and log-probabilities bit for bit,
+    over two calls (the second reuses the recorded graph) with eager work and syncs in between."""
+    print("ar decode: graph vs eager", flush=True)
+    eager = StaticARSampler(int4_policy, graph=False)
+    graphed = StaticARSampler(int4_policy, graph=True)
+    for call, (n_text, n_img, seed) in enumerate(((7, 24, 21), (11, 20, 22), (7, 24, 21))):
+        cond, uncond, cmask, umask = make_inputs(3, n_text, torch.bfloat16, "cuda:0", seed=seed)
+        torch.manual_seed(seed)
+        want_t, want_lp = eager.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=n_img)
+        torch.cuda.synchronize()
+        torch.manual_seed(seed)
+        got_t, got_lp = graphed.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=n_img)
+        torch.cuda.synchronize()
+        assert torch.equal(got_t, want_t), (call, got_t, want_t)
+        assert torch.equal(got_lp, want_lp), call
+        assert len(want_t.unique()) > n_img // 2
+    (sess,) = graphed._sessions.values()
+    assert sess.graph is not None
+
+
+@pytest.mark.gpu
+def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy):
+    """Same int4 policy through the reference loop (dynamic cache, torch formulas for the tail):
+    same tokens under the same seed; log-probabilities within a bf16 rounding of the log-softmax."""
+    print("ar decode: static fused vs reference loop", flush=True)
+    cond, uncond, cmask, umask = make_inputs(3, 7, torch.bfloat16, "cuda:0")
+    torch.manual_seed(31)
+    want_t, want_lp = reference_loop(int4_policy, cond, uncond, cmask, umask, 5.0, 1.0, 16)
+    for graph in (False, True):
+        torch.manual_seed(31)
+        got_t, got_lp = StaticARSampler(int4_policy, graph=graph).sample_image_tokens(
+            cond, uncond, cmask, umask, image_token_num=16)
+        torch.cuda.synchronize()
+        assert torch.equal(got_t, want_t), (graph, got_t, want_t)
+        torch.testing.assert_close(got_lp, want_lp, rtol=2 ** -7, atol=2 ** -7)

@@ -1,0 +1,202 @@
+"""Image-token sampling over a static KV cache, one HIP graph replay per decode step.
+
+Stands for ``JanusProPolicy.sample_image_tokens`` (``vrl/models/families/janus_pro/policy.py:476-525``)
+and the step it loops over (``_sample_ar_step``, ``policy.py:624-731``), with the same
+arguments, the same results and the same use of the random stream:
+
+* The reference keeps one KV cache per row, concatenates the rows before every trunk call and
+  splits them afterwards (``policy.py:664-682``, ``vrl/models/ar.py:42-110``: a copy of the whole
+  cache per token), rebuilds the attention masks with ``torch.cat`` (``policy.py:701-720``) and
+  reads row positions back to the host twice per token (``policy.py:638``, ``:730``).  When all
+  rows advance together, as they do in ``sample_image_tokens``, split-then-concat is the identity
+  and the positions are known on the host, so here the trunk writes into one preallocated
+  ``StaticCache`` whose length counter lives on the device, the attention mask is one
+  ``[2B, L_max]`` buffer (prompt mask, then ones) and nothing is read back until the end.
+* A decode step then has no host-dependent control flow and fixed addresses, so it is recorded
+  once as a HIP graph (trunk, head, CFG combine, draw, log-probability, next-token embedding,
+  write of token and log-probability at a device-side position) and replayed ``L_img - 2`` times.
+  The prompt pass and the first decode step run eagerly (the latter doubles as the warm-up a
+  capture needs).
+* The tail after the head is one launch (:func:`visionrl_amd.ops.cfg_sample`) when the logits are
+  bf16 on a GPU, and the reference's torch formulas otherwise; both draw through
+  ``exponential_`` exactly as ``torch.multinomial`` does, so a seeded rollout
+  (``vrl/models/families/janus_pro/executor.py:147-151`` seeds the global generator) samples the
+  same tokens as the reference loop.
+
+Rows that advance at different positions (the ``step_ar`` contract used with the token scheduler,
+``policy.py:527-572``) are not covered: that path keeps the reference implementation.
+"""
+
+from __future__ import annotations
+
+import types
+from typing import Any
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+
+__all__ = ["StaticARSampler", "install_static_ar_sampler"]
+
+
+def _round_up(n: int, to: int) -> int:
+    return (n + to - 1) // to * to
+
+
+class _Session:
+    """Buffers and the recorded step for one (rows, cache length, guidance, temperature) shape."""
+
+    def __init__(self, sampler: "StaticARSampler", rows2: int, hidden: int, max_len: int,
+                 dtype: torch.dtype, device: torch.device, cfg_weight: float, temperature: float,
+                 mask_dtype: torch.dtype):
+        from transformers.cache_utils import StaticCache
+
+        self.sampler = sampler
+        self.rows2, self.max_len = rows2, max_len
+        self.cfg_weight, self.temperature = float(cfg_weight), float(temperature)
+        trunk = sampler.trunk
+        self.cache = StaticCache(config=trunk.config, max_cache_len=max_len)
+        self.cur = torch.zeros((rows2, 1, hidden), dtype=dtype, device=device)
+        self.mask = torch.ones((rows2, max_len), dtype=mask_dtype, device=device)
+        self.tokens = torch.zeros((rows2 // 2, max_len), dtype=torch.long, device=device)
+        self.logprobs = torch.zeros((rows2 // 2, max_len), dtype=torch.float32, device=device)
+        self.img_pos = torch.zeros(1, dtype=torch.long, device=device)
+        self.graph = None
+
+    # -- one call of sample_image_tokens starts here
+    def begin(self, mask: torch.Tensor) -> None:
+        self.cache.reset()
+        self.mask.fill_(1)
+        self.mask[:, :mask.shape[1]].copy_(mask)
+        self.img_pos.zero_()
+
+    def tail(self, hidden: torch.Tensor) -> None:
+        """Head, guided draw, log-probability, bookkeeping, next input (``policy.py:684-700``)."""
+        s = self.sampler
+        logits = s.base.gen_head(hidden).squeeze(1)
+        if s.fused_tail and logits.dtype == torch.bfloat16 and logits.is_cuda:
+            sampled, lp = ops.cfg_sample(logits.contiguous(), self.cfg_weight, self.temperature)
+        else:
+            cond, uncond = logits.chunk(2, dim=0)
+            guided = uncond + self.cfg_weight * (cond - uncond)
+            probs = F.softmax(guided / self.temperature, dim=-1)
+            sampled = torch.multinomial(probs, num_samples=1).squeeze(-1)
+            lp = F.log_softmax(cond / self.temperature, dim=-1).gather(-1, sampled.unsqueeze(-1)).squeeze(-1)
+        self.tokens.index_copy_(1, self.img_pos, sampled.unsqueeze(1))
+        self.logprobs.index_copy_(1, self.img_pos, lp.to(torch.float32).unsqueeze(1))
+        self.img_pos.add_(1)
+        nxt = s.base.prepare_gen_img_embeds(torch.cat([sampled, sampled], dim=0).unsqueeze(-1))
+        self.cur.copy_(nxt.reshape(self.cur.shape))
+
+    def prefill(self, embeds: torch.Tensor) -> None:
+        out = self.sampler.trunk(inputs_embeds=embeds, attention_mask=self.mask, use_cache=True,
+                                 past_key_values=self.cache)
+        self.tail(out.last_hidden_state[:, -1:, :])
+
+    def step(self) -> None:
+        out = self.sampler.trunk(inputs_embeds=self.cur, attention_mask=self.mask, use_cache=True,
+                                 past_key_values=self.cache)
+        self.tail(out.last_hidden_state[:, -1:, :])
+
+    def capture(self) -> None:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.step()
+        self.graph = graph
+
+
+class StaticARSampler:
+    """``sample_image_tokens`` of a Janus-Pro style policy over a static cache and a HIP graph.
+
+    ``policy`` is duck-typed: ``_lm_trunk()`` returns the Hugging Face ``LlamaModel``
+    (``policy.py:240-266``), ``_base()`` the module holding ``gen_head`` and
+    ``prepare_gen_img_embeds`` (``policy.py:226-238``), ``config`` the defaults
+    (``cfg_weight``, ``temperature``, ``image_token_num``).  ``graph=False`` runs every step
+    eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
+    for the part after the head.
+    """
+
+    def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True,
+                 length_bucket: int = 64, max_sessions: int = 2):
+        self.policy = policy
+        self.trunk = policy._lm_trunk()
+        self.base = policy._base()
+        for name in ("gen_head", "prepare_gen_img_embeds"):
+            if not hasattr(self.base, name):
+                raise TypeError(f"policy._base() has no {name}")
+        self.graph = bool(graph)
+        self.fused_tail = bool(fused_tail)
+        self.length_bucket = int(length_bucket)
+        self.max_sessions = int(max_sessions)
+        self._sessions: dict = {}
+
+    def _defaults(self, cfg_weight, temperature, image_token_num):
+        conf = getattr(self.policy, "config", None)
+        cfg = cfg_weight if cfg_weight is not None else getattr(conf, "cfg_weight", None)
+        temp = temperature if temperature is not None else getattr(conf, "temperature", None)
+        n_img = image_token_num or getattr(conf, "image_token_num", None)
+        if cfg is None or temp is None or not n_img:
+            raise ValueError("cfg_weight, temperature and image_token_num need a value or a policy.config default")
+        if not float(temp) > 0:
+            raise ValueError("temperature must be positive")
+        return float(cfg), float(temp), int(n_img)
+
+    def _session(self, key, make):
+        sess = self._sessions.pop(key, None)
+        if sess is None:
+            while len(self._sessions) >= self.max_sessions:   # oldest first: caches are GBs at 1B scale
+                self._sessions.pop(next(iter(self._sessions)))
+            sess = make()
+        self._sessions[key] = sess
+        return sess
+
+    @torch.no_grad()
+    def sample_image_tokens(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,
+                            cond_attention_mask: torch.Tensor, uncond_attention_mask: torch.Tensor, *,
+                            cfg_weight: float | None = None, temperature: float | None = None,
+                            image_token_num: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """Returns ``(image_token_ids int64 [B, L_img], logprobs float32 [B, L_img])``."""
+        cfg, temp, n_img = self._defaults(cfg_weight, temperature, image_token_num)
+        if cond_inputs_embeds.dim() != 3 or cond_inputs_embeds.shape != uncond_inputs_embeds.shape:
+            raise ValueError("cond and uncond embeddings must both be [B, L_text, H]")
+        B, n_text, hidden = cond_inputs_embeds.shape
+        if tuple(cond_attention_mask.shape) != (B, n_text) or tuple(uncond_attention_mask.shape) != (B, n_text):
+            raise ValueError("attention masks must be [B, L_text]")
+        device, dtype = cond_inputs_embeds.device, cond_inputs_embeds.dtype
+        max_len = _round_up(n_text + n_img, self.length_bucket)
+        use_graph = self.graph and device.type == "cuda"
+        key = (2 * B, hidden, max_len, dtype, device, cfg, temp, cond_attention_mask.dtype)
+        sess = self._session(key, lambda: _Session(self, 2 * B, hidden, max_len, dtype, device, cfg, temp,
+                                                   cond_attention_mask.dtype))
+        sess.begin(torch.cat([cond_attention_mask, uncond_attention_mask], dim=0))
+        sess.prefill(torch.cat([cond_inputs_embeds, uncond_inputs_embeds], dim=0))
+        left = n_img - 1
+        if use_graph and left > 0:
+            if sess.graph is None:
+                sess.step()          # a real step, and the warm-up the capture needs
+                left -= 1
+                if left > 0:
+                    sess.capture()   # records, does not run
+            for _ in range(left):
+                sess.graph.replay()
+        else:
+            for _ in range(left):
+                sess.step()
+        return sess.tokens[:, :n_img].clone(), sess.logprobs[:, :n_img].clone()
+
+
+def install_static_ar_sampler(policy: Any, **options) -> StaticARSampler:
+    """Make ``policy.sample_image_tokens`` (what ``JanusProPipelineExecutor.forward`` calls,
+    ``vrl/models/families/janus_pro/executor.py:197-203``) run through a :class:`StaticARSampler`."""
+    sampler = StaticARSampler(policy, **options)
+
+    def sample_image_tokens(self, cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                            uncond_attention_mask, *, cfg_weight=None, temperature=None, image_token_num=None):
+        return sampler.sample_image_tokens(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                                           uncond_attention_mask, cfg_weight=cfg_weight,
+                                           temperature=temperature, image_token_num=image_token_num)
+
+    policy.sample_image_tokens = types.MethodType(sample_image_tokens, policy)
+    policy._static_ar_sampler = sampler
+    return sampler
