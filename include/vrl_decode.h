@@ -1,0 +1,64 @@
+/*
+ * C ABI of the decode-step kernels that sit between the int4 linears of a Llama decoder layer.
+ *
+ * One decode step of the reference calls the Hugging Face LlamaModel on a single new token per
+ * row (vrl/models/families/janus_pro/policy.py:673-678) after concatenating per-row KV caches
+ * (policy.py:664-671, vrl/models/ar.py:42-110).  Between the linears that vrl_int4.h covers, each
+ * decoder layer of that model computes, on bf16 tensors (every tensor op in fp32, result rounded
+ * to bf16):
+ *   h      = residual + sublayer_output                       (LlamaDecoderLayer.forward)
+ *   normed = weight * bf16( h * rsqrt(mean(h^2) + eps) )      (LlamaRMSNorm.forward)
+ *   q, k   = x * cos + rotate_half(x) * sin                   (apply_rotary_pos_emb)
+ *   cache[position] = k, v;  out = softmax(q . K^T * scaling + mask) . V   (Cache.update, sdpa)
+ * These entry points compute exactly that for one new token per row over a preallocated cache,
+ * with the position held in device memory so that a recorded HIP graph can be replayed.
+ *
+ * Conventions as in vrl_int4.h: caller-owned device memory, calls only enqueue on `hip_stream`
+ * of the current device, no allocation, no synchronisation, no state; return 0, a hipError_t
+ * value, or a VRL_INT4_E* code (nothing is enqueued then).
+ */
+#ifndef VRL_DECODE_H
+#define VRL_DECODE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Residual add and RMSNorm of M rows of K bf16 values (K % 8 == 0, K <= 16384):
+ *   h = residual ? bf16(x + residual) : x;   y = weight * bf16(h * rsqrt(mean(h^2) + eps))
+ * `h_out` receives h when it is not NULL (required when residual is given; may alias x or
+ * residual).  Stands for `residual + hidden_states` followed by input_layernorm /
+ * post_attention_layernorm / the model's final norm.  All pointers 16-byte aligned.
+ */
+int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const void *weight, void *h_out,
+                         void *y, int M, int K, float eps, void *hip_stream);
+
+/*
+ * Rotary embedding, cache append and attention of one new token per row.
+ *   q        bf16 [M, n_heads * D]       query projections of the new token, row stride q_stride elements
+ *   k, v     bf16 [M, n_kv_heads * D]    key / value projections, row stride kv_stride elements
+ *   k_cache, v_cache  bf16 [M, n_kv_heads, L_max, D]   (the layout of transformers' StaticLayer)
+ *   cos, sin bf16 [L_max, D]             rotary tables, row p = position p
+ *   mask     uint8 [M, L_max]            1 = this cache slot may be attended (0 = prompt padding)
+ *   position int64 device scalar p, 0 <= p < L_max: the slot the new token takes
+ *   out      bf16 [M, n_heads * D]
+ * Row m, head h: q and k are rotated with row p of the tables (each product and the sum rounded
+ * to bf16, as the tensor ops do), the rotated k and v are written to slot p of the cache, and
+ * out = softmax(q . K[0..p]^T * scaling, masked slots excluded) . V[0..p] with fp32 scores and
+ * accumulation.  D is 64 or 128; n_heads % n_kv_heads == 0; L_max <= 8192.  A position outside
+ * [0, L_max) makes the call a no-op on the device.  Calls for different layers (different
+ * caches) are independent; two calls on the same cache must be ordered by the stream.
+ */
+int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                              void *k_cache, void *v_cache, const void *cos, const void *sin,
+                              const void *mask, const int64_t *position, void *out,
+                              int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                              void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VRL_DECODE_H */

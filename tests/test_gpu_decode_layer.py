@@ -1,0 +1,155 @@
+"""The decode-step kernels between the linears against their oracle (and against the library
+modules they stand for, run on the device)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decode_oracle as d
+from oracle import int4_oracle as o
+from tests._util import bf16_to_bits, bits_to_bf16
+from tests.test_decode_oracle import attn_case, rand_bits, ulp_distance
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops_mod():
+    from visionrl_amd import ops
+    return ops
+
+
+def say(*what):
+    print("decode layer:", *what, flush=True)
+
+
+@pytest.mark.parametrize("M,K,with_residual", [(1, 2048, False), (2, 2048, True), (32, 2048, True), (3, 4096, True),
+                                               (5, 264, True), (2, 16384, False), (7, 3072, True)])
+def test_add_rmsnorm_parity(ops_mod, M, K, with_residual):
+    say("add_rmsnorm", M, K, with_residual)
+    rng = np.random.default_rng(31 * K + M)
+    x, res, w = rand_bits(rng, (M, K)), rand_bits(rng, (M, K), 4.0), rand_bits(rng, (K,), 0.5)
+    h_want, y_want = d.add_rmsnorm(x, res if with_residual else None, w, 1e-6)
+    xt, rt, wt = bits_to_bf16(x, DEV), bits_to_bf16(res, DEV), bits_to_bf16(w, DEV)
+    h, y = ops_mod.add_rmsnorm(xt, wt, 1e-6, rt if with_residual else None)
+    torch.cuda.synchronize()
+    assert (bf16_to_bits(h) == h_want).all()
+    dist = ulp_distance(bf16_to_bits(y), y_want)
+    assert dist.max() <= 1 and (dist > 0).mean() < 2e-3, (dist.max(), (dist > 0).mean())
+    if with_residual:   # in place: h over the residual stream
+        h2, y2 = ops_mod.add_rmsnorm(xt, wt, 1e-6, rt, h_out=rt)
+        torch.cuda.synchronize()
+        assert h2 is rt and torch.equal(h2, h) and torch.equal(y2, y)
+
+
+def test_add_rmsnorm_equals_the_library_module_on_the_device(ops_mod):
+    from transformers.models.llama.modeling_llama import LlamaRMSNorm
+
+    say("add_rmsnorm vs LlamaRMSNorm")
+    torch.manual_seed(0)
+    norm = LlamaRMSNorm(2048, eps=1e-6).to(torch.bfloat16).to(DEV)
+    with torch.no_grad():
+        norm.weight.normal_(1.0, 0.2)
+        x = torch.randn(32, 2048, device=DEV).to(torch.bfloat16)
+        res = (torch.randn(32, 2048, device=DEV) * 5).to(torch.bfloat16)
+        want_h = res + x
+        want = norm(want_h)
+    h, y = ops_mod.add_rmsnorm(x, norm.weight.data, 1e-6, res)
+    torch.cuda.synchronize()
+    assert torch.equal(h, want_h)
+    dist = ulp_distance(bf16_to_bits(y), bf16_to_bits(want))
+    assert dist.max() <= 1 and (dist > 0).mean() < 2e-3
+
+
+def run_attn(ops_mod, c):
+    t = {k: (bits_to_bf16(c[k], DEV) if k in ("q", "k", "v", "kc", "vc", "cos", "sin") else None) for k in c}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([c["p"]], dtype=torch.int64, device=DEV)
+    out = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], t["kc"], t["vc"], t["cos"], t["sin"], mask, pos,
+                                   c["scaling"])
+    torch.cuda.synchronize()
+    return out, t["kc"], t["vc"]
+
+
+ATTN_CASES = [
+    # M, H, Hkv, D, L, p
+    (2, 16, 16, 128, 640, 37), (2, 16, 16, 128, 640, 639), (32, 16, 16, 128, 128, 100), (3, 4, 4, 64, 64, 0),
+    (3, 4, 4, 64, 64, 1), (2, 8, 2, 128, 96, 15), (2, 8, 2, 128, 96, 16), (2, 8, 2, 128, 96, 17), (1, 6, 3, 64, 48, 47),
+    (2, 4, 1, 64, 8192, 5000),
+]
+
+
+@pytest.mark.parametrize("M,H,Hkv,D,L,p", ATTN_CASES)
+def test_rope_attn_decode_parity(ops_mod, M, H, Hkv, D, L, p):
+    say("rope_attn", M, H, Hkv, D, L, p)
+    c = attn_case(1000 + p + L, M, H, Hkv, D, L, p)
+    want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
+                                                c["mask"], p, H, Hkv, c["scaling"])
+    out, kc, vc = run_attn(ops_mod, c)
+    # cache: slot p holds the rotated key and the value bit for bit, nothing else moved
+    assert (bf16_to_bits(kc) == kc_want).all() and (bf16_to_bits(vc) == vc_want).all()
+    got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)
+    # fp32 scores and accumulation, one bf16 rounding of the result
+    tol = 0.51 * o.bf16_ulp(want.astype(np.float32)) + 2e-5 * np.abs(want).max()
+    assert (np.abs(got - want) <= tol).all(), np.abs(got - want).max()
+
+
+def test_rope_attn_masks_and_strided_inputs(ops_mod):
+    say("rope_attn masks, fused qkv buffer")
+    M, H, D, L, p = 2, 4, 64, 32, 20
+    c = attn_case(5, M, H, H, D, L, p)
+    c["mask"][:] = 0
+    c["mask"][:, 4] = 1           # one slot allowed: the output is that slot's value row
+    out, _, _ = run_attn(ops_mod, c)
+    assert (bf16_to_bits(out) == c["vc"][:, :, 4, :].reshape(M, H * D)).all()
+    c["mask"][:] = 0              # nothing allowed: zeros, not NaN
+    out, _, _ = run_attn(ops_mod, c)
+    assert (bf16_to_bits(out) & 0x7FFF == 0).all()
+    # q, k, v as column blocks of one [M, 3*H*D] buffer (how a fused projection would hand them over)
+    c = attn_case(6, M, H, H, D, L, p)
+    want, _, _ = run_attn(ops_mod, c)
+    qkv = torch.cat([bits_to_bf16(c[n], DEV) for n in ("q", "k", "v")], dim=1)
+    q, k, v = qkv[:, :H * D], qkv[:, H * D:2 * H * D], qkv[:, 2 * H * D:]
+    got = ops_mod.rope_attn_decode(q, k, v, bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV),
+                                   bits_to_bf16(c["cos"], DEV), bits_to_bf16(c["sin"], DEV),
+                                   torch.from_numpy(c["mask"]).to(DEV),
+                                   torch.tensor([p], dtype=torch.int64, device=DEV), c["scaling"])
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
+def test_position_outside_the_cache_is_a_no_op(ops_mod):
+    say("rope_attn position out of range")
+    c = attn_case(8, 2, 2, 2, 64, 16, 3)
+    for bad in (-1, 16, 1 << 40):
+        c["p"] = 3
+        t_out = torch.full((2, 128), 7.0, dtype=torch.bfloat16, device=DEV)
+        kc, vc = bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV)
+        ops_mod.rope_attn_decode(bits_to_bf16(c["q"], DEV), bits_to_bf16(c["k"], DEV), bits_to_bf16(c["v"], DEV),
+                                 kc, vc, bits_to_bf16(c["cos"], DEV), bits_to_bf16(c["sin"], DEV),
+                                 torch.from_numpy(c["mask"]).to(DEV),
+                                 torch.tensor([bad], dtype=torch.int64, device=DEV), c["scaling"], out=t_out)
+        torch.cuda.synchronize()
+        assert (t_out == 7.0).all() and (bf16_to_bits(kc) == c["kc"]).all() and (bf16_to_bits(vc) == c["vc"]).all()
+
+
+def test_wrappers_reject_contract_violations(ops_mod):
+    x = torch.zeros(2, 256, dtype=torch.bfloat16, device=DEV)
+    w = torch.ones(256, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops_mod.add_rmsnorm(x.float(), w, 1e-6)
+    with pytest.raises(ValueError):
+        ops_mod.add_rmsnorm(x, w[:128], 1e-6)
+    with pytest.raises(ValueError):
+        ops_mod.add_rmsnorm(x[:, :132].contiguous(), w[:132].contiguous(), 1e-6)   # K % 8
+    c = attn_case(9, 2, 2, 2, 64, 16, 3)
+    args = [bits_to_bf16(c[n], DEV) for n in ("q", "k", "v", "kc", "vc", "cos", "sin")]
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([3], dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(*args, mask.long(), pos, 0.125)
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(*args, mask, pos.int(), 0.125)
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(args[0][:, :100], *args[1:], mask, pos, 0.125)

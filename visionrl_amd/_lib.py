@@ -28,6 +28,8 @@ SYMBOLS = (
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
     "vrl_cfg_sample_bf16",
+    "vrl_add_rmsnorm_bf16",
+    "vrl_rope_attn_decode_bf16",
 )
 
 
@@ -99,6 +101,11 @@ def _bind(lib):
     lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
     lib.vrl_cfg_sample_bf16.restype = ci
     lib.vrl_cfg_sample_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_float, ctypes.c_float, vp]
+    lib.vrl_add_rmsnorm_bf16.restype = ci
+    lib.vrl_add_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_float, vp]
+    lib.vrl_rope_attn_decode_bf16.restype = ci
+    lib.vrl_rope_attn_decode_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
+                                              ci, ci, ci, ci, ci, ctypes.c_float, vp]
 
 
 def load():

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libvrl_int4.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["int4_gemv.hip", "cfg_sample.hip"]
+SOURCES = ["int4_gemv.hip", "cfg_sample.hip", "decode_layer.hip"]
 
 HIPCC_FLAGS = [
     "-O3",

@@ -1,0 +1,329 @@
+// The parts of a Llama decoder layer between its linears, for one new token per row:
+// residual add + RMSNorm, and rotary embedding + cache append + attention over a static cache.
+//
+// Restates, with the roundings torch applies to bf16 tensors (each tensor op computes in fp32
+// and rounds its result to bf16), what the trunk call of a decode step runs between the
+// projections (vrl/models/families/janus_pro/policy.py:673-678 -> transformers LlamaDecoderLayer.forward,
+// LlamaRMSNorm.forward, apply_rotary_pos_emb, StaticLayer.update, sdpa_attention_forward):
+//   h = bf16(residual + x);  normed = bf16(weight * bf16(h * rsqrt(mean(h^2) + eps)))
+//   q' = bf16(bf16(q * cos) + bf16(rotate_half(q) * sin)), same for k
+//   cache[p] = k', v;  out = bf16(softmax(q' . K^T * scaling, masked slots out) . V)
+// The attention keeps scores and probabilities in fp32 (the library kernel it stands for rounds
+// the probabilities to bf16 before the second product), so it agrees with it to a bf16 rounding
+// of the output, not bit for bit.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/vrl_decode.h"
+#include "../../include/vrl_int4.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+constexpr int THREADS = 256;
+constexpr int WAVES = THREADS / WAVE;
+constexpr int MAX_NORM_K = 16384;
+constexpr int MAX_CACHE_LEN = 8192;
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
+
+// round to nearest even through the hardware conversion, value kept in a float
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float v) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v);
+}
+__device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+    return v;
+}
+
+// every thread returns the block's total; `red` holds WAVES floats and is free for reuse afterwards
+template <bool MAX>
+__device__ __forceinline__ float block_reduce(float v, float *red) {
+    v = MAX ? wave_max(v) : wave_sum(v);
+    __syncthreads();  // earlier readers of red are done
+    if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int k = 1; k < WAVES; ++k) r = MAX ? fmaxf(r, red[k]) : r + red[k];
+    return r;
+}
+
+// ---------------------------------------------------------------- residual add + RMSNorm
+template <bool ADD>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_kernel(const uint16_t *x, const uint16_t *residual,
+                                                              const uint16_t *__restrict__ weight,
+                                                              uint16_t *h_out, uint16_t *__restrict__ y,
+                                                              int K, float eps) {
+    extern __shared__ __align__(16) uint16_t hs[];  // the row after the add, K values
+    __shared__ float red[WAVES];
+    const long row = (long)blockIdx.x * K;
+    float ss = 0.0f;
+    for (int i = threadIdx.x * 8; i < K; i += THREADS * 8) {
+        uint4 xv = *reinterpret_cast<const uint4 *>(x + row + i);
+        if (ADD) {
+            const uint4 rv = *reinterpret_cast<const uint4 *>(residual + row + i);
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, rw[4] = {rv.x, rv.y, rv.z, rv.w};
+            uint32_t hw[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t lo = f32_to_bf16_bits(bf16_to_f32(rw[e] & 0xFFFFu) + bf16_to_f32(xw[e] & 0xFFFFu));
+                const uint32_t hi = f32_to_bf16_bits(bf16_to_f32(rw[e] >> 16) + bf16_to_f32(xw[e] >> 16));
+                hw[e] = lo | (hi << 16);
+            }
+            xv = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+        }
+        const uint32_t w4[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = bf16_to_f32(w4[e] & 0xFFFFu), hi = bf16_to_f32(w4[e] >> 16);
+            ss += lo * lo;
+            ss += hi * hi;
+        }
+        *reinterpret_cast<uint4 *>(hs + i) = xv;
+        if (h_out) *reinterpret_cast<uint4 *>(h_out + row + i) = xv;
+    }
+    const float total = block_reduce<false>(ss, red);
+    const float r = rsqrtf(total * (1.0f / (float)K) + eps);  // mean as sum * (1/K), as the tensor op does
+    for (int i = threadIdx.x * 8; i < K; i += THREADS * 8) {  // every thread reads back what it wrote
+        const uint4 hv = *reinterpret_cast<const uint4 *>(hs + i);
+        const uint4 wv = *reinterpret_cast<const uint4 *>(weight + i);
+        const uint32_t h4[4] = {hv.x, hv.y, hv.z, hv.w}, w4[4] = {wv.x, wv.y, wv.z, wv.w};
+        uint32_t o4[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = round_bf16(bf16_to_f32(h4[e] & 0xFFFFu) * r);
+            const float hi = round_bf16(bf16_to_f32(h4[e] >> 16) * r);
+            o4[e] = f32_to_bf16_bits(bf16_to_f32(w4[e] & 0xFFFFu) * lo) |
+                    (f32_to_bf16_bits(bf16_to_f32(w4[e] >> 16) * hi) << 16);
+        }
+        *reinterpret_cast<uint4 *>(y + row + i) = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+    }
+}
+
+// ---------------------------------------------------------------- rotary + cache append + attention
+struct AttnArgs {
+    const uint16_t *q, *k, *v;
+    uint16_t *k_cache, *v_cache;
+    const uint16_t *cos, *sin;
+    const uint8_t *mask;
+    const long long *position;
+    uint16_t *out;
+    int q_stride, kv_stride;
+    int n_heads, n_kv_heads, L_max;
+    float scaling;
+};
+
+template <int VEC>
+__device__ __forceinline__ void load_bf16_vec(const uint16_t *p, float (&f)[VEC]) {
+    if (VEC == 8) {
+        const uint4 w = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
+            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
+        }
+    } else {
+        const uint2 w = *reinterpret_cast<const uint2 *>(p);
+        const uint32_t u[2] = {w.x, w.y};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
+            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
+        }
+    }
+}
+
+// One workgroup per (head, row).  Sixteen lanes share a cache slot (D / 16 values each), so a wave
+// reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the workgroup sixteen.
+template <int D>
+__global__ __launch_bounds__(THREADS) void rope_attn_decode_kernel(AttnArgs a) {
+    constexpr int VEC = D / 16;
+    extern __shared__ __align__(16) float smem[];
+    float *qs = smem;                // rotated query
+    float *ks = qs + D;              // rotated key of the new token
+    float *vs = ks + D;              // value of the new token
+    float *part = vs + D;            // WAVES x D partial outputs
+    float *red = part + WAVES * D;   // WAVES
+    float *sc = red + WAVES;         // scores, then probabilities, of slots 0..p
+
+    const long long p64 = *a.position;
+    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the grid
+    const int p = (int)p64;
+    const int h = blockIdx.x, m = blockIdx.y;
+    const int group = a.n_heads / a.n_kv_heads;
+    const int hk = h / group;
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int sub = lane >> 4, l16 = lane & 15;
+    const long cache_base = ((long)m * a.n_kv_heads + hk) * a.L_max * D;
+    const uint8_t *mask = a.mask + (long)m * a.L_max;
+
+    if (tid < D) {
+        const uint16_t *qrow = a.q + (long)m * a.q_stride + h * D;
+        const uint16_t *krow = a.k + (long)m * a.kv_stride + hk * D;
+        const uint16_t *vrow = a.v + (long)m * a.kv_stride + hk * D;
+        const int partner = tid < D / 2 ? tid + D / 2 : tid - D / 2;
+        const float sign = tid < D / 2 ? -1.0f : 1.0f;  // rotate_half: (-x2, x1)
+        const float c = bf16_to_f32(a.cos[(long)p * D + tid]), s = bf16_to_f32(a.sin[(long)p * D + tid]);
+        const float qe = round_bf16(round_bf16(bf16_to_f32(qrow[tid]) * c) +
+                                    round_bf16(sign * bf16_to_f32(qrow[partner]) * s));
+        const float ke = round_bf16(round_bf16(bf16_to_f32(krow[tid]) * c) +
+                                    round_bf16(sign * bf16_to_f32(krow[partner]) * s));
+        qs[tid] = qe;
+        ks[tid] = ke;
+        vs[tid] = bf16_to_f32(vrow[tid]);
+        if (h % group == 0) {  // one workgroup per kv head appends; readers of slot p use their own copy
+            a.k_cache[cache_base + (long)p * D + tid] = (uint16_t)f32_to_bf16_bits(ke);
+            a.v_cache[cache_base + (long)p * D + tid] = vrow[tid];
+        }
+    }
+    __syncthreads();
+
+    float qreg[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) qreg[i] = qs[l16 * VEC + i];
+    const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
+    const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
+
+    // scores of the cached slots 0..p-1
+#pragma unroll 4
+    for (int j0 = 0; j0 < p; j0 += 4 * WAVES) {
+        const int j = j0 + wave * 4 + sub;
+        const int jj = j < p ? j : p - 1;  // in range: the loop runs only when p >= 1
+        float kf[VEC];
+        load_bf16_vec<VEC>(kc + (long)jj * D, kf);
+        float dot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) dot += qreg[i] * kf[i];
+        dot += __shfl_xor(dot, 1, WAVE);
+        dot += __shfl_xor(dot, 2, WAVE);
+        dot += __shfl_xor(dot, 4, WAVE);
+        dot += __shfl_xor(dot, 8, WAVE);
+        if (l16 == 0 && j < p) sc[j] = mask[j] ? dot * a.scaling : -INFINITY;
+    }
+    if (wave == 0) {  // the new token's own slot
+        float dot = 0.0f;
+        for (int d = lane; d < D; d += WAVE) dot += qs[d] * ks[d];
+        dot = wave_sum(dot);
+        if (lane == 0) sc[p] = mask[p] ? dot * a.scaling : -INFINITY;
+    }
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int j = tid; j <= p; j += THREADS) mx = fmaxf(mx, sc[j]);
+    mx = block_reduce<true>(mx, red);
+    if (mx == -INFINITY) mx = 0.0f;  // every slot masked: probabilities and output become zero
+    float sum = 0.0f;
+    for (int j = tid; j <= p; j += THREADS) {  // each thread rewrites the entries it read
+        const float e = expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+    sum = block_reduce<false>(sum, red);  // its barriers also publish the probabilities
+
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+#pragma unroll 4
+    for (int j0 = 0; j0 < p; j0 += 4 * WAVES) {
+        const int j = j0 + wave * 4 + sub;
+        const int jj = j < p ? j : p - 1;
+        float vf[VEC];
+        load_bf16_vec<VEC>(vc + (long)jj * D, vf);
+        const float w = j < p ? sc[jj] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] += w * vf[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        acc[i] += __shfl_xor(acc[i], 16, WAVE);
+        acc[i] += __shfl_xor(acc[i], 32, WAVE);
+    }
+    if (sub == 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[wave * D + l16 * VEC + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < D) {
+        float o = sc[p] * vs[tid];
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) o += part[w * D + tid];
+        o = sum > 0.0f ? o / sum : 0.0f;
+        a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)f32_to_bf16_bits(o);
+    }
+}
+
+bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+}  // namespace
+
+extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const void *weight, void *h_out,
+                                    void *y, int M, int K, float eps, void *hip_stream) {
+    if (!x || !weight || !y || (residual && !h_out)) return VRL_INT4_ENULL;
+    if (M < 1 || M > (1 << 20) || K < 8 || K % 8 != 0 || K > MAX_NORM_K || !(eps >= 0.0f)) return VRL_INT4_ESHAPE;
+    if (misaligned(x, 16) || misaligned(weight, 16) || misaligned(y, 16) || misaligned(residual, 16) ||
+        misaligned(h_out, 16))
+        return VRL_INT4_EALIGN;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    const size_t lds = (size_t)K * sizeof(uint16_t);
+    auto xs = static_cast<const uint16_t *>(x);
+    auto rs = static_cast<const uint16_t *>(residual);
+    auto ws = static_cast<const uint16_t *>(weight);
+    auto hs = static_cast<uint16_t *>(h_out);
+    auto ys = static_cast<uint16_t *>(y);
+    if (residual)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<true>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_kernel<false>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
+    return (int)hipGetLastError();
+}
+
+extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                         void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                         const void *mask, const int64_t *position, void *out,
+                                         int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                         void *hip_stream) {
+    if (!q || !k || !v || !k_cache || !v_cache || !cos || !sin || !mask || !position || !out) return VRL_INT4_ENULL;
+    if (M < 1 || M > 65535 || n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || n_heads > 65535 ||
+        (D != 64 && D != 128) || L_max < 1 || L_max > MAX_CACHE_LEN || q_stride < n_heads * D ||
+        kv_stride < n_kv_heads * D || q_stride % 8 != 0 || kv_stride % 8 != 0)
+        return VRL_INT4_ESHAPE;
+    if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(k_cache, 16) ||
+        misaligned(v_cache, 16) || misaligned(cos, 2) || misaligned(sin, 2) || misaligned(position, 8) ||
+        misaligned(out, 2))
+        return VRL_INT4_EALIGN;
+    AttnArgs a;
+    a.q = static_cast<const uint16_t *>(q);
+    a.k = static_cast<const uint16_t *>(k);
+    a.v = static_cast<const uint16_t *>(v);
+    a.k_cache = static_cast<uint16_t *>(k_cache);
+    a.v_cache = static_cast<uint16_t *>(v_cache);
+    a.cos = static_cast<const uint16_t *>(cos);
+    a.sin = static_cast<const uint16_t *>(sin);
+    a.mask = static_cast<const uint8_t *>(mask);
+    a.position = reinterpret_cast<const long long *>(position);
+    a.out = static_cast<uint16_t *>(out);
+    a.q_stride = q_stride;
+    a.kv_stride = kv_stride;
+    a.n_heads = n_heads;
+    a.n_kv_heads = n_kv_heads;
+    a.L_max = L_max;
+    a.scaling = scaling;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    const size_t lds = (size_t)(3 * D + WAVES * D + WAVES + L_max) * sizeof(float);
+    if (D == 128)
+        hipLaunchKernelGGL(rope_attn_decode_kernel<128>, dim3(n_heads, M), dim3(THREADS), lds, stream, a);
+    else
+        hipLaunchKernelGGL(rope_attn_decode_kernel<64>, dim3(n_heads, M), dim3(THREADS), lds, stream, a);
+    return (int)hipGetLastError();
+}

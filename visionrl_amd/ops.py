@@ -25,7 +25,8 @@ from .int4_format import check_packed
 
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
-           "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample"]
+           "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "add_rmsnorm",
+           "rope_attn_decode"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -497,3 +498,84 @@ class DirectCall:
         if rc:
             _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
         return outs
+
+
+# ---------------------------------------------------------------------- decode-step kernels around the linears
+def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None,
+                *, h_out: torch.Tensor | None = None, y: torch.Tensor | None = None):
+    """``LlamaRMSNorm`` of ``h = x (+ residual)`` over bf16 rows ``[M, K]``: returns ``(h, normed)``.
+
+    The residual add of ``LlamaDecoderLayer.forward`` and the norm that follows it, in one launch
+    (reached from ``vrl/models/families/janus_pro/policy.py:673-678``).  ``h_out`` / ``y`` may be
+    given to reuse buffers; without a residual ``h`` is ``x`` itself.
+    """
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("x must be contiguous bfloat16 [M, K]")
+    dev = _require_device("x", x)
+    M, K = x.shape
+    if weight.dtype != torch.bfloat16 or tuple(weight.shape) != (K,) or not weight.is_contiguous():
+        raise ValueError(f"weight must be contiguous bfloat16 [{K}]")
+    _require_device("weight", weight, dev)
+    for name, t in (("residual", residual), ("h_out", h_out), ("y", y)):
+        if t is not None:
+            if t.dtype != torch.bfloat16 or tuple(t.shape) != (M, K) or not t.is_contiguous():
+                raise ValueError(f"{name} must be contiguous bfloat16 [{M}, {K}]")
+            _require_device(name, t, dev)
+    if y is None:
+        y = torch.empty_like(x)
+    if residual is not None and h_out is None:
+        h_out = torch.empty_like(x)
+    with _on(dev):
+        rc = _lib.load().vrl_add_rmsnorm_bf16(
+            x.data_ptr(), residual.data_ptr() if residual is not None else None, weight.data_ptr(),
+            h_out.data_ptr() if h_out is not None else None, y.data_ptr(), M, K, float(eps), _stream_handle(dev))
+    _lib.check(rc, "vrl_add_rmsnorm_bf16")
+    return (h_out if h_out is not None else x), y
+
+
+def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+                     v_cache: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mask: torch.Tensor,
+                     position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rotary embedding, cache append and attention for one new token per row, one launch.
+
+    ``q [M, H*D]``, ``k, v [M, Hkv*D]`` bf16 (rows may be strided views of one buffer), caches
+    ``[M, Hkv, L, D]`` bf16 (the layout of transformers' ``StaticLayer``; slot ``position`` is
+    written), ``cos, sin [L, D]`` bf16, ``mask [M, L]`` uint8, ``position`` an int64 device
+    scalar.  Stands for ``apply_rotary_pos_emb``, ``Cache.update`` and the attention of
+    ``LlamaAttention.forward`` (reached from ``vrl/models/families/janus_pro/policy.py:673-678``).
+    """
+    dev = _require_device("k_cache", k_cache)
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.dtype != torch.bfloat16 or \
+            v_cache.dtype != torch.bfloat16 or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise ValueError("caches must be contiguous bfloat16 [M, Hkv, L, D] of one shape")
+    M, Hkv, L, D = k_cache.shape
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dtype != torch.bfloat16 or t.dim() != 2 or t.shape[0] != M or t.stride(1) != 1:
+            raise ValueError(f"{name} must be bfloat16 [{M}, heads * {D}] with unit inner stride")
+        if t.device != dev:
+            raise ValueError(f"{name} is on {t.device}, expected {dev}")
+    if q.shape[1] % D != 0 or tuple(k.shape) != (M, Hkv * D) or tuple(v.shape) != (M, Hkv * D) or \
+            k.stride(0) != v.stride(0):
+        raise ValueError("q must hold whole heads and k, v be [M, Hkv * D] with one row stride")
+    H = q.shape[1] // D
+    for name, t in (("cos", cos), ("sin", sin)):
+        if t.dtype != torch.bfloat16 or tuple(t.shape) != (L, D) or not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous bfloat16 [{L}, {D}]")
+        _require_device(name, t, dev)
+    if mask.dtype != torch.uint8 or tuple(mask.shape) != (M, L) or not mask.is_contiguous():
+        raise ValueError(f"mask must be contiguous uint8 [{M}, {L}]")
+    if position.dtype != torch.int64 or position.numel() != 1:
+        raise ValueError("position must be an int64 tensor with one element")
+    for name, t in (("v_cache", v_cache), ("mask", mask), ("position", position)):
+        _require_device(name, t, dev)
+    if out is None:
+        out = torch.empty((M, H * D), dtype=torch.bfloat16, device=dev)
+    elif out.dtype != torch.bfloat16 or tuple(out.shape) != (M, H * D) or not out.is_contiguous():
+        raise ValueError(f"out must be contiguous bfloat16 [{M}, {H * D}]")
+    with _on(dev):
+        rc = _lib.load().vrl_rope_attn_decode_bf16(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), k_cache.data_ptr(),
+            v_cache.data_ptr(), cos.data_ptr(), sin.data_ptr(), mask.data_ptr(), position.data_ptr(),
+            out.data_ptr(), M, H, Hkv, D, L, float(scaling), _stream_handle(dev))
+    _lib.check(rc, "vrl_rope_attn_decode_bf16")
+    return out
