@@ -397,7 +397,8 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
 
     ``reference_style`` is the loop of vrl/models/families/janus_pro/policy.py:624-731 with the trunk's
     dynamic cache and the torch formulas for the tail, without its per-row cache copies and host
-    read-backs (so a lower bound for the reference); ``static_*`` is visionrl_amd.ar_decode.
+    read-backs (so a lower bound for the reference); ``static_*`` is visionrl_amd.ar_decode over the
+    trunk module, ``native_*`` the same with the trunk as visionrl_amd.decode_step (7 launches per layer).
     """
     import types
 
@@ -479,7 +480,7 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
         entry = out.setdefault(f"B{B}", {})
         entry["bf16_reference_style_ms_per_token"] = per_token_ms(
             lambda: reference_style(policy, *inputs[B], tokens))
-        sampler = StaticARSampler(policy, graph=True, fused_tail=False)
+        sampler = StaticARSampler(policy, graph=True, fused_tail=False, native=False)
         entry["bf16_static_hip_graph_ms_per_token"] = per_token_ms(
             lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
         del sampler
@@ -491,10 +492,11 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
         if only is None:
             entry["int4_reference_style_ms_per_token"] = per_token_ms(
                 lambda: reference_style(policy, *inputs[B], tokens))
-        for name, graph in (("int4_static_eager", False), ("int4_static_hip_graph", True)):
+        for name, graph, native in (("int4_static_eager", False, False), ("int4_static_hip_graph", True, False),
+                                    ("int4_native_eager", False, True), ("int4_native_hip_graph", True, True)):
             if only is not None and name != only:
                 continue
-            sampler = StaticARSampler(policy, graph=graph)
+            sampler = StaticARSampler(policy, graph=graph, native=native)
             entry[f"{name}_ms_per_token"] = per_token_ms(
                 lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
             del sampler
@@ -589,7 +591,7 @@ def main():
     from visionrl_amd import ops
 
     if args.ar_decode:
-        print(json.dumps(ar_decode_loop(device, only="int4_static_hip_graph", batches=(args.ar_decode,))))
+        print(json.dumps(ar_decode_loop(device, only="int4_native_hip_graph", batches=(args.ar_decode,))))
         return
     if args.single_calls:
         for M in (1, 32):

@@ -13,7 +13,7 @@ import pytest
 from visionrl_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "vrl_int4.h")
+HEADERS = [os.path.join(ROOT, "include", name) for name in ("vrl_int4.h", "vrl_decode.h")]
 
 
 @pytest.fixture(scope="module")
@@ -22,9 +22,11 @@ def lib():
 
 
 def declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(vrl_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+        names |= set(re.findall(r"\b(vrl_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -164,6 +166,32 @@ def test_direct_prepacked_validation(lib):
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002
     probs[1].y, probs[1].M, probs[1].K = p, 32, 16384  # LDS holds 4 such rows: 8 slabs, 9 with the first problem
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
+
+
+def test_decode_layer_validation(lib):
+    keep, p = buf(1 << 16)
+    norm = lib.vrl_add_rmsnorm_bf16
+    assert norm(None, None, p, None, p, 1, 256, 1e-6, None) == 1003
+    assert norm(p, p, p, None, p, 1, 256, 1e-6, None) == 1003       # a residual needs somewhere to put h
+    assert norm(p, None, p, None, p, 0, 256, 1e-6, None) == 1001
+    assert norm(p, None, p, None, p, 1, 260, 1e-6, None) == 1001    # K % 8
+    assert norm(p, None, p, None, p, 1, 16392, 1e-6, None) == 1001  # K beyond what one workgroup stages
+    assert norm(p, None, p, None, p, 1, 256, -1.0, None) == 1001
+    assert norm(p + 2, None, p, None, p, 1, 256, 1e-6, None) == 1002
+    attn = lib.vrl_rope_attn_decode_bf16
+    ok = dict(q=p, k=p, v=p, qs=256, ks=256, kc=p, vc=p, cos=p, sin=p, mask=p, pos=p, out=p,
+              M=1, H=4, Hkv=4, D=64, L=16, scale=0.125)
+
+    def call(**over):
+        a = dict(ok, **over)
+        return attn(a["q"], a["k"], a["v"], a["qs"], a["ks"], a["kc"], a["vc"], a["cos"], a["sin"], a["mask"],
+                    a["pos"], a["out"], a["M"], a["H"], a["Hkv"], a["D"], a["L"], a["scale"], None)
+
+    assert call(pos=None) == 1003 and call(mask=None) == 1003
+    assert call(D=96) == 1001 and call(Hkv=3) == 1001 and call(L=0) == 1001 and call(L=8193) == 1001
+    assert call(qs=128) == 1001          # rows narrower than the heads they hold
+    assert call(ks=260) == 1001          # row stride must keep rows 16-byte aligned
+    assert call(kc=p + 8) == 1002 and call(pos=p + 4) == 1002
 
 
 def test_cfg_sample_validation(lib):

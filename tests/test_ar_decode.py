@@ -170,12 +170,13 @@ def int4_policy():
 
 
 @pytest.mark.gpu
-def test_graph_replays_equal_eager_steps(int4_policy):
+@pytest.mark.parametrize("native", [False, True])
+def test_graph_replays_equal_eager_steps(int4_policy, native):
     """Every replayed step against the same step run eagerly: tokens and log-probabilities bit for bit,
     over two calls (the second reuses the recorded graph) with eager work and syncs in between."""
-    print("ar decode: graph vs eager", flush=True)
-    eager = StaticARSampler(int4_policy, graph=False)
-    graphed = StaticARSampler(int4_policy, graph=True)
+    print("ar decode: graph vs eager, native trunk", native, flush=True)
+    eager = StaticARSampler(int4_policy, graph=False, native=native)
+    graphed = StaticARSampler(int4_policy, graph=True, native=native)
     for call, (n_text, n_img, seed) in enumerate(((7, 24, 21), (11, 20, 22), (7, 24, 21))):
         cond, uncond, cmask, umask = make_inputs(3, n_text, torch.bfloat16, "cuda:0", seed=seed)
         torch.manual_seed(seed)
@@ -188,21 +189,84 @@ def test_graph_replays_equal_eager_steps(int4_policy):
         assert torch.equal(got_lp, want_lp), call
         assert len(want_t.unique()) > n_img // 2
     (sess,) = graphed._sessions.values()
-    assert sess.graph is not None
+    assert sess.graph is not None and bool(sess.native) == native
 
 
 @pytest.mark.gpu
 def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy):
     """Same int4 policy through the reference loop (dynamic cache, torch formulas for the tail):
-    same tokens under the same seed; log-probabilities within a bf16 rounding of the log-softmax."""
+    same tokens under the same seed; log-probabilities within a bf16 rounding of the log-softmax.
+    The trunk stays the module here (``native=False``): the native trunk agrees with it to bf16
+    roundings only, which the tests below bound."""
     print("ar decode: static fused vs reference loop", flush=True)
     cond, uncond, cmask, umask = make_inputs(3, 7, torch.bfloat16, "cuda:0")
     torch.manual_seed(31)
     want_t, want_lp = reference_loop(int4_policy, cond, uncond, cmask, umask, 5.0, 1.0, 16)
     for graph in (False, True):
         torch.manual_seed(31)
-        got_t, got_lp = StaticARSampler(int4_policy, graph=graph).sample_image_tokens(
+        got_t, got_lp = StaticARSampler(int4_policy, graph=graph, native=False).sample_image_tokens(
             cond, uncond, cmask, umask, image_token_num=16)
         torch.cuda.synchronize()
         assert torch.equal(got_t, want_t), (graph, got_t, want_t)
         torch.testing.assert_close(got_lp, want_lp, rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.gpu
+def test_native_trunk_tracks_the_module_trunk(int4_policy):
+    """Teacher-forced: both trunks consume the same inputs step after step, each over its own cache;
+    hidden states and appended cache rows stay within bf16 roundings of each other."""
+    print("ar decode: native trunk vs module trunk", flush=True)
+    rows, n_text, steps = 6, 7, 12
+    cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=41)
+    sessions = []
+    for native in (True, False):
+        sampler = StaticARSampler(int4_policy, graph=False, native=native)
+        torch.manual_seed(41)
+        sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=1)   # prompt pass only
+        (sess,) = sampler._sessions.values()
+        sessions.append((sampler, sess))
+    (_, nat), (_, mod) = sessions
+    assert nat.native and not mod.native
+    assert nat.native.launches == 7 * LAYERS + 1
+    trunk = int4_policy._lm_trunk()
+    gen = torch.Generator(device="cuda:0").manual_seed(42)
+    worst = 0.0
+    with torch.no_grad():
+        for t in range(steps):
+            emb = torch.randn((rows, 1, HIDDEN), generator=gen, device="cuda:0").to(torch.bfloat16)
+            nat.cur.copy_(emb)
+            got = nat.native.run().float().clone()
+            nat.slot.add_(1)
+            want = trunk(inputs_embeds=emb, attention_mask=mod.mask, use_cache=True,
+                         past_key_values=mod.cache).last_hidden_state[:, -1].float()
+            torch.cuda.synchronize()
+            err = (got - want).abs()
+            worst = max(worst, err.max().item())
+            # normalised hidden states are O(1): a few bf16 steps (2^-8 relative) through two layers
+            assert err.max().item() <= 0.08 and err.mean().item() <= 0.008, (t, err.max().item(), err.mean().item())
+    for layer_n, layer_m in zip(nat.cache.layers, mod.cache.layers):
+        for a, b in ((layer_n.keys, layer_m.keys), (layer_n.values, layer_m.values)):
+            a, b = a[:, :, :n_text + steps].float(), b[:, :, :n_text + steps].float()
+            assert torch.equal(a[:, :, :n_text], b[:, :, :n_text])                 # the prompt pass is shared code
+            assert (a - b).abs().max().item() <= 0.05 * b.abs().max().item()
+            assert (a[:, :, n_text + steps:] == 0).all()
+    print("ar decode: worst hidden-state difference", worst, flush=True)
+
+
+@pytest.mark.gpu
+def test_native_sampling_agrees_with_the_module_path_on_independent_draws(int4_policy):
+    """Two image tokens for 16 rows: the first comes from the shared prompt pass (identical), the
+    second from one decode step of either trunk under the same noise: draws flip only at near-ties."""
+    print("ar decode: native vs module sampling", flush=True)
+    cond, uncond, cmask, umask = make_inputs(16, 7, torch.bfloat16, "cuda:0", seed=51)
+    out = []
+    for native in (True, False):
+        torch.manual_seed(52)
+        out.append(StaticARSampler(int4_policy, graph=False, native=native).sample_image_tokens(
+            cond, uncond, cmask, umask, image_token_num=2))
+    torch.cuda.synchronize()
+    (t_n, lp_n), (t_m, lp_m) = out
+    assert torch.equal(t_n[:, 0], t_m[:, 0]) and torch.equal(lp_n[:, 0], lp_m[:, 0])
+    same = t_n[:, 1] == t_m[:, 1]
+    assert same.sum().item() >= 14, (t_n[:, 1], t_m[:, 1])
+    assert (lp_n[same, 1] - lp_m[same, 1]).abs().max().item() <= 0.25

@@ -328,3 +328,34 @@ def test_grouped_siblings_hand_results_over_by_tensor_identity():
     # more rows than the plan-free launch takes: every module on its own
     big = torch.randn(40, 512, device=dev).to(torch.bfloat16)
     assert torch.equal(q(big), alone[0](big)) and k._handed is None
+
+
+@pytest.mark.gpu
+def test_prompt_sized_calls_go_through_the_library_gemm():
+    """More than 32 rows (the prompt pass): bit-exact weight tile, then the library GEMM, for the plain
+    and the fused gate|up module, prepacked or not."""
+    import torch.nn.functional as F
+
+    dev = "cuda:0"
+    torch.manual_seed(4)
+    lin = nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev)
+    gate = nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev)
+    up = nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev)
+    x = torch.randn(4, 20, 512, device=dev).to(torch.bfloat16)   # 80 rows
+    q = Int4Linear.from_linear(lin, 128)
+    gu = Int4GateUpSiLU(Int4Linear.from_linear(gate, 128), Int4Linear.from_linear(up, 128))
+    for prepacked in (False, True):
+        if prepacked:
+            q.prepack_(), gu.prepack_()
+            assert q._packed is not None and gu._packed is not None
+        y = q(x)
+        assert torch.equal(y, F.linear(x, q.dequantize()))
+        from visionrl_amd import ops
+
+        w = ops.int4_dequant(gu.qweight, gu.scales, gu.qzeros, 128)
+        g, u = F.linear(x, w).chunk(2, dim=-1)
+        got = gu(x)
+        assert got.shape == (4, 20, 64) and torch.equal(got, F.silu(g) * u)
+        # and it stays within a bf16 rounding or two of the fused decode kernel's fp32 epilogue
+        small = gu(x[:1, :8])
+        assert (small.float() - got[:1, :8].float()).abs().max().item() <= 2.0 ** -6 * max(1.0, got.abs().max().item())

@@ -17,6 +17,10 @@ arguments, the same results and the same use of the random stream:
   write of token and log-probability at a device-side position) and replayed ``L_img - 2`` times.
   The prompt pass and the first decode step run eagerly (the latter doubles as the warm-up a
   capture needs).
+* When the trunk's projections are prepacked int4 modules, the trunk part of the step runs as
+  seven launches per layer over the same cache tensors (:mod:`visionrl_amd.decode_step`) instead
+  of the module's some thirty tensor ops per layer; results then agree with the module path to
+  bf16 roundings of the hidden states (the attention keeps fp32 probabilities), not bit for bit.
 * The tail after the head is one launch (:func:`visionrl_amd.ops.cfg_sample`) when the logits are
   bf16 on a GPU, and the reference's torch formulas otherwise; both draw through
   ``exponential_`` exactly as ``torch.multinomial`` does, so a seeded rollout
@@ -36,6 +40,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
+from .decode_step import NativeDecodeTrunk
 
 __all__ = ["StaticARSampler", "install_static_ar_sampler"]
 
@@ -62,6 +67,9 @@ class _Session:
         self.tokens = torch.zeros((rows2 // 2, max_len), dtype=torch.long, device=device)
         self.logprobs = torch.zeros((rows2 // 2, max_len), dtype=torch.float32, device=device)
         self.img_pos = torch.zeros(1, dtype=torch.long, device=device)
+        self.mask_u8 = torch.ones((rows2, max_len), dtype=torch.uint8, device=device)
+        self.slot = torch.zeros(1, dtype=torch.long, device=device)   # cache slot of the next new token
+        self.native = None     # NativeDecodeTrunk once the cache exists, False if the trunk does not qualify
         self.graph = None
 
     # -- one call of sample_image_tokens starts here
@@ -69,6 +77,8 @@ class _Session:
         self.cache.reset()
         self.mask.fill_(1)
         self.mask[:, :mask.shape[1]].copy_(mask)
+        self.mask_u8.copy_(self.mask != 0)
+        self.slot.fill_(mask.shape[1])
         self.img_pos.zero_()
 
     def tail(self, hidden: torch.Tensor) -> None:
@@ -93,11 +103,22 @@ class _Session:
         out = self.sampler.trunk(inputs_embeds=embeds, attention_mask=self.mask, use_cache=True,
                                  past_key_values=self.cache)
         self.tail(out.last_hidden_state[:, -1:, :])
+        if self.native is None:   # the cache tensors exist from here on
+            self.native = False
+            s = self.sampler
+            if s.native and self.cur.is_cuda and self.cur.dtype == torch.bfloat16 and \
+                    NativeDecodeTrunk.unsupported(s.trunk, self.rows2, self.max_len) is None:
+                self.native = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot)
 
     def step(self) -> None:
-        out = self.sampler.trunk(inputs_embeds=self.cur, attention_mask=self.mask, use_cache=True,
-                                 past_key_values=self.cache)
-        self.tail(out.last_hidden_state[:, -1:, :])
+        if self.native:
+            hidden = self.native.run().view(self.rows2, 1, -1)
+        else:
+            out = self.sampler.trunk(inputs_embeds=self.cur, attention_mask=self.mask, use_cache=True,
+                                     past_key_values=self.cache)
+            hidden = out.last_hidden_state[:, -1:, :]
+        self.tail(hidden)
+        self.slot.add_(1)
 
     def capture(self) -> None:
         graph = torch.cuda.CUDAGraph()
@@ -114,10 +135,13 @@ class StaticARSampler:
     ``prepare_gen_img_embeds`` (``policy.py:226-238``), ``config`` the defaults
     (``cfg_weight``, ``temperature``, ``image_token_num``).  ``graph=False`` runs every step
     eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
-    for the part after the head.
+    for the part after the head.  With ``native`` (the default) the trunk of a decode step runs as
+    :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (seven launches per layer) when the policy
+    went through ``apply_int4_to_policy`` with its defaults and carries no adapters; otherwise, and
+    for the prompt pass, the trunk module itself is called.
     """
 
-    def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True,
+    def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True, native: bool = True,
                  length_bucket: int = 64, max_sessions: int = 2):
         self.policy = policy
         self.trunk = policy._lm_trunk()
@@ -127,6 +151,7 @@ class StaticARSampler:
                 raise TypeError(f"policy._base() has no {name}")
         self.graph = bool(graph)
         self.fused_tail = bool(fused_tail)
+        self.native = bool(native)
         self.length_bucket = int(length_bucket)
         self.max_sessions = int(max_sessions)
         self._sessions: dict = {}

@@ -11,10 +11,15 @@ convention and route the arithmetic to the HIP library; the weights are frozen
 from __future__ import annotations
 
 import torch
+import torch.nn.functional as F
 from torch import nn
 
 from . import ops
 from .int4_format import check_packed, pack_nibbles, quantize_minmax
+
+# Calls with more activation rows than this (the prompt pass) rebuild the bf16 weight (bit-exact
+# tile, one launch) and hand the product to the library GEMM; the GEMV kernels are for decode.
+GEMM_ROWS = 32
 
 
 def _rows(x: torch.Tensor, in_features: int) -> torch.Tensor:
@@ -140,7 +145,10 @@ class Int4Linear(nn.Module):
                     packed = None
             else:
                 packed = None
-            if packed is None:
+            if packed is None and M > GEMM_ROWS:
+                # prompt-sized call: the GEMV kernels would stream the weight once per 16 rows
+                y = F.linear(rows, self.dequantize())
+            elif packed is None:
                 y = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=rows.device)
                 ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
         if self.bias is not None:
@@ -185,6 +193,10 @@ class Int4GateUpSiLU(nn.Module):
         if packed is not None and not torch.compiler.is_compiling() and rows.shape[0] <= self._direct_rows \
                 and packed.blob.device == rows.device:
             y = self._call(rows)[0]
+        elif rows.shape[0] > GEMM_ROWS and not torch.compiler.is_compiling():
+            w = ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
+            gate, up = F.linear(rows, w).chunk(2, dim=-1)   # prompt-sized call: one library GEMM
+            y = F.silu(gate) * up
         else:
             y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         return y.reshape(*x.shape[:-1], self.intermediate_size)
