@@ -392,8 +392,9 @@ def decode_tail(device, steps: int):
     return out
 
 
-def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16)):
-    """ms per image token of the whole decode loop on a Janus-Pro-1B shaped policy (random weights).
+def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16), prompt: int = 304):
+    """ms per decode step of the image-token loop on a Janus-Pro-1B shaped policy (random weights), at
+    cache lengths around the middle of a 576-token image (a 304-token context, then 48 tokens).
 
     ``reference_style`` is the loop of vrl/models/families/janus_pro/policy.py:624-731 with the trunk's
     dynamic cache and the torch formulas for the tail, without its per-row cache copies and host
@@ -455,14 +456,19 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
         return toks, lps
 
     def per_token_ms(fn):
-        fn()   # warm-up (and graph capture where there is one)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / tokens
+        """fn(n) samples n image tokens; the prompt pass and the first token are timed apart (n = 1)
+        and subtracted, so the figure is the cost of one decode step at cache lengths
+        prompt .. prompt + tokens."""
+        def timed(n):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn(n)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3
+        fn(tokens)   # warm-up (and graph capture where there is one)
+        return (timed(tokens) - min(timed(1), timed(1))) / (tokens - 1)
 
-    out = {"tokens_per_call": tokens, "prompt_tokens": 16,
+    out = {"tokens_per_call": tokens, "prompt_tokens": prompt,
            "model": "LlamaModel 24 x (2048, 5632), 16 heads, head 2048->16384, random weights"}
     with torch.device(device):
         torch.manual_seed(0)
@@ -472,17 +478,17 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
     inputs = {}
     for B in batches:
         g = torch.Generator(device=device).manual_seed(7000 + B)
-        inputs[B] = (torch.randn((B, 16, HIDDEN), generator=g, device=device).to(torch.bfloat16),
-                     torch.randn((B, 16, HIDDEN), generator=g, device=device).to(torch.bfloat16),
-                     torch.ones((B, 16), dtype=torch.long, device=device),
-                     torch.ones((B, 16), dtype=torch.long, device=device))
+        inputs[B] = (torch.randn((B, prompt, HIDDEN), generator=g, device=device).to(torch.bfloat16),
+                     torch.randn((B, prompt, HIDDEN), generator=g, device=device).to(torch.bfloat16),
+                     torch.ones((B, prompt), dtype=torch.long, device=device),
+                     torch.ones((B, prompt), dtype=torch.long, device=device))
     for B in batches if only is None else ():
         entry = out.setdefault(f"B{B}", {})
         entry["bf16_reference_style_ms_per_token"] = per_token_ms(
-            lambda: reference_style(policy, *inputs[B], tokens))
+            lambda n: reference_style(policy, *inputs[B], n))
         sampler = StaticARSampler(policy, graph=True, fused_tail=False, native=False)
         entry["bf16_static_hip_graph_ms_per_token"] = per_token_ms(
-            lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
+            lambda n: sampler.sample_image_tokens(*inputs[B], image_token_num=n))
         del sampler
         torch.cuda.empty_cache()
     apply_int4_to_policy(policy, group_size=GROUP)
@@ -491,14 +497,14 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
         entry = out.setdefault(f"B{B}", {})
         if only is None:
             entry["int4_reference_style_ms_per_token"] = per_token_ms(
-                lambda: reference_style(policy, *inputs[B], tokens))
+                lambda n: reference_style(policy, *inputs[B], n))
         for name, graph, native in (("int4_static_eager", False, False), ("int4_static_hip_graph", True, False),
                                     ("int4_native_eager", False, True), ("int4_native_hip_graph", True, True)):
             if only is not None and name != only:
                 continue
             sampler = StaticARSampler(policy, graph=graph, native=native)
             entry[f"{name}_ms_per_token"] = per_token_ms(
-                lambda: sampler.sample_image_tokens(*inputs[B], image_token_num=tokens))
+                lambda n: sampler.sample_image_tokens(*inputs[B], image_token_num=n))
             del sampler
             torch.cuda.empty_cache()
     return out

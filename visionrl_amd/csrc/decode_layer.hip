@@ -8,9 +8,9 @@
 //   h = bf16(residual + x);  normed = bf16(weight * bf16(h * rsqrt(mean(h^2) + eps)))
 //   q' = bf16(bf16(q * cos) + bf16(rotate_half(q) * sin)), same for k
 //   cache[p] = k', v;  out = bf16(softmax(q' . K^T * scaling, masked slots out) . V)
-// The attention keeps scores and probabilities in fp32 (the library kernel it stands for rounds
-// the probabilities to bf16 before the second product), so it agrees with it to a bf16 rounding
-// of the output, not bit for bit.
+// The attention keeps scores, probabilities and a running softmax in fp32 (the library kernel it
+// stands for rounds the probabilities to bf16 before the second product), so it agrees with it to
+// a bf16 rounding of the output, not bit for bit.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -123,39 +123,61 @@ struct AttnArgs {
     float scaling;
 };
 
+// Raw cache vectors: D / 16 bf16 values of one slot per lane (16 or 8 bytes).
 template <int VEC>
-__device__ __forceinline__ void load_bf16_vec(const uint16_t *p, float (&f)[VEC]) {
-    if (VEC == 8) {
-        const uint4 w = *reinterpret_cast<const uint4 *>(p);
-        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
-            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
-        }
+struct RawVec {
+    uint32_t w[VEC / 2];
+};
+
+template <int VEC>
+__device__ __forceinline__ RawVec<VEC> load_raw(const uint16_t *p) {
+    RawVec<VEC> r;
+    if constexpr (VEC == 8) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        r.w[0] = v.x, r.w[1] = v.y, r.w[2] = v.z, r.w[3] = v.w;
     } else {
-        const uint2 w = *reinterpret_cast<const uint2 *>(p);
-        const uint32_t u[2] = {w.x, w.y};
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
-            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
-        }
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        r.w[0] = v.x, r.w[1] = v.y;
     }
+    return r;
 }
 
-// One workgroup per (head, row).  Sixteen lanes share a cache slot (D / 16 values each), so a wave
-// reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the workgroup sixteen.
+// Running softmax state of a set of slots: their maximum score m, sum of exp(score - m), and
+// the exp-weighted sum of value rows (the lane's VEC columns of it).
+template <int VEC>
+struct Partial {
+    float m, l, acc[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const float (&acc2)[VEC]) {
+    const float m = fmaxf(a.m, m2);
+    const float ref = m == -INFINITY ? 0.0f : m;  // both empty: keep zeros, avoid inf - inf
+    const float c1 = __expf(a.m - ref), c2 = __expf(m2 - ref);
+    a.m = m;
+    a.l = a.l * c1 + l2 * c2;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) a.acc[i] = a.acc[i] * c1 + acc2[i] * c2;
+}
+
+constexpr int ATT_THREADS = 1024;
+constexpr int ATT_WAVES = ATT_THREADS / WAVE;
+constexpr int ATT_UNROLL = 4;  // slots per 16-lane group in flight (keys and values: 8 vector loads per lane)
+
+// One workgroup of 16 waves per (head, row).  Sixteen lanes share a cache slot (D / 16 values
+// each), so a wave reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the
+// workgroup 64.  Every 16-lane group keeps its own running softmax over the slots it visits
+// (key and value loads of ATT_UNROLL slots are issued together: values do not wait for scores);
+// the groups, the waves and the new token's own slot are merged at the end.
 template <int D>
-__global__ __launch_bounds__(THREADS) void rope_attn_decode_kernel(AttnArgs a) {
+__global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs a) {
     constexpr int VEC = D / 16;
-    extern __shared__ __align__(16) float smem[];
-    float *qs = smem;                // rotated query
-    float *ks = qs + D;              // rotated key of the new token
-    float *vs = ks + D;              // value of the new token
-    float *part = vs + D;            // WAVES x D partial outputs
-    float *red = part + WAVES * D;   // WAVES
-    float *sc = red + WAVES;         // scores, then probabilities, of slots 0..p
+    __shared__ float qs[D];                 // rotated query
+    __shared__ float ks[D];                 // rotated key of the new token
+    __shared__ float vs[D];                 // value of the new token
+    __shared__ float pm[ATT_WAVES], pl[ATT_WAVES];
+    __shared__ float pacc[ATT_WAVES][D];
+    __shared__ float s_new;                 // score of the new token's own slot
 
     const long long p64 = *a.position;
     if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the grid
@@ -192,73 +214,90 @@ __global__ __launch_bounds__(THREADS) void rope_attn_decode_kernel(AttnArgs a) {
     float qreg[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) qreg[i] = qs[l16 * VEC + i];
-    const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
-    const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
-
-    // scores of the cached slots 0..p-1
-#pragma unroll 4
-    for (int j0 = 0; j0 < p; j0 += 4 * WAVES) {
-        const int j = j0 + wave * 4 + sub;
-        const int jj = j < p ? j : p - 1;  // in range: the loop runs only when p >= 1
-        float kf[VEC];
-        load_bf16_vec<VEC>(kc + (long)jj * D, kf);
-        float dot = 0.0f;
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) dot += qreg[i] * kf[i];
-        dot += __shfl_xor(dot, 1, WAVE);
-        dot += __shfl_xor(dot, 2, WAVE);
-        dot += __shfl_xor(dot, 4, WAVE);
-        dot += __shfl_xor(dot, 8, WAVE);
-        if (l16 == 0 && j < p) sc[j] = mask[j] ? dot * a.scaling : -INFINITY;
-    }
     if (wave == 0) {  // the new token's own slot
         float dot = 0.0f;
         for (int d = lane; d < D; d += WAVE) dot += qs[d] * ks[d];
         dot = wave_sum(dot);
-        if (lane == 0) sc[p] = mask[p] ? dot * a.scaling : -INFINITY;
+        if (lane == 0) s_new = mask[p] ? dot * a.scaling : -INFINITY;
     }
-    __syncthreads();
+    const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
+    const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
 
-    float mx = -INFINITY;
-    for (int j = tid; j <= p; j += THREADS) mx = fmaxf(mx, sc[j]);
-    mx = block_reduce<true>(mx, red);
-    if (mx == -INFINITY) mx = 0.0f;  // every slot masked: probabilities and output become zero
-    float sum = 0.0f;
-    for (int j = tid; j <= p; j += THREADS) {  // each thread rewrites the entries it read
-        const float e = expf(sc[j] - mx);
-        sc[j] = e;
-        sum += e;
-    }
-    sum = block_reduce<false>(sum, red);  // its barriers also publish the probabilities
+    Partial<VEC> st;
+    st.m = -INFINITY;
+    st.l = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) st.acc[i] = 0.0f;
 
-    float acc[VEC];
+    // cached slots 0..p-1: slot j0 + u * 64 + wave * 4 + sub for u = 0..ATT_UNROLL-1
+    for (int j0 = 0; j0 < p; j0 += 4 * ATT_WAVES * ATT_UNROLL) {
+        RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
+        bool live[ATT_UNROLL];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
-#pragma unroll 4
-    for (int j0 = 0; j0 < p; j0 += 4 * WAVES) {
-        const int j = j0 + wave * 4 + sub;
-        const int jj = j < p ? j : p - 1;
-        float vf[VEC];
-        load_bf16_vec<VEC>(vc + (long)jj * D, vf);
-        const float w = j < p ? sc[jj] : 0.0f;
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const int j = j0 + u * 4 * ATT_WAVES + wave * 4 + sub;
+            const int jj = j < p ? j : p - 1;  // in range: the loop runs only when p >= 1
+            kraw[u] = load_raw<VEC>(kc + (long)jj * D);
+            vraw[u] = load_raw<VEC>(vc + (long)jj * D);
+            live[u] = j < p && mask[jj] != 0;
+        }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] += w * vf[i];
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < VEC / 2; ++i) {
+                dot += qreg[2 * i] * bf16_to_f32(kraw[u].w[i] & 0xFFFFu);
+                dot += qreg[2 * i + 1] * bf16_to_f32(kraw[u].w[i] >> 16);
+            }
+            dot += __shfl_xor(dot, 1, WAVE);
+            dot += __shfl_xor(dot, 2, WAVE);
+            dot += __shfl_xor(dot, 4, WAVE);
+            dot += __shfl_xor(dot, 8, WAVE);
+            const float s = live[u] ? dot * a.scaling : -INFINITY;
+            float vf[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC / 2; ++i) {
+                vf[2 * i] = bf16_to_f32(vraw[u].w[i] & 0xFFFFu);
+                vf[2 * i + 1] = bf16_to_f32(vraw[u].w[i] >> 16);
+            }
+            merge<VEC>(st, s, 1.0f, vf);
+        }
     }
+    // the four 16-lane groups of the wave
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        acc[i] += __shfl_xor(acc[i], 16, WAVE);
-        acc[i] += __shfl_xor(acc[i], 32, WAVE);
+    for (int off = 16; off <= 32; off <<= 1) {
+        const float m2 = __shfl_xor(st.m, off, WAVE), l2 = __shfl_xor(st.l, off, WAVE);
+        float acc2[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc2[i] = __shfl_xor(st.acc[i], off, WAVE);
+        merge<VEC>(st, m2, l2, acc2);
     }
     if (sub == 0) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) part[wave * D + l16 * VEC + i] = acc[i];
+        for (int i = 0; i < VEC; ++i) pacc[wave][l16 * VEC + i] = st.acc[i];
+    }
+    if (lane == 0) {
+        pm[wave] = st.m;
+        pl[wave] = st.l;
     }
     __syncthreads();
     if (tid < D) {
-        float o = sc[p] * vs[tid];
+        float mx = s_new;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) o += part[w * D + tid];
-        o = sum > 0.0f ? o / sum : 0.0f;
+        for (int w = 0; w < ATT_WAVES; ++w) mx = fmaxf(mx, pm[w]);
+        float o = 0.0f, sum = 0.0f;
+        if (mx != -INFINITY) {  // else every slot is masked: the output is zero
+            const float cn = __expf(s_new - mx);
+            o = cn * vs[tid];
+            sum = cn;
+#pragma unroll
+            for (int w = 0; w < ATT_WAVES; ++w) {
+                const float c = __expf(pm[w] - mx);
+                o += c * pacc[w][tid];
+                sum += c * pl[w];
+            }
+            o /= sum;
+        }
         a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)f32_to_bf16_bits(o);
     }
 }
@@ -320,10 +359,9 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
     a.L_max = L_max;
     a.scaling = scaling;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const size_t lds = (size_t)(3 * D + WAVES * D + WAVES + L_max) * sizeof(float);
     if (D == 128)
-        hipLaunchKernelGGL(rope_attn_decode_kernel<128>, dim3(n_heads, M), dim3(THREADS), lds, stream, a);
+        hipLaunchKernelGGL(rope_attn_decode_kernel<128>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
     else
-        hipLaunchKernelGGL(rope_attn_decode_kernel<64>, dim3(n_heads, M), dim3(THREADS), lds, stream, a);
+        hipLaunchKernelGGL(rope_attn_decode_kernel<64>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
     return (int)hipGetLastError();
 }
