@@ -149,6 +149,29 @@ typedef struct vrl_int4_plan_info {
  */
 int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream);
 
+/*
+ * The same launch with the residual add and the RMSNorm that precede the linears of a decoder
+ * layer applied to the activations on their way in (LlamaDecoderLayer.forward:
+ * `hidden_states = residual + hidden_states`, then input_layernorm / post_attention_layernorm,
+ * then q|k|v or gate|up; reached from policy.py:673-678):
+ *   h = residual ? bf16(x + residual) : x;   x' = weight * bf16(h * rsqrt(mean(h^2) + eps))
+ * and every problem multiplies x' (never written to memory) instead of x.  All problems share
+ * the input: problems[i].x == norm->x, same M and K, K <= 4096.  `h_out`, when not NULL,
+ * receives h ([M, K]); it must not be the memory of x or residual (workgroups read those
+ * while another one writes h).  Roundings are those of the tensor ops (see vrl_decode.h).
+ */
+typedef struct vrl_int4_norm {
+    const void *x;        /* bf16 [M, K]: output of the previous sublayer (or the embedding) */
+    const void *residual; /* bf16 [M, K] residual stream, NULL for none */
+    const void *weight;   /* bf16 [K] norm weight */
+    void *h_out;          /* bf16 [M, K] or NULL */
+    float eps;
+    int32_t reserved;
+} vrl_int4_norm;
+
+int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_problems,
+                                      const vrl_int4_norm *norm, void *hip_stream);
+
 size_t vrl_int4_grouped_plan_size(int n_problems);
 
 /* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems)) and *info. */

@@ -227,7 +227,7 @@ def test_native_trunk_tracks_the_module_trunk(int4_policy):
         sessions.append((sampler, sess))
     (_, nat), (_, mod) = sessions
     assert nat.native and not mod.native
-    assert nat.native.launches == 7 * LAYERS + 1
+    assert nat.native.launches == 5 * LAYERS + 1
     trunk = int4_policy._lm_trunk()
     gen = torch.Generator(device="cuda:0").manual_seed(42)
     worst = 0.0

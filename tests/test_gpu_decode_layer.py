@@ -153,3 +153,73 @@ def test_wrappers_reject_contract_violations(ops_mod):
         ops_mod.rope_attn_decode(*args, mask, pos.int(), 0.125)
     with pytest.raises(ValueError):
         ops_mod.rope_attn_decode(args[0][:, :100], *args[1:], mask, pos, 0.125)
+
+
+# ------------------------------------------------------------------ add + norm applied while the linears stage their input
+NORM_FUSED_CASES = [
+    # M, K, [N...], fused gate|up, residual
+    (1, 2048, [2048, 2048, 2048], False, True), (2, 2048, [2048, 512, 512], False, True),
+    (32, 2048, [2048, 2048, 2048], False, True), (2, 2048, [2 * 5632], True, True), (32, 2048, [2 * 704], True, True),
+    (3, 4096, [256], False, False), (5, 640, [48, 80], False, True), (16, 1536, [64], False, True),
+    (9, 2048, [100], False, False),
+]
+
+
+@pytest.mark.parametrize("M,K,Ns,fused,with_residual", NORM_FUSED_CASES)
+def test_norm_fused_launch_parity(ops_mod, M, K, Ns, fused, with_residual):
+    from tests._util import assert_gemv_close, to_device
+
+    say("norm-fused launch", M, K, Ns, fused, with_residual)
+    G = 128
+    rng = np.random.default_rng(7 * K + M)
+    x, res, wn = rand_bits(rng, (M, K)), rand_bits(rng, (M, K), 4.0), rand_bits(rng, (K,), 0.5)
+    h_want, xn = d.add_rmsnorm(x, res if with_residual else None, wn, 1e-6)
+    xt, rt, wt = bits_to_bf16(x, DEV), bits_to_bf16(res, DEV), bits_to_bf16(wn, DEV)
+    h_out = torch.zeros_like(xt)
+    probs, checks = [], []
+    for i, N in enumerate(Ns):
+        ops = o.make_operands(4000 + i + N, M, K, N, G)
+        ops["x_bits"] = xn                       # what the tiles must have multiplied
+        dd = to_device(ops, DEV)
+        probs.append((xt, ops_mod.int4_prepack(dd["qweight"], dd["scales"], dd["qzeros"], G), fused))
+        checks.append(ops)
+    outs = ops_mod.DirectGemv(probs, norm=(rt if with_residual else None, wt, 1e-6, h_out)).launch()
+    torch.cuda.synchronize()
+    assert (bf16_to_bits(h_out) == h_want).all()
+    for y, ops in zip(outs, checks):
+        if not fused:
+            assert_gemv_close(bf16_to_bits(y), ops, G, "norm-fused")
+            continue
+        ref = o.gate_up_silu_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+        got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
+        tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
+        assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all()
+    # against the two-launch form on the device: same h, outputs within a rounding of the normalised row
+    h2, normed = ops_mod.add_rmsnorm(xt, wt, 1e-6, rt if with_residual else None)
+    two = ops_mod.DirectGemv([(normed, pw, f) for _, pw, f in probs]).launch()
+    torch.cuda.synchronize()
+    assert torch.equal(h2, h_out)
+    for a, b in zip(outs, two):
+        close = (a.float() - b.float()).abs() <= 2.0 ** -6 * b.float().abs() + 2.0 ** -7
+        assert close.all() and (a != b).float().mean().item() < 0.02
+
+
+def test_norm_fused_launch_rejects(ops_mod):
+    G, M, K = 128, 2, 256
+    ops = o.make_operands(1, M, K, 32, G)
+    from tests._util import to_device
+    dd = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(dd["qweight"], dd["scales"], dd["qzeros"], G)
+    x, w = dd["x"], torch.ones(K, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(x, pw, False), (x.clone(), pw, False)], norm=(None, w, 1e-6, None))   # two inputs
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(x, pw, False)], norm=(None, w[:128], 1e-6, None))
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(x, pw, False)], norm=(None, w, 1e-6, x)).launch()                     # h over x
+    big = o.make_operands(2, 1, 8192, 16, G)
+    db = to_device(big, DEV)
+    pwb = ops_mod.int4_prepack(db["qweight"], db["scales"], db["qzeros"], G)
+    with pytest.raises(ValueError):
+        ops_mod.DirectGemv([(db["x"], pwb, False)],
+                           norm=(None, torch.ones(8192, dtype=torch.bfloat16, device=DEV), 1e-6, None)).launch()

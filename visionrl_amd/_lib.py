@@ -24,6 +24,7 @@ SYMBOLS = (
     "vrl_int4_prepacked_bytes",
     "vrl_int4_prepack",
     "vrl_int4_gemv_prepacked_bf16",
+    "vrl_int4_gemv_prepacked_norm_bf16",
     "vrl_int4_grouped_plan_size",
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
@@ -53,6 +54,19 @@ class Problem(ctypes.Structure):
         ("fused_gate_up", ctypes.c_int32),
         ("prepacked", ctypes.c_int32),
         ("reserved", ctypes.c_int32 * 2),
+    ]
+
+
+class Norm(ctypes.Structure):
+    """Mirror of ``vrl_int4_norm``."""
+
+    _fields_ = [
+        ("x", ctypes.c_void_p),
+        ("residual", ctypes.c_void_p),
+        ("weight", ctypes.c_void_p),
+        ("h_out", ctypes.c_void_p),
+        ("eps", ctypes.c_float),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -92,6 +106,8 @@ def _bind(lib):
     lib.vrl_int4_prepack.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     lib.vrl_int4_gemv_prepacked_bf16.restype = ci
     lib.vrl_int4_gemv_prepacked_bf16.argtypes = [ctypes.POINTER(Problem), ci, vp]
+    lib.vrl_int4_gemv_prepacked_norm_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_norm_bf16.argtypes = [ctypes.POINTER(Problem), ci, ctypes.POINTER(Norm), vp]
     lib.vrl_int4_grouped_plan_size.restype = ctypes.c_size_t
     lib.vrl_int4_grouped_plan_size.argtypes = [ci]
     lib.vrl_int4_grouped_plan_build.restype = ci

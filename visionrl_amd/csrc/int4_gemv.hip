@@ -318,9 +318,9 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int KS, int TW>
+template <bool FUSED, int KS, int TW, bool NORM>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
-    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW>;
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM>;
     if (lds > 64 * 1024) {
         static bool raised = false;  // per instantiation; the attribute is a property of the function
         if (!raised) {
@@ -334,13 +334,13 @@ int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_
     return (int)hipGetLastError();
 }
 
-template <bool FUSED>
+template <bool FUSED, bool NORM>
 int launch_direct_shape(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
-    if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1>(args, workgroups, lds, stream);
-    if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4>(args, workgroups, lds, stream);
-    if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1>(args, workgroups, lds, stream);
-    if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2>(args, workgroups, lds, stream);
-    if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1, NORM>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4, NORM>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1, NORM>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2, NORM>(args, workgroups, lds, stream);
+    if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1, NORM>(args, workgroups, lds, stream);
     return VRL_INT4_EPLAN;
 }
 
@@ -439,7 +439,8 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     return (int)hipGetLastError();
 }
 
-int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {
+static int direct_launch(const vrl_int4_problem *problems, int n_problems, const vrl_int4_norm *norm,
+                         void *hip_stream) {
     if (!problems) return VRL_INT4_ENULL;
     if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
     bool fused_any = false;
@@ -463,6 +464,24 @@ int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problem
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
     memset(&args, 0, sizeof args);
+    if (norm) {
+        // one normalised input for every problem of the launch: same rows, same K, x is the un-normed tensor
+        const vrl_int4_problem &q0 = problems[0];
+        if (!norm->x || !norm->weight) return VRL_INT4_ENULL;
+        if (q0.K > NORM_MAX_K || !(norm->eps >= 0.0f)) return VRL_INT4_ESHAPE;
+        for (int i = 0; i < n_problems; ++i)
+            if (problems[i].x != norm->x || problems[i].M != q0.M || problems[i].K != q0.K) return VRL_INT4_ESHAPE;
+        if (norm->h_out && (norm->h_out == norm->x || norm->h_out == norm->residual)) return VRL_INT4_ESHAPE;
+        if ((reinterpret_cast<uintptr_t>(norm->residual) | reinterpret_cast<uintptr_t>(norm->weight) |
+             reinterpret_cast<uintptr_t>(norm->h_out)) & 15u)
+            return VRL_INT4_EALIGN;
+        args.norm.x0 = static_cast<const uint16_t *>(norm->x);
+        args.norm.residual = static_cast<const uint16_t *>(norm->residual);
+        args.norm.weight = static_cast<const uint16_t *>(norm->weight);
+        args.norm.h_out = static_cast<uint16_t *>(norm->h_out);
+        args.norm.eps = norm->eps;
+        args.norm.enabled = 1;
+    }
     long workgroups = 0;
     size_t x_bytes = 0;
     for (int i = 0; i < n_problems; ++i) {
@@ -483,7 +502,7 @@ int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problem
             p.M = std::min<int>((int)rows, q.M - m0);
             p.N = q.N; p.K = q.K; p.G = q.G;
             p.fused = q.fused_gate_up ? 1 : 0;
-            p.prepacked = 1;
+            p.prepacked = 1 | (norm && i == 0 ? PP_WRITE_H : 0);  // the first problem's slabs write h
             p.kc = kc;
             p.tile_begin = (int)workgroups;  // first workgroup of the record
             workgroups += (tiles + tw - 1) / tw;
@@ -503,8 +522,21 @@ int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problem
     }
     const size_t lds = xz_bytes + red;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    return fused_any ? launch_direct_shape<true>(args, ks, tw, (int)workgroups, lds, stream)
-                     : launch_direct_shape<false>(args, ks, tw, (int)workgroups, lds, stream);
+    if (norm)
+        return fused_any ? launch_direct_shape<true, true>(args, ks, tw, (int)workgroups, lds, stream)
+                         : launch_direct_shape<false, true>(args, ks, tw, (int)workgroups, lds, stream);
+    return fused_any ? launch_direct_shape<true, false>(args, ks, tw, (int)workgroups, lds, stream)
+                     : launch_direct_shape<false, false>(args, ks, tw, (int)workgroups, lds, stream);
+}
+
+int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {
+    return direct_launch(problems, n_problems, nullptr, hip_stream);
+}
+
+int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_problems,
+                                      const vrl_int4_norm *norm, void *hip_stream) {
+    if (!norm) return VRL_INT4_ENULL;
+    return direct_launch(problems, n_problems, norm, hip_stream);
 }
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {

@@ -118,6 +118,105 @@ __device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int
     }
 }
 
+// Residual add and RMSNorm applied while the activations are staged (plan-free launches only):
+// the record's x points into `x0`, a sublayer output; what the tiles multiply is
+//   weight * bf16(h * rsqrt(mean(h^2) + eps)),  h = residual ? bf16(x + residual) : x
+// with the roundings LlamaDecoderLayer.forward / LlamaRMSNorm.forward apply to bf16 tensors.
+// Every workgroup normalises the rows it stages (one wave per row, the row kept in registers);
+// the first workgroup of a record flagged PP_WRITE_H also writes h to `h_out`.
+struct NormArgs {
+    const uint16_t *x0;        // base of the activation tensor the records' x point into
+    const uint16_t *residual;  // same shape as x0, or nullptr
+    const uint16_t *weight;    // [K]
+    uint16_t *h_out;           // same shape as x0, or nullptr; never the memory of x0 or residual
+    float eps;
+    int32_t enabled;
+};
+constexpr int PP_WRITE_H = 4;       // DevProblem::prepacked bit
+constexpr int NORM_MAX_K = 4096;    // eight 16-byte words per lane hold a row
+
+template <int NW>  // 16-byte words per lane that hold a row: K <= NW * 512
+__device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
+                                                  int xstride, int nwaves, bool write_h) {
+    typedef __attribute__((address_space(1))) u32x4_t *gptr_w4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int nthreads = nwaves * WAVE;
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+    // k beyond K reads as zero; so does the row behind the activation rows if the record has one
+    const int padw = (kext - p.K) >> 3;
+    for (int idx = threadIdx.x; idx < p.M * padw; idx += nthreads) {
+        const int m = idx / padw;
+        *reinterpret_cast<u32x4_t *>(xs + m * xstride + p.K + ((idx - m * padw) << 3)) = zero;
+    }
+    if (p.prepacked & PP_ZERO_ROW)
+        for (int j = threadIdx.x; j < (kext >> 3); j += nthreads)
+            *reinterpret_cast<u32x4_t *>(xs + p.M * xstride + (j << 3)) = zero;
+    const long base = p.x - n.x0;
+    const float inv_k = 1.0f / (float)p.K;
+    for (int m = wave; m < p.M; m += nwaves) {
+        const long row = base + (long)m * p.K;
+        u32x4_t h[NW], rv[NW], wv[NW];
+        // one memory round trip: the row, its residual and the norm weight are requested together
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            const int k = (i * WAVE + lane) << 3;
+            h[i] = rv[i] = wv[i] = zero;
+            if (k < p.K) {
+                h[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.x0 + row + k));
+                if (n.residual) rv[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.residual + row + k));
+                wv[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.weight + k));
+            }
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            const int k = (i * WAVE + lane) << 3;
+            if (k < p.K) {
+                if (n.residual) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        h[i][e] = pack_bf16_rne(
+                            bf16_bits_to_f32(rv[i][e] & 0xFFFFu) + bf16_bits_to_f32(h[i][e] & 0xFFFFu),
+                            bf16_bits_to_f32(rv[i][e] >> 16) + bf16_bits_to_f32(h[i][e] >> 16));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float lo = bf16_bits_to_f32(h[i][e] & 0xFFFFu), hi = bf16_bits_to_f32(h[i][e] >> 16);
+                    ss += lo * lo;
+                    ss += hi * hi;
+                }
+                if (write_h) *(gptr_w4)(uintptr_t)(n.h_out + row + k) = h[i];
+            }
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE);
+        const float r = rsqrtf(ss * inv_k + n.eps);
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            const int k = (i * WAVE + lane) << 3;
+            if (k < p.K) {
+                u32x4_t y;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t xn = pack_bf16_rne(bf16_bits_to_f32(h[i][e] & 0xFFFFu) * r,
+                                                      bf16_bits_to_f32(h[i][e] >> 16) * r);
+                    y[e] = pack_bf16_rne(bf16_bits_to_f32(wv[i][e] & 0xFFFFu) * bf16_bits_to_f32(xn & 0xFFFFu),
+                                         bf16_bits_to_f32(wv[i][e] >> 16) * bf16_bits_to_f32(xn >> 16));
+                }
+                *reinterpret_cast<u32x4_t *>(xs + m * xstride + k) = y;
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void stage_x_norm(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
+                                             int xstride, int nwaves, bool write_h) {
+    // rows up to 2048 wide keep half the registers (the 16-wave workgroups have 128 per lane)
+    if (p.K <= NORM_MAX_K / 2) stage_x_norm_rows<NORM_MAX_K / (16 * WAVE)>(p, n, kext, xs, xstride, nwaves, write_h);
+    else stage_x_norm_rows<NORM_MAX_K / (8 * WAVE)>(p, n, kext, xs, xstride, nwaves, write_h);
+}
+
 struct PPGroup {
     bf16x4_t bdiag;  // B operand of the 4x4x4 product: scale at k' = lane % 4, zero elsewhere
     f32x4_t cq;      // C operand: -(128 + z) * scale in all four rows
@@ -406,8 +505,9 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // o_proj, ...).  A workgroup carries TW such tiles at once (KS * TW waves), so that one
 // staging of the activations serves TW tiles: that matters once x is tens of KB (8+ rows).
 // LDS: staged activations, then TW x (KS - 1) x RS partial tiles.
-template <bool FUSED, int KS, int TW, int GQ>
-__device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+template <bool FUSED, int KS, int TW, int GQ, bool NORM>
+__device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
+                                                 const NormArgs &norm) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tw = wave / KS, kw = wave % KS;  // tile of the round, share of K
@@ -426,7 +526,11 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, work ? tile : t0, sc0);
     if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
     __syncthreads();
-    stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
+    if constexpr (NORM)
+        stage_x_norm(p, norm, nsc * PP_SC, xs, xstride, KS * TW,
+                     t0 == 0 && (p.prepacked & PP_WRITE_H) && norm.h_out != nullptr);
+    else
+        stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
     __syncthreads();
     for (int base = t0; base < t1; base += TW) {
         tile = base + tw;
@@ -456,16 +560,17 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 }
 
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
-template <bool FUSED, int KS, int TW>
-__device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+template <bool FUSED, int KS, int TW, bool NORM>
+__device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem,
+                                               const NormArgs &norm) {
     if (FUSED && p.fused) {
-        if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1>(p, t0, t1, smem);
-        else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2>(p, t0, t1, smem);
-        else split_segment_pp<FUSED, KS, TW, 4>(p, t0, t1, smem);
+        if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1, NORM>(p, t0, t1, smem, norm);
+        else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM>(p, t0, t1, smem, norm);
+        else split_segment_pp<FUSED, KS, TW, 4, NORM>(p, t0, t1, smem, norm);
     } else {
-        if (p.G == 128) split_segment_pp<false, KS, TW, 1>(p, t0, t1, smem);
-        else if (p.G == 64) split_segment_pp<false, KS, TW, 2>(p, t0, t1, smem);
-        else split_segment_pp<false, KS, TW, 4>(p, t0, t1, smem);
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM>(p, t0, t1, smem, norm);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM>(p, t0, t1, smem, norm);
+        else split_segment_pp<false, KS, TW, 4, NORM>(p, t0, t1, smem, norm);
     }
 }
 
@@ -483,7 +588,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
-        split_by_group<FUSED, WPB, 1>(p, a, b, smem);
+        split_by_group<FUSED, WPB, 1, false>(p, a, b, smem, NormArgs{});
         t = seg_end;
     }
 }
@@ -498,9 +603,10 @@ struct DirectArgs {
     int32_t n;
     int32_t pad;
     DevProblem recs[DIRECT_MAX];  // tile_begin holds the record's first workgroup here
+    NormArgs norm;                // read by the NORM instantiations only
 };
 
-template <bool FUSED, int KS, int TW>
+template <bool FUSED, int KS, int TW, bool NORM>
 __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int g = blockIdx.x;
@@ -510,7 +616,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
     const int t0 = (g - p.tile_begin) * TW;
-    split_by_group<FUSED, KS, TW>(p, t0, min(tiles, t0 + TW), smem);
+    split_by_group<FUSED, KS, TW, NORM>(p, t0, min(tiles, t0 + TW), smem, a.norm);
 }
 
 }  // namespace

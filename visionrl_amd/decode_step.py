@@ -4,12 +4,14 @@ The trunk call of a decode step (``vrl/models/families/janus_pro/policy.py:673-6
 Hugging Face ``LlamaModel`` on one new token per row: per layer some thirty small tensor ops
 between the seven linears (norm in four ops, rotary in eight, cache update, mask building,
 attention, residual adds).  At decode sizes every one of them is a launch that costs more than
-the arithmetic in it.  :class:`NativeDecodeTrunk` runs the same layer as seven launches:
+the arithmetic in it.  :class:`NativeDecodeTrunk` runs the same layer as five launches:
 
-    add + RMSNorm -> q|k|v (one int4 launch) -> rotary + cache append + attention -> o_proj
-    -> add + RMSNorm -> gate|up + SiLU (one int4 launch) -> down_proj
+    [add + RMSNorm ->] q|k|v (one int4 launch) -> rotary + cache append + attention -> o_proj
+    -> [add + RMSNorm ->] gate|up + SiLU (one int4 launch) -> down_proj
 
-with the residual add of the previous sublayer folded into the next norm, over the same
+where the residual add of the previous sublayer and the norm are applied by the int4 launch that
+follows them while it stages its input (for hidden sizes up to 4096; a launch of their own
+otherwise), over the same
 ``StaticCache`` tensors the prompt pass filled (``[rows, kv_heads, L_max, head_dim]``), the cache
 slot of the new token held in device memory, and every buffer preallocated, so that the whole
 step can be recorded as one HIP graph.  Arithmetic follows the library's roundings (each tensor
@@ -21,6 +23,8 @@ says why a trunk does not qualify, and callers then keep the module path.
 """
 
 from __future__ import annotations
+
+import ctypes
 
 import torch
 
@@ -99,33 +103,52 @@ class NativeDecodeTrunk:
             cos, sin = trunk.rotary_emb(cur, position_ids=torch.arange(self.max_len, device=dev)[None])
         self.cos, self.sin = cos[0].contiguous(), sin[0].contiguous()
         new = lambda n: torch.empty((rows, n), dtype=torch.bfloat16, device=dev)
-        self.h, self.normed, self.attn = new(hidden), new(hidden), new(H * D)
-        self._keep = [cache, cur, mask, slot]
+        # the residual stream alternates between two buffers: a launch that adds to it reads one and
+        # writes the other (its workgroups read the old stream while one of them writes the new one)
+        streams = [new(hidden), new(hidden)]
+        self.normed, self.attn = new(hidden), new(H * D)
+        self._keep = [cache, cur, mask, slot, streams]
         lib = _lib.load()
-        x2d = cur.view(rows, hidden)
-        calls = []   # (function, argument tuple without the stream)
-        pending = None   # output of the previous sublayer, still to be added to the residual stream
+        fuse_norm = hidden <= 4096   # the linears normalise their input while staging it
+        calls = []       # (function, argument tuple without the stream)
+        state = {"x": cur.view(rows, hidden), "res": None, "flip": 0}   # x: sublayer output not yet added to res
 
-        def norm(module, x, residual):
+        def norm_weight(module):
             w = module.weight.data
-            if w.dtype != torch.bfloat16 or tuple(w.shape) != (hidden,):
-                raise TypeError("norm weights must be bfloat16 [hidden]")
+            if w.dtype != torch.bfloat16 or tuple(w.shape) != (hidden,) or not w.is_contiguous():
+                raise TypeError("norm weights must be contiguous bfloat16 [hidden]")
             self._keep.append(w)
-            calls.append((lib.vrl_add_rmsnorm_bf16, (x.data_ptr(), residual.data_ptr() if residual is not None else None,
-                                                     w.data_ptr(), self.h.data_ptr(), self.normed.data_ptr(),
-                                                     rows, hidden, float(module.variance_epsilon))))
+            return w, float(module.variance_epsilon)
 
-        def gemv(problems):
-            launch = ops.DirectGemv(problems)
+        def gemv(problems, norm=None):
+            launch = ops.DirectGemv(problems, norm=norm)
             self._keep.append(launch)
-            calls.append((lib.vrl_int4_gemv_prepacked_bf16, (launch.table, len(launch.table))))
+            if norm is None:
+                calls.append((lib.vrl_int4_gemv_prepacked_bf16, (launch.table, len(launch.table))))
+            else:
+                calls.append((lib.vrl_int4_gemv_prepacked_norm_bf16,
+                              (launch.table, len(launch.table), ctypes.byref(launch.norm))))
             return launch.outputs
+
+        def normed_gemv(module, weights, fused):
+            """h = res + x; the linears over norm(h); afterwards res = h."""
+            w, eps = norm_weight(module)
+            h_out = streams[state["flip"]]
+            state["flip"] ^= 1
+            if fuse_norm:
+                outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
+            else:
+                calls.append((lib.vrl_add_rmsnorm_bf16,
+                              (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,
+                               w.data_ptr(), h_out.data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+                outs = gemv([(self.normed, pw, fused) for pw in weights])
+            state["res"] = h_out
+            return outs
 
         for i, layer in enumerate(trunk.layers):
             attn, mlp = layer.self_attn, layer.mlp
-            norm(layer.input_layernorm, x2d if pending is None else pending, None if pending is None else self.h)
-            q, k, v = gemv([(self.normed, attn.q_proj._packed, False), (self.normed, attn.k_proj._packed, False),
-                            (self.normed, attn.v_proj._packed, False)])
+            q, k, v = normed_gemv(layer.input_layernorm,
+                                  [attn.q_proj._packed, attn.k_proj._packed, attn.v_proj._packed], False)
             if q.shape[1] != H * D or k.shape[1] != Hkv * D or v.shape[1] != Hkv * D:
                 raise TypeError(f"layers[{i}] projections do not match the attention geometry")
             keys, values = cache.layers[i].keys, cache.layers[i].values
@@ -137,11 +160,13 @@ class NativeDecodeTrunk:
                            values.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), mask.data_ptr(),
                            slot.data_ptr(), self.attn.data_ptr(), rows, H, Hkv, D, self.max_len,
                            float(attn.scaling))))
-            (o,) = gemv([(self.attn, attn.o_proj._packed, False)])
-            norm(layer.post_attention_layernorm, o, self.h)
-            (act,) = gemv([(self.normed, mlp.gate_up._packed, True)])
-            (pending,) = gemv([(act, mlp.down_proj._packed, False)])
-        norm(trunk.norm, pending, self.h)
+            (state["x"],) = gemv([(self.attn, attn.o_proj._packed, False)])
+            (act,) = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
+            (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])
+        w, eps = norm_weight(trunk.norm)
+        calls.append((lib.vrl_add_rmsnorm_bf16,
+                      (state["x"].data_ptr(), state["res"].data_ptr(), w.data_ptr(),
+                       streams[state["flip"]].data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
         self._calls = calls
         self.launches = len(calls)
 

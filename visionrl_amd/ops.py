@@ -319,9 +319,10 @@ class DirectGemv:
     MAX_ROWS = 32
     MAX_RECORDS = 8   # row slabs of all problems of one launch
 
-    def __init__(self, problems, outputs=None):
+    def __init__(self, problems, outputs=None, norm=None):
         if not 1 <= len(problems) <= self.MAX_PROBLEMS:
             raise ValueError(f"DirectGemv takes 1 to {self.MAX_PROBLEMS} problems")
+        self.norm = None
         self._keep = []
         self.outputs = []
         self.table = (_lib.Problem * len(problems))()
@@ -355,11 +356,40 @@ class DirectGemv:
             rec.M, rec.N, rec.K, rec.G = x.shape[0], pw.N, pw.K, pw.group_size
             rec.fused_gate_up, rec.prepacked = (1 if fused else 0), 1
         self.device = dev
+        if norm is not None:
+            self._set_norm(problems, *norm)
+
+    def _set_norm(self, problems, residual, weight, eps, h_out):
+        """``norm=(residual | None, weight, eps, h_out | None)``: every problem then multiplies
+        ``weight * rmsnorm(x + residual)`` instead of its ``x`` (the same tensor for all of them), the
+        add and norm of ``LlamaDecoderLayer.forward`` in front of q|k|v or gate|up; ``h_out``
+        receives ``x + residual`` and must be a buffer of its own."""
+        x = problems[0][0]
+        if any(prob[0] is not x for prob in problems):
+            raise ValueError("a normalised launch takes one input tensor for all its problems")
+        if weight.dtype != torch.bfloat16 or tuple(weight.shape) != (x.shape[1],) or not weight.is_contiguous():
+            raise ValueError(f"norm weight must be contiguous bfloat16 [{x.shape[1]}]")
+        _require_device("norm weight", weight, self.device)
+        for name, t in (("residual", residual), ("h_out", h_out)):
+            if t is not None:
+                if t.dtype != torch.bfloat16 or t.shape != x.shape or not t.is_contiguous():
+                    raise ValueError(f"{name} must be contiguous bfloat16 {tuple(x.shape)}")
+                _require_device(name, t, self.device)
+        rec = _lib.Norm()
+        rec.x, rec.weight, rec.eps = x.data_ptr(), weight.data_ptr(), float(eps)
+        rec.residual = residual.data_ptr() if residual is not None else None
+        rec.h_out = h_out.data_ptr() if h_out is not None else None
+        self.norm = rec
+        self._keep.append((residual, weight, h_out))
 
     def launch(self):
         lib = _lib.load()
         with _on(self.device):
-            rc = lib.vrl_int4_gemv_prepacked_bf16(self.table, len(self.table), _stream_handle(self.device))
+            if self.norm is not None:
+                rc = lib.vrl_int4_gemv_prepacked_norm_bf16(self.table, len(self.table), ctypes.byref(self.norm),
+                                                           _stream_handle(self.device))
+            else:
+                rc = lib.vrl_int4_gemv_prepacked_bf16(self.table, len(self.table), _stream_handle(self.device))
         _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
         return self.outputs
 
