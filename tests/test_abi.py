@@ -168,6 +168,38 @@ def test_direct_prepacked_validation(lib):
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
 
 
+def test_norm_fused_launch_validation(lib):
+    keep, p = buf(1 << 16)
+    probs = (_lib.Problem * 2)()
+    for rec in probs:
+        rec.x = rec.qweight = rec.y = p
+        rec.M, rec.N, rec.K, rec.G, rec.prepacked = 1, 64, 256, 128, 1
+    norm = _lib.Norm()
+    norm.x, norm.weight, norm.eps = p, p, 1e-6
+    f = lib.vrl_int4_gemv_prepacked_norm_bf16
+    assert f(probs, 2, None, None) == 1003
+    norm.weight = None
+    assert f(probs, 2, ctypes.byref(norm), None) == 1003
+    norm.weight = p
+    probs[1].x = p + 512                      # every problem reads the one normalised input
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+    probs[1].x, probs[1].M = p, 2             # ... with the same rows
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+    probs[1].M = 1
+    norm.h_out = p                            # h may not overwrite what other workgroups still read
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+    norm.h_out, norm.residual = p + 4096, p + 4096
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+    norm.h_out, norm.residual = None, p + 8
+    assert f(probs, 2, ctypes.byref(norm), None) == 1002
+    norm.residual, norm.eps = None, -1.0
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+    norm.eps = 1e-6
+    for rec in probs:
+        rec.K = 8192                          # a row must fit the registers of one wave
+    assert f(probs, 2, ctypes.byref(norm), None) == 1001
+
+
 def test_decode_layer_validation(lib):
     keep, p = buf(1 << 16)
     norm = lib.vrl_add_rmsnorm_bf16
