@@ -58,6 +58,34 @@ int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q
                               int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
                               void *hip_stream);
 
+/*
+ * LoRA adapters on top of an int4 projection, for the decode step of a policy whose attention
+ * projections carry PEFT adapters (vrl/models/families/janus_pro/policy.py:298-324: rank 32 on
+ * q/k/v/o by default, policy.py:81-88); the wrapper computes
+ *   result = base_layer(x) + lora_B(lora_A(x)) * scaling
+ * Two launches per group of projections that share an input x [M, K] (bf16, M <= 32):
+ *   vrl_lora_down_bf16:    t[m, off_i + j] = sum_k x[m,k] * A_i[j,k]         for every adapter i
+ *   vrl_lora_up_add_bf16:  y_i[m,n] = bf16( y_i[m,n] + scaling_i * sum_j t[m, off_i + j] * B_i[n,j] )
+ * with t a float32 [M, r_total] scratch buffer of the caller's, off_i the sum of the ranks before
+ * adapter i.  Adapter weights are float32 (what PEFT keeps by default: everything in fp32, one
+ * rounding when the result returns to bf16) or bf16 (weights_fp32 = 0: t, the up-projection and its
+ * scaled value are rounded to bf16 as the bf16 modules round them).  1 <= n_adapters <= 4,
+ * r <= 256, r_total <= 512, K % 8 == 0, pointers 16-byte aligned.
+ */
+typedef struct vrl_lora_adapter {
+    const void *A;     /* [r, K] row-major */
+    const void *B;     /* [N, r] row-major */
+    void *y;           /* bf16 [M, N], updated in place by vrl_lora_up_add_bf16 */
+    int32_t N, r;
+    float scaling;
+    int32_t weights_fp32;
+} vrl_lora_adapter;
+
+int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adapters, int n_adapters,
+                       float *t, void *hip_stream);
+int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
+                         void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

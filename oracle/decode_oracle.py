@@ -91,3 +91,27 @@ def rope_attn_decode(q_bits, k_bits, v_bits, k_cache_bits, v_cache_bits, cos_bit
         e = np.exp(s)
         out[:, h] = np.einsum("ml,mld->md", e / e.sum(axis=-1, keepdims=True), vf[:, hk])
     return out.reshape(M, n_heads * D), kc, vc
+
+
+def lora_add(y_bits, x_bits, A, B, scaling: float, weights_fp32: bool):
+    """``result = base + lora_B(lora_A(x)) * scaling`` of a PEFT LoRA wrapper, bf16 bits out.
+
+    ``peft`` is not part of the reference tree (named only in an error message,
+    ``vrl/models/families/janus_pro/policy.py:301-306``, ">=0.12"); this restates its published
+    ``lora.Linear.forward``: with float32 adapter weights (its default, ``autocast_adapter_dtype``)
+    the input is upcast, both products, the scaling and the sum with the bf16 base output are
+    float32 and the result is rounded to bf16 once; with bf16 adapter weights every module output
+    (``lora_A(x)``, ``lora_B(.)``, ``* scaling``, the sum) is rounded to bf16.  ``A [r, K]`` and
+    ``B [N, r]`` are float arrays holding the weights' values.  Sums are float64 here.
+    """
+    x = bf16_bits_to_f32(x_bits).astype(np.float64)
+    y = bf16_bits_to_f32(y_bits).astype(np.float64)
+    t = x @ np.asarray(A, dtype=np.float64).T
+    if not weights_fp32:
+        t = _rnd(t).astype(np.float64)
+    u = t @ np.asarray(B, dtype=np.float64).T
+    if weights_fp32:
+        delta = u * float(np.float32(scaling))
+    else:
+        delta = _rnd(_rnd(u).astype(np.float64) * float(np.float32(scaling))).astype(np.float64)
+    return f32_to_bf16_bits((y + delta).astype(np.float32))

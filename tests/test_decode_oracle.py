@@ -22,6 +22,15 @@ def ulp_distance(a_bits, b_bits):
     return np.abs(key(a_bits) - key(b_bits))
 
 
+def within_one_step_of(got_bits, want_bits, operand_bits):
+    """|got - want| <= one bf16 step at the magnitude of the larger of result and operand (a sum that
+    cancels is only as exact as its operands' steps); returns the fraction of differing elements."""
+    got, want = o.bf16_bits_to_f32(got_bits).astype(np.float64), o.bf16_bits_to_f32(want_bits).astype(np.float64)
+    ref = np.maximum(np.abs(want), np.abs(o.bf16_bits_to_f32(operand_bits).astype(np.float64)))
+    assert (np.abs(got - want) <= o.bf16_ulp(ref.astype(np.float32))).all(), np.abs(got - want).max()
+    return float((got_bits != want_bits).mean())
+
+
 @pytest.mark.parametrize("M,K,with_residual", [(2, 2048, True), (3, 256, False), (5, 4096, True), (1, 3072, True)])
 def test_add_rmsnorm_matches_llama_rmsnorm(M, K, with_residual):
     from transformers.models.llama.modeling_llama import LlamaRMSNorm
@@ -128,3 +137,39 @@ def test_rope_attn_closed_forms():
     want = o.bf16_bits_to_f32(vc[:, :, :10, :]).astype(np.float64).mean(axis=2).reshape(M, H * D)
     assert np.abs(out - want).max() <= 1e-12
     assert (vc[:, :, 9, :].reshape(M, H * D) == c["v"]).all() and (vc[:, :, 10:, :] == c["vc"][:, :, 10:, :]).all()
+
+
+@pytest.mark.parametrize("fp32", [True, False])
+def test_lora_add_matches_the_wrapper_formula_in_torch(fp32):
+    """``base(x) + lora_B(lora_A(x)) * scaling`` with torch modules on the CPU, in the two dtypes a
+    PEFT wrapper runs its adapter in."""
+    from torch import nn
+
+    rng = np.random.default_rng(3 + fp32)
+    M, K, N, r, scaling = 5, 512, 96, 16, 2.0
+    x, y = rand_bits(rng, (M, K)), rand_bits(rng, (M, N), 2.0)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    torch.manual_seed(int(fp32))
+    lora_a, lora_b = nn.Linear(K, r, bias=False).to(dtype), nn.Linear(r, N, bias=False).to(dtype)
+    with torch.no_grad():
+        lora_b.weight.normal_(0, 0.05)
+        result, xt = bits_to_bf16(y), bits_to_bf16(x)
+        want = (result + lora_b(lora_a(xt.to(dtype))) * scaling).to(torch.bfloat16)
+    got = d.lora_add(y, x, lora_a.weight.detach().float().numpy(), lora_b.weight.detach().float().numpy(), scaling, fp32)
+    assert within_one_step_of(got, bf16_to_bits(want), y) < 0.02   # summation order inside the library products
+
+
+def test_lora_add_closed_forms():
+    rng = np.random.default_rng(9)
+    M, K, N, r = 3, 64, 24, 8
+    x, y = rand_bits(rng, (M, K)), rand_bits(rng, (M, N))
+    A, B = rng.standard_normal((r, K)).astype(np.float32), np.zeros((N, r), dtype=np.float32)
+    assert (d.lora_add(y, x, A, B, 2.0, True) == y).all()          # a fresh adapter (B = 0) changes nothing
+    # rank-one adapter picking x[:, 0] into column 5: y[:, 5] + 2 * x[:, 0], one rounding
+    A[:] = 0
+    A[0, 0] = 1.0
+    B[5, 0] = 1.0
+    got = d.lora_add(y, x, A, B, 2.0, True)
+    want = y.copy()
+    want[:, 5] = o.f32_to_bf16_bits(o.bf16_bits_to_f32(y[:, 5]) + 2.0 * o.bf16_bits_to_f32(x[:, 0]))
+    assert (got == want).all()

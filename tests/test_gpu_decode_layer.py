@@ -8,7 +8,7 @@ import torch
 from oracle import decode_oracle as d
 from oracle import int4_oracle as o
 from tests._util import bf16_to_bits, bits_to_bf16
-from tests.test_decode_oracle import attn_case, rand_bits, ulp_distance
+from tests.test_decode_oracle import attn_case, rand_bits, ulp_distance, within_one_step_of
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -223,3 +223,61 @@ def test_norm_fused_launch_rejects(ops_mod):
     with pytest.raises(ValueError):
         ops_mod.DirectGemv([(db["x"], pwb, False)],
                            norm=(None, torch.ones(8192, dtype=torch.bfloat16, device=DEV), 1e-6, None)).launch()
+
+
+# ------------------------------------------------------------------ LoRA adapters over int4 projections
+@pytest.mark.parametrize("M,K,shapes,fp32", [
+    (2, 2048, [(2048, 32), (2048, 32), (2048, 32)], True), (32, 2048, [(2048, 32), (512, 32), (512, 32)], True),
+    (2, 2048, [(2048, 32)], False), (7, 640, [(100, 8), (48, 16)], True), (32, 4096, [(4096, 64)], False),
+    (1, 5632, [(2048, 256)], True),
+])
+def test_lora_add_parity(ops_mod, M, K, shapes, fp32):
+    say("lora add", M, K, shapes, fp32)
+    rng = np.random.default_rng(K + M + len(shapes))
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    x = rand_bits(rng, (M, K))
+    xt = bits_to_bf16(x, DEV)
+    adapters, checks = [], []
+    for i, (N, r) in enumerate(shapes):
+        A = torch.from_numpy((rng.standard_normal((r, K)) * K ** -0.5).astype(np.float32)).to(dtype)
+        B = torch.from_numpy((rng.standard_normal((N, r)) * 0.1).astype(np.float32)).to(dtype)
+        y = rand_bits(rng, (M, N), 2.0)
+        yt = bits_to_bf16(y, DEV)
+        scaling = 2.0 if i % 2 == 0 else 0.75
+        adapters.append((A.to(DEV), B.to(DEV), scaling, yt))
+        checks.append((y, A.float().numpy(), B.float().numpy(), scaling, yt))
+    ops_mod.LoraAdd(xt, adapters).launch()
+    torch.cuda.synchronize()
+    for y, A, B, scaling, yt in checks:
+        want = d.lora_add(y, x, A, B, scaling, fp32)
+        assert within_one_step_of(bf16_to_bits(yt), want, y) < 0.02
+
+
+def test_lora_add_sees_in_place_weight_updates_and_rejects_misuse(ops_mod):
+    say("lora add: weight sync, contract")
+    rng = np.random.default_rng(1)
+    M, K, N, r = 2, 256, 64, 8
+    x = rand_bits(rng, (M, K))
+    xt = bits_to_bf16(x, DEV)
+    A = torch.zeros(r, K, device=DEV)
+    B = torch.zeros(N, r, device=DEV)
+    y0 = rand_bits(rng, (M, N))
+    yt = bits_to_bf16(y0, DEV)
+    launch = ops_mod.LoraAdd(xt, [(A, B, 2.0, yt)])
+    launch.launch()
+    torch.cuda.synchronize()
+    assert (bf16_to_bits(yt) == y0).all()                      # B = 0: nothing added
+    A.copy_(torch.randn(r, K, device=DEV) * 0.1)               # what a LoRA weight sync does
+    B.copy_(torch.randn(N, r, device=DEV) * 0.1)
+    launch.launch()
+    torch.cuda.synchronize()
+    want = d.lora_add(y0, x, A.cpu().numpy(), B.cpu().numpy(), 2.0, True)
+    within_one_step_of(bf16_to_bits(yt), want, y0)
+    with pytest.raises(ValueError):
+        ops_mod.LoraAdd(xt, [(A, B.to(torch.bfloat16), 2.0, yt)])       # mixed dtypes
+    with pytest.raises(ValueError):
+        ops_mod.LoraAdd(xt, [(A[:, :128].contiguous(), B, 2.0, yt)])    # A does not take x
+    with pytest.raises(ValueError):
+        ops_mod.LoraAdd(xt, [(A, B, 2.0, yt)] * 5)
+    with pytest.raises(ValueError):
+        ops_mod.LoraAdd(xt, [(A[:4].contiguous(), B[:, :4].contiguous(), 2.0, yt)]).launch()   # rank % 8

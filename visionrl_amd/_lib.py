@@ -31,6 +31,8 @@ SYMBOLS = (
     "vrl_cfg_sample_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
+    "vrl_lora_down_bf16",
+    "vrl_lora_up_add_bf16",
 )
 
 
@@ -67,6 +69,20 @@ class Norm(ctypes.Structure):
         ("h_out", ctypes.c_void_p),
         ("eps", ctypes.c_float),
         ("reserved", ctypes.c_int32),
+    ]
+
+
+class LoraAdapter(ctypes.Structure):
+    """Mirror of ``vrl_lora_adapter``."""
+
+    _fields_ = [
+        ("A", ctypes.c_void_p),
+        ("B", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("N", ctypes.c_int32),
+        ("r", ctypes.c_int32),
+        ("scaling", ctypes.c_float),
+        ("weights_fp32", ctypes.c_int32),
     ]
 
 
@@ -119,6 +135,10 @@ def _bind(lib):
     lib.vrl_cfg_sample_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_float, ctypes.c_float, vp]
     lib.vrl_add_rmsnorm_bf16.restype = ci
     lib.vrl_add_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_float, vp]
+    lib.vrl_lora_down_bf16.restype = ci
+    lib.vrl_lora_down_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
+    lib.vrl_lora_up_add_bf16.restype = ci
+    lib.vrl_lora_up_add_bf16.argtypes = [vp, ci, ctypes.POINTER(LoraAdapter), ci, vp]
     lib.vrl_rope_attn_decode_bf16.restype = ci
     lib.vrl_rope_attn_decode_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                               ci, ci, ci, ci, ci, ctypes.c_float, vp]

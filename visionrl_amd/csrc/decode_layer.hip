@@ -14,6 +14,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
 
 #include "../../include/vrl_decode.h"
 #include "../../include/vrl_int4.h"
@@ -302,6 +303,118 @@ __global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs 
     }
 }
 
+// ---------------------------------------------------------------- LoRA adapters over an int4 projection
+constexpr int LORA_MAX_ADAPTERS = 4;
+constexpr int LORA_MAX_ROWS = 32;
+constexpr int LORA_MAX_RANK = 256;
+constexpr int LORA_MAX_TOTAL = 512;
+
+struct LoraArgs {
+    vrl_lora_adapter ad[LORA_MAX_ADAPTERS];
+    int32_t off[LORA_MAX_ADAPTERS + 1];  // first column of each adapter in t
+    int32_t n, M, K;
+};
+
+__device__ __forceinline__ void load8(const void *base, long index, bool fp32, float (&f)[8]) {
+    if (fp32) {
+        const float4 a = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index);
+        const float4 b = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index + 4);
+        f[0] = a.x, f[1] = a.y, f[2] = a.z, f[3] = a.w, f[4] = b.x, f[5] = b.y, f[6] = b.z, f[7] = b.w;
+    } else {
+        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + index);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
+            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
+        }
+    }
+}
+
+// One wave per adapter row j: the row of A walks past in 8-value pieces, every activation row keeps
+// an accumulator (the activations come from cache: all waves read the same M rows).
+__global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__restrict__ x, LoraArgs a,
+                                                            float *__restrict__ t) {
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int col = blockIdx.x * WAVES + wave;  // column of t
+    const int total = a.off[a.n];
+    if (col >= total) return;  // wave-uniform, no barrier below
+    int i = 0;
+#pragma unroll
+    for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
+        if (k < a.n && a.off[k] <= col) i = k;
+    const vrl_lora_adapter ad = a.ad[i];
+    const long arow = (long)(col - a.off[i]) * a.K;
+    const bool fp32 = ad.weights_fp32 != 0;
+    float acc[LORA_MAX_ROWS];
+#pragma unroll
+    for (int m = 0; m < LORA_MAX_ROWS; ++m) acc[m] = 0.0f;
+    for (int k = lane * 8; k < a.K; k += WAVE * 8) {
+        float af[8];
+        load8(ad.A, arow + k, fp32, af);
+#pragma unroll
+        for (int m = 0; m < LORA_MAX_ROWS; ++m) {
+            if (m < a.M) {
+                float xf[8];
+                load8(x, (long)m * a.K + k, false, xf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[m] += xf[e] * af[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < LORA_MAX_ROWS; ++m) {
+        if (m < a.M) {
+            float v = wave_sum(acc[m]);
+            if (!fp32) v = round_bf16(v);  // lora_A's output tensor is bf16 then
+            if (lane == 0) t[(long)m * total + col] = v;
+        }
+    }
+}
+
+// One thread per output column: its row of B in registers piece by piece, t staged in LDS.
+__global__ __launch_bounds__(THREADS) void lora_up_add_kernel(const float *__restrict__ t, LoraArgs a) {
+    extern __shared__ __align__(16) float ts[];  // M x r of this adapter
+    const int i = blockIdx.y;
+    const vrl_lora_adapter ad = a.ad[i];
+    const int total = a.off[a.n], r = ad.r;
+    for (int idx = threadIdx.x; idx < a.M * r; idx += THREADS) {
+        const int m = idx / r;
+        ts[idx] = t[(long)m * total + a.off[i] + (idx - m * r)];
+    }
+    __syncthreads();
+    const int n = blockIdx.x * THREADS + threadIdx.x;
+    if (n >= ad.N) return;
+    const bool fp32 = ad.weights_fp32 != 0;
+    uint16_t *y = static_cast<uint16_t *>(ad.y);
+    float u[LORA_MAX_ROWS];
+#pragma unroll
+    for (int m = 0; m < LORA_MAX_ROWS; ++m) u[m] = 0.0f;
+    for (int j = 0; j < r; j += 8) {  // r % 8 == 0
+        float bf[8];
+        load8(ad.B, (long)n * r + j, fp32, bf);
+#pragma unroll
+        for (int m = 0; m < LORA_MAX_ROWS; ++m) {
+            if (m < a.M) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) u[m] += ts[m * r + j + e] * bf[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < LORA_MAX_ROWS; ++m) {
+        if (m < a.M) {
+            const long at = (long)m * ad.N + n;
+            float delta = u[m];
+            if (!fp32) delta = round_bf16(round_bf16(delta) * ad.scaling);  // lora_B's output, then * scaling
+            else delta *= ad.scaling;
+            y[at] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(y[at]) + delta);
+        }
+    }
+}
+
+int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y);
+
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 }  // namespace
@@ -363,5 +476,59 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
         hipLaunchKernelGGL(rope_attn_decode_kernel<128>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
     else
         hipLaunchKernelGGL(rope_attn_decode_kernel<64>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+namespace {
+int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y) {
+    if (!adapters) return VRL_INT4_ENULL;
+    if (n < 1 || n > LORA_MAX_ADAPTERS || M < 1 || M > LORA_MAX_ROWS || K < 8 || K % 8 != 0) return VRL_INT4_ESHAPE;
+    a.n = n;
+    a.M = M;
+    a.K = K;
+    a.off[0] = 0;
+    for (int i = 0; i < n; ++i) {
+        const vrl_lora_adapter &ad = adapters[i];
+        if (!ad.A || !ad.B || (need_y && !ad.y)) return VRL_INT4_ENULL;
+        if (ad.r < 8 || ad.r % 8 != 0 || ad.r > LORA_MAX_RANK || ad.N < 1) return VRL_INT4_ESHAPE;
+        if (misaligned(ad.A, 16) || misaligned(ad.B, 16) || misaligned(ad.y, 2)) return VRL_INT4_EALIGN;
+        a.ad[i] = ad;
+        a.off[i + 1] = a.off[i] + ad.r;
+    }
+    for (int i = n; i < LORA_MAX_ADAPTERS; ++i) a.off[i + 1] = a.off[n];
+    if (a.off[n] > LORA_MAX_TOTAL) return VRL_INT4_ESHAPE;
+    return VRL_INT4_OK;
+}
+}  // namespace
+
+extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adapters, int n_adapters,
+                                  float *t, void *hip_stream) {
+    if (!x || !t) return VRL_INT4_ENULL;
+    if (misaligned(x, 16) || misaligned(t, 4)) return VRL_INT4_EALIGN;
+    LoraArgs a;
+    memset(&a, 0, sizeof a);
+    const int rc = lora_args(a, M, K, adapters, n_adapters, false);
+    if (rc != VRL_INT4_OK) return rc;
+    const int total = a.off[a.n];
+    hipLaunchKernelGGL(lora_down_kernel, dim3((total + WAVES - 1) / WAVES), dim3(THREADS), 0,
+                       reinterpret_cast<hipStream_t>(hip_stream), static_cast<const uint16_t *>(x), a, t);
+    return (int)hipGetLastError();
+}
+
+extern "C" int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
+                                    void *hip_stream) {
+    if (!t) return VRL_INT4_ENULL;
+    if (misaligned(t, 4)) return VRL_INT4_EALIGN;
+    LoraArgs a;
+    memset(&a, 0, sizeof a);
+    const int rc = lora_args(a, M, 8, adapters, n_adapters, true);
+    if (rc != VRL_INT4_OK) return rc;
+    int max_n = 0, max_r = 0;
+    for (int i = 0; i < a.n; ++i) {
+        max_n = a.ad[i].N > max_n ? a.ad[i].N : max_n;
+        max_r = a.ad[i].r > max_r ? a.ad[i].r : max_r;
+    }
+    hipLaunchKernelGGL(lora_up_add_kernel, dim3((max_n + THREADS - 1) / THREADS, a.n), dim3(THREADS),
+                       (size_t)M * max_r * sizeof(float), reinterpret_cast<hipStream_t>(hip_stream), t, a);
     return (int)hipGetLastError();
 }

@@ -26,7 +26,7 @@ from .int4_format import check_packed
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
            "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "add_rmsnorm",
-           "rope_attn_decode"]
+           "rope_attn_decode", "LoraAdd"]
 
 
 def _stream_handle(device: torch.device) -> int:
@@ -609,3 +609,52 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
             out.data_ptr(), M, H, Hkv, D, L, float(scaling), _stream_handle(dev))
     _lib.check(rc, "vrl_rope_attn_decode_bf16")
     return out
+
+
+class LoraAdd:
+    """LoRA adapters added onto the outputs of int4 projections that share an input: two launches.
+
+    ``adapters`` is a list of ``(A [r, K], B [N, r], scaling, y [M, N])`` with ``A``/``B`` the
+    ``lora_A`` / ``lora_B`` weights of a PEFT wrapper (float32 or bfloat16, kept by reference: an
+    in-place weight sync is seen by the next launch) and ``y`` the bf16 output of the base
+    projection, updated in place: ``y += scaling * (x A^T) B^T`` with the roundings the wrapper's
+    own forward applies (``vrl/models/families/janus_pro/policy.py:298-324`` attaches the adapters).
+    ``x`` is the fixed bf16 ``[M <= 32, K]`` input buffer of the group.
+    """
+
+    def __init__(self, x: torch.Tensor, adapters):
+        if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_contiguous():
+            raise ValueError("x must be contiguous bfloat16 [M, K]")
+        dev = _require_device("x", x)
+        M, K = x.shape
+        if not 1 <= len(adapters) <= 4:
+            raise ValueError("1 to 4 adapters per group")
+        self.table = (_lib.LoraAdapter * len(adapters))()
+        total = 0
+        for rec, (A, B, scaling, y) in zip(self.table, adapters):
+            if A.dtype != B.dtype or A.dtype not in (torch.float32, torch.bfloat16):
+                raise ValueError("adapter weights must both be float32 or both bfloat16")
+            if A.dim() != 2 or B.dim() != 2 or A.shape[1] != K or B.shape[1] != A.shape[0] or \
+                    not A.is_contiguous() or not B.is_contiguous():
+                raise ValueError(f"adapter weights must be contiguous A [r, {K}] and B [N, r]")
+            r, N = A.shape[0], B.shape[0]
+            if y.dtype != torch.bfloat16 or tuple(y.shape) != (M, N) or not y.is_contiguous():
+                raise ValueError(f"y must be contiguous bfloat16 [{M}, {N}]")
+            for name, t in (("A", A), ("B", B), ("y", y)):
+                _require_device(name, t, dev)
+            rec.A, rec.B, rec.y, rec.N, rec.r = A.data_ptr(), B.data_ptr(), y.data_ptr(), N, r
+            rec.scaling, rec.weights_fp32 = float(scaling), int(A.dtype == torch.float32)
+            total += r
+        self.t = torch.empty((M, total), dtype=torch.float32, device=dev)
+        self.x, self.M, self.K, self.device = x, M, K, dev
+        self._keep = list(adapters)
+
+    def launch(self):
+        lib = _lib.load()
+        stream = _stream_handle(self.device)
+        with _on(self.device):
+            rc = lib.vrl_lora_down_bf16(self.x.data_ptr(), self.M, self.K, self.table, len(self.table),
+                                        self.t.data_ptr(), stream)
+            _lib.check(rc, "vrl_lora_down_bf16")
+            rc = lib.vrl_lora_up_add_bf16(self.t.data_ptr(), self.M, self.table, len(self.table), stream)
+            _lib.check(rc, "vrl_lora_up_add_bf16")
