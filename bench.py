@@ -491,8 +491,47 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
             lambda n: sampler.sample_image_tokens(*inputs[B], image_token_num=n))
         del sampler
         torch.cuda.empty_cache()
+    class LoraWrapper(nn.Module):
+        """The forward of a PEFT LoRA wrapper (not installed here) with the reference's defaults:
+        rank 32, alpha 64, float32 adapter weights on q/k/v/o_proj (policy.py:81-88, :298-324)."""
+
+        def __init__(self, base, r=32, alpha=64):
+            super().__init__()
+            self.base_layer = base
+            self.lora_A = nn.ModuleDict({"default": nn.Linear(base.in_features, r, bias=False)})
+            self.lora_B = nn.ModuleDict({"default": nn.Linear(r, base.out_features, bias=False)})
+            self.scaling, self.active_adapters = {"default": alpha / r}, ["default"]
+            self.merged = self.disable_adapters = False
+            nn.init.normal_(self.lora_B["default"].weight, std=0.01)
+
+        def forward(self, x):
+            a, b = self.lora_A["default"], self.lora_B["default"]
+            return (self.base_layer(x) + b(a(x.to(a.weight.dtype))) * self.scaling["default"]).to(x.dtype)
+
+    def with_adapters(on: bool):
+        for layer in policy._lm_trunk().layers:
+            for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+                mod = getattr(layer.self_attn, name)
+                if on and not isinstance(mod, LoraWrapper):
+                    setattr(layer.self_attn, name, LoraWrapper(mod).to(device))
+                elif not on and isinstance(mod, LoraWrapper):
+                    setattr(layer.self_attn, name, mod.base_layer)
+
     apply_int4_to_policy(policy, group_size=GROUP)
     torch.cuda.empty_cache()
+    if only in (None, "int4_lora_native_hip_graph"):
+        with_adapters(True)
+        for B in batches:
+            entry = out.setdefault(f"B{B}", {})
+            for name, native in (("int4_lora_static_hip_graph", False), ("int4_lora_native_hip_graph", True)):
+                if only is not None and name != only:
+                    continue
+                sampler = StaticARSampler(policy, graph=True, native=native)
+                entry[f"{name}_ms_per_token"] = per_token_ms(
+                    lambda n: sampler.sample_image_tokens(*inputs[B], image_token_num=n))
+                del sampler
+                torch.cuda.empty_cache()
+        with_adapters(False)
     for B in batches:
         entry = out.setdefault(f"B{B}", {})
         if only is None:
@@ -574,6 +613,7 @@ def main():
                     help="run just the grouped decode-step launches (for profilers)")
     ap.add_argument("--single-calls", action="store_true",
                     help="loop single-GEMV launches over distinct weights per shape and exit (for profilers)")
+    ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
     ap.add_argument("--ar-decode", type=int, default=0, metavar="B",
                     help="run only the recorded decode loop at batch B on the int4 policy and exit (for profilers)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -597,7 +637,8 @@ def main():
     from visionrl_amd import ops
 
     if args.ar_decode:
-        print(json.dumps(ar_decode_loop(device, only="int4_native_hip_graph", batches=(args.ar_decode,))))
+        which = "int4_lora_native_hip_graph" if args.lora else "int4_native_hip_graph"
+        print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,))))
         return
     if args.single_calls:
         for M in (1, 32):

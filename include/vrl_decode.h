@@ -69,8 +69,8 @@ int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q
  * with t a float32 [M, r_total] scratch buffer of the caller's, off_i the sum of the ranks before
  * adapter i.  Adapter weights are float32 (what PEFT keeps by default: everything in fp32, one
  * rounding when the result returns to bf16) or bf16 (weights_fp32 = 0: t, the up-projection and its
- * scaled value are rounded to bf16 as the bf16 modules round them).  1 <= n_adapters <= 4,
- * r <= 256, r_total <= 512, K % 8 == 0, pointers 16-byte aligned.
+ * scaled value are rounded to bf16 as the bf16 modules round them); one type per launch.
+ * 1 <= n_adapters <= 4, r % 8 == 0, r <= 64, K % 8 == 0, pointers 16-byte aligned.
  */
 typedef struct vrl_lora_adapter {
     const void *A;     /* [r, K] row-major */

@@ -270,3 +270,105 @@ def test_native_sampling_agrees_with_the_module_path_on_independent_draws(int4_p
     same = t_n[:, 1] == t_m[:, 1]
     assert same.sum().item() >= 14, (t_n[:, 1], t_m[:, 1])
     assert (lp_n[same, 1] - lp_m[same, 1]).abs().max().item() <= 0.25
+
+
+# ------------------------------------------------------------------ LoRA adapters on the attention projections
+class LoraWrapper(nn.Module):
+    """The attributes and the forward of peft's ``lora.Linear`` that matter at rollout time
+    (``vrl/models/families/janus_pro/policy.py:298-324`` wraps q/k/v/o_proj with it): the frozen
+    projection in ``base_layer``, one adapter named "default", the adapter run in its own dtype
+    on the upcast input and the sum cast back."""
+
+    def __init__(self, base, r=8, alpha=16, dtype=torch.float32):
+        super().__init__()
+        self.base_layer = base
+        self.lora_A = nn.ModuleDict({"default": nn.Linear(base.in_features, r, bias=False).to(dtype)})
+        self.lora_B = nn.ModuleDict({"default": nn.Linear(r, base.out_features, bias=False).to(dtype)})
+        self.scaling = {"default": alpha / r}
+        self.active_adapters = ["default"]
+        self.merged = False
+        self.disable_adapters = False
+        with torch.no_grad():
+            self.lora_B["default"].weight.normal_(0.0, 0.05)   # a trained adapter, not a fresh (zero) one
+
+    def forward(self, x):
+        result = self.base_layer(x)
+        a, b = self.lora_A["default"], self.lora_B["default"]
+        result = result + b(a(x.to(a.weight.dtype))) * self.scaling["default"]
+        return result.to(x.dtype)
+
+
+def lora_policy(dtype):
+    from visionrl_amd.policy_glue import apply_int4_to_policy
+
+    policy = StubPolicy(torch.bfloat16, "cuda:0")
+    torch.manual_seed(7)
+    for layer in policy._lm_trunk().layers:
+        for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            setattr(layer.self_attn, name, LoraWrapper(getattr(layer.self_attn, name), dtype=dtype).to("cuda:0"))
+    summary = apply_int4_to_policy(policy, group_size=128)
+    assert summary["linears"] == 7 * LAYERS and summary["qkv_groups"] == LAYERS
+    return policy
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_native_trunk_with_lora_adapters_tracks_the_module_trunk(dtype):
+    """As above with adapters on q/k/v/o: the native layer adds them with two launches per group; a
+    weight sync in place (``load_lora_state``) reaches it without rebuilding anything."""
+    from visionrl_amd.policy_glue import load_lora_state
+
+    print("ar decode: native trunk with LoRA", dtype, flush=True)
+    policy = lora_policy(dtype)
+    rows, n_text, steps = 4, 6, 6
+    cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=61)
+    sessions = []
+    for native in (True, False):
+        sampler = StaticARSampler(policy, graph=False, native=native)
+        torch.manual_seed(61)
+        sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=1)
+        (sess,) = sampler._sessions.values()
+        sessions.append(sess)
+    nat, mod = sessions
+    assert nat.native and not mod.native
+    assert nat.native.launches == (5 + 1 + 4) * LAYERS + 1   # norm of its own, 2 x (down, up) per layer
+    trunk = policy._lm_trunk()
+    gen = torch.Generator(device="cuda:0").manual_seed(62)
+
+    def compare(n):
+        with torch.no_grad():
+            for t in range(n):
+                emb = torch.randn((rows, 1, HIDDEN), generator=gen, device="cuda:0").to(torch.bfloat16)
+                nat.cur.copy_(emb)
+                got = nat.native.run().float().clone()
+                nat.slot.add_(1)
+                want = trunk(inputs_embeds=emb, attention_mask=mod.mask, use_cache=True,
+                             past_key_values=mod.cache).last_hidden_state[:, -1].float()
+                torch.cuda.synchronize()
+                err = (got - want).abs()
+                assert err.max().item() <= 0.08 and err.mean().item() <= 0.008, (t, err.max().item())
+        return got
+
+    before = compare(steps)
+    # the adapters matter: without them the hidden states differ by far more than the tolerance
+    bare = trunk.layers[0].self_attn.q_proj
+    state = {k: torch.randn_like(v) * 0.05 for k, v in trunk.state_dict().items() if "lora_" in k}
+    summary = load_lora_state(trunk, state)
+    assert summary["loaded"] == 8 * LAYERS
+    assert torch.equal(bare.lora_B["default"].weight.data, state["layers.0.self_attn.q_proj.lora_B.default.weight"])
+    after = compare(steps)          # same launches, same pointers, new adapter values: still tracks the modules
+    assert (after - before).abs().max().item() > 0.1
+
+
+@pytest.mark.gpu
+def test_graph_replays_equal_eager_steps_with_lora():
+    print("ar decode: graph vs eager with LoRA", flush=True)
+    policy = lora_policy(torch.float32)
+    cond, uncond, cmask, umask = make_inputs(2, 7, torch.bfloat16, "cuda:0", seed=71)
+    out = []
+    for graph in (False, True):
+        torch.manual_seed(71)
+        out.append(StaticARSampler(policy, graph=graph).sample_image_tokens(cond, uncond, cmask, umask,
+                                                                             image_token_num=16))
+    torch.cuda.synchronize()
+    assert torch.equal(out[0][0], out[1][0]) and torch.equal(out[0][1], out[1][1])

@@ -229,7 +229,7 @@ def test_norm_fused_launch_rejects(ops_mod):
 @pytest.mark.parametrize("M,K,shapes,fp32", [
     (2, 2048, [(2048, 32), (2048, 32), (2048, 32)], True), (32, 2048, [(2048, 32), (512, 32), (512, 32)], True),
     (2, 2048, [(2048, 32)], False), (7, 640, [(100, 8), (48, 16)], True), (32, 4096, [(4096, 64)], False),
-    (1, 5632, [(2048, 256)], True),
+    (1, 5632, [(2048, 64)], True), (9, 1024, [(96, 40), (64, 8)], False),
 ])
 def test_lora_add_parity(ops_mod, M, K, shapes, fp32):
     say("lora add", M, K, shapes, fp32)
@@ -281,3 +281,5 @@ def test_lora_add_sees_in_place_weight_updates_and_rejects_misuse(ops_mod):
         ops_mod.LoraAdd(xt, [(A, B, 2.0, yt)] * 5)
     with pytest.raises(ValueError):
         ops_mod.LoraAdd(xt, [(A[:4].contiguous(), B[:, :4].contiguous(), 2.0, yt)]).launch()   # rank % 8
+    with pytest.raises(ValueError):
+        ops_mod.LoraAdd(xt, [(A, B, 2.0, yt), (A.to(torch.bfloat16), B.to(torch.bfloat16), 2.0, yt)])   # one type per launch

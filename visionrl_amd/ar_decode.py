@@ -18,7 +18,7 @@ arguments, the same results and the same use of the random stream:
   The prompt pass and the first decode step run eagerly (the latter doubles as the warm-up a
   capture needs).
 * When the trunk's projections are prepacked int4 modules, the trunk part of the step runs as
-  seven launches per layer over the same cache tensors (:mod:`visionrl_amd.decode_step`) instead
+  five launches per layer over the same cache tensors (:mod:`visionrl_amd.decode_step`) instead
   of the module's some thirty tensor ops per layer; results then agree with the module path to
   bf16 roundings of the hidden states (the attention keeps fp32 probabilities), not bit for bit.
 * The tail after the head is one launch (:func:`visionrl_amd.ops.cfg_sample`) when the logits are
@@ -108,7 +108,10 @@ class _Session:
             s = self.sampler
             if s.native and self.cur.is_cuda and self.cur.dtype == torch.bfloat16 and \
                     NativeDecodeTrunk.unsupported(s.trunk, self.rows2, self.max_len) is None:
-                self.native = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot)
+                try:
+                    self.native = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot)
+                except (TypeError, ValueError):   # something the native launches do not take: module path
+                    self.native = False
 
     def step(self) -> None:
         if self.native:
@@ -136,9 +139,9 @@ class StaticARSampler:
     (``cfg_weight``, ``temperature``, ``image_token_num``).  ``graph=False`` runs every step
     eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
     for the part after the head.  With ``native`` (the default) the trunk of a decode step runs as
-    :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (seven launches per layer) when the policy
-    went through ``apply_int4_to_policy`` with its defaults and carries no adapters; otherwise, and
-    for the prompt pass, the trunk module itself is called.
+    :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (five launches per layer, ten with LoRA
+    adapters on the attention projections) when the policy went through ``apply_int4_to_policy``
+    with its defaults; otherwise, and for the prompt pass, the trunk module itself is called.
     """
 
     def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True, native: bool = True,

@@ -35,15 +35,37 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float v) {
 }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to_bf16_bits(v)); }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
+// Cross-lane sums through DPP (register-to-register, no trip through the LDS crossbar that
+// __shfl_xor takes).  A DPP row is 16 lanes: two quad permutes and two mirrors leave every lane of
+// a row with the row's sum; the four rows of a wave meet through readlane.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141>(v);  // row_half_mirror
+    v += dpp_move<0x140>(v);  // row_mirror
     return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
     return v;
+}
+__device__ __forceinline__ float lane_of(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_of(v, 0), lane_of(v, 16)), fmaxf(lane_of(v, 32), lane_of(v, 48)));
 }
 
 // every thread returns the block's total; `red` holds WAVES floats and is free for reuse afterwards
@@ -250,10 +272,7 @@ __global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs 
                 dot += qreg[2 * i] * bf16_to_f32(kraw[u].w[i] & 0xFFFFu);
                 dot += qreg[2 * i + 1] * bf16_to_f32(kraw[u].w[i] >> 16);
             }
-            dot += __shfl_xor(dot, 1, WAVE);
-            dot += __shfl_xor(dot, 2, WAVE);
-            dot += __shfl_xor(dot, 4, WAVE);
-            dot += __shfl_xor(dot, 8, WAVE);
+            dot = row16_sum(dot);  // the sixteen lanes that share the slot
             const float s = live[u] ? dot * a.scaling : -INFINITY;
             float vf[VEC];
 #pragma unroll
@@ -306,8 +325,8 @@ __global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs 
 // ---------------------------------------------------------------- LoRA adapters over an int4 projection
 constexpr int LORA_MAX_ADAPTERS = 4;
 constexpr int LORA_MAX_ROWS = 32;
-constexpr int LORA_MAX_RANK = 256;
-constexpr int LORA_MAX_TOTAL = 512;
+constexpr int LORA_MAX_RANK = 64;
+constexpr int LORA_MAX_TOTAL = 256;
 
 struct LoraArgs {
     vrl_lora_adapter ad[LORA_MAX_ADAPTERS];
@@ -315,8 +334,9 @@ struct LoraArgs {
     int32_t n, M, K;
 };
 
-__device__ __forceinline__ void load8(const void *base, long index, bool fp32, float (&f)[8]) {
-    if (fp32) {
+template <bool FP32>
+__device__ __forceinline__ void load8(const void *base, long index, float (&f)[8]) {
+    if constexpr (FP32) {
         const float4 a = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index);
         const float4 b = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index + 4);
         f[0] = a.x, f[1] = a.y, f[2] = a.z, f[3] = a.w, f[4] = b.x, f[5] = b.y, f[6] = b.z, f[7] = b.w;
@@ -331,86 +351,146 @@ __device__ __forceinline__ void load8(const void *base, long index, bool fp32, f
     }
 }
 
-// One wave per adapter row j: the row of A walks past in 8-value pieces, every activation row keeps
-// an accumulator (the activations come from cache: all waves read the same M rows).
+// Both kernels are written without data-dependent branches: rows beyond M repeat row M - 1
+// (clamped index), which costs arithmetic but keeps every load of a lane in flight at once.
+// MB bounds the rows a build handles (8 or 32); FP32 is the adapters' weight type.
+
+// One workgroup per column of t (an adapter row j): its four waves take interleaved 512-value
+// pieces of K; a lane holds 8 values of the A row and requests the matching 8 values of sixteen
+// activation rows at a time, then every row's partial sum is reduced over the wave and the four
+// waves meet in LDS.
+template <bool FP32, int MB>
 __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__restrict__ x, LoraArgs a,
                                                             float *__restrict__ t) {
+    __shared__ float part[WAVES][LORA_MAX_ROWS];
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int col = blockIdx.x * WAVES + wave;  // column of t
+    const int col = blockIdx.x;
     const int total = a.off[a.n];
-    if (col >= total) return;  // wave-uniform, no barrier below
     int i = 0;
 #pragma unroll
     for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
         if (k < a.n && a.off[k] <= col) i = k;
-    const vrl_lora_adapter ad = a.ad[i];
-    const long arow = (long)(col - a.off[i]) * a.K;
-    const bool fp32 = ad.weights_fp32 != 0;
-    float acc[LORA_MAX_ROWS];
+    const void *A = a.ad[0].A;
+    int first = 0;
 #pragma unroll
-    for (int m = 0; m < LORA_MAX_ROWS; ++m) acc[m] = 0.0f;
-    for (int k = lane * 8; k < a.K; k += WAVE * 8) {
+    for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
+        if (k == i) A = a.ad[k].A, first = a.off[k];   // scalar selects, no indexing of the argument block
+    const long arow = (long)(col - first) * a.K;
+    constexpr int RB = MB < 16 ? MB : 16;  // rows requested together
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+    for (int k = (wave * WAVE + lane) * 8; k < a.K; k += THREADS * 8) {
         float af[8];
-        load8(ad.A, arow + k, fp32, af);
+        load8<FP32>(A, arow + k, af);
 #pragma unroll
-        for (int m = 0; m < LORA_MAX_ROWS; ++m) {
-            if (m < a.M) {
-                float xf[8];
-                load8(x, (long)m * a.K + k, false, xf);
+        for (int m0 = 0; m0 < MB; m0 += RB) {
+            uint4 xr[RB];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[m] += xf[e] * af[e];
+            for (int u = 0; u < RB; ++u) {
+                const int m = m0 + u < a.M ? m0 + u : a.M - 1;
+                xr[u] = *reinterpret_cast<const uint4 *>(x + (long)m * a.K + k);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // all requests of the batch before the first use
+#pragma unroll
+            for (int u = 0; u < RB; ++u) {
+                const uint32_t w[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc[m0 + u] += bf16_to_f32(w[e] & 0xFFFFu) * af[2 * e] + bf16_to_f32(w[e] >> 16) * af[2 * e + 1];
             }
         }
     }
 #pragma unroll
-    for (int m = 0; m < LORA_MAX_ROWS; ++m) {
-        if (m < a.M) {
-            float v = wave_sum(acc[m]);
-            if (!fp32) v = round_bf16(v);  // lora_A's output tensor is bf16 then
-            if (lane == 0) t[(long)m * total + col] = v;
+    for (int m = 0; m < MB; ++m) {
+        const float v = wave_sum(acc[m]);
+        if (lane == 0) part[wave][m] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < a.M) {
+        float v = part[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += part[w][threadIdx.x];
+        if (!FP32) v = round_bf16(v);  // lora_A's output tensor is bf16 then
+        t[(long)threadIdx.x * total + col] = v;
+    }
+}
+
+// One thread per output column, 64 columns per workgroup: t of the adapter staged in LDS, the
+// column's row of B (up to RB values, zero beyond the rank) in registers, 16-byte LDS reads shared
+// by the wave.  Rows are walked by a plain loop (the products of a row land in LDS), then the base
+// outputs are fetched and rewritten eight rows at a time.
+constexpr int UP_THREADS = 64;
+template <bool FP32, int RB>
+__global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__restrict__ t, LoraArgs a) {
+    extern __shared__ __align__(16) float ts[];  // M x r of this adapter, then M x UP_THREADS products
+    const int i = blockIdx.y;
+    vrl_lora_adapter ad = a.ad[0];
+    int first = 0;
+#pragma unroll
+    for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
+        if (k == i) ad = a.ad[k], first = a.off[k];
+    const int total = a.off[a.n], r = ad.r;
+    if (blockIdx.x * UP_THREADS >= ad.N) return;  // uniform: adapters of one launch differ in width
+    float *us = ts + a.M * r;
+    {   // t of this adapter: rows of r floats (r % 8 == 0), four at a time, requests issued together
+        const int r4 = r >> 2, count = a.M * r4;
+#pragma unroll 4
+        for (int idx = threadIdx.x; idx < count; idx += UP_THREADS) {
+            const int m = idx / r4;
+            *reinterpret_cast<float4 *>(ts + 4 * idx) =
+                *reinterpret_cast<const float4 *>(t + (long)m * total + first + 4 * (idx - m * r4));
+        }
+    }
+    const int n = blockIdx.x * UP_THREADS + threadIdx.x;
+    const int nn = n < ad.N ? n : ad.N - 1;  // lanes past the last column repeat it and store nothing
+    uint16_t *y = static_cast<uint16_t *>(ad.y);
+    float bf[RB];
+#pragma unroll
+    for (int g = 0; g < RB / 8; ++g) {
+        float piece[8];
+        load8<FP32>(ad.B, (long)nn * r + (8 * g < r ? 8 * g : r - 8), piece);
+        const float keep = 8 * g < r ? 1.0f : 0.0f;   // beyond the rank: zeros
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bf[8 * g + e] = piece[e] * keep;
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int m = 0; m < a.M; ++m) {
+        const float *row = ts + m * r;
+        float u = 0.0f;
+#pragma unroll
+        for (int g = 0; g < RB / 4; ++g) {
+            const float4 tv = *reinterpret_cast<const float4 *>(row + (4 * g < r ? 4 * g : r - 4));  // x 0 beyond r
+            u += tv.x * bf[4 * g] + tv.y * bf[4 * g + 1] + tv.z * bf[4 * g + 2] + tv.w * bf[4 * g + 3];
+        }
+        us[m * UP_THREADS + threadIdx.x] = u;  // read back by the same thread only
+    }
+    if (n >= ad.N) return;
+    for (int m0 = 0; m0 < a.M; m0 += 8) {
+        uint16_t base[8];
+#pragma unroll
+        for (int d = 0; d < 8; ++d) base[d] = y[(long)(m0 + d < a.M ? m0 + d : a.M - 1) * ad.N + n];
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+            const int m = m0 + d < a.M ? m0 + d : a.M - 1;  // rows past the end rewrite row M - 1 with its own value
+            float delta = us[m * UP_THREADS + threadIdx.x];
+            if (!FP32) delta = round_bf16(round_bf16(delta) * ad.scaling);  // lora_B's output, then * scaling
+            else delta *= ad.scaling;
+            y[(long)m * ad.N + n] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(base[d]) + delta);
         }
     }
 }
 
-// One thread per output column: its row of B in registers piece by piece, t staged in LDS.
-__global__ __launch_bounds__(THREADS) void lora_up_add_kernel(const float *__restrict__ t, LoraArgs a) {
-    extern __shared__ __align__(16) float ts[];  // M x r of this adapter
-    const int i = blockIdx.y;
-    const vrl_lora_adapter ad = a.ad[i];
-    const int total = a.off[a.n], r = ad.r;
-    for (int idx = threadIdx.x; idx < a.M * r; idx += THREADS) {
-        const int m = idx / r;
-        ts[idx] = t[(long)m * total + a.off[i] + (idx - m * r)];
-    }
-    __syncthreads();
-    const int n = blockIdx.x * THREADS + threadIdx.x;
-    if (n >= ad.N) return;
-    const bool fp32 = ad.weights_fp32 != 0;
-    uint16_t *y = static_cast<uint16_t *>(ad.y);
-    float u[LORA_MAX_ROWS];
-#pragma unroll
-    for (int m = 0; m < LORA_MAX_ROWS; ++m) u[m] = 0.0f;
-    for (int j = 0; j < r; j += 8) {  // r % 8 == 0
-        float bf[8];
-        load8(ad.B, (long)n * r + j, fp32, bf);
-#pragma unroll
-        for (int m = 0; m < LORA_MAX_ROWS; ++m) {
-            if (m < a.M) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) u[m] += ts[m * r + j + e] * bf[e];
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < LORA_MAX_ROWS; ++m) {
-        if (m < a.M) {
-            const long at = (long)m * ad.N + n;
-            float delta = u[m];
-            if (!fp32) delta = round_bf16(round_bf16(delta) * ad.scaling);  // lora_B's output, then * scaling
-            else delta *= ad.scaling;
-            y[at] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(y[at]) + delta);
-        }
-    }
+template <bool FP32, int MB>
+void launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_t stream) {
+    hipLaunchKernelGGL((lora_down_kernel<FP32, MB>), dim3(a.off[a.n]), dim3(THREADS), 0, stream, x, a, t);
+}
+
+template <bool FP32, int RB>
+void launch_lora_up(const float *t, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
+    hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>), dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n),
+                       dim3(UP_THREADS), (size_t)a.M * (max_r + UP_THREADS) * sizeof(float), stream, t, a);
 }
 
 int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y);
@@ -492,6 +572,7 @@ int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n
         if (!ad.A || !ad.B || (need_y && !ad.y)) return VRL_INT4_ENULL;
         if (ad.r < 8 || ad.r % 8 != 0 || ad.r > LORA_MAX_RANK || ad.N < 1) return VRL_INT4_ESHAPE;
         if (misaligned(ad.A, 16) || misaligned(ad.B, 16) || misaligned(ad.y, 2)) return VRL_INT4_EALIGN;
+        if ((ad.weights_fp32 != 0) != (adapters[0].weights_fp32 != 0)) return VRL_INT4_ESHAPE;  // one type per launch
         a.ad[i] = ad;
         a.off[i + 1] = a.off[i] + ad.r;
     }
@@ -509,9 +590,11 @@ extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_ad
     memset(&a, 0, sizeof a);
     const int rc = lora_args(a, M, K, adapters, n_adapters, false);
     if (rc != VRL_INT4_OK) return rc;
-    const int total = a.off[a.n];
-    hipLaunchKernelGGL(lora_down_kernel, dim3((total + WAVES - 1) / WAVES), dim3(THREADS), 0,
-                       reinterpret_cast<hipStream_t>(hip_stream), static_cast<const uint16_t *>(x), a, t);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    auto xs = static_cast<const uint16_t *>(x);
+    const bool fp32 = a.ad[0].weights_fp32 != 0;
+    if (M <= 8) fp32 ? launch_lora_down<true, 8>(xs, a, t, stream) : launch_lora_down<false, 8>(xs, a, t, stream);
+    else fp32 ? launch_lora_down<true, 32>(xs, a, t, stream) : launch_lora_down<false, 32>(xs, a, t, stream);
     return (int)hipGetLastError();
 }
 
@@ -528,7 +611,11 @@ extern "C" int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapte
         max_n = a.ad[i].N > max_n ? a.ad[i].N : max_n;
         max_r = a.ad[i].r > max_r ? a.ad[i].r : max_r;
     }
-    hipLaunchKernelGGL(lora_up_add_kernel, dim3((max_n + THREADS - 1) / THREADS, a.n), dim3(THREADS),
-                       (size_t)M * max_r * sizeof(float), reinterpret_cast<hipStream_t>(hip_stream), t, a);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    const bool fp32 = a.ad[0].weights_fp32 != 0;
+    if (fp32) max_r <= 32 ? launch_lora_up<true, 32>(t, a, max_n, max_r, stream)
+                          : launch_lora_up<true, 64>(t, a, max_n, max_r, stream);
+    else max_r <= 32 ? launch_lora_up<false, 32>(t, a, max_n, max_r, stream)
+                     : launch_lora_up<false, 64>(t, a, max_n, max_r, stream);
     return (int)hipGetLastError();
 }

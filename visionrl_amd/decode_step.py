@@ -18,8 +18,12 @@ step can be recorded as one HIP graph.  Arithmetic follows the library's roundin
 op in fp32, rounded to bf16); the attention keeps its probabilities in fp32.
 
 Needs a trunk whose projections were swapped for prepacked :class:`Int4Linear` modules with the
-fused MLP (``apply_int4_to_policy`` defaults) and carry no adapter; :meth:`NativeDecodeTrunk.unsupported`
-says why a trunk does not qualify, and callers then keep the module path.
+fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry one active LoRA
+adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
+the norm as a launch of its own (the adapters read the normalised row) and two more launches per
+adapter group (down-projection of all adapters that share the input, up-projection added onto the
+int4 outputs).  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not qualify, and
+callers then keep the module path.
 """
 
 from __future__ import annotations
@@ -42,6 +46,53 @@ def _plain_int4(module, name: str):
     if module.bias is not None:
         raise TypeError(f"{name} has a bias")
     return module._packed
+
+
+def _adapter_of(module, name: str):
+    """``(A, B, scaling)`` of the one active LoRA adapter of a PEFT-style wrapper.
+
+    Reads the attributes of peft's ``lora.Linear`` (``lora_A`` / ``lora_B`` module dicts keyed by
+    adapter name, ``scaling``, ``active_adapters``, ``merged``, ``disable_adapters``, ``use_dora``;
+    the wrappers ``policy.py:298-324`` attaches); a plain pair of linears with a float
+    ``scaling`` attribute is taken too.  The weights are returned by reference, so an in-place
+    weight sync reaches the launches that hold them.
+    """
+    if getattr(module, "merged", False) or getattr(module, "disable_adapters", False):
+        raise TypeError(f"{name}: merged or disabled adapters")
+    lora_a, lora_b, scaling = module.lora_A, module.lora_B, getattr(module, "scaling", 1.0)
+    if hasattr(lora_a, "keys"):
+        active = getattr(module, "active_adapters", None) or getattr(module, "active_adapter", "default")
+        active = [active] if isinstance(active, str) else list(active)
+        active = [key for key in active if key in lora_a]
+        if len(active) != 1:
+            raise TypeError(f"{name}: exactly one active adapter is supported, found {active}")
+        key = active[0]
+        if getattr(module, "use_dora", None) and module.use_dora.get(key):
+            raise TypeError(f"{name}: DoRA adapters keep the module path")
+        drop = getattr(module, "lora_dropout", None)
+        drop = drop[key] if drop is not None and key in drop else None
+        if isinstance(drop, torch.nn.Dropout) and drop.p > 0 and drop.training:
+            raise TypeError(f"{name}: adapter dropout is active")
+        lora_a, lora_b = lora_a[key], lora_b[key]
+        scaling = scaling[key] if hasattr(scaling, "keys") else scaling
+    if getattr(lora_a, "bias", None) is not None or getattr(lora_b, "bias", None) is not None:
+        raise TypeError(f"{name}: adapter linears with a bias")
+    A, B = lora_a.weight.data, lora_b.weight.data
+    if A.dtype != B.dtype or A.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"{name}: adapter weights must both be float32 or both bfloat16")
+    if A.shape[0] % 8 != 0 or A.shape[0] > 64 or not A.is_contiguous() or not B.is_contiguous():
+        raise TypeError(f"{name}: adapter rank {A.shape[0]} (a multiple of 8 up to 64)")
+    return A, B, float(scaling)
+
+
+def _projection(module, name: str):
+    """``(prepacked weight, adapter or None)`` of a bare int4 projection or a LoRA wrapper around one."""
+    if isinstance(module, Int4Linear):
+        return _plain_int4(module, name), None
+    base = getattr(module, "base_layer", None)
+    if not isinstance(base, Int4Linear) or not hasattr(module, "lora_A") or not hasattr(module, "lora_B"):
+        raise TypeError(f"{name} is {type(module).__name__}: neither an Int4Linear nor a LoRA wrapper around one")
+    return _plain_int4(base, name + ".base_layer"), _adapter_of(module, name)
 
 
 class NativeDecodeTrunk:
@@ -67,7 +118,7 @@ class NativeDecodeTrunk:
                 return f"hidden size {conf.hidden_size}"
             for i, layer in enumerate(trunk.layers):
                 attn, mlp = layer.self_attn, layer.mlp
-                packed = [_plain_int4(getattr(attn, n), f"layers[{i}].self_attn.{n}")
+                packed = [_projection(getattr(attn, n), f"layers[{i}].self_attn.{n}")[0]
                           for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
                 if not isinstance(mlp, Int4LlamaMLP) or getattr(mlp.gate_up, "_packed", None) is None:
                     return f"layers[{i}].mlp is not a prepacked fused int4 MLP"
@@ -130,25 +181,40 @@ class NativeDecodeTrunk:
                               (launch.table, len(launch.table), ctypes.byref(launch.norm))))
             return launch.outputs
 
-        def normed_gemv(module, weights, fused):
+        def lora(x, outs, adapters):
+            """outs[i] += adapter i applied to x, for the projections that carry one: two launches."""
+            todo = [(A, B, s, y) for y, ad in zip(outs, adapters) if ad is not None for A, B, s in [ad]]
+            if not todo:
+                return
+            launch = ops.LoraAdd(x, todo)
+            self._keep.append(launch)
+            n = len(launch.table)
+            calls.append((lib.vrl_lora_down_bf16, (x.data_ptr(), rows, x.shape[1], launch.table, n,
+                                                   launch.t.data_ptr())))
+            calls.append((lib.vrl_lora_up_add_bf16, (launch.t.data_ptr(), rows, launch.table, n)))
+
+        def normed_gemv(module, weights, fused, adapters=()):
             """h = res + x; the linears over norm(h); afterwards res = h."""
             w, eps = norm_weight(module)
             h_out = streams[state["flip"]]
             state["flip"] ^= 1
-            if fuse_norm:
+            if fuse_norm and not any(ad is not None for ad in adapters):
                 outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
             else:
                 calls.append((lib.vrl_add_rmsnorm_bf16,
                               (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,
                                w.data_ptr(), h_out.data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
                 outs = gemv([(self.normed, pw, fused) for pw in weights])
+                lora(self.normed, outs, adapters)   # adapters read the normalised row, so it is written out
             state["res"] = h_out
             return outs
 
         for i, layer in enumerate(trunk.layers):
             attn, mlp = layer.self_attn, layer.mlp
-            q, k, v = normed_gemv(layer.input_layernorm,
-                                  [attn.q_proj._packed, attn.k_proj._packed, attn.v_proj._packed], False)
+            proj = {n: _projection(getattr(attn, n), f"layers[{i}].self_attn.{n}")
+                    for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
+            q, k, v = normed_gemv(layer.input_layernorm, [proj[n][0] for n in ("q_proj", "k_proj", "v_proj")],
+                                  False, [proj[n][1] for n in ("q_proj", "k_proj", "v_proj")])
             if q.shape[1] != H * D or k.shape[1] != Hkv * D or v.shape[1] != Hkv * D:
                 raise TypeError(f"layers[{i}] projections do not match the attention geometry")
             keys, values = cache.layers[i].keys, cache.layers[i].values
@@ -160,7 +226,9 @@ class NativeDecodeTrunk:
                            values.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), mask.data_ptr(),
                            slot.data_ptr(), self.attn.data_ptr(), rows, H, Hkv, D, self.max_len,
                            float(attn.scaling))))
-            (state["x"],) = gemv([(self.attn, attn.o_proj._packed, False)])
+            outs = gemv([(self.attn, proj["o_proj"][0], False)])
+            lora(self.attn, outs, [proj["o_proj"][1]])
+            (state["x"],) = outs
             (act,) = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
             (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])
         w, eps = norm_weight(trunk.norm)

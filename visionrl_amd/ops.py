@@ -615,7 +615,8 @@ class LoraAdd:
     """LoRA adapters added onto the outputs of int4 projections that share an input: two launches.
 
     ``adapters`` is a list of ``(A [r, K], B [N, r], scaling, y [M, N])`` with ``A``/``B`` the
-    ``lora_A`` / ``lora_B`` weights of a PEFT wrapper (float32 or bfloat16, kept by reference: an
+    ``lora_A`` / ``lora_B`` weights of a PEFT wrapper (float32 or bfloat16, rank a multiple of 8 up
+    to 64, kept by reference: an
     in-place weight sync is seen by the next launch) and ``y`` the bf16 output of the base
     projection, updated in place: ``y += scaling * (x A^T) B^T`` with the roundings the wrapper's
     own forward applies (``vrl/models/families/janus_pro/policy.py:298-324`` attaches the adapters).
@@ -632,8 +633,8 @@ class LoraAdd:
         self.table = (_lib.LoraAdapter * len(adapters))()
         total = 0
         for rec, (A, B, scaling, y) in zip(self.table, adapters):
-            if A.dtype != B.dtype or A.dtype not in (torch.float32, torch.bfloat16):
-                raise ValueError("adapter weights must both be float32 or both bfloat16")
+            if A.dtype != B.dtype or A.dtype not in (torch.float32, torch.bfloat16) or A.dtype != adapters[0][0].dtype:
+                raise ValueError("adapter weights of one launch must all be float32 or all bfloat16")
             if A.dim() != 2 or B.dim() != 2 or A.shape[1] != K or B.shape[1] != A.shape[0] or \
                     not A.is_contiguous() or not B.is_contiguous():
                 raise ValueError(f"adapter weights must be contiguous A [r, {K}] and B [N, r]")
