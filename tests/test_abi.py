@@ -226,6 +226,28 @@ def test_decode_layer_validation(lib):
     assert call(kc=p + 8) == 1002 and call(pos=p + 4) == 1002
 
 
+def test_lora_validation(lib):
+    keep, p = buf(1 << 16)
+    ads = (_lib.LoraAdapter * 2)()
+    for ad in ads:
+        ad.A, ad.B, ad.y, ad.N, ad.r, ad.scaling, ad.weights_fp32 = p, p, p, 64, 8, 2.0, 1
+    down, up = lib.vrl_lora_down_bf16, lib.vrl_lora_up_add_bf16
+    assert down(None, 1, 256, ads, 2, p, None) == 1003 and down(p, 1, 256, None, 2, p, None) == 1003
+    assert down(p, 1, 256, ads, 2, None, None) == 1003 and up(None, 1, ads, 2, None) == 1003
+    assert down(p, 0, 256, ads, 2, p, None) == 1001 and down(p, 33, 256, ads, 2, p, None) == 1001   # rows
+    assert down(p, 1, 260, ads, 2, p, None) == 1001 and down(p, 1, 256, ads, 5, p, None) == 1001    # K % 8, adapters
+    ads[1].r = 12
+    assert down(p, 1, 256, ads, 2, p, None) == 1001       # rank % 8
+    ads[1].r = 72
+    assert down(p, 1, 256, ads, 2, p, None) == 1001       # rank beyond 64
+    ads[1].r, ads[1].weights_fp32 = 8, 0
+    assert down(p, 1, 256, ads, 2, p, None) == 1001       # one weight type per launch
+    ads[1].weights_fp32, ads[1].A = 1, p + 8
+    assert down(p, 1, 256, ads, 2, p, None) == 1002
+    ads[1].A, ads[1].y = p, None
+    assert up(p, 1, ads, 2, None) == 1003                 # the up-projection needs somewhere to add to
+
+
 def test_cfg_sample_validation(lib):
     keep, p = buf(4096)
     f = lib.vrl_cfg_sample_bf16
