@@ -183,17 +183,18 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
     for (int i = 0; i < VEC; ++i) a.acc[i] = a.acc[i] * c1 + acc2[i] * c2;
 }
 
-constexpr int ATT_THREADS = 1024;
-constexpr int ATT_WAVES = ATT_THREADS / WAVE;
-constexpr int ATT_UNROLL = 4;  // slots per 16-lane group in flight (keys and values: 8 vector loads per lane)
+constexpr int ATT_MAX_WAVES = 16;
 
-// One workgroup of 16 waves per (head, row).  Sixteen lanes share a cache slot (D / 16 values
+// One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
+// keep many requests in flight), 8 when there are at least two per CU (several then share a CU
+// and overlap each other's prologue and epilogue).  Sixteen lanes share a cache slot (D / 16 values
 // each), so a wave reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the
 // workgroup 64.  Every 16-lane group keeps its own running softmax over the slots it visits
 // (key and value loads of ATT_UNROLL slots are issued together: values do not wait for scores);
 // the groups, the waves and the new token's own slot are merged at the end.
-template <int D>
-__global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs a) {
+// ATT_UNROLL: slots per 16-lane group in flight (keys and values: 2 * ATT_UNROLL vector loads per lane)
+template <int D, int ATT_WAVES, int ATT_UNROLL>
+__global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnArgs a) {
     constexpr int VEC = D / 16;
     __shared__ float qs[D];                 // rotated query
     __shared__ float ks[D];                 // rotated key of the new token
@@ -212,6 +213,25 @@ __global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs 
     const int sub = lane >> 4, l16 = lane & 15;
     const long cache_base = ((long)m * a.n_kv_heads + hk) * a.L_max * D;
     const uint8_t *mask = a.mask + (long)m * a.L_max;
+    const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
+    const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
+    constexpr int STEP = 4 * ATT_WAVES * ATT_UNROLL;  // slots the workgroup visits per batch
+
+    // The cached slots do not depend on the new token: the first batch of keys and values is
+    // requested before anything else and arrives while the query is rotated.
+    RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
+    bool live[ATT_UNROLL];
+    auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs p >= 1
+#pragma unroll
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const int j = j0 + u * 4 * ATT_WAVES + wave * 4 + sub;
+            const int jj = j < p ? j : p - 1;  // slots past the end repeat the last one and are not counted
+            kraw[u] = load_raw<VEC>(kc + (long)jj * D);
+            vraw[u] = load_raw<VEC>(vc + (long)jj * D);
+            live[u] = j < p && mask[jj] != 0;
+        }
+    };
+    if (p > 0) request(0);
 
     if (tid < D) {
         const uint16_t *qrow = a.q + (long)m * a.q_stride + h * D;
@@ -243,27 +263,15 @@ __global__ __launch_bounds__(ATT_THREADS) void rope_attn_decode_kernel(AttnArgs 
         dot = wave_sum(dot);
         if (lane == 0) s_new = mask[p] ? dot * a.scaling : -INFINITY;
     }
-    const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
-    const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
-
     Partial<VEC> st;
     st.m = -INFINITY;
     st.l = 0.0f;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) st.acc[i] = 0.0f;
 
-    // cached slots 0..p-1: slot j0 + u * 64 + wave * 4 + sub for u = 0..ATT_UNROLL-1
-    for (int j0 = 0; j0 < p; j0 += 4 * ATT_WAVES * ATT_UNROLL) {
-        RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
-        bool live[ATT_UNROLL];
-#pragma unroll
-        for (int u = 0; u < ATT_UNROLL; ++u) {
-            const int j = j0 + u * 4 * ATT_WAVES + wave * 4 + sub;
-            const int jj = j < p ? j : p - 1;  // in range: the loop runs only when p >= 1
-            kraw[u] = load_raw<VEC>(kc + (long)jj * D);
-            vraw[u] = load_raw<VEC>(vc + (long)jj * D);
-            live[u] = j < p && mask[jj] != 0;
-        }
+    // cached slots 0..p-1, a batch per trip; the batch of the first trip is already on its way
+    for (int j0 = 0; j0 < p; j0 += STEP) {
+        if (j0 > 0) request(j0);
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             float dot = 0.0f;
@@ -552,10 +560,14 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
     a.L_max = L_max;
     a.scaling = scaling;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    if (D == 128)
-        hipLaunchKernelGGL(rope_attn_decode_kernel<128>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
-    else
-        hipLaunchKernelGGL(rope_attn_decode_kernel<64>, dim3(n_heads, M), dim3(ATT_THREADS), 0, stream, a);
+    const bool many = (long)n_heads * M >= 512;
+    const dim3 grid(n_heads, M);
+    // few workgroups: 16 waves each (256 slots per trip); many: 8 waves, several workgroups per CU
+    // (a deeper unroll of the 16-wave form, 512 slots per trip, measured slower)
+    if (D == 128 && many) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 8, 4>), grid, dim3(8 * WAVE), 0, stream, a);
+    else if (D == 128) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4>), grid, dim3(16 * WAVE), 0, stream, a);
+    else if (many) hipLaunchKernelGGL((rope_attn_decode_kernel<64, 8, 4>), grid, dim3(8 * WAVE), 0, stream, a);
+    else hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4>), grid, dim3(16 * WAVE), 0, stream, a);
     return (int)hipGetLastError();
 }
 
