@@ -23,17 +23,17 @@ HIDDEN, INTER, HEADS, LAYERS, VOCAB_IMG = 256, 512, 4, 2, 1024
 
 
 class StubMMGPT(nn.Module):
-    def __init__(self, dtype):
+    def __init__(self, dtype, hidden=HIDDEN, inter=INTER, heads=HEADS, layers=LAYERS, vocab=VOCAB_IMG, kv_heads=None):
         super().__init__()
         from transformers import LlamaConfig, LlamaModel
 
-        cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=LAYERS,
-                          num_attention_heads=HEADS, num_key_value_heads=HEADS, vocab_size=128,
-                          max_position_embeddings=256)
+        cfg = LlamaConfig(hidden_size=hidden, intermediate_size=inter, num_hidden_layers=layers,
+                          num_attention_heads=heads, num_key_value_heads=kv_heads or heads, vocab_size=128,
+                          max_position_embeddings=1024)
         torch.manual_seed(0)
         self.language_model = types.SimpleNamespace(model=LlamaModel(cfg).to(dtype).eval())
-        self.gen_head = nn.Linear(HIDDEN, VOCAB_IMG, bias=False).to(dtype)
-        self.gen_embed = nn.Embedding(VOCAB_IMG, HIDDEN).to(dtype)
+        self.gen_head = nn.Linear(hidden, vocab, bias=False).to(dtype)
+        self.gen_embed = nn.Embedding(vocab, hidden).to(dtype)
         with torch.no_grad():   # spread the logits so that draws are not all near-ties
             self.gen_head.weight.mul_(8.0)
 
@@ -42,8 +42,8 @@ class StubMMGPT(nn.Module):
 
 
 class StubPolicy:
-    def __init__(self, dtype=torch.float32, device="cpu"):
-        self.mmgpt = StubMMGPT(dtype)
+    def __init__(self, dtype=torch.float32, device="cpu", **shape):
+        self.mmgpt = StubMMGPT(dtype, **shape)
         self.mmgpt.language_model.model.to(device)
         self.mmgpt.to(device)
         self.config = types.SimpleNamespace(cfg_weight=5.0, temperature=1.0, image_token_num=12)
@@ -55,10 +55,10 @@ class StubPolicy:
         return self.mmgpt.language_model.model
 
 
-def make_inputs(B, n_text, dtype, device, seed=3):
+def make_inputs(B, n_text, dtype, device, seed=3, hidden=HIDDEN):
     g = torch.Generator().manual_seed(seed)
-    cond = torch.randn(B, n_text, HIDDEN, generator=g).to(dtype).to(device)
-    uncond = torch.randn(B, n_text, HIDDEN, generator=g).to(dtype).to(device)
+    cond = torch.randn(B, n_text, hidden, generator=g).to(dtype).to(device)
+    uncond = torch.randn(B, n_text, hidden, generator=g).to(dtype).to(device)
     cmask = torch.ones(B, n_text, dtype=torch.long)
     umask = torch.ones(B, n_text, dtype=torch.long)
     for b in range(B):   # left padding of different lengths, as the tokenizer produces
@@ -372,3 +372,62 @@ def test_graph_replays_equal_eager_steps_with_lora():
                                                                              image_token_num=16))
     torch.cuda.synchronize()
     assert torch.equal(out[0][0], out[1][0]) and torch.equal(out[0][1], out[1][1])
+
+
+# ------------------------------------------------------------------ the real layer shapes
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,kv_heads,lora", [(1, 16, False), (16, 16, False), (16, 4, True)])
+def test_native_trunk_at_janus_layer_shapes(B, kv_heads, lora):
+    """Two decoder layers of the Janus-Pro-1B geometry (2048 hidden, 16 heads of 128, 5632 intermediate,
+    16384 image tokens): the 128-wide heads, the row slabs of down_proj and the 32-row launches are on
+    the path here.  Native trunk against module trunk (teacher-forced), recorded graph against eager
+    steps, and the same seed sampling the same tokens twice (what the reference's own determinism test
+    asks of the loop, tests/engine/generation/test_pipeline_janus_pro.py:337-400)."""
+    from visionrl_amd.policy_glue import apply_int4_to_policy
+
+    print("ar decode: Janus layer shapes", B, kv_heads, lora, flush=True)
+    hidden = 2048
+    policy = StubPolicy(torch.bfloat16, "cuda:0", hidden=hidden, inter=5632, heads=16, layers=2, vocab=16384,
+                        kv_heads=kv_heads)
+    if lora:
+        torch.manual_seed(5)
+        for layer in policy._lm_trunk().layers:
+            for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
+                setattr(layer.self_attn, name,
+                        LoraWrapper(getattr(layer.self_attn, name), r=32, alpha=64).to("cuda:0"))
+    apply_int4_to_policy(policy, group_size=128)
+    rows, n_text, steps = 2 * B, 40, 5
+    cond, uncond, cmask, umask = make_inputs(B, n_text, torch.bfloat16, "cuda:0", seed=81, hidden=hidden)
+    sessions = []
+    for native in (True, False):
+        sampler = StaticARSampler(policy, graph=False, native=native)
+        torch.manual_seed(81)
+        sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=1)
+        (sess,) = sampler._sessions.values()
+        sessions.append(sess)
+    nat, mod = sessions
+    assert nat.native and not mod.native
+    trunk = policy._lm_trunk()
+    gen = torch.Generator(device="cuda:0").manual_seed(82)
+    with torch.no_grad():
+        for t in range(steps):
+            emb = torch.randn((rows, 1, hidden), generator=gen, device="cuda:0").to(torch.bfloat16)
+            nat.cur.copy_(emb)
+            got = nat.native.run().float().clone()
+            nat.slot.add_(1)
+            want = trunk(inputs_embeds=emb, attention_mask=mod.mask, use_cache=True,
+                         past_key_values=mod.cache).last_hidden_state[:, -1].float()
+            torch.cuda.synchronize()
+            err = (got - want).abs()
+            assert err.max().item() <= 0.1 and err.mean().item() <= 0.008, (t, err.max().item(), err.mean().item())
+    del sessions, nat, mod
+    out = []
+    for graph in (False, True, True):
+        torch.manual_seed(83)
+        out.append(StaticARSampler(policy, graph=graph).sample_image_tokens(cond, uncond, cmask, umask,
+                                                                             image_token_num=10))
+    torch.cuda.synchronize()
+    for tokens, logprobs in out[1:]:
+        assert torch.equal(tokens, out[0][0]) and torch.equal(logprobs, out[0][1])
+    assert out[0][0].shape == (B, 10) and (out[0][0] >= 0).all() and (out[0][0] < 16384).all()
+    assert (out[0][1] <= 0).all() and torch.isfinite(out[0][1]).all()
