@@ -158,6 +158,111 @@ def test_install_replaces_the_policy_method():
     assert torch.equal(got[0], want[0]) and policy._static_ar_sampler is sampler
 
 
+# ------------------------------------------------------------------ the step API under a token scheduler
+class Seq:
+    """What ``step_ar`` reads of the scheduler's ``ActiveSequence`` (vrl/engine/ar/sequence.py:21-61)."""
+
+    def __init__(self, row, max_new_tokens):
+        self.sample_id, self.metadata, self.position, self.max_new_tokens = f"s{row}", {"row_index": row}, 0, max_new_tokens
+
+    @property
+    def finished(self):
+        return self.position >= self.max_new_tokens
+
+
+def scheduled_loop(policy, inputs, n_img, batch_size):
+    """The executor's loop (vrl/models/families/janus_pro/executor.py:373-413) with the scheduler's
+    grouping (vrl/engine/ar/token_scheduler.py:59-90): first pending position, at most batch_size rows."""
+    state = policy.init_ar_state(*inputs, cfg_weight=5.0, temperature=1.0, image_token_num=n_img)
+    pending = [Seq(row, n_img) for row in range(inputs[0].shape[0])]
+    results = []
+    while pending:
+        position = pending[0].position
+        batch = [seq for seq in pending if seq.position == position][:batch_size]
+        results.append(policy.step_ar(state, batch))
+        for seq in batch:
+            seq.position += 1
+        chosen = {id(seq) for seq in batch}
+        pending = [seq for seq in pending if id(seq) not in chosen] + [seq for seq in batch if not seq.finished]
+    return policy.finalize_ar_state(state), results
+
+
+def test_step_api_in_lockstep_samples_what_the_reference_loop_samples():
+    policy = StubPolicy()
+    inputs = make_inputs(3, 6, torch.float32, "cpu", seed=9)
+    torch.manual_seed(13)
+    want_t, want_lp = reference_loop(policy, *inputs, 5.0, 1.0, 7)
+    install_static_ar_sampler(policy, graph=False, fused_tail=False)
+    torch.manual_seed(13)
+    (got_t, got_lp), results = scheduled_loop(policy, inputs, 7, batch_size=3)
+    assert torch.equal(got_t, want_t)
+    torch.testing.assert_close(got_lp, want_lp, rtol=1e-5, atol=1e-5)
+    assert len(results) == 7
+    for p, res in enumerate(results):      # the per-step results carry the same tokens, in row order
+        assert res.sequence_ids == ["s0", "s1", "s2"] and res.positions == [p] * 3
+        assert torch.equal(res.token, want_t[:, p]) and res.replay_extras == {}
+        torch.testing.assert_close(res.log_prob, want_lp[:, p], rtol=1e-5, atol=1e-5)
+
+
+def test_step_api_contract():
+    policy = StubPolicy()
+    inputs = make_inputs(3, 6, torch.float32, "cpu", seed=9)
+    sampler = install_static_ar_sampler(policy, graph=False, fused_tail=False)
+    state = policy.init_ar_state(*inputs, image_token_num=2)
+    seqs = [Seq(row, 2) for row in range(3)]
+    with pytest.raises(ValueError, match="at least one"):
+        policy.step_ar(state, [])
+    with pytest.raises(ValueError, match="row indices"):
+        policy.step_ar(state, [Seq(7, 2)])
+    with pytest.raises(ValueError, match="together"):
+        policy.step_ar(state, seqs[:2])                  # this stand-in has no step functions of its own to take over
+    seqs[1].position = 1
+    with pytest.raises(ValueError, match="positions must match within"):
+        policy.step_ar(state, seqs)
+    seqs[1].position = 0
+    policy.step_ar(state, seqs)
+    with pytest.raises(ValueError, match="state's position"):
+        policy.step_ar(state, seqs)                      # the sequences were not advanced
+    for seq in seqs:
+        seq.position = 1
+    policy.step_ar(state, seqs)
+    for seq in seqs:
+        seq.position = 2
+    with pytest.raises(ValueError, match="finished"):
+        policy.step_ar(state, seqs)
+    tokens, logprobs = policy.finalize_ar_state(state)
+    assert tokens.shape == (3, 2) and torch.equal(tokens, state.token_ids) and sampler is policy._static_ar_sampler
+
+
+def test_partial_batches_go_to_the_policys_own_step_functions():
+    calls = []
+
+    class WithStepApi(StubPolicy):
+        def init_ar_state(self, *args, **kwargs):
+            calls.append(("init", kwargs["image_token_num"]))
+            return {"steps": 0}
+
+        def step_ar(self, state, sequences, *, generator=None):
+            state["steps"] += 1
+            calls.append(("step", [seq.metadata["row_index"] for seq in sequences]))
+            return "their result"
+
+        def finalize_ar_state(self, state):
+            return "their tokens", state["steps"]
+
+    policy = WithStepApi()
+    inputs = make_inputs(3, 6, torch.float32, "cpu", seed=9)
+    install_static_ar_sampler(policy, graph=False, fused_tail=False)
+    final, results = scheduled_loop(policy, inputs, 2, batch_size=2)
+    assert final == ("their tokens", 4) and results == ["their result"] * 4
+    assert calls == [("init", 2), ("step", [0, 1]), ("step", [2]), ("step", [0, 1]), ("step", [2])]
+    # a full batch keeps the static loop, whatever the policy has
+    calls.clear()
+    torch.manual_seed(1)
+    (tokens, _), _ = scheduled_loop(policy, inputs, 2, batch_size=3)
+    assert calls == [] and tokens.shape == (3, 2)
+
+
 # ------------------------------------------------------------------ GPU: int4 modules, fused tail, HIP graph
 @pytest.fixture(scope="module")
 def int4_policy():
@@ -358,6 +463,25 @@ def test_native_trunk_with_lora_adapters_tracks_the_module_trunk(dtype):
     assert torch.equal(bare.lora_B["default"].weight.data, state["layers.0.self_attn.q_proj.lora_B.default.weight"])
     after = compare(steps)          # same launches, same pointers, new adapter values: still tracks the modules
     assert (after - before).abs().max().item() > 0.1
+
+
+@pytest.mark.gpu
+def test_step_api_with_recorded_steps_equals_sample_image_tokens(int4_policy):
+    """The scheduler-driven form over recorded graphs: same tokens as one ``sample_image_tokens`` call,
+    twice in a row (the second generation replays from its first decode step on)."""
+    print("ar decode: step API over graphs", flush=True)
+    inputs = make_inputs(3, 7, torch.bfloat16, "cuda:0", seed=91)
+    sampler = StaticARSampler(int4_policy, graph=True)
+    holder = types.SimpleNamespace(init_ar_state=sampler.init_ar_state, step_ar=sampler.step_ar,
+                                   finalize_ar_state=sampler.finalize_ar_state)
+    for seed in (92, 93):
+        torch.manual_seed(seed)
+        want = StaticARSampler(int4_policy, graph=False).sample_image_tokens(*inputs, image_token_num=9)
+        torch.manual_seed(seed)
+        got, results = scheduled_loop(holder, inputs, 9, batch_size=3)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        assert torch.equal(torch.stack([r.token for r in results], dim=1), want[0])
 
 
 @pytest.mark.gpu

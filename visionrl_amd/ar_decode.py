@@ -27,12 +27,16 @@ arguments, the same results and the same use of the random stream:
   (``vrl/models/families/janus_pro/executor.py:147-151`` seeds the global generator) samples the
   same tokens as the reference loop.
 
-Rows that advance at different positions (the ``step_ar`` contract used with the token scheduler,
-``policy.py:527-572``) are not covered: that path keeps the reference implementation.
+The step API the executor's token scheduler drives (``init_ar_state`` / ``step_ar`` /
+``finalize_ar_state``, ``policy.py:527-622``, ``executor.py:373-413``) is covered for what the
+scheduler does by default: every row of the chunk stepped together at one position.  A generation
+whose scheduler batch is smaller than the chunk (rows at different positions) is handed to the
+policy's own step functions.
 """
 
 from __future__ import annotations
 
+import dataclasses
 import types
 from typing import Any
 
@@ -42,11 +46,47 @@ import torch.nn.functional as F
 from . import ops
 from .decode_step import NativeDecodeTrunk
 
-__all__ = ["StaticARSampler", "install_static_ar_sampler"]
+__all__ = ["StaticARSampler", "StaticARState", "StaticARStepResult", "install_static_ar_sampler"]
 
 
 def _round_up(n: int, to: int) -> int:
     return (n + to - 1) // to * to
+
+
+@dataclasses.dataclass
+class StaticARStepResult:
+    """Fields of the reference's ``ARStepResult`` (``vrl/models/ar.py:26-39``)."""
+
+    sequence_ids: list
+    positions: list
+    token: Any
+    log_prob: Any
+    replay_extras: dict = dataclasses.field(default_factory=dict)
+
+
+@dataclasses.dataclass
+class StaticARState:
+    """What ``init_ar_state`` hands to ``step_ar`` / ``finalize_ar_state``: the rows of one chunk,
+    advancing together over one static cache (the counterpart of ``JanusProARState``,
+    ``policy.py:114-130``, whose per-row caches and masks have no equivalent here)."""
+
+    session: Any
+    inputs: Any                    # prompt embeddings and masks until the first step consumed them
+    cfg_weight: float
+    temperature: float
+    image_token_num: int
+    batch_size: int
+    position: int = 0
+    reference: Any = None          # the policy's own (init_ar_state, step_ar, finalize_ar_state), if it has them
+    delegate: Any = None           # their state, once a partial batch sent the generation their way
+
+    @property
+    def token_ids(self) -> torch.Tensor:
+        return self.session.tokens[:, :self.image_token_num]
+
+    @property
+    def logprobs(self) -> torch.Tensor:
+        return self.session.logprobs[:, :self.image_token_num]
 
 
 class _Session:
@@ -179,12 +219,13 @@ class StaticARSampler:
         self._sessions[key] = sess
         return sess
 
+    # -- the step API (init_ar_state / step_ar / finalize_ar_state, policy.py:527-622) ---------------
     @torch.no_grad()
-    def sample_image_tokens(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,
-                            cond_attention_mask: torch.Tensor, uncond_attention_mask: torch.Tensor, *,
-                            cfg_weight: float | None = None, temperature: float | None = None,
-                            image_token_num: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
-        """Returns ``(image_token_ids int64 [B, L_img], logprobs float32 [B, L_img])``."""
+    def init_ar_state(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,
+                      cond_attention_mask: torch.Tensor, uncond_attention_mask: torch.Tensor, *,
+                      cfg_weight: float | None = None, temperature: float | None = None,
+                      image_token_num: int | None = None) -> "StaticARState":
+        """State for a generation whose rows advance together; nothing runs until the first step."""
         cfg, temp, n_img = self._defaults(cfg_weight, temperature, image_token_num)
         if cond_inputs_embeds.dim() != 3 or cond_inputs_embeds.shape != uncond_inputs_embeds.shape:
             raise ValueError("cond and uncond embeddings must both be [B, L_text, H]")
@@ -193,31 +234,104 @@ class StaticARSampler:
             raise ValueError("attention masks must be [B, L_text]")
         device, dtype = cond_inputs_embeds.device, cond_inputs_embeds.dtype
         max_len = _round_up(n_text + n_img, self.length_bucket)
-        use_graph = self.graph and device.type == "cuda"
         key = (2 * B, hidden, max_len, dtype, device, cfg, temp, cond_attention_mask.dtype)
         sess = self._session(key, lambda: _Session(self, 2 * B, hidden, max_len, dtype, device, cfg, temp,
                                                    cond_attention_mask.dtype))
-        sess.begin(torch.cat([cond_attention_mask, uncond_attention_mask], dim=0))
-        sess.prefill(torch.cat([cond_inputs_embeds, uncond_inputs_embeds], dim=0))
-        left = n_img - 1
-        if use_graph and left > 0:
+        return StaticARState(session=sess, inputs=(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                                                   uncond_attention_mask),
+                             cfg_weight=cfg, temperature=temp, image_token_num=n_img, batch_size=B)
+
+    def _advance(self, state: "StaticARState") -> None:
+        """One token for every row: the prompt pass first, then eager / recorded decode steps."""
+        sess = state.session
+        if state.position >= state.image_token_num:
+            raise ValueError("the generation has already finished sampling")
+        if state.position == 0:
+            cond, uncond, cmask, umask = state.inputs
+            sess.begin(torch.cat([cmask, umask], dim=0))
+            sess.prefill(torch.cat([cond, uncond], dim=0))
+            state.inputs = None
+        elif self.graph and sess.cur.is_cuda:
+            if sess.graph is None and state.position >= 2:
+                sess.capture()           # after one eager decode step: records, does not run
             if sess.graph is None:
-                sess.step()          # a real step, and the warm-up the capture needs
-                left -= 1
-                if left > 0:
-                    sess.capture()   # records, does not run
-            for _ in range(left):
+                sess.step()              # a real step, and the warm-up the capture needs
+            else:
                 sess.graph.replay()
         else:
-            for _ in range(left):
-                sess.step()
-        return sess.tokens[:, :n_img].clone(), sess.logprobs[:, :n_img].clone()
+            sess.step()
+        state.position += 1
+
+    @torch.no_grad()
+    def step_ar(self, state: "StaticARState", sequences, *, generator=None) -> "StaticARStepResult":
+        """One scheduled token step (``JanusProPolicy.step_ar``, ``policy.py:527-572``) for all rows at once.
+
+        ``sequences`` are the scheduler's active sequences (``metadata["row_index"]``, ``position``,
+        ``sample_id``).  The token scheduler hands over every row of a chunk at one position unless
+        it was given a smaller batch size (``executor.py:396-413``); a partial batch on the first
+        step switches the whole generation to the policy's own step functions, later it is an error.
+        """
+        del generator   # like the reference: the draw uses the global generator
+        if not sequences:
+            raise ValueError("step_ar requires at least one ActiveSequence")
+        if state.delegate is not None:
+            return state.reference[1](state.delegate, sequences)
+        B = state.batch_size
+        rows = [int(seq.metadata.get("row_index", -1)) for seq in sequences]
+        if any(row < 0 or row >= B for row in rows):
+            raise ValueError(f"invalid Janus row indices: {rows}")
+        positions = [int(seq.position) for seq in sequences]
+        if len(set(positions)) != 1:
+            raise ValueError("ActiveSequence positions must match within one AR step")
+        if rows != list(range(B)):
+            if state.position == 0 and state.reference is not None:
+                cond, uncond, cmask, umask = state.inputs
+                state.delegate = state.reference[0](cond, uncond, cmask, umask, cfg_weight=state.cfg_weight,
+                                                    temperature=state.temperature,
+                                                    image_token_num=state.image_token_num)
+                return state.reference[1](state.delegate, sequences)
+            raise ValueError("the static decode loop steps all rows of a chunk together, in row order; "
+                             f"got rows {rows} of {B}")
+        if positions[0] != state.position:
+            raise ValueError("ActiveSequence positions must match the state's position")
+        p = state.position
+        self._advance(state)
+        sess = state.session
+        return StaticARStepResult(sequence_ids=[str(seq.sample_id) for seq in sequences], positions=positions,
+                                  token=sess.tokens[:, p].clone(), log_prob=sess.logprobs[:, p].clone())
+
+    @torch.no_grad()
+    def finalize_ar_state(self, state: "StaticARState") -> tuple[torch.Tensor, torch.Tensor]:
+        """``(image_token_ids, logprobs)`` of the rows sampled so far up to ``image_token_num``."""
+        if state.delegate is not None:
+            return state.reference[2](state.delegate)
+        n = state.image_token_num
+        return state.session.tokens[:, :n].clone(), state.session.logprobs[:, :n].clone()
+
+    @torch.no_grad()
+    def sample_image_tokens(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,
+                            cond_attention_mask: torch.Tensor, uncond_attention_mask: torch.Tensor, *,
+                            cfg_weight: float | None = None, temperature: float | None = None,
+                            image_token_num: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """Returns ``(image_token_ids int64 [B, L_img], logprobs float32 [B, L_img])``."""
+        state = self.init_ar_state(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                                   uncond_attention_mask, cfg_weight=cfg_weight, temperature=temperature,
+                                   image_token_num=image_token_num)
+        while state.position < state.image_token_num:
+            self._advance(state)
+        return self.finalize_ar_state(state)
 
 
 def install_static_ar_sampler(policy: Any, **options) -> StaticARSampler:
-    """Make ``policy.sample_image_tokens`` (what ``JanusProPipelineExecutor.forward`` calls,
-    ``vrl/models/families/janus_pro/executor.py:197-203``) run through a :class:`StaticARSampler`."""
+    """Route ``policy.sample_image_tokens`` (what ``JanusProPipelineExecutor.forward`` calls,
+    ``vrl/models/families/janus_pro/executor.py:197-203``) and the step API the executor's token
+    scheduler drives (``init_ar_state`` / ``step_ar`` / ``finalize_ar_state``, ``executor.py:373-413``)
+    through a :class:`StaticARSampler`.  The policy's own step functions, if it has them, stay
+    reachable: a generation whose first scheduled batch is not the whole chunk is handed to them."""
     sampler = StaticARSampler(policy, **options)
+    names = ("init_ar_state", "step_ar", "finalize_ar_state")
+    reference = tuple(getattr(policy, name, None) for name in names)
+    reference = reference if all(callable(fn) for fn in reference) else None
 
     def sample_image_tokens(self, cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
                             uncond_attention_mask, *, cfg_weight=None, temperature=None, image_token_num=None):
@@ -225,6 +339,23 @@ def install_static_ar_sampler(policy: Any, **options) -> StaticARSampler:
                                            uncond_attention_mask, cfg_weight=cfg_weight,
                                            temperature=temperature, image_token_num=image_token_num)
 
+    def init_ar_state(self, cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask, uncond_attention_mask, *,
+                      cfg_weight=None, temperature=None, image_token_num=None):
+        state = sampler.init_ar_state(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                                      uncond_attention_mask, cfg_weight=cfg_weight, temperature=temperature,
+                                      image_token_num=image_token_num)
+        state.reference = reference
+        return state
+
+    def step_ar(self, state, sequences, *, generator=None):
+        return sampler.step_ar(state, sequences, generator=generator)
+
+    def finalize_ar_state(self, state):
+        return sampler.finalize_ar_state(state)
+
     policy.sample_image_tokens = types.MethodType(sample_image_tokens, policy)
+    policy.init_ar_state = types.MethodType(init_ar_state, policy)
+    policy.step_ar = types.MethodType(step_ar, policy)
+    policy.finalize_ar_state = types.MethodType(finalize_ar_state, policy)
     policy._static_ar_sampler = sampler
     return sampler
