@@ -80,6 +80,32 @@ __device__ __forceinline__ void block_reduce2(float &a, float &b, float (*lds)[W
     }
 }
 
+// VEC = 8: every thread takes 8 consecutive vocabulary entries per step with 16-byte loads, all
+// steps of a walk requested before the first is used (V % 8 == 0, 16-byte aligned rows); VEC = 1
+// is the form for any V.
+template <int VEC>
+__device__ __forceinline__ void load_entries(const uint16_t *p, uint16_t (&v)[VEC]) {
+    if constexpr (VEC == 8) {
+        const uint4 w = *reinterpret_cast<const uint4 *>(p);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[2 * e] = (uint16_t)(u[e] & 0xFFFFu);
+            v[2 * e + 1] = (uint16_t)(u[e] >> 16);
+        }
+    } else {
+        v[0] = *p;
+    }
+}
+
+__device__ __forceinline__ void scaled_pair(float c, float u, float w, float inv_t, float &gt, float &ct) {
+    const float d = round_bf16(c - u);
+    const float g = round_bf16(u + round_bf16(w * d));
+    gt = round_bf16(g * inv_t);
+    ct = round_bf16(c * inv_t);
+}
+
+template <int VEC>
 __global__ __launch_bounds__(THREADS) void cfg_sample_kernel(const uint16_t *__restrict__ logits,
                                                              const uint16_t *__restrict__ noise,
                                                              long long *__restrict__ sampled,
@@ -94,37 +120,60 @@ __global__ __launch_bounds__(THREADS) void cfg_sample_kernel(const uint16_t *__r
     r.uncond = logits + (long)(B + b) * V;
     r.noise = noise + (long)b * V;
 
+    constexpr int STEP = THREADS * VEC;
     // walk 1: maxima of guided / T and of cond / T
     float mg = -INFINITY, mc = -INFINITY;
-    for (int i = threadIdx.x; i < V; i += THREADS) {
-        float gt, ct;
-        scaled_logits(r, i, w, inv_t, gt, ct);
-        mg = fmaxf(mg, gt);
-        mc = fmaxf(mc, ct);
+#pragma unroll 4
+    for (int i = threadIdx.x * VEC; i < V; i += STEP) {
+        uint16_t cb[VEC], ub[VEC];
+        load_entries<VEC>(r.cond + i, cb);
+        load_entries<VEC>(r.uncond + i, ub);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float gt, ct;
+            scaled_pair(bf16_to_f32(cb[e]), bf16_to_f32(ub[e]), w, inv_t, gt, ct);
+            mg = fmaxf(mg, gt);
+            mc = fmaxf(mc, ct);
+        }
     }
     block_reduce2<true>(mg, mc, red);
 
     // walk 2: the two softmax denominators
     float sg = 0.0f, sc = 0.0f;
-    for (int i = threadIdx.x; i < V; i += THREADS) {
-        float gt, ct;
-        scaled_logits(r, i, w, inv_t, gt, ct);
-        sg += expf(gt - mg);
-        sc += expf(ct - mc);
+#pragma unroll 4
+    for (int i = threadIdx.x * VEC; i < V; i += STEP) {
+        uint16_t cb[VEC], ub[VEC];
+        load_entries<VEC>(r.cond + i, cb);
+        load_entries<VEC>(r.uncond + i, ub);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float gt, ct;
+            scaled_pair(bf16_to_f32(cb[e]), bf16_to_f32(ub[e]), w, inv_t, gt, ct);
+            sg += expf(gt - mg);
+            sc += expf(ct - mc);
+        }
     }
     block_reduce2<false>(sg, sc, red);
 
     // walk 3: argmax of probs / q, lowest index among equal maxima
     float bv = -INFINITY;
     int bi = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < V; i += THREADS) {
-        float gt, ct;
-        scaled_logits(r, i, w, inv_t, gt, ct);
-        const float p = round_bf16(expf(gt - mg) / sg);
-        const float ratio = round_bf16(p / bf16_to_f32(r.noise[i]));
-        if (ratio > bv || (ratio == bv && i < bi) || (ratio != ratio && bv == bv)) {
-            bv = ratio;   // a NaN ratio wins over numbers, as in torch's argmax
-            bi = i;
+#pragma unroll 4
+    for (int i = threadIdx.x * VEC; i < V; i += STEP) {
+        uint16_t cb[VEC], ub[VEC], nb[VEC];
+        load_entries<VEC>(r.cond + i, cb);
+        load_entries<VEC>(r.uncond + i, ub);
+        load_entries<VEC>(r.noise + i, nb);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float gt, ct;
+            scaled_pair(bf16_to_f32(cb[e]), bf16_to_f32(ub[e]), w, inv_t, gt, ct);
+            const float p = round_bf16(expf(gt - mg) / sg);
+            const float ratio = round_bf16(p / bf16_to_f32(nb[e]));
+            if (ratio > bv || (ratio == bv && i + e < bi) || (ratio != ratio && bv == bv)) {
+                bv = ratio;   // a NaN ratio wins over numbers, as in torch's argmax
+                bi = i + e;
+            }
         }
     }
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
@@ -172,7 +221,9 @@ extern "C" int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_
     if ((reinterpret_cast<uintptr_t>(logits) & 1u) || (reinterpret_cast<uintptr_t>(noise) & 1u) ||
         (reinterpret_cast<uintptr_t>(sampled) & 7u) || (reinterpret_cast<uintptr_t>(logprob) & 3u))
         return VRL_INT4_EALIGN;
-    hipLaunchKernelGGL(cfg_sample_kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
+    const bool wide = V % 8 == 0 && ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(noise)) & 15u) == 0;
+    auto kernel = wide ? &cfg_sample_kernel<8> : &cfg_sample_kernel<1>;
+    hipLaunchKernelGGL(kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint16_t *>(logits), static_cast<const uint16_t *>(noise),
                        reinterpret_cast<long long *>(sampled), logprob, B, V, cfg_weight, 1.0f / temperature);
     return (int)hipGetLastError();
