@@ -500,18 +500,20 @@ def test_graph_replays_equal_eager_steps_with_lora():
 
 # ------------------------------------------------------------------ the real layer shapes
 @pytest.mark.gpu
-@pytest.mark.parametrize("B,kv_heads,lora", [(1, 16, False), (16, 16, False), (16, 4, True)])
-def test_native_trunk_at_janus_layer_shapes(B, kv_heads, lora):
+@pytest.mark.parametrize("B,kv_heads,lora,hidden,inter,heads", [
+    (1, 16, False, 2048, 5632, 16), (16, 16, False, 2048, 5632, 16), (16, 4, True, 2048, 5632, 16),
+    (1, 32, False, 4096, 11008, 32), (16, 32, True, 4096, 11008, 32),      # the 7B-class layer
+])
+def test_native_trunk_at_janus_layer_shapes(B, kv_heads, lora, hidden, inter, heads):
     """Two decoder layers of the Janus-Pro-1B geometry (2048 hidden, 16 heads of 128, 5632 intermediate,
-    16384 image tokens): the 128-wide heads, the row slabs of down_proj and the 32-row launches are on
-    the path here.  Native trunk against module trunk (teacher-forced), recorded graph against eager
+    16384 image tokens) and of the 7B-class one (4096, 32 heads, 11008): the 128-wide heads, the row
+    slabs of down_proj, the 32-row launches and the 4096-wide normalising launches are on the path here.  Native trunk against module trunk (teacher-forced), recorded graph against eager
     steps, and the same seed sampling the same tokens twice (what the reference's own determinism test
     asks of the loop, tests/engine/generation/test_pipeline_janus_pro.py:337-400)."""
     from visionrl_amd.policy_glue import apply_int4_to_policy
 
-    print("ar decode: Janus layer shapes", B, kv_heads, lora, flush=True)
-    hidden = 2048
-    policy = StubPolicy(torch.bfloat16, "cuda:0", hidden=hidden, inter=5632, heads=16, layers=2, vocab=16384,
+    print("ar decode: Janus layer shapes", B, kv_heads, lora, hidden, inter, heads, flush=True)
+    policy = StubPolicy(torch.bfloat16, "cuda:0", hidden=hidden, inter=inter, heads=heads, layers=2, vocab=16384,
                         kv_heads=kv_heads)
     if lora:
         torch.manual_seed(5)
