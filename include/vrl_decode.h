@@ -86,6 +86,32 @@ int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adap
 int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
                          void *hip_stream);
 
+/*
+ * vrl_rope_attn_decode_bf16 with the up-projections of the q, k, v adapters added while the new
+ * token's projections are read, in place of a vrl_lora_up_add_bf16 launch between the int4 launch
+ * and the attention: q, k, v hold the base projections' outputs, `t` the down-projections of the
+ * group (vrl_lora_down_bf16), and the kernel attends with (and appends to the cache)
+ *   q' = bf16(q + scaling_q * t[:, off_q : off_q + r_q] . B_q^T), likewise k', v'
+ * with the roundings described above.  A NULL B means the projection has no adapter; at least one
+ * must be given.  q, k and v themselves are left as they are.
+ */
+typedef struct vrl_attn_lora {
+    const float *t;          /* [M, t_stride] float32, 16-byte aligned */
+    int32_t t_stride;        /* a multiple of 4 */
+    int32_t weights_fp32;    /* type of every B: 1 float32, 0 bf16 */
+    const void *q_B, *k_B, *v_B;   /* [n_heads * D, r_q], [n_kv_heads * D, r_k], [n_kv_heads * D, r_v] */
+    int32_t r[3];            /* ranks (q, k, v): multiples of 8 up to 64 */
+    int32_t offset[3];       /* first column of each adapter in t, a multiple of 4 */
+    float scaling[3];
+    int32_t reserved;
+} vrl_attn_lora;
+
+int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                   void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                   const void *mask, const int64_t *position, void *out,
+                                   int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                   const vrl_attn_lora *lora, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

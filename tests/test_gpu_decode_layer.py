@@ -283,3 +283,54 @@ def test_lora_add_sees_in_place_weight_updates_and_rejects_misuse(ops_mod):
         ops_mod.LoraAdd(xt, [(A[:4].contiguous(), B[:, :4].contiguous(), 2.0, yt)]).launch()   # rank % 8
     with pytest.raises(ValueError):
         ops_mod.LoraAdd(xt, [(A, B, 2.0, yt), (A.to(torch.bfloat16), B.to(torch.bfloat16), 2.0, yt)])   # one type per launch
+
+
+@pytest.mark.parametrize("M,H,Hkv,D,fp32,which", [(2, 16, 16, 128, True, "qkv"), (32, 16, 16, 128, True, "qkv"),
+                                                   (3, 8, 2, 64, False, "qv"), (5, 4, 4, 64, True, "k")])
+def test_attention_adds_the_qkv_adapters_itself(ops_mod, M, H, Hkv, D, fp32, which):
+    """``rope_attn_decode(..., lora=group)`` against the two-launch form (up-projection onto q, k, v,
+    then the plain attention): the appended cache rows and the output agree to a rounding of the
+    adapter sums' order."""
+    say("attention with adapters", M, H, Hkv, D, fp32, which)
+    L, p, K, r = 96, 41, 256, 16
+    c = attn_case(300 + M, M, H, Hkv, D, L, p)
+    rng = np.random.default_rng(M + D)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    x = bits_to_bf16(rand_bits(rng, (M, K)), DEV)
+    t = {n: bits_to_bf16(c[n], DEV) for n in ("q", "k", "v", "cos", "sin")}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([p], dtype=torch.int64, device=DEV)
+
+    def adapters(q, k, v):
+        gen = torch.Generator().manual_seed(5)
+        ads = []
+        for name, y in (("q", q), ("k", k), ("v", v)):
+            if name in which:
+                A = (torch.randn(r, K, generator=gen) * K ** -0.5).to(dtype).to(DEV)
+                B = (torch.randn(y.shape[1], r, generator=gen) * 0.2).to(dtype).to(DEV)
+                ads.append((A, B, 2.0, y))
+        return ads
+
+    # two launches: y += up(down(x)), then attention
+    q1, k1, v1 = t["q"].clone(), t["k"].clone(), t["v"].clone()
+    kc1, vc1 = bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV)
+    ops_mod.LoraAdd(x, adapters(q1, k1, v1)).launch()
+    want = ops_mod.rope_attn_decode(q1, k1, v1, kc1, vc1, t["cos"], t["sin"], mask, pos, c["scaling"])
+    # one: down only, the attention adds the rest
+    q2, k2, v2 = t["q"].clone(), t["k"].clone(), t["v"].clone()
+    kc2, vc2 = bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV)
+    group = ops_mod.LoraAdd(x, adapters(q2, k2, v2))
+    group.launch_down()
+    got = ops_mod.rope_attn_decode(q2, k2, v2, kc2, vc2, t["cos"], t["sin"], mask, pos, c["scaling"], lora=group)
+    torch.cuda.synchronize()
+    assert torch.equal(q2, t["q"]) and torch.equal(k2, t["k"]) and torch.equal(v2, t["v"])   # inputs untouched
+    assert not torch.equal(q1, t["q"]) or "q" not in which
+    for a, b in ((kc2, kc1), (vc2, vc1)):
+        assert torch.equal(a[:, :, :p], b[:, :, :p]) and torch.equal(a[:, :, p + 1:], b[:, :, p + 1:])
+        within_one_step_of(bf16_to_bits(a[:, :, p]), bf16_to_bits(b[:, :, p]), bf16_to_bits(b[:, :, p]))
+        assert (a[:, :, p] != b[:, :, p]).float().mean().item() < 0.02
+    diff = (got.float() - want.float()).abs()
+    assert diff.max().item() <= 2.0 ** -6 * max(1.0, want.float().abs().max().item())
+    assert (got != want).float().mean().item() < 0.05
+    with pytest.raises(ValueError):   # a group over other outputs
+        ops_mod.rope_attn_decode(q1, k1, v1, kc1, vc1, t["cos"], t["sin"], mask, pos, c["scaling"], lora=group)

@@ -31,6 +31,7 @@ SYMBOLS = (
     "vrl_cfg_sample_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
+    "vrl_rope_attn_decode_lora_bf16",
     "vrl_lora_down_bf16",
     "vrl_lora_up_add_bf16",
 )
@@ -86,6 +87,23 @@ class LoraAdapter(ctypes.Structure):
     ]
 
 
+class AttnLora(ctypes.Structure):
+    """Mirror of ``vrl_attn_lora``."""
+
+    _fields_ = [
+        ("t", ctypes.c_void_p),
+        ("t_stride", ctypes.c_int32),
+        ("weights_fp32", ctypes.c_int32),
+        ("q_B", ctypes.c_void_p),
+        ("k_B", ctypes.c_void_p),
+        ("v_B", ctypes.c_void_p),
+        ("r", ctypes.c_int32 * 3),
+        ("offset", ctypes.c_int32 * 3),
+        ("scaling", ctypes.c_float * 3),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
 class PlanInfo(ctypes.Structure):
     """Mirror of ``vrl_int4_plan_info``."""
 
@@ -135,6 +153,10 @@ def _bind(lib):
     lib.vrl_cfg_sample_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_float, ctypes.c_float, vp]
     lib.vrl_add_rmsnorm_bf16.restype = ci
     lib.vrl_add_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_float, vp]
+    lib.vrl_rope_attn_decode_lora_bf16.restype = ci
+    lib.vrl_rope_attn_decode_lora_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
+                                                   ci, ci, ci, ci, ci, ctypes.c_float,
+                                                   ctypes.POINTER(AttnLora), vp]
     lib.vrl_lora_down_bf16.restype = ci
     lib.vrl_lora_down_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
     lib.vrl_lora_up_add_bf16.restype = ci

@@ -26,6 +26,7 @@ constexpr int THREADS = 256;
 constexpr int WAVES = THREADS / WAVE;
 constexpr int MAX_NORM_K = 16384;
 constexpr int MAX_CACHE_LEN = 8192;
+constexpr int LORA_MAX_RANK = 64;
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
 
@@ -144,6 +145,13 @@ struct AttnArgs {
     int q_stride, kv_stride;
     int n_heads, n_kv_heads, L_max;
     float scaling;
+    // adapters whose up-projection is added while q, k, v are read (LORA instantiations only)
+    const float *t;          // [M, t_stride] down-projections
+    int t_stride;
+    const void *lb[3];       // B [N, r] of the q, k, v adapter, nullptr for none
+    int lr[3], loff[3];      // rank, first column in t
+    float lscale[3];
+    int lfp32;
 };
 
 // Raw cache vectors: D / 16 bf16 values of one slot per lane (16 or 8 bytes).
@@ -193,7 +201,33 @@ constexpr int ATT_MAX_WAVES = 16;
 // (key and value loads of ATT_UNROLL slots are issued together: values do not wait for scores);
 // the groups, the waves and the new token's own slot are merged at the end.
 // ATT_UNROLL: slots per 16-lane group in flight (keys and values: 2 * ATT_UNROLL vector loads per lane)
-template <int D, int ATT_WAVES, int ATT_UNROLL>
+// base + scaling * sum_j t[j] * B[n, j] with the roundings of the adapter wrapper's forward (see the
+// LoRA kernels below): what the projection's output would hold after its up-projection launch.
+template <bool FP32>
+__device__ __forceinline__ float lora_fixed(float base, const void *B, int r, float scale, const float *t, long n) {
+    if (!B) return base;  // uniform
+    float u = 0.0f;
+    for (int j = 0; j < r; j += 8) {  // r % 8 == 0
+        float bf[8];
+        if constexpr (FP32) {
+            const float4 x = *reinterpret_cast<const float4 *>(static_cast<const float *>(B) + n * r + j);
+            const float4 y = *reinterpret_cast<const float4 *>(static_cast<const float *>(B) + n * r + j + 4);
+            bf[0] = x.x, bf[1] = x.y, bf[2] = x.z, bf[3] = x.w, bf[4] = y.x, bf[5] = y.y, bf[6] = y.z, bf[7] = y.w;
+        } else {
+            const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(B) + n * r + j);
+            const uint32_t x[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bf[2 * e] = bf16_to_f32(x[e] & 0xFFFFu), bf[2 * e + 1] = bf16_to_f32(x[e] >> 16);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u += t[j + e] * bf[e];
+    }
+    const float delta = FP32 ? u * scale : round_bf16(round_bf16(u) * scale);
+    return round_bf16(base + delta);
+}
+
+// LORA: 0 none, 1 float32 adapter weights, 2 bf16 adapter weights
+template <int D, int ATT_WAVES, int ATT_UNROLL, int LORA>
 __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnArgs a) {
     constexpr int VEC = D / 16;
     __shared__ float qs[D];                 // rotated query
@@ -233,23 +267,45 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     };
     if (p > 0) request(0);
 
+    if constexpr (LORA != 0) {
+        // q, k, v of this head with their adapters added, through LDS (the rotation pairs columns)
+        if (tid < D) {
+            const float *trow = a.t + (long)m * a.t_stride;
+            const long nq = (long)h * D + tid, nk = (long)hk * D + tid;
+            qs[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.q[(long)m * a.q_stride + nq]), a.lb[0], a.lr[0], a.lscale[0],
+                                            trow + a.loff[0], nq);
+            ks[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.k[(long)m * a.kv_stride + nk]), a.lb[1], a.lr[1], a.lscale[1],
+                                            trow + a.loff[1], nk);
+            vs[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.v[(long)m * a.kv_stride + nk]), a.lb[2], a.lr[2], a.lscale[2],
+                                            trow + a.loff[2], nk);
+        }
+        __syncthreads();
+    }
+    float q_own = 0.0f, q_pair = 0.0f, k_own = 0.0f, k_pair = 0.0f, v_own = 0.0f;
     if (tid < D) {
-        const uint16_t *qrow = a.q + (long)m * a.q_stride + h * D;
-        const uint16_t *krow = a.k + (long)m * a.kv_stride + hk * D;
-        const uint16_t *vrow = a.v + (long)m * a.kv_stride + hk * D;
         const int partner = tid < D / 2 ? tid + D / 2 : tid - D / 2;
+        if constexpr (LORA != 0) {
+            q_own = qs[tid], q_pair = qs[partner], k_own = ks[tid], k_pair = ks[partner], v_own = vs[tid];
+        } else {
+            const uint16_t *qrow = a.q + (long)m * a.q_stride + h * D;
+            const uint16_t *krow = a.k + (long)m * a.kv_stride + hk * D;
+            q_own = bf16_to_f32(qrow[tid]), q_pair = bf16_to_f32(qrow[partner]);
+            k_own = bf16_to_f32(krow[tid]), k_pair = bf16_to_f32(krow[partner]);
+            v_own = bf16_to_f32(a.v[(long)m * a.kv_stride + hk * D + tid]);
+        }
+    }
+    if constexpr (LORA != 0) __syncthreads();  // everyone has read its pair before the rotated values go in
+    if (tid < D) {
         const float sign = tid < D / 2 ? -1.0f : 1.0f;  // rotate_half: (-x2, x1)
         const float c = bf16_to_f32(a.cos[(long)p * D + tid]), s = bf16_to_f32(a.sin[(long)p * D + tid]);
-        const float qe = round_bf16(round_bf16(bf16_to_f32(qrow[tid]) * c) +
-                                    round_bf16(sign * bf16_to_f32(qrow[partner]) * s));
-        const float ke = round_bf16(round_bf16(bf16_to_f32(krow[tid]) * c) +
-                                    round_bf16(sign * bf16_to_f32(krow[partner]) * s));
+        const float qe = round_bf16(round_bf16(q_own * c) + round_bf16(sign * q_pair * s));
+        const float ke = round_bf16(round_bf16(k_own * c) + round_bf16(sign * k_pair * s));
         qs[tid] = qe;
         ks[tid] = ke;
-        vs[tid] = bf16_to_f32(vrow[tid]);
+        vs[tid] = v_own;
         if (h % group == 0) {  // one workgroup per kv head appends; readers of slot p use their own copy
             a.k_cache[cache_base + (long)p * D + tid] = (uint16_t)f32_to_bf16_bits(ke);
-            a.v_cache[cache_base + (long)p * D + tid] = vrow[tid];
+            a.v_cache[cache_base + (long)p * D + tid] = (uint16_t)f32_to_bf16_bits(v_own);
         }
     }
     __syncthreads();
@@ -333,7 +389,6 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
 // ---------------------------------------------------------------- LoRA adapters over an int4 projection
 constexpr int LORA_MAX_ADAPTERS = 4;
 constexpr int LORA_MAX_ROWS = 32;
-constexpr int LORA_MAX_RANK = 64;
 constexpr int LORA_MAX_TOTAL = 256;
 
 struct LoraArgs {
@@ -528,11 +583,23 @@ extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const v
     return (int)hipGetLastError();
 }
 
-extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
-                                         void *k_cache, void *v_cache, const void *cos, const void *sin,
-                                         const void *mask, const int64_t *position, void *out,
-                                         int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
-                                         void *hip_stream) {
+namespace {
+template <int LORA>
+void launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
+    const bool many = (long)a.n_heads * M >= 512;
+    const dim3 grid(a.n_heads, M);
+    // few workgroups: 16 waves each (256 slots per trip); many: 8 waves, several workgroups per CU
+    // (a deeper unroll of the 16-wave form, 512 slots per trip, measured slower)
+    if (D == 128 && many) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 8, 4, LORA>), grid, dim3(8 * WAVE), 0, stream, a);
+    else if (D == 128) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4, LORA>), grid, dim3(16 * WAVE), 0, stream, a);
+    else if (many) hipLaunchKernelGGL((rope_attn_decode_kernel<64, 8, 4, LORA>), grid, dim3(8 * WAVE), 0, stream, a);
+    else hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4, LORA>), grid, dim3(16 * WAVE), 0, stream, a);
+}
+
+int attn_decode(const void *q, const void *k, const void *v, int q_stride, int kv_stride, void *k_cache,
+                void *v_cache, const void *cos, const void *sin, const void *mask, const int64_t *position,
+                void *out, int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                const vrl_attn_lora *lora, void *hip_stream) {
     if (!q || !k || !v || !k_cache || !v_cache || !cos || !sin || !mask || !position || !out) return VRL_INT4_ENULL;
     if (M < 1 || M > 65535 || n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || n_heads > 65535 ||
         (D != 64 && D != 128) || L_max < 1 || L_max > MAX_CACHE_LEN || q_stride < n_heads * D ||
@@ -543,6 +610,7 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
         misaligned(out, 2))
         return VRL_INT4_EALIGN;
     AttnArgs a;
+    memset(&a, 0, sizeof a);
     a.q = static_cast<const uint16_t *>(q);
     a.k = static_cast<const uint16_t *>(k);
     a.v = static_cast<const uint16_t *>(v);
@@ -560,15 +628,53 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
     a.L_max = L_max;
     a.scaling = scaling;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    const bool many = (long)n_heads * M >= 512;
-    const dim3 grid(n_heads, M);
-    // few workgroups: 16 waves each (256 slots per trip); many: 8 waves, several workgroups per CU
-    // (a deeper unroll of the 16-wave form, 512 slots per trip, measured slower)
-    if (D == 128 && many) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 8, 4>), grid, dim3(8 * WAVE), 0, stream, a);
-    else if (D == 128) hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4>), grid, dim3(16 * WAVE), 0, stream, a);
-    else if (many) hipLaunchKernelGGL((rope_attn_decode_kernel<64, 8, 4>), grid, dim3(8 * WAVE), 0, stream, a);
-    else hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4>), grid, dim3(16 * WAVE), 0, stream, a);
+    if (!lora) {
+        launch_attn<0>(a, M, D, stream);
+        return (int)hipGetLastError();
+    }
+    if (!lora->t) return VRL_INT4_ENULL;
+    if (misaligned(lora->t, 16) || lora->t_stride < 8 || lora->t_stride % 4 != 0) return VRL_INT4_ESHAPE;
+    const void *bs[3] = {lora->q_B, lora->k_B, lora->v_B};
+    bool any = false;
+    for (int i = 0; i < 3; ++i) {
+        a.lb[i] = bs[i];
+        a.lr[i] = lora->r[i];
+        a.loff[i] = lora->offset[i];
+        a.lscale[i] = lora->scaling[i];
+        if (!bs[i]) continue;
+        any = true;
+        if (lora->r[i] < 8 || lora->r[i] % 8 != 0 || lora->r[i] > LORA_MAX_RANK || lora->offset[i] < 0 ||
+            lora->offset[i] % 4 != 0 || lora->offset[i] + lora->r[i] > lora->t_stride)
+            return VRL_INT4_ESHAPE;
+        if (misaligned(bs[i], 16)) return VRL_INT4_EALIGN;
+    }
+    if (!any) return VRL_INT4_ENULL;
+    a.t = lora->t;
+    a.t_stride = lora->t_stride;
+    a.lfp32 = lora->weights_fp32;
+    if (lora->weights_fp32) launch_attn<1>(a, M, D, stream);
+    else launch_attn<2>(a, M, D, stream);
     return (int)hipGetLastError();
+}
+}  // namespace
+
+extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                         void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                         const void *mask, const int64_t *position, void *out,
+                                         int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                         void *hip_stream) {
+    return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, position, out, M, n_heads,
+                       n_kv_heads, D, L_max, scaling, nullptr, hip_stream);
+}
+
+extern "C" int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, int q_stride,
+                                              int kv_stride, void *k_cache, void *v_cache, const void *cos,
+                                              const void *sin, const void *mask, const int64_t *position, void *out,
+                                              int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                              const vrl_attn_lora *lora, void *hip_stream) {
+    if (!lora) return VRL_INT4_ENULL;
+    return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, position, out, M, n_heads,
+                       n_kv_heads, D, L_max, scaling, lora, hip_stream);
 }
 
 namespace {

@@ -20,9 +20,9 @@ op in fp32, rounded to bf16); the attention keeps its probabilities in fp32.
 Needs a trunk whose projections were swapped for prepacked :class:`Int4Linear` modules with the
 fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry one active LoRA
 adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
-the norm as a launch of its own (the adapters read the normalised row) and two more launches per
-adapter group (down-projection of all adapters that share the input, up-projection added onto the
-int4 outputs).  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not qualify, and
+the norm as a launch of its own (the adapters read the normalised row), a down-projection launch
+for the q|k|v adapters (their up-projections are added by the attention launch as it reads q, k, v)
+and a down- and an up-projection launch for o_proj's: nine launches.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not qualify, and
 callers then keep the module path.
 """
 
@@ -181,23 +181,28 @@ class NativeDecodeTrunk:
                               (launch.table, len(launch.table), ctypes.byref(launch.norm))))
             return launch.outputs
 
-        def lora(x, outs, adapters):
-            """outs[i] += adapter i applied to x, for the projections that carry one: two launches."""
+        def lora(x, outs, adapters, up=True):
+            """outs[i] += adapter i applied to x, for the projections that carry one: a down-projection
+            launch and, unless the consumer adds the up-projection itself (``up=False``: the attention
+            does for q, k, v), an up-projection launch.  Returns the group or ``None``."""
             todo = [(A, B, s, y) for y, ad in zip(outs, adapters) if ad is not None for A, B, s in [ad]]
             if not todo:
-                return
+                return None
             launch = ops.LoraAdd(x, todo)
             self._keep.append(launch)
             n = len(launch.table)
             calls.append((lib.vrl_lora_down_bf16, (x.data_ptr(), rows, x.shape[1], launch.table, n,
                                                    launch.t.data_ptr())))
-            calls.append((lib.vrl_lora_up_add_bf16, (launch.t.data_ptr(), rows, launch.table, n)))
+            if up:
+                calls.append((lib.vrl_lora_up_add_bf16, (launch.t.data_ptr(), rows, launch.table, n)))
+            return launch
 
-        def normed_gemv(module, weights, fused, adapters=()):
-            """h = res + x; the linears over norm(h); afterwards res = h."""
+        def normed_gemv(module, weights, fused, adapters=(), up=True):
+            """h = res + x; the linears over norm(h); afterwards res = h.  Returns (outputs, adapter group)."""
             w, eps = norm_weight(module)
             h_out = streams[state["flip"]]
             state["flip"] ^= 1
+            group = None
             if fuse_norm and not any(ad is not None for ad in adapters):
                 outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
             else:
@@ -205,31 +210,35 @@ class NativeDecodeTrunk:
                               (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,
                                w.data_ptr(), h_out.data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
                 outs = gemv([(self.normed, pw, fused) for pw in weights])
-                lora(self.normed, outs, adapters)   # adapters read the normalised row, so it is written out
+                group = lora(self.normed, outs, adapters, up)   # adapters read the normalised row, so it is written out
             state["res"] = h_out
-            return outs
+            return outs, group
 
         for i, layer in enumerate(trunk.layers):
             attn, mlp = layer.self_attn, layer.mlp
             proj = {n: _projection(getattr(attn, n), f"layers[{i}].self_attn.{n}")
                     for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
-            q, k, v = normed_gemv(layer.input_layernorm, [proj[n][0] for n in ("q_proj", "k_proj", "v_proj")],
-                                  False, [proj[n][1] for n in ("q_proj", "k_proj", "v_proj")])
+            (q, k, v), group = normed_gemv(layer.input_layernorm,
+                                           [proj[n][0] for n in ("q_proj", "k_proj", "v_proj")], False,
+                                           [proj[n][1] for n in ("q_proj", "k_proj", "v_proj")], up=False)
             if q.shape[1] != H * D or k.shape[1] != Hkv * D or v.shape[1] != Hkv * D:
                 raise TypeError(f"layers[{i}] projections do not match the attention geometry")
             keys, values = cache.layers[i].keys, cache.layers[i].values
             if tuple(keys.shape) != (rows, Hkv, self.max_len, D) or keys.dtype != torch.bfloat16 or \
                     not keys.is_contiguous() or not values.is_contiguous():
                 raise ValueError(f"cache layer {i} is not bfloat16 [rows, kv_heads, L_max, head_dim]")
-            calls.append((lib.vrl_rope_attn_decode_bf16,
-                          (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), keys.data_ptr(),
-                           values.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), mask.data_ptr(),
-                           slot.data_ptr(), self.attn.data_ptr(), rows, H, Hkv, D, self.max_len,
-                           float(attn.scaling))))
+            attn_args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), keys.data_ptr(),
+                         values.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), mask.data_ptr(),
+                         slot.data_ptr(), self.attn.data_ptr(), rows, H, Hkv, D, self.max_len, float(attn.scaling))
+            if group is None:
+                calls.append((lib.vrl_rope_attn_decode_bf16, attn_args))
+            else:   # the attention adds the up-projections of the q, k, v adapters while it reads them
+                calls.append((lib.vrl_rope_attn_decode_lora_bf16,
+                              (*attn_args, ctypes.byref(group.attn_record(q, k, v)))))
             outs = gemv([(self.attn, proj["o_proj"][0], False)])
             lora(self.attn, outs, [proj["o_proj"][1]])
             (state["x"],) = outs
-            (act,) = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
+            (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
             (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])
         w, eps = norm_weight(trunk.norm)
         calls.append((lib.vrl_add_rmsnorm_bf16,

@@ -565,7 +565,8 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: tor
 
 def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mask: torch.Tensor,
-                     position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None) -> torch.Tensor:
+                     position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None,
+                     lora: "LoraAdd | None" = None) -> torch.Tensor:
     """Rotary embedding, cache append and attention for one new token per row, one launch.
 
     ``q [M, H*D]``, ``k, v [M, Hkv*D]`` bf16 (rows may be strided views of one buffer), caches
@@ -573,6 +574,8 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
     written), ``cos, sin [L, D]`` bf16, ``mask [M, L]`` uint8, ``position`` an int64 device
     scalar.  Stands for ``apply_rotary_pos_emb``, ``Cache.update`` and the attention of
     ``LlamaAttention.forward`` (reached from ``vrl/models/families/janus_pro/policy.py:673-678``).
+    ``lora`` is a :class:`LoraAdd` over exactly the q, k, v outputs passed here whose down-projection
+    was launched: the attention then adds the up-projections itself (q, k, v stay as they are).
     """
     dev = _require_device("k_cache", k_cache)
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.dtype != torch.bfloat16 or \
@@ -602,11 +605,15 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
         out = torch.empty((M, H * D), dtype=torch.bfloat16, device=dev)
     elif out.dtype != torch.bfloat16 or tuple(out.shape) != (M, H * D) or not out.is_contiguous():
         raise ValueError(f"out must be contiguous bfloat16 [{M}, {H * D}]")
-    with _on(dev):
-        rc = _lib.load().vrl_rope_attn_decode_bf16(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), k_cache.data_ptr(),
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), k_cache.data_ptr(),
             v_cache.data_ptr(), cos.data_ptr(), sin.data_ptr(), mask.data_ptr(), position.data_ptr(),
-            out.data_ptr(), M, H, Hkv, D, L, float(scaling), _stream_handle(dev))
+            out.data_ptr(), M, H, Hkv, D, L, float(scaling))
+    with _on(dev):
+        if lora is None:
+            rc = _lib.load().vrl_rope_attn_decode_bf16(*args, _stream_handle(dev))
+        else:
+            rc = _lib.load().vrl_rope_attn_decode_lora_bf16(*args, ctypes.byref(lora.attn_record(q, k, v)),
+                                                            _stream_handle(dev))
     _lib.check(rc, "vrl_rope_attn_decode_bf16")
     return out
 
@@ -650,12 +657,41 @@ class LoraAdd:
         self.x, self.M, self.K, self.device = x, M, K, dev
         self._keep = list(adapters)
 
-    def launch(self):
-        lib = _lib.load()
-        stream = _stream_handle(self.device)
+    def launch_down(self):
+        """``t = x . A^T`` for every adapter of the group."""
         with _on(self.device):
-            rc = lib.vrl_lora_down_bf16(self.x.data_ptr(), self.M, self.K, self.table, len(self.table),
-                                        self.t.data_ptr(), stream)
-            _lib.check(rc, "vrl_lora_down_bf16")
-            rc = lib.vrl_lora_up_add_bf16(self.t.data_ptr(), self.M, self.table, len(self.table), stream)
-            _lib.check(rc, "vrl_lora_up_add_bf16")
+            rc = _lib.load().vrl_lora_down_bf16(self.x.data_ptr(), self.M, self.K, self.table, len(self.table),
+                                                self.t.data_ptr(), _stream_handle(self.device))
+        _lib.check(rc, "vrl_lora_down_bf16")
+
+    def launch_up(self):
+        """``y_i += scaling_i * t_i . B_i^T`` for every adapter of the group."""
+        with _on(self.device):
+            rc = _lib.load().vrl_lora_up_add_bf16(self.t.data_ptr(), self.M, self.table, len(self.table),
+                                                  _stream_handle(self.device))
+        _lib.check(rc, "vrl_lora_up_add_bf16")
+
+    def launch(self):
+        self.launch_down()
+        self.launch_up()
+
+    def attn_record(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+        """The ``vrl_attn_lora`` record that lets the attention launch add this group's up-projections
+        to ``q``, ``k``, ``v`` (the outputs this group was built over; others have no adapter)."""
+        rec = _lib.AttnLora()
+        rec.t, rec.t_stride = self.t.data_ptr(), self.t.shape[1]
+        rec.weights_fp32 = self.table[0].weights_fp32
+        offset, found = 0, 0
+        slots = {q.data_ptr(): 0, k.data_ptr(): 1, v.data_ptr(): 2}
+        for ad in self.table:
+            i = slots.get(ad.y)
+            if i is None:
+                raise ValueError("the adapter group holds an output that is not q, k or v of this call")
+            setattr(rec, ("q_B", "k_B", "v_B")[i], ad.B)
+            rec.r[i], rec.offset[i], rec.scaling[i] = ad.r, offset, ad.scaling
+            offset += ad.r
+            found += 1
+        if not found:
+            raise ValueError("no adapter")
+        self._attn_record = rec   # kept alive for a launch that is only enqueued
+        return rec
