@@ -546,6 +546,17 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
                 lambda n: sampler.sample_image_tokens(*inputs[B], image_token_num=n))
             del sampler
             torch.cuda.empty_cache()
+        if only is None:   # a whole image: 40-token prompt, 576 image tokens, prompt pass included
+            short = tuple(t[:, :40].contiguous() for t in inputs[B])
+            sampler = StaticARSampler(policy)
+            sampler.sample_image_tokens(*short, image_token_num=576)   # records the step for this shape
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            sampler.sample_image_tokens(*short, image_token_num=576)
+            torch.cuda.synchronize()
+            entry["int4_native_hip_graph_s_per_576_token_image_batch"] = time.perf_counter() - t0
+            del sampler
+            torch.cuda.empty_cache()
     return out
 
 
