@@ -100,12 +100,6 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t *__restrict
 // -------------------------------------------------------------------------
 constexpr int GEN_MT = 4;  // activation rows per pass
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
-    return v;
-}
-
 __device__ __forceinline__ void generic_row_dot(const DevProblem &p, int n, int m0, int mt,
                                                 float acc[GEN_MT]) {
     const int lane = threadIdx.x & (WAVE - 1);

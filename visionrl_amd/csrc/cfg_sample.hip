@@ -15,6 +15,7 @@
 #include <stdint.h>
 
 #include "../../include/vrl_int4.h"
+#include "wave_reduce.hpp"
 
 namespace {
 
@@ -46,18 +47,6 @@ __device__ __forceinline__ void scaled_logits(const Row &r, int i, float w, floa
     const float g = round_bf16(u + round_bf16(w * d));
     gt = round_bf16(g * inv_t);
     ct = round_bf16(c * inv_t);
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
-    return v;
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, WAVE);
-    return v;
 }
 
 template <bool MAX>

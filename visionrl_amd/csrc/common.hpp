@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "../../include/vrl_int4.h"
+#include "wave_reduce.hpp"
 
 namespace {
 

@@ -18,6 +18,7 @@
 
 #include "../../include/vrl_decode.h"
 #include "../../include/vrl_int4.h"
+#include "wave_reduce.hpp"
 
 namespace {
 
@@ -35,39 +36,6 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float v) {
     return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v);
 }
 __device__ __forceinline__ float round_bf16(float v) { return bf16_to_f32(f32_to_bf16_bits(v)); }
-
-// Cross-lane sums through DPP (register-to-register, no trip through the LDS crossbar that
-// __shfl_xor takes).  A DPP row is 16 lanes: two quad permutes and two mirrors leave every lane of
-// a row with the row's sum; the four rows of a wave meet through readlane.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float row16_sum(float v) {
-    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
-    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
-    v += dpp_move<0x141>(v);  // row_half_mirror
-    v += dpp_move<0x140>(v);  // row_mirror
-    return v;
-}
-__device__ __forceinline__ float row16_max(float v) {
-    v = fmaxf(v, dpp_move<0xB1>(v));
-    v = fmaxf(v, dpp_move<0x4E>(v));
-    v = fmaxf(v, dpp_move<0x141>(v));
-    v = fmaxf(v, dpp_move<0x140>(v));
-    return v;
-}
-__device__ __forceinline__ float lane_of(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-__device__ __forceinline__ float wave_sum(float v) {
-    v = row16_sum(v);
-    return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
-}
-__device__ __forceinline__ float wave_max(float v) {
-    v = row16_max(v);
-    return fmaxf(fmaxf(lane_of(v, 0), lane_of(v, 16)), fmaxf(lane_of(v, 32), lane_of(v, 48)));
-}
 
 // every thread returns the block's total; `red` holds WAVES floats and is free for reuse afterwards
 template <bool MAX>
@@ -151,7 +119,6 @@ struct AttnArgs {
     const void *lb[3];       // B [N, r] of the q, k, v adapter, nullptr for none
     int lr[3], loff[3];      // rank, first column in t
     float lscale[3];
-    int lfp32;
 };
 
 // Raw cache vectors: D / 16 bf16 values of one slot per lane (16 or 8 bytes).
@@ -191,7 +158,6 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
     for (int i = 0; i < VEC; ++i) a.acc[i] = a.acc[i] * c1 + acc2[i] * c2;
 }
 
-constexpr int ATT_MAX_WAVES = 16;
 
 // One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
 // keep many requests in flight), 8 when there are at least two per CU (several then share a CU
@@ -556,10 +522,30 @@ void launch_lora_up(const float *t, const LoraArgs &a, int max_n, int max_r, hip
                        dim3(UP_THREADS), (size_t)a.M * (max_r + UP_THREADS) * sizeof(float), stream, t, a);
 }
 
-int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y);
-
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
+
+// host side: one argument block for both LoRA launches
+int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y) {
+    if (!adapters) return VRL_INT4_ENULL;
+    if (n < 1 || n > LORA_MAX_ADAPTERS || M < 1 || M > LORA_MAX_ROWS || K < 8 || K % 8 != 0) return VRL_INT4_ESHAPE;
+    a.n = n;
+    a.M = M;
+    a.K = K;
+    a.off[0] = 0;
+    for (int i = 0; i < n; ++i) {
+        const vrl_lora_adapter &ad = adapters[i];
+        if (!ad.A || !ad.B || (need_y && !ad.y)) return VRL_INT4_ENULL;
+        if (ad.r < 8 || ad.r % 8 != 0 || ad.r > LORA_MAX_RANK || ad.N < 1) return VRL_INT4_ESHAPE;
+        if (misaligned(ad.A, 16) || misaligned(ad.B, 16) || misaligned(ad.y, 2)) return VRL_INT4_EALIGN;
+        if ((ad.weights_fp32 != 0) != (adapters[0].weights_fp32 != 0)) return VRL_INT4_ESHAPE;  // one type per launch
+        a.ad[i] = ad;
+        a.off[i + 1] = a.off[i] + ad.r;
+    }
+    for (int i = n; i < LORA_MAX_ADAPTERS; ++i) a.off[i + 1] = a.off[n];
+    if (a.off[n] > LORA_MAX_TOTAL) return VRL_INT4_ESHAPE;
+    return VRL_INT4_OK;
+}
 }  // namespace
 
 extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const void *weight, void *h_out,
@@ -651,7 +637,6 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
     if (!any) return VRL_INT4_ENULL;
     a.t = lora->t;
     a.t_stride = lora->t_stride;
-    a.lfp32 = lora->weights_fp32;
     if (lora->weights_fp32) launch_attn<1>(a, M, D, stream);
     else launch_attn<2>(a, M, D, stream);
     return (int)hipGetLastError();
@@ -677,28 +662,6 @@ extern "C" int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, cons
                        n_kv_heads, D, L_max, scaling, lora, hip_stream);
 }
 
-namespace {
-int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y) {
-    if (!adapters) return VRL_INT4_ENULL;
-    if (n < 1 || n > LORA_MAX_ADAPTERS || M < 1 || M > LORA_MAX_ROWS || K < 8 || K % 8 != 0) return VRL_INT4_ESHAPE;
-    a.n = n;
-    a.M = M;
-    a.K = K;
-    a.off[0] = 0;
-    for (int i = 0; i < n; ++i) {
-        const vrl_lora_adapter &ad = adapters[i];
-        if (!ad.A || !ad.B || (need_y && !ad.y)) return VRL_INT4_ENULL;
-        if (ad.r < 8 || ad.r % 8 != 0 || ad.r > LORA_MAX_RANK || ad.N < 1) return VRL_INT4_ESHAPE;
-        if (misaligned(ad.A, 16) || misaligned(ad.B, 16) || misaligned(ad.y, 2)) return VRL_INT4_EALIGN;
-        if ((ad.weights_fp32 != 0) != (adapters[0].weights_fp32 != 0)) return VRL_INT4_ESHAPE;  // one type per launch
-        a.ad[i] = ad;
-        a.off[i + 1] = a.off[i] + ad.r;
-    }
-    for (int i = n; i < LORA_MAX_ADAPTERS; ++i) a.off[i + 1] = a.off[n];
-    if (a.off[n] > LORA_MAX_TOTAL) return VRL_INT4_ESHAPE;
-    return VRL_INT4_OK;
-}
-}  // namespace
 
 extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adapters, int n_adapters,
                                   float *t, void *hip_stream) {

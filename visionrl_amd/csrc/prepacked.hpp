@@ -135,23 +135,6 @@ struct NormArgs {
 constexpr int PP_WRITE_H = 4;       // DevProblem::prepacked bit
 constexpr int NORM_MAX_K = 4096;    // eight 16-byte words per lane hold a row
 
-// wave-wide sum through DPP (two quad permutes, two mirrors: every lane of a 16-lane row holds the
-// row's sum) and readlane for the four rows: register-to-register, no LDS crossbar
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
-    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
-    v += dpp_move<0x141>(v);  // row_half_mirror
-    v += dpp_move<0x140>(v);  // row_mirror
-    auto lane_of = [](float x, int lane) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
-    };
-    return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
-}
-
 template <int NW>  // 16-byte words per lane that hold a row: K <= NW * 512
 __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
                                                   int xstride, int nwaves, bool write_h) {
@@ -206,7 +189,7 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
                 if (write_h) *(gptr_w4)(uintptr_t)(n.h_out + row + k) = h[i];
             }
         }
-        ss = wave_sum_dpp(ss);
+        ss = wave_sum(ss);
         const float r = rsqrtf(ss * inv_k + n.eps);
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
