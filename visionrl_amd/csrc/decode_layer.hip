@@ -276,41 +276,60 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     }
     __syncthreads();
 
-    float qreg[VEC];
+    // the lane's VEC values of the rotated query as bf16 pairs (exact: they are bf16 values), so that a
+    // key word needs no conversion: v_dot2_f32_bf16 takes two products per instruction
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    bf16x2_t qpair[VEC / 2];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) qreg[i] = qs[l16 * VEC + i];
+    for (int i = 0; i < VEC / 2; ++i) {
+        const uint32_t bits = f32_to_bf16_bits(qs[l16 * VEC + 2 * i]) | (f32_to_bf16_bits(qs[l16 * VEC + 2 * i + 1]) << 16);
+        qpair[i] = __builtin_bit_cast(bf16x2_t, bits);
+    }
     if (wave == 0) {  // the new token's own slot
         float dot = 0.0f;
         for (int d = lane; d < D; d += WAVE) dot += qs[d] * ks[d];
         dot = wave_sum(dot);
         if (lane == 0) s_new = mask[p] ? dot * a.scaling : -INFINITY;
     }
+
     Partial<VEC> st;
     st.m = -INFINITY;
     st.l = 0.0f;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) st.acc[i] = 0.0f;
 
-    // cached slots 0..p-1, a batch per trip; the batch of the first trip is already on its way
+    // cached slots 0..p-1, a batch per trip; the batch of the first trip is already on its way.
+    // The running softmax is rescaled once per batch: one maximum over the batch's scores and the
+    // state, one exponential per score and one for the state.
     for (int j0 = 0; j0 < p; j0 += STEP) {
         if (j0 > 0) request(j0);
+        float sc[ATT_UNROLL];
+        float mx = st.m;
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             float dot = 0.0f;
 #pragma unroll
-            for (int i = 0; i < VEC / 2; ++i) {
-                dot += qreg[2 * i] * bf16_to_f32(kraw[u].w[i] & 0xFFFFu);
-                dot += qreg[2 * i + 1] * bf16_to_f32(kraw[u].w[i] >> 16);
-            }
+            for (int i = 0; i < VEC / 2; ++i)
+                dot = __builtin_amdgcn_fdot2_f32_bf16(qpair[i], __builtin_bit_cast(bf16x2_t, kraw[u].w[i]), dot, false);
             dot = row16_sum(dot);  // the sixteen lanes that share the slot
-            const float s = live[u] ? dot * a.scaling : -INFINITY;
-            float vf[VEC];
+            sc[u] = live[u] ? dot * a.scaling : -INFINITY;
+            mx = fmaxf(mx, sc[u]);
+        }
+        const float ref = mx == -INFINITY ? 0.0f : mx;  // nothing attendable yet: keep zeros, avoid inf - inf
+        const float c0 = __expf(st.m - ref);
+        st.m = mx;
+        st.l *= c0;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) st.acc[i] *= c0;
+#pragma unroll
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const float w = __expf(sc[u] - ref);
+            st.l += w;
 #pragma unroll
             for (int i = 0; i < VEC / 2; ++i) {
-                vf[2 * i] = bf16_to_f32(vraw[u].w[i] & 0xFFFFu);
-                vf[2 * i + 1] = bf16_to_f32(vraw[u].w[i] >> 16);
+                st.acc[2 * i] += w * bf16_to_f32(vraw[u].w[i] & 0xFFFFu);
+                st.acc[2 * i + 1] += w * bf16_to_f32(vraw[u].w[i] >> 16);
             }
-            merge<VEC>(st, s, 1.0f, vf);
         }
     }
     // the four 16-lane groups of the wave
