@@ -557,3 +557,32 @@ def test_native_trunk_at_janus_layer_shapes(B, kv_heads, lora, hidden, inter, he
         assert torch.equal(tokens, out[0][0]) and torch.equal(logprobs, out[0][1])
     assert out[0][0].shape == (B, 10) and (out[0][0] >= 0).all() and (out[0][0] < 16384).all()
     assert (out[0][1] <= 0).all() and torch.isfinite(out[0][1]).all()
+
+
+@pytest.mark.gpu
+def test_adapter_state_changes_invalidate_the_recorded_step():
+    """Disabling the adapters (what the policy's reference-policy context does, policy.py:21) between two
+    generations: the second one must not replay a step recorded with them."""
+    print("ar decode: adapter state change", flush=True)
+    policy = lora_policy(torch.float32)
+    inputs = make_inputs(2, 7, torch.bfloat16, "cuda:0", seed=95)
+    sampler = StaticARSampler(policy, graph=True)
+    torch.manual_seed(96)
+    with_adapters = sampler.sample_image_tokens(*inputs, image_token_num=8)
+    (sess,) = sampler._sessions.values()
+    first_graph = sess.graph
+    assert sess.native and first_graph is not None
+    wrappers = [getattr(layer.self_attn, n) for layer in policy._lm_trunk().layers
+                for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+
+    for w in wrappers:
+        w.disable_adapters = True
+        w.forward = types.MethodType(lambda self, x: self.base_layer(x), w)
+    torch.manual_seed(96)
+    without = sampler.sample_image_tokens(*inputs, image_token_num=8)
+    torch.cuda.synchronize()
+    assert sess.graph is not first_graph and not sess.native   # disabled adapters: this stand-in keeps the module path
+    torch.manual_seed(96)
+    want = StaticARSampler(policy, graph=False, native=False).sample_image_tokens(*inputs, image_token_num=8)
+    assert torch.equal(without[0], want[0]) and torch.equal(without[1], want[1])
+    assert not torch.equal(without[1], with_adapters[1])

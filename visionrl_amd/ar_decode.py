@@ -44,7 +44,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
-from .decode_step import NativeDecodeTrunk
+from .decode_step import NativeDecodeTrunk, trunk_signature
 
 __all__ = ["StaticARSampler", "StaticARState", "StaticARStepResult", "install_static_ar_sampler"]
 
@@ -111,9 +111,13 @@ class _Session:
         self.slot = torch.zeros(1, dtype=torch.long, device=device)   # cache slot of the next new token
         self.native = None     # NativeDecodeTrunk once the cache exists, False if the trunk does not qualify
         self.graph = None
+        self.signature = None  # of the trunk's modules and adapter state the launch list / graph were made for
 
     # -- one call of sample_image_tokens starts here
     def begin(self, mask: torch.Tensor) -> None:
+        signature = trunk_signature(self.sampler.trunk)
+        if signature != self.signature:   # modules swapped, adapters merged / disabled / switched: start over
+            self.signature, self.native, self.graph = signature, None, None
         self.cache.reset()
         self.mask.fill_(1)
         self.mask[:, :mask.shape[1]].copy_(mask)

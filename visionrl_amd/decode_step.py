@@ -35,7 +35,7 @@ import torch
 from . import _lib, ops
 from .linear import Int4Linear, Int4LlamaMLP
 
-__all__ = ["NativeDecodeTrunk"]
+__all__ = ["NativeDecodeTrunk", "trunk_signature"]
 
 
 def _plain_int4(module, name: str):
@@ -93,6 +93,25 @@ def _projection(module, name: str):
     if not isinstance(base, Int4Linear) or not hasattr(module, "lora_A") or not hasattr(module, "lora_B"):
         raise TypeError(f"{name} is {type(module).__name__}: neither an Int4Linear nor a LoRA wrapper around one")
     return _plain_int4(base, name + ".base_layer"), _adapter_of(module, name)
+
+
+def trunk_signature(trunk) -> tuple:
+    """What a recorded decode step bakes in besides tensor addresses: which module objects serve the
+    projections and the state of their adapters (merged, disabled, active names, scaling).  A
+    recorded step or a native launch list is valid while this value is unchanged; weight values may
+    change in place."""
+    sig = []
+    for layer in trunk.layers:
+        for owner, names in ((layer.self_attn, ("q_proj", "k_proj", "v_proj", "o_proj")), (layer, ("mlp",))):
+            for name in names:
+                mod = getattr(owner, name, None)
+                active = getattr(mod, "active_adapters", None) or getattr(mod, "active_adapter", None)
+                active = tuple(active) if isinstance(active, (list, tuple)) else active
+                scaling = getattr(mod, "scaling", None)
+                scaling = tuple(sorted(scaling.items())) if hasattr(scaling, "items") else scaling
+                sig.append((id(mod), bool(getattr(mod, "merged", False)),
+                            bool(getattr(mod, "disable_adapters", False)), active, scaling))
+    return tuple(sig)
 
 
 class NativeDecodeTrunk:
