@@ -194,6 +194,22 @@ def test_runtime_spec_options_and_builder_wrapper():
         spec, lambda s: types.SimpleNamespace(policy=StubPolicy(), metadata={"model_path": "stub"}))
     assert bundle.metadata["int4"]["linears"] == 7 * LAYERS
     assert isinstance(bundle.policy._base().gen_head, Int4Linear)
+    assert bundle.metadata["int4"]["static_sampler"] is False    # this stand-in has no sample_image_tokens to replace
+
+    class Sampling(StubPolicy):                                   # a policy with the loop and what the loop needs
+        def __init__(self):
+            super().__init__()
+            self.mmgpt.prepare_gen_img_embeds = lambda ids: None
+
+        def sample_image_tokens(self, *args, **kwargs):
+            raise AssertionError("replaced by the static sampler")
+
+    for wanted in (True, False):
+        spec.extra["int4"] = {"static_sampler": wanted}
+        b = build_int4_runtime_bundle(spec, lambda s: types.SimpleNamespace(policy=Sampling(), metadata={}))
+        assert b.metadata["int4"]["static_sampler"] is wanted
+        assert hasattr(b.policy, "_static_ar_sampler") is wanted
+        assert (b.policy.sample_image_tokens.__func__ is not Sampling.sample_image_tokens) is wanted
     plain = build_int4_runtime_bundle(types.SimpleNamespace(extra={}),
                                       lambda s: types.SimpleNamespace(policy=StubPolicy(), metadata={}))
     assert "int4" not in plain.metadata

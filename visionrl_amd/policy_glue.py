@@ -13,7 +13,9 @@ Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
 * ``builder.py:11-33``, ``:77-113`` and ``vrl/distributed/ray/rollout/worker.py:143-163``:
   rollout workers build the policy from a ``RuntimeBuildSpec`` whose ``extra``
   dict is the only channel for new scalar options; ``extra["int4"]`` carries
-  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true}``.
+  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true,
+  "static_sampler": true}`` (the last one routes ``sample_image_tokens`` and the step API through
+  :mod:`visionrl_amd.ar_decode`).
 
 * ``vrl/distributed/ray/rollout/worker.py:55-71``: a rollout worker applies synced trainer
   weights through ``policy.load_trainable_state(state)``, which the Janus-Pro policy does not
@@ -171,7 +173,7 @@ def int4_options_from_spec(spec: Any) -> dict | None:
         opt = {}
     if not isinstance(opt, dict):
         raise TypeError('RuntimeBuildSpec.extra["int4"] must be true or a dict of options')
-    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack", "group_qkv"}
+    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack", "group_qkv", "static_sampler"}
     unknown = set(opt) - allowed
     if unknown:
         raise ValueError(f'unknown keys in extra["int4"]: {sorted(unknown)}')
@@ -180,7 +182,8 @@ def int4_options_from_spec(spec: Any) -> dict | None:
             "fuse_mlp": bool(opt.get("fuse_mlp", True)),
             "head": bool(opt.get("head", True)),
             "prepack": bool(opt.get("prepack", True)),
-            "group_qkv": bool(opt.get("group_qkv", True))}
+            "group_qkv": bool(opt.get("group_qkv", True)),
+            "static_sampler": bool(opt.get("static_sampler", True))}
 
 
 def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
@@ -192,7 +195,17 @@ def build_int4_runtime_bundle(spec: Any, builder: Callable[[Any], Any]) -> Any:
     bundle = builder(spec)
     opt = int4_options_from_spec(spec)
     if opt is not None:
+        static_sampler = opt.pop("static_sampler")
         summary = apply_int4_to_policy(bundle.policy, **opt)
+        summary["static_sampler"] = False
+        if static_sampler and hasattr(bundle.policy, "sample_image_tokens"):
+            from .ar_decode import install_static_ar_sampler
+
+            try:   # the image-token loop over a static cache and recorded decode steps
+                install_static_ar_sampler(bundle.policy)
+                summary["static_sampler"] = True
+            except (TypeError, AttributeError):   # not a Janus-Pro shaped policy: leave its own loop
+                pass
         meta = getattr(bundle, "metadata", None)
         if isinstance(meta, dict):
             meta["int4"] = summary
