@@ -334,3 +334,67 @@ def test_attention_adds_the_qkv_adapters_itself(ops_mod, M, H, Hkv, D, fp32, whi
     assert (got != want).float().mean().item() < 0.05
     with pytest.raises(ValueError):   # a group over other outputs
         ops_mod.rope_attn_decode(q1, k1, v1, kc1, vc1, t["cos"], t["sin"], mask, pos, c["scaling"], lora=group)
+
+
+# ------------------------------------------------------------------ seeded random shapes through every decode-layer launch
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes(ops_mod, seed):
+    """Twenty random cases per seed for each launch: ragged row counts, grouped-query heads, padding
+    masks, positions anywhere in the cache, ranks and widths that do not divide the workgroup shapes."""
+    from tests._util import assert_gemv_close, to_device
+
+    rng = np.random.default_rng(seed)
+    for case in range(20):
+        M = int(rng.integers(1, 33))
+        # residual add + norm, alone and inside an int4 launch
+        K = int(rng.choice([128, 256, 640, 1024, 2048, 3072, 4096]))
+        say("random", seed, case, "norm", M, K)
+        x, res, wn = rand_bits(rng, (M, K)), rand_bits(rng, (M, K), 3.0), rand_bits(rng, (K,), 0.7)
+        use_res = bool(rng.integers(0, 2))
+        h_want, xn = d.add_rmsnorm(x, res if use_res else None, wn, 1e-5)
+        xt, rt, wt = bits_to_bf16(x, DEV), bits_to_bf16(res, DEV), bits_to_bf16(wn, DEV)
+        h, y = ops_mod.add_rmsnorm(xt, wt, 1e-5, rt if use_res else None)
+        torch.cuda.synchronize()
+        assert (bf16_to_bits(h) == h_want).all()
+        assert ulp_distance(bf16_to_bits(y), xn).max() <= 1
+        N = int(rng.integers(1, 20)) * 16 + int(rng.choice([0, 0, 4]))
+        ops = o.make_operands(int(rng.integers(1 << 30)), M, K, N, 128)
+        ops["x_bits"] = xn
+        dd = to_device(ops, DEV)
+        pw = ops_mod.int4_prepack(dd["qweight"], dd["scales"], dd["qzeros"], 128)
+        h_out = torch.empty_like(xt)
+        (yn,) = ops_mod.DirectGemv([(xt, pw, False)], norm=(rt if use_res else None, wt, 1e-5, h_out)).launch()
+        torch.cuda.synchronize()
+        assert (bf16_to_bits(h_out) == h_want).all()
+        assert_gemv_close(bf16_to_bits(yn), ops, 128, f"random norm-fused {seed}/{case}")
+        # attention
+        D = int(rng.choice([64, 128]))
+        Hkv = int(rng.choice([1, 2, 4]))
+        H = Hkv * int(rng.choice([1, 2, 4]))
+        L = int(rng.integers(1, 40)) * 8
+        p = int(rng.integers(0, L))
+        Ma = min(M, 8)
+        say("random", seed, case, "attention", Ma, H, Hkv, D, L, p)
+        c = attn_case(int(rng.integers(1 << 30)), Ma, H, Hkv, D, L, p)
+        c["mask"] = (rng.random((Ma, L)) > 0.2).astype(np.uint8)
+        c["mask"][:, p] = 1
+        want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
+                                                    c["mask"], p, H, Hkv, c["scaling"])
+        out, kc, vc = run_attn(ops_mod, c)
+        assert (bf16_to_bits(kc) == kc_want).all() and (bf16_to_bits(vc) == vc_want).all()
+        got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)
+        tol = 0.51 * o.bf16_ulp(want.astype(np.float32)) + 2e-5 * np.abs(want).max()
+        assert (np.abs(got - want) <= tol).all(), (seed, case, np.abs(got - want).max())
+        # adapters
+        r = int(rng.integers(1, 9)) * 8
+        Nl = int(rng.integers(1, 300))
+        fp32 = bool(rng.integers(0, 2))
+        say("random", seed, case, "lora", M, K, Nl, r, fp32)
+        dtype = torch.float32 if fp32 else torch.bfloat16
+        A = torch.from_numpy((rng.standard_normal((r, K)) * K ** -0.5).astype(np.float32)).to(dtype)
+        B = torch.from_numpy((rng.standard_normal((Nl, r)) * 0.1).astype(np.float32)).to(dtype)
+        y0 = rand_bits(rng, (M, Nl), 2.0)
+        yt = bits_to_bf16(y0, DEV)
+        ops_mod.LoraAdd(xt, [(A.to(DEV), B.to(DEV), 1.5, yt)]).launch()
+        torch.cuda.synchronize()
+        within_one_step_of(bf16_to_bits(yt), d.lora_add(y0, x, A.float().numpy(), B.float().numpy(), 1.5, fp32), y0)
