@@ -31,6 +31,8 @@
 // canonical triple), prepacked.hpp (repack, stream and latency kernels over the MFMA-shaped blob), this file
 // (the grouped stream kernel that dispatches to both halves, plan building, launchers, the C ABI).
 
+#include <atomic>
+
 #include "prepacked.hpp"
 
 namespace {
@@ -322,12 +324,16 @@ template <bool FUSED, int KS, int TW, bool NORM>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
     auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM>;
     if (lds > 64 * 1024) {
-        static bool raised = false;  // per instantiation; the attribute is a property of the function
-        if (!raised) {
+        // once per instantiation and device: the attribute belongs to the function on that device
+        static std::atomic<uint64_t> raised{0};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(raised.load(std::memory_order_relaxed) & bit)) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)DIRECT_LDS_CAP);
             if (e != hipSuccess) return (int)e;
-            raised = true;
+            raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
