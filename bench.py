@@ -627,6 +627,9 @@ def main():
     ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
     ap.add_argument("--ar-decode", type=int, default=0, metavar="B",
                     help="run only the recorded decode loop at batch B on the int4 policy and exit (for profilers)")
+    ap.add_argument("--attn-decode", type=int, default=0, metavar="ROWS",
+                    help="run 8 attention decode launches (16 heads x 128, slot 330 of 384) over distinct caches "
+                         "at ROWS rows and exit (for counter runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run plain 1 GiB device copies and exit (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -647,6 +650,21 @@ def main():
         return
     from visionrl_amd import ops
 
+    if args.attn_decode:
+        rows, heads, dim, slots, at = args.attn_decode, 16, 128, 384, 330
+        new = lambda *shape: torch.randn(shape, device=device).to(torch.bfloat16)
+        q, k, v = new(rows, heads * dim), new(rows, heads * dim), new(rows, heads * dim)
+        caches = [(new(rows, heads, slots, dim), new(rows, heads, slots, dim)) for _ in range(8)]
+        cos, sin = new(slots, dim), new(slots, dim)
+        mask = torch.ones((rows, slots), dtype=torch.uint8, device=device)
+        pos = torch.tensor([at], dtype=torch.int64, device=device)
+        out = torch.empty((rows, heads * dim), dtype=torch.bfloat16, device=device)
+        for kc, vc in caches:
+            ops.rope_attn_decode(q, k, v, kc, vc, cos, sin, mask, pos, dim ** -0.5, out=out)
+        torch.cuda.synchronize()
+        print(json.dumps({"attn_decode_launches": len(caches), "rows": rows,
+                          "cache_bytes_read_per_launch": rows * heads * at * dim * 2 * 2}))
+        return
     if args.ar_decode:
         which = "int4_lora_native_hip_graph" if args.lora else "int4_native_hip_graph"
         print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,))))
