@@ -320,9 +320,9 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int KS, int TW, bool NORM>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG = false>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
-    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM>;
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG>;
     if (lds > 64 * 1024) {
         // once per instantiation and device: the attribute belongs to the function on that device
         static std::atomic<uint64_t> raised{0};
@@ -341,7 +341,11 @@ int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_
 }
 
 template <bool FUSED, bool NORM>
-int launch_direct_shape(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
+int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int workgroups, size_t lds,
+                        hipStream_t stream) {
+    if constexpr (!NORM) {
+        if (xg) return launch_direct<FUSED, 16, 1, false, true>(args, workgroups, lds, stream);
+    }
     if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1, NORM>(args, workgroups, lds, stream);
     if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4, NORM>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1, NORM>(args, workgroups, lds, stream);
@@ -466,6 +470,8 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // activation rows a workgroup carries several tiles so that one staging of x serves them
     const int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
     const int tw = max_m >= 8 ? 16 / ks : 1;
+    // long K with one super-chunk per wave: the waves fetch their own activations, nothing is staged
+    const bool xg = !norm && ks == 16 && max_nsc <= 16;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
@@ -494,7 +500,7 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         const vrl_int4_problem &q = problems[i];
         const int kc = pp_nsc(q.K) * PP_SC;
         const size_t row_bytes = (size_t)(kc + XPAD) * 2;
-        long rows = (long)((DIRECT_LDS_CAP - red) / row_bytes);
+        long rows = xg ? MAX_TILE_M : (long)((DIRECT_LDS_CAP - red) / row_bytes);
         if (rows > MAX_TILE_M) rows = MAX_TILE_M;
         if (rows < 1) return VRL_INT4_ESHAPE;
         const int out_cols = q.fused_gate_up ? q.N / 2 : q.N;
@@ -521,18 +527,18 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     for (int i = 0; i < args.n; ++i) {
         DevProblem &p = args.recs[i];
         const size_t need = (size_t)(p.M + 1) * (p.kc + XPAD) * 2;
-        if (p.M < MAX_TILE_M && need + red <= 32 * 1024) {
+        if (!xg && p.M < MAX_TILE_M && need + red <= 32 * 1024) {
             p.prepacked |= PP_ZERO_ROW;
             xz_bytes = std::max(xz_bytes, need);
         }
     }
-    const size_t lds = xz_bytes + red;
+    const size_t lds = xg ? red : xz_bytes + red;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     if (norm)
-        return fused_any ? launch_direct_shape<true, true>(args, ks, tw, (int)workgroups, lds, stream)
-                         : launch_direct_shape<false, true>(args, ks, tw, (int)workgroups, lds, stream);
-    return fused_any ? launch_direct_shape<true, false>(args, ks, tw, (int)workgroups, lds, stream)
-                     : launch_direct_shape<false, false>(args, ks, tw, (int)workgroups, lds, stream);
+        return fused_any ? launch_direct_shape<true, true>(args, ks, tw, false, (int)workgroups, lds, stream)
+                         : launch_direct_shape<false, true>(args, ks, tw, false, (int)workgroups, lds, stream);
+    return fused_any ? launch_direct_shape<true, false>(args, ks, tw, xg, (int)workgroups, lds, stream)
+                     : launch_direct_shape<false, false>(args, ks, tw, xg, (int)workgroups, lds, stream);
 }
 
 int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {

@@ -320,11 +320,14 @@ __device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t,
 // for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
 // if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
 // never runs dry between tiles.
-template <int MB, bool FUSED, int GQ>
+// XG: the A operand of the one super-chunk the call covers (sc1 == sc0 + 1) was fetched into registers by
+// the caller (xpre[b][4 * d + dd]) instead of being staged in LDS.
+template <int MB, bool FUSED, int GQ, bool XG = false>
 __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
                                                int next_tile, const uint16_t *xs, int xstride,
                                                int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
-                                               f32x4_t (&acc)[FUSED ? 2 : 1][MB]) {
+                                               f32x4_t (&acc)[FUSED ? 2 : 1][MB],
+                                               const u32x4_t (*xpre)[16] = nullptr) {
     constexpr int RS = FUSED ? 2 : 1;
     const int lane = threadIdx.x & (WAVE - 1);
     const int lc = lane & 15;
@@ -369,9 +372,13 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                 bf16x8_t xa[MB];
 #pragma unroll
                 for (int b = 0; b < MB; ++b) {
-                    const int m = min(16 * b + lc, pad_row);
-                    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
-                    xa[b] = __builtin_bit_cast(bf16x8_t, raw);
+                    if constexpr (XG) {
+                        xa[b] = __builtin_bit_cast(bf16x8_t, xpre[b][4 * d + dd]);
+                    } else {
+                        const int m = min(16 * b + lc, pad_row);
+                        const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xs + m * xstride + kloc + 8 * dd);
+                        xa[b] = __builtin_bit_cast(bf16x8_t, raw);
+                    }
                 }
 #pragma unroll
                 for (int r = 0; r < RS; ++r) {
@@ -504,16 +511,22 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // o_proj, ...).  A workgroup carries TW such tiles at once (KS * TW waves), so that one
 // staging of the activations serves TW tiles: that matters once x is tens of KB (8+ rows).
 // LDS: staged activations, then TW x (KS - 1) x RS partial tiles.
-template <bool FUSED, int KS, int TW, int GQ, bool NORM>
+// XG (plan-free launches of long K, one super-chunk per wave): no staging at all.  With K split over
+// the waves and one tile per workgroup every activation value is used by exactly one wave, so each
+// wave fetches its own A operand (16 rows x 512 k: sixteen 16-byte buffer loads per lane, zeros for
+// rows beyond M and k beyond K through the buffer's range check) while its weights arrive; LDS
+// holds only the partial tiles, and 16 rows per record fit whatever K is.
+template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
                                                  const NormArgs &norm) {
     constexpr int RS = FUSED ? 2 : 1;
+    static_assert(!XG || (TW == 1 && !NORM), "register-fed activations: one tile per workgroup, no norm");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tw = wave / KS, kw = wave % KS;  // tile of the round, share of K
     const int lane = threadIdx.x & (WAVE - 1);
     uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
     const int xstride = p.kc + XPAD;
-    const int xrows = p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0);
+    const int xrows = XG ? 0 : p.M + ((p.prepacked & PP_ZERO_ROW) ? 1 : 0);
     f32x4_t *red = reinterpret_cast<f32x4_t *>(smem + (size_t)xrows * xstride * 2) + tw * (KS - 1) * RS * WAVE;
     const int nsc = pp_nsc(p.K);
     const int per = (nsc + KS - 1) / KS;
@@ -524,13 +537,22 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     bool work = sc0 < sc1 && tile < t1;  // wave-uniform
     PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, work ? tile : t0, sc0);
     if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
-    __syncthreads();
-    if constexpr (NORM)
-        stage_x_norm(p, norm, nsc * PP_SC, xs, xstride, KS * TW,
-                     t0 == 0 && (p.prepacked & PP_WRITE_H) && norm.h_out != nullptr);
-    else
-        stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
-    __syncthreads();
+    u32x4_t xpre[1][16];
+    if constexpr (XG) {
+        const int lc = lane & 15, kbase = sc0 * PP_SC + (lane >> 4) * 128;  // the lane's row and 128-k span
+        const rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.x), 0, p.M * p.K * 2, 0x00020000);
+        const uint32_t voff = (work && lc < p.M && kbase < p.K) ? (uint32_t)(lc * p.K + kbase) * 2u : PP_OUT_OF_RANGE;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xpre[0][i] = __builtin_amdgcn_raw_buffer_load_b128(xr, voff + 16u * i, 0, 0);
+    } else {
+        __syncthreads();
+        if constexpr (NORM)
+            stage_x_norm(p, norm, nsc * PP_SC, xs, xstride, KS * TW,
+                         t0 == 0 && (p.prepacked & PP_WRITE_H) && norm.h_out != nullptr);
+        else
+            stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
+        __syncthreads();
+    }
     for (int base = t0; base < t1; base += TW) {
         tile = base + tw;
         const int next = tile + TW < t1 ? tile + TW : -1;
@@ -538,7 +560,10 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 #pragma unroll
         for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if (work) {
-            stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
+            if constexpr (XG)
+                stream_rows_pp<1, FUSED, GQ, true>(p, rsrc, cur, next, nullptr, 0, sc0, sc1, ring, acc, xpre);
+            else
+                stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
             if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
         }
         if (kw != 0) {
@@ -559,17 +584,17 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 }
 
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
-template <bool FUSED, int KS, int TW, bool NORM>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG>
 __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem,
                                                const NormArgs &norm) {
     if (FUSED && p.fused) {
-        if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1, NORM>(p, t0, t1, smem, norm);
-        else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM>(p, t0, t1, smem, norm);
-        else split_segment_pp<FUSED, KS, TW, 4, NORM>(p, t0, t1, smem, norm);
+        if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm);
+        else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
+        else split_segment_pp<FUSED, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
     } else {
-        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM>(p, t0, t1, smem, norm);
-        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM>(p, t0, t1, smem, norm);
-        else split_segment_pp<false, KS, TW, 4, NORM>(p, t0, t1, smem, norm);
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
+        else split_segment_pp<false, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
     }
 }
 
@@ -587,7 +612,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
-        split_by_group<FUSED, WPB, 1, false>(p, a, b, smem, NormArgs{});
+        split_by_group<FUSED, WPB, 1, false, false>(p, a, b, smem, NormArgs{});
         t = seg_end;
     }
 }
@@ -605,7 +630,7 @@ struct DirectArgs {
     NormArgs norm;                // read by the NORM instantiations only
 };
 
-template <bool FUSED, int KS, int TW, bool NORM>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG>
 __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int g = blockIdx.x;
@@ -615,7 +640,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
     const int t0 = (g - p.tile_begin) * TW;
-    split_by_group<FUSED, KS, TW, NORM>(p, t0, min(tiles, t0 + TW), smem, a.norm);
+    split_by_group<FUSED, KS, TW, NORM, XG>(p, t0, min(tiles, t0 + TW), smem, a.norm);
 }
 
 }  // namespace
