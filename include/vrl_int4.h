@@ -142,8 +142,8 @@ typedef struct vrl_int4_plan_info {
  * prepacked weight, or the q|k|v / gate|up linears of one decoder layer, policy.py:673-678):
  * the records travel as kernel arguments, the waves of a workgroup split K of a 16-column
  * tile.  Meant for decode and rollout batches (the launch is one memory round trip).  Every
- * problem must have prepacked = 1; activations are taken in slabs of at most 16 rows that
- * fit LDS (fewer rows per slab for long K), and all slabs of a call together may number at
+ * problem must have prepacked = 1; activations are taken in slabs of at most 16 rows (fewer
+ * for K > 8192, where a slab must fit LDS), and all slabs of a call together may number at
  * most 8 (for K = 2048: three problems of 32 rows), else VRL_INT4_ESHAPE and the caller uses
  * a grouped plan or vrl_int4_gemv_bf16.  scales and qzeros of the records are ignored.
  */
