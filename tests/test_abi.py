@@ -244,7 +244,9 @@ def test_lora_validation(lib):
     assert down(p, 1, 256, ads, 2, p, None) == 1001       # one weight type per launch
     ads[1].weights_fp32, ads[1].A = 1, p + 8
     assert down(p, 1, 256, ads, 2, p, None) == 1002
-    ads[1].A, ads[1].y = p, None
+    ads[1].A = p
+    assert down(p, 1, 256, ads, 2, p + 4, None) == 1002 and up(p + 4, 1, ads, 2, None) == 1002   # t is read 16 bytes at a time
+    ads[1].y = None
     assert up(p, 1, ads, 2, None) == 1003                 # the up-projection needs somewhere to add to
 
 

@@ -159,14 +159,6 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
 }
 
 
-// One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
-// keep many requests in flight), 8 when there are at least two per CU (several then share a CU
-// and overlap each other's prologue and epilogue).  Sixteen lanes share a cache slot (D / 16 values
-// each), so a wave reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the
-// workgroup 64.  Every 16-lane group keeps its own running softmax over the slots it visits
-// (key and value loads of ATT_UNROLL slots are issued together: values do not wait for scores);
-// the groups, the waves and the new token's own slot are merged at the end.
-// ATT_UNROLL: slots per 16-lane group in flight (keys and values: 2 * ATT_UNROLL vector loads per lane)
 // base + scaling * sum_j t[j] * B[n, j] with the roundings of the adapter wrapper's forward (see the
 // LoRA kernels below): what the projection's output would hold after its up-projection launch.
 template <bool FP32>
@@ -192,6 +184,14 @@ __device__ __forceinline__ float lora_fixed(float base, const void *B, int r, fl
     return round_bf16(base + delta);
 }
 
+// One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
+// keep many requests in flight), 8 when there are at least two per CU (several then share a CU
+// and overlap each other's prologue and epilogue).  Sixteen lanes share a cache slot (D / 16 values
+// each), so a wave reads four consecutive slots (4 * D * 2 bytes, contiguous) per load and the
+// workgroup 64.  Every 16-lane group keeps its own running softmax over the slots it visits
+// (key and value loads of ATT_UNROLL slots are issued together: values do not wait for scores);
+// the groups, the waves and the new token's own slot are merged at the end.
+// ATT_UNROLL: slots per 16-lane group in flight (keys and values: 2 * ATT_UNROLL vector loads per lane)
 // LORA: 0 none, 1 float32 adapter weights, 2 bf16 adapter weights
 template <int D, int ATT_WAVES, int ATT_UNROLL, int LORA>
 __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnArgs a) {
@@ -685,7 +685,7 @@ extern "C" int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, cons
 extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adapters, int n_adapters,
                                   float *t, void *hip_stream) {
     if (!x || !t) return VRL_INT4_ENULL;
-    if (misaligned(x, 16) || misaligned(t, 4)) return VRL_INT4_EALIGN;
+    if (misaligned(x, 16) || misaligned(t, 16)) return VRL_INT4_EALIGN;
     LoraArgs a;
     memset(&a, 0, sizeof a);
     const int rc = lora_args(a, M, K, adapters, n_adapters, false);
@@ -701,7 +701,7 @@ extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_ad
 extern "C" int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
                                     void *hip_stream) {
     if (!t) return VRL_INT4_ENULL;
-    if (misaligned(t, 4)) return VRL_INT4_EALIGN;
+    if (misaligned(t, 16)) return VRL_INT4_EALIGN;
     LoraArgs a;
     memset(&a, 0, sizeof a);
     const int rc = lora_args(a, M, 8, adapters, n_adapters, true);
