@@ -344,7 +344,9 @@ template <bool FUSED, bool NORM>
 int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int workgroups, size_t lds,
                         hipStream_t stream) {
     if constexpr (!NORM) {
-        if (xg) return launch_direct<FUSED, 16, 1, false, true>(args, workgroups, lds, stream);
+        if (xg && ks == 16) return launch_direct<FUSED, 16, 1, false, true>(args, workgroups, lds, stream);
+        if (xg && ks == 8) return launch_direct<FUSED, 8, 1, false, true>(args, workgroups, lds, stream);
+        if (xg) return launch_direct<FUSED, 4, 1, false, true>(args, workgroups, lds, stream);
     }
     if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1, NORM>(args, workgroups, lds, stream);
     if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4, NORM>(args, workgroups, lds, stream);
@@ -455,6 +457,7 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
     bool fused_any = false;
     int max_nsc = 1, max_m = 1;
+    long slab_tiles = 0;  // 16-column tiles x 16-row slabs of the launch
     for (int i = 0; i < n_problems; ++i) {
         const vrl_int4_problem &q = problems[i];
         if (!q.prepacked) return VRL_INT4_ESHAPE;
@@ -465,13 +468,16 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         fused_any |= q.fused_gate_up != 0;
         max_nsc = std::max(max_nsc, pp_nsc(q.K));
         max_m = std::max(max_m, q.M);
+        slab_tiles += (long)(((q.fused_gate_up ? q.N / 2 : q.N) + 15) / 16) * ((q.M + MAX_TILE_M - 1) / MAX_TILE_M);
     }
     // KS waves split K of a tile (one super-chunk each where K allows); with 8 or more
     // activation rows a workgroup carries several tiles so that one staging of x serves them
     const int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
-    const int tw = max_m >= 8 ? 16 / ks : 1;
-    // long K with one super-chunk per wave: the waves fetch their own activations, nothing is staged
-    const bool xg = !norm && ks == 16 && max_nsc <= 16;
+    // One super-chunk per wave: the waves can fetch their own activations, with nothing staged and one
+    // tile per workgroup.  Long K always does; shorter K with 8+ rows does while the launch is small
+    // (every tile then fetches its rows from L2 itself: for a wide matrix one staging per TW tiles wins).
+    const bool xg = !norm && max_nsc <= ks && (ks == 16 || (max_m >= 8 && slab_tiles <= 2L * device_cu_count()));
+    const int tw = (max_m >= 8 && !xg) ? 16 / ks : 1;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
