@@ -108,7 +108,8 @@ def check_against_oracle(sampled, logprob, lb, nb, w, T):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,V,w,T", [(1, 16384, 5.0, 1.0), (16, 16384, 5.0, 1.0), (3, 1000, 1.5, 0.7),
-                                     (2, 17, 0.0, 2.0), (5, 65536 + 24, 7.5, 0.9), (16, 16384, 1.0, 1.0)])
+                                     (2, 17, 0.0, 2.0), (5, 65536 + 24, 7.5, 0.9), (16, 16384, 1.0, 1.0),
+                                     (2, 8192, 3.0, 1.0), (4, 8192 + 64, 5.0, 1.3)])
 def test_cfg_sample_matches_oracle(ops_mod, B, V, w, T):
     print(f"[case] cfg_sample B={B} V={V} w={w} T={T}", flush=True)
     lb, nb = make_logits(40 + B + V, B, V)

@@ -8,8 +8,10 @@
 //   sampled = multinomial(probs, 1)                   = argmax(probs / q), q ~ Exp(1) drawn by the caller
 //                                                       with the call torch.multinomial makes itself
 //   lp      = log_softmax(cond / T)[sampled]
-// One workgroup per batch row walks the row three times (maxima, sums, draw); the row
-// (6 bytes per vocabulary entry) stays in cache between the walks.
+// One workgroup per batch row, three passes over the row (maxima, sums, draw).  The kernel is bound
+// by instruction issue on the row's one CU, so a row of up to 16384 entries is read once and its
+// scaled logits and exponentials stay in registers between the passes; longer (or unaligned) rows
+// are walked three times and stay in cache between the walks (6 bytes per vocabulary entry).
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -25,12 +27,9 @@ constexpr int WAVES = THREADS / WAVE;
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
 
-// round to nearest even, NaN kept quiet: what a torch bf16 kernel stores
+// round to nearest even through the hardware conversion (NaN stays NaN): what a torch bf16 kernel stores
 __device__ __forceinline__ float round_bf16(float v) {
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return __builtin_bit_cast(float, u | 0x00400000u);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return __builtin_bit_cast(float, u & 0xFFFF0000u);
+    return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)v) << 16);
 }
 
 struct Row {
@@ -38,16 +37,6 @@ struct Row {
     const uint16_t *uncond;
     const uint16_t *noise;
 };
-
-// guided / T and cond / T of one vocabulary entry, as bf16 values held in floats
-__device__ __forceinline__ void scaled_logits(const Row &r, int i, float w, float inv_t, float &gt, float &ct) {
-    const float c = bf16_to_f32(r.cond[i]);
-    const float u = bf16_to_f32(r.uncond[i]);
-    const float d = round_bf16(c - u);
-    const float g = round_bf16(u + round_bf16(w * d));
-    gt = round_bf16(g * inv_t);
-    ct = round_bf16(c * inv_t);
-}
 
 template <bool MAX>
 __device__ __forceinline__ void block_reduce2(float &a, float &b, float (*lds)[WAVES]) {
@@ -87,11 +76,43 @@ __device__ __forceinline__ void load_entries(const uint16_t *p, uint16_t (&v)[VE
     }
 }
 
+// guided / T and cond / T of one vocabulary entry (c, u: its two logits), as bf16 values held in floats
 __device__ __forceinline__ void scaled_pair(float c, float u, float w, float inv_t, float &gt, float &ct) {
     const float d = round_bf16(c - u);
     const float g = round_bf16(u + round_bf16(w * d));
     gt = round_bf16(g * inv_t);
     ct = round_bf16(c * inv_t);
+}
+
+// the better of two draws: the larger ratio, the lower index among equals, a NaN over any number (torch's argmax)
+__device__ __forceinline__ void take_better(float &bv, int &bi, float ov, int oi) {
+    const bool other_nan = ov != ov, mine_nan = bv != bv;
+    const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
+    if (take) {
+        bv = ov;
+        bi = oi;
+    }
+}
+
+// the workgroup's best draw, then the row's two outputs
+__device__ __forceinline__ void finish_row(const Row &r, float bv, int bi, float mc, float sc, float w, float inv_t,
+                                           int V, long long *sampled, float *logprob, float *best_v, int *best_i) {
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) take_better(bv, bi, __shfl_xor(bv, off, WAVE), __shfl_xor(bi, off, WAVE));
+    if (lane == 0) {
+        best_v[wave] = bv;
+        best_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < WAVES; ++k) take_better(bv, bi, best_v[k], best_i[k]);
+        if (bi >= V) bi = 0;  // V >= 1, so only if every ratio compared false: cannot happen for finite input
+        float gt, ct;
+        scaled_pair(bf16_to_f32(r.cond[bi]), bf16_to_f32(r.uncond[bi]), w, inv_t, gt, ct);
+        sampled[blockIdx.x] = bi;
+        logprob[blockIdx.x] = round_bf16(ct - mc - logf(sc));
+    }
 }
 
 template <int VEC>
@@ -165,40 +186,81 @@ __global__ __launch_bounds__(THREADS) void cfg_sample_kernel(const uint16_t *__r
             }
         }
     }
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    finish_row(r, bv, bi, mc, sc, w, inv_t, V, sampled, logprob, best_v, best_i);
+}
+
+// Rows of at most STEPS * 8192 entries (V % 8 == 0, 16-byte aligned): every thread reads its 8 * STEPS
+// entries once; same arithmetic and the same order of sums as the walking kernel.
+template <int STEPS>
+__global__ __launch_bounds__(THREADS) void cfg_sample_resident_kernel(const uint16_t *__restrict__ logits,
+                                                                      const uint16_t *__restrict__ noise,
+                                                                      long long *__restrict__ sampled,
+                                                                      float *__restrict__ logprob, int B, int V,
+                                                                      float w, float inv_t) {
+    __shared__ float red[2][WAVES];
+    __shared__ float best_v[WAVES];
+    __shared__ int best_i[WAVES];
+    const int b = blockIdx.x;
+    Row r;
+    r.cond = logits + (long)b * V;
+    r.uncond = logits + (long)(B + b) * V;
+    r.noise = noise + (long)b * V;
+    constexpr int N = 8 * STEPS;
+    uint16_t cb[STEPS][8], ub[STEPS][8], nb[STEPS][8];
 #pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, WAVE);
-        const int oi = __shfl_xor(bi, off, WAVE);
-        const bool other_nan = ov != ov, mine_nan = bv != bv;
-        const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
-        if (take) {
-            bv = ov;
-            bi = oi;
+    for (int s = 0; s < STEPS; ++s) {   // entries past the end repeat the thread's first in-range ones, uncounted
+        const int i = (s * THREADS + threadIdx.x) * 8;
+        const int ii = i < V ? i : 0;
+        load_entries<8>(r.cond + ii, cb[s]);
+        load_entries<8>(r.uncond + ii, ub[s]);
+        load_entries<8>(r.noise + ii, nb[s]);
+    }
+    float gt[N], ct[N];
+    float mg = -INFINITY, mc = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        const bool in = (s * THREADS + threadIdx.x) * 8 < V;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            scaled_pair(bf16_to_f32(cb[s][e]), bf16_to_f32(ub[s][e]), w, inv_t, gt[8 * s + e], ct[8 * s + e]);
+            mg = fmaxf(mg, in ? gt[8 * s + e] : -INFINITY);
+            mc = fmaxf(mc, in ? ct[8 * s + e] : -INFINITY);
         }
     }
-    if (lane == 0) {
-        best_v[wave] = bv;
-        best_i[wave] = bi;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int k = 1; k < WAVES; ++k) {
-            const float ov = best_v[k];
-            const int oi = best_i[k];
-            const bool other_nan = ov != ov, mine_nan = bv != bv;
-            const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
-            if (take) {
-                bv = ov;
-                bi = oi;
+    block_reduce2<true>(mg, mc, red);
+    float sg = 0.0f, sc = 0.0f;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        const bool in = (s * THREADS + threadIdx.x) * 8 < V;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            gt[8 * s + e] = expf(gt[8 * s + e] - mg);   // kept for the draw
+            const float ec = expf(ct[8 * s + e] - mc);
+            if (in) {
+                sg += gt[8 * s + e];
+                sc += ec;
             }
         }
-        if (bi >= V) bi = 0;  // V >= 1, so only if every ratio compared false: cannot happen for finite input
-        float gt, ct;
-        scaled_logits(r, bi, w, inv_t, gt, ct);
-        sampled[b] = bi;
-        logprob[b] = round_bf16(ct - mc - logf(sc));
     }
+    block_reduce2<false>(sg, sc, red);
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        const int i = (s * THREADS + threadIdx.x) * 8;
+        if (i < V) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = round_bf16(gt[8 * s + e] / sg);
+                const float ratio = round_bf16(p / bf16_to_f32(nb[s][e]));
+                if (ratio > bv || (ratio == bv && i + e < bi) || (ratio != ratio && bv == bv)) {
+                    bv = ratio;
+                    bi = i + e;
+                }
+            }
+        }
+    }
+    finish_row(r, bv, bi, mc, sc, w, inv_t, V, sampled, logprob, best_v, best_i);
 }
 
 }  // namespace
@@ -211,7 +273,10 @@ extern "C" int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_
         (reinterpret_cast<uintptr_t>(sampled) & 7u) || (reinterpret_cast<uintptr_t>(logprob) & 3u))
         return VRL_INT4_EALIGN;
     const bool wide = V % 8 == 0 && ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(noise)) & 15u) == 0;
-    auto kernel = wide ? &cfg_sample_kernel<8> : &cfg_sample_kernel<1>;
+    auto kernel = !wide ? &cfg_sample_kernel<1>
+                  : V <= THREADS * 8 ? &cfg_sample_resident_kernel<1>
+                  : V <= THREADS * 16 ? &cfg_sample_resident_kernel<2>
+                                      : &cfg_sample_kernel<8>;
     hipLaunchKernelGGL(kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint16_t *>(logits), static_cast<const uint16_t *>(noise),
                        reinterpret_cast<long long *>(sampled), logprob, B, V, cfg_weight, 1.0f / temperature);
