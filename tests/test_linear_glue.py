@@ -375,3 +375,35 @@ def test_prompt_sized_calls_go_through_the_library_gemm():
         # and it stays within a bf16 rounding or two of the fused decode kernel's fp32 epilogue
         small = gu(x[:1, :8])
         assert (small.float() - got[:1, :8].float()).abs().max().item() <= 2.0 ** -6 * max(1.0, got.abs().max().item())
+
+
+@pytest.mark.gpu
+def test_gradient_reaches_the_input_of_a_quantised_layer():
+    """A train-time replay over the frozen int4 base (inputs that carry a gradient, any row count): the
+    modules multiply by the dequantised weight through autograd-recorded ops, so ``x.grad`` is that of
+    the explicit bf16 product; without a gradient the same decode-sized call takes the HIP launch."""
+    import torch.nn.functional as F
+
+    dev = "cuda:0"
+    torch.manual_seed(5)
+    q = Int4Linear.from_linear(nn.Linear(512, 96, bias=True).to(torch.bfloat16).to(dev), 128).prepack_()
+    gu = Int4GateUpSiLU(Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128),
+                        Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128)).prepack_()
+    for rows in (2, 48):
+        x = torch.randn(rows, 512, device=dev).to(torch.bfloat16).requires_grad_(True)
+        ref = x.detach().clone().requires_grad_(True)
+        y = q(x)
+        assert y.requires_grad
+        y.float().square().sum().backward()
+        (F.linear(ref, q.dequantize()) + q.bias).float().square().sum().backward()
+        assert torch.equal(x.grad, ref.grad)
+        x.grad = ref.grad = None
+        z = gu(x)
+        assert z.requires_grad
+        z.float().sum().backward()
+        from visionrl_amd import ops
+        g, u = F.linear(ref, ops.int4_dequant(gu.qweight, gu.scales, gu.qzeros, 128)).chunk(2, dim=-1)
+        (F.silu(g) * u).float().sum().backward()
+        assert torch.equal(x.grad, ref.grad)
+        with torch.no_grad():
+            assert not q(x).requires_grad and not gu(x).requires_grad

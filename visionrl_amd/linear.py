@@ -5,7 +5,9 @@ The reference calls its decode linears as plain modules, ``module(x[..., K]) ->
 (``vrl/models/families/janus_pro/policy.py:673-678`` for the Llama trunk,
 ``policy.py:138-160`` for ``gen_head``).  These modules keep that calling
 convention and route the arithmetic to the HIP library; the weights are frozen
-(no gradient flows into the packed tensors).
+(no gradient flows into the packed tensors).  A call whose input carries a gradient
+(a train-time replay over the quantised base, e.g. under LoRA adapters) multiplies by
+the dequantised weight through the library GEMM, so the gradient reaches the input.
 """
 
 from __future__ import annotations
@@ -20,6 +22,11 @@ from .int4_format import check_packed, pack_nibbles, quantize_minmax
 # Calls with more activation rows than this (the prompt pass) rebuild the bf16 weight (bit-exact
 # tile, one launch) and hand the product to the library GEMM; the GEMV kernels are for decode.
 GEMM_ROWS = 32
+
+
+def _wants_grad(x: torch.Tensor) -> bool:
+    """The HIP launches are not recorded by autograd: such calls take the dequant + GEMM route."""
+    return torch.is_grad_enabled() and x.requires_grad
 
 
 def _rows(x: torch.Tensor, in_features: int) -> torch.Tensor:
@@ -127,6 +134,8 @@ class Int4Linear(nn.Module):
             self._handed = None
         if torch.compiler.is_compiling():
             y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
+        elif _wants_grad(x):
+            y = F.linear(rows, self.dequantize())
         elif handed is not None and handed[0] is x:  # computed by the group leader's launch
             y = handed[1]
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
@@ -190,10 +199,11 @@ class Int4GateUpSiLU(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
         packed = getattr(self, "_packed", None)
-        if packed is not None and not torch.compiler.is_compiling() and rows.shape[0] <= self._direct_rows \
-                and packed.blob.device == rows.device:
+        grad = _wants_grad(x) and not torch.compiler.is_compiling()
+        if packed is not None and not grad and not torch.compiler.is_compiling() \
+                and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
             y = self._call(rows)[0]
-        elif rows.shape[0] > GEMM_ROWS and not torch.compiler.is_compiling():
+        elif (grad or rows.shape[0] > GEMM_ROWS) and not torch.compiler.is_compiling():
             w = ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
             gate, up = F.linear(rows, w).chunk(2, dim=-1)   # prompt-sized call: one library GEMM
             y = F.silu(gate) * up
