@@ -401,12 +401,13 @@ __device__ __forceinline__ void load8(const void *base, long index, float (&f)[8
 
 // Both kernels are written without data-dependent branches: rows beyond M repeat row M - 1
 // (clamped index), which costs arithmetic but keeps every load of a lane in flight at once.
-// MB bounds the rows a build handles (8 or 32); FP32 is the adapters' weight type.
+// MB is the number of rows a workgroup handles (8 or 16; blockIdx.y picks the row block); FP32 is the
+// adapters' weight type.
 
-// One workgroup per column of t (an adapter row j): its four waves take interleaved 512-value
-// pieces of K; a lane holds 8 values of the A row and requests the matching 8 values of sixteen
-// activation rows at a time, then every row's partial sum is reduced over the wave and the four
-// waves meet in LDS.
+// One workgroup per column of t (an adapter row j) and block of MB rows: its four waves take
+// interleaved 512-value pieces of K; a lane holds 8 values of the A row and requests the matching 8
+// values of all its activation rows at once, then every row's partial sum is reduced over the wave
+// and the four waves meet in LDS.
 template <bool FP32, int MB>
 __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__restrict__ x, LoraArgs a,
                                                             float *__restrict__ t) {
@@ -424,29 +425,24 @@ __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__re
     for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
         if (k == i) A = a.ad[k].A, first = a.off[k];   // scalar selects, no indexing of the argument block
     const long arow = (long)(col - first) * a.K;
-    constexpr int RB = MB < 16 ? MB : 16;  // rows requested together
+    const int m_lo = blockIdx.y * MB, rows = min(MB, a.M - m_lo);
+    x += (long)m_lo * a.K;
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
     for (int k = (wave * WAVE + lane) * 8; k < a.K; k += THREADS * 8) {
         float af[8];
         load8<FP32>(A, arow + k, af);
+        uint4 xr[MB];
 #pragma unroll
-        for (int m0 = 0; m0 < MB; m0 += RB) {
-            uint4 xr[RB];
+        for (int u = 0; u < MB; ++u) xr[u] = *reinterpret_cast<const uint4 *>(x + (long)(u < rows ? u : rows - 1) * a.K + k);
+        __builtin_amdgcn_sched_barrier(0);  // all requests before the first use
 #pragma unroll
-            for (int u = 0; u < RB; ++u) {
-                const int m = m0 + u < a.M ? m0 + u : a.M - 1;
-                xr[u] = *reinterpret_cast<const uint4 *>(x + (long)m * a.K + k);
-            }
-            __builtin_amdgcn_sched_barrier(0);  // all requests of the batch before the first use
+        for (int u = 0; u < MB; ++u) {
+            const uint32_t w[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
 #pragma unroll
-            for (int u = 0; u < RB; ++u) {
-                const uint32_t w[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    acc[m0 + u] += bf16_to_f32(w[e] & 0xFFFFu) * af[2 * e] + bf16_to_f32(w[e] >> 16) * af[2 * e + 1];
-            }
+            for (int e = 0; e < 4; ++e)
+                acc[u] += bf16_to_f32(w[e] & 0xFFFFu) * af[2 * e] + bf16_to_f32(w[e] >> 16) * af[2 * e + 1];
         }
     }
 #pragma unroll
@@ -455,23 +451,24 @@ __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__re
         if (lane == 0) part[wave][m] = v;
     }
     __syncthreads();
-    if (threadIdx.x < a.M) {
+    if (threadIdx.x < rows) {
         float v = part[0][threadIdx.x];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) v += part[w][threadIdx.x];
         if (!FP32) v = round_bf16(v);  // lora_A's output tensor is bf16 then
-        t[(long)threadIdx.x * total + col] = v;
+        t[(long)(m_lo + threadIdx.x) * total + col] = v;
     }
 }
 
-// One thread per output column, 64 columns per workgroup: t of the adapter staged in LDS, the
-// column's row of B (up to RB values, zero beyond the rank) in registers, 16-byte LDS reads shared
-// by the wave.  Rows are walked by a plain loop (the products of a row land in LDS), then the base
-// outputs are fetched and rewritten eight rows at a time.
+// One thread per output column, 64 columns per workgroup, eight rows per workgroup (blockIdx.z): t of
+// the adapter and those rows staged in LDS, the column's row of B (up to RB values, zero beyond the
+// rank) in registers, 16-byte LDS reads shared by the wave.  The rows' products are formed while
+// their base outputs are on the way (one memory round trip per workgroup).
 constexpr int UP_THREADS = 64;
+constexpr int UP_ROWS = 8;
 template <bool FP32, int RB>
 __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__restrict__ t, LoraArgs a) {
-    extern __shared__ __align__(16) float ts[];  // M x r of this adapter, then M x UP_THREADS products
+    extern __shared__ __align__(16) float ts[];  // UP_ROWS x r of this adapter
     const int i = blockIdx.y;
     vrl_lora_adapter ad = a.ad[0];
     int first = 0;
@@ -480,19 +477,23 @@ __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__
         if (k == i) ad = a.ad[k], first = a.off[k];
     const int total = a.off[a.n], r = ad.r;
     if (blockIdx.x * UP_THREADS >= ad.N) return;  // uniform: adapters of one launch differ in width
-    float *us = ts + a.M * r;
+    const int m_lo = blockIdx.z * UP_ROWS, rows = min(UP_ROWS, a.M - m_lo);
+    const int n = blockIdx.x * UP_THREADS + threadIdx.x;
+    const int nn = n < ad.N ? n : ad.N - 1;  // lanes past the last column repeat it and store nothing
+    uint16_t *y = static_cast<uint16_t *>(ad.y);
+    uint16_t base[UP_ROWS];
+#pragma unroll
+    for (int d = 0; d < UP_ROWS; ++d)  // rows past the end repeat the last one and are not stored
+        base[d] = y[(long)(m_lo + (d < rows ? d : rows - 1)) * ad.N + nn];
     {   // t of this adapter: rows of r floats (r % 8 == 0), four at a time, requests issued together
-        const int r4 = r >> 2, count = a.M * r4;
+        const int r4 = r >> 2, count = rows * r4;
 #pragma unroll 4
         for (int idx = threadIdx.x; idx < count; idx += UP_THREADS) {
             const int m = idx / r4;
             *reinterpret_cast<float4 *>(ts + 4 * idx) =
-                *reinterpret_cast<const float4 *>(t + (long)m * total + first + 4 * (idx - m * r4));
+                *reinterpret_cast<const float4 *>(t + (long)(m_lo + m) * total + first + 4 * (idx - m * r4));
         }
     }
-    const int n = blockIdx.x * UP_THREADS + threadIdx.x;
-    const int nn = n < ad.N ? n : ad.N - 1;  // lanes past the last column repeat it and store nothing
-    uint16_t *y = static_cast<uint16_t *>(ad.y);
     float bf[RB];
 #pragma unroll
     for (int g = 0; g < RB / 8; ++g) {
@@ -503,42 +504,36 @@ __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__
         for (int e = 0; e < 8; ++e) bf[8 * g + e] = piece[e] * keep;
     }
     __syncthreads();
-#pragma unroll 2
-    for (int m = 0; m < a.M; ++m) {
-        const float *row = ts + m * r;
-        float u = 0.0f;
-#pragma unroll
-        for (int g = 0; g < RB / 4; ++g) {
-            const float4 tv = *reinterpret_cast<const float4 *>(row + (4 * g < r ? 4 * g : r - 4));  // x 0 beyond r
-            u += tv.x * bf[4 * g] + tv.y * bf[4 * g + 1] + tv.z * bf[4 * g + 2] + tv.w * bf[4 * g + 3];
-        }
-        us[m * UP_THREADS + threadIdx.x] = u;  // read back by the same thread only
-    }
     if (n >= ad.N) return;
-    for (int m0 = 0; m0 < a.M; m0 += 8) {
-        uint16_t base[8];
 #pragma unroll
-        for (int d = 0; d < 8; ++d) base[d] = y[(long)(m0 + d < a.M ? m0 + d : a.M - 1) * ad.N + n];
+    for (int d = 0; d < UP_ROWS; ++d) {
+        if (d < rows) {   // uniform
+            const float *row = ts + d * r;
+            float u = 0.0f;
 #pragma unroll
-        for (int d = 0; d < 8; ++d) {
-            const int m = m0 + d < a.M ? m0 + d : a.M - 1;  // rows past the end rewrite row M - 1 with its own value
-            float delta = us[m * UP_THREADS + threadIdx.x];
-            if (!FP32) delta = round_bf16(round_bf16(delta) * ad.scaling);  // lora_B's output, then * scaling
-            else delta *= ad.scaling;
-            y[(long)m * ad.N + n] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(base[d]) + delta);
+            for (int g = 0; g < RB / 4; ++g) {
+                const float4 tv = *reinterpret_cast<const float4 *>(row + (4 * g < r ? 4 * g : r - 4));  // x 0 beyond r
+                u += tv.x * bf[4 * g] + tv.y * bf[4 * g + 1] + tv.z * bf[4 * g + 2] + tv.w * bf[4 * g + 3];
+            }
+            float delta;
+            if (!FP32) delta = round_bf16(round_bf16(u) * ad.scaling);  // lora_B's output, then * scaling
+            else delta = u * ad.scaling;
+            y[(long)(m_lo + d) * ad.N + n] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(base[d]) + delta);
         }
     }
 }
 
 template <bool FP32, int MB>
 void launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_t stream) {
-    hipLaunchKernelGGL((lora_down_kernel<FP32, MB>), dim3(a.off[a.n]), dim3(THREADS), 0, stream, x, a, t);
+    hipLaunchKernelGGL((lora_down_kernel<FP32, MB>), dim3(a.off[a.n], (a.M + MB - 1) / MB), dim3(THREADS), 0, stream,
+                       x, a, t);
 }
 
 template <bool FP32, int RB>
 void launch_lora_up(const float *t, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
-    hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>), dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n),
-                       dim3(UP_THREADS), (size_t)a.M * (max_r + UP_THREADS) * sizeof(float), stream, t, a);
+    hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>),
+                       dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n, (a.M + UP_ROWS - 1) / UP_ROWS),
+                       dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, a);
 }
 
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
@@ -694,7 +689,7 @@ extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_ad
     auto xs = static_cast<const uint16_t *>(x);
     const bool fp32 = a.ad[0].weights_fp32 != 0;
     if (M <= 8) fp32 ? launch_lora_down<true, 8>(xs, a, t, stream) : launch_lora_down<false, 8>(xs, a, t, stream);
-    else fp32 ? launch_lora_down<true, 32>(xs, a, t, stream) : launch_lora_down<false, 32>(xs, a, t, stream);
+    else fp32 ? launch_lora_down<true, 16>(xs, a, t, stream) : launch_lora_down<false, 16>(xs, a, t, stream);
     return (int)hipGetLastError();
 }
 
