@@ -159,29 +159,22 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
 }
 
 
-// base + scaling * sum_j t[j] * B[n, j] with the roundings of the adapter wrapper's forward (see the
-// LoRA kernels below): what the projection's output would hold after its up-projection launch.
+// eight consecutive adapter weights (float32 or bf16) as floats
 template <bool FP32>
-__device__ __forceinline__ float lora_fixed(float base, const void *B, int r, float scale, const float *t, long n) {
-    if (!B) return base;  // uniform
-    float u = 0.0f;
-    for (int j = 0; j < r; j += 8) {  // r % 8 == 0
-        float bf[8];
-        if constexpr (FP32) {
-            const float4 x = *reinterpret_cast<const float4 *>(static_cast<const float *>(B) + n * r + j);
-            const float4 y = *reinterpret_cast<const float4 *>(static_cast<const float *>(B) + n * r + j + 4);
-            bf[0] = x.x, bf[1] = x.y, bf[2] = x.z, bf[3] = x.w, bf[4] = y.x, bf[5] = y.y, bf[6] = y.z, bf[7] = y.w;
-        } else {
-            const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(B) + n * r + j);
-            const uint32_t x[4] = {w.x, w.y, w.z, w.w};
+__device__ __forceinline__ void load8(const void *base, long index, float (&f)[8]) {
+    if constexpr (FP32) {
+        const float4 a = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index);
+        const float4 b = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index + 4);
+        f[0] = a.x, f[1] = a.y, f[2] = a.z, f[3] = a.w, f[4] = b.x, f[5] = b.y, f[6] = b.z, f[7] = b.w;
+    } else {
+        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + index);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) bf[2 * e] = bf16_to_f32(x[e] & 0xFFFFu), bf[2 * e + 1] = bf16_to_f32(x[e] >> 16);
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
+            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) u += t[j + e] * bf[e];
     }
-    const float delta = FP32 ? u * scale : round_bf16(round_bf16(u) * scale);
-    return round_bf16(base + delta);
 }
 
 // One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
@@ -234,16 +227,57 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     if (p > 0) request(0);
 
     if constexpr (LORA != 0) {
-        // q, k, v of this head with their adapters added, through LDS (the rotation pairs columns)
+        // q, k, v of this head with their adapters added: base + scaling * sum_j t[j] * B[n, j] with the
+        // roundings of the adapter wrapper's forward (what the projection's output would hold after an
+        // up-projection launch).  NS threads share an output column, each taking eight ranks per trip
+        // (the requests of a trip are independent: one memory round trip); the partial sums meet in
+        // LDS in a fixed order, and the values go on through LDS because the rotation pairs columns.
+        constexpr bool FP32 = LORA == 1;
+        constexpr int NS = ATT_WAVES * WAVE / D;
+        __shared__ float lpart[3][NS][D];
+        const int col = tid % D, slice = tid / D;   // the slice is uniform over a wave (D >= 64)
+        const float *trow = a.t + (long)m * a.t_stride;
+        const long ncol[3] = {(long)h * D + col, (long)hk * D + col, (long)hk * D + col};
+        float base3[3] = {0.0f, 0.0f, 0.0f};
         if (tid < D) {
-            const float *trow = a.t + (long)m * a.t_stride;
-            const long nq = (long)h * D + tid, nk = (long)hk * D + tid;
-            qs[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.q[(long)m * a.q_stride + nq]), a.lb[0], a.lr[0], a.lscale[0],
-                                            trow + a.loff[0], nq);
-            ks[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.k[(long)m * a.kv_stride + nk]), a.lb[1], a.lr[1], a.lscale[1],
-                                            trow + a.loff[1], nk);
-            vs[tid] = lora_fixed<LORA == 1>(bf16_to_f32(a.v[(long)m * a.kv_stride + nk]), a.lb[2], a.lr[2], a.lscale[2],
-                                            trow + a.loff[2], nk);
+            base3[0] = bf16_to_f32(a.q[(long)m * a.q_stride + ncol[0]]);
+            base3[1] = bf16_to_f32(a.k[(long)m * a.kv_stride + ncol[1]]);
+            base3[2] = bf16_to_f32(a.v[(long)m * a.kv_stride + ncol[2]]);
+        }
+        float u3[3] = {0.0f, 0.0f, 0.0f};
+        for (int j = slice * 8; j < LORA_MAX_RANK; j += NS * 8) {   // one trip unless a rank exceeds 8 * NS
+            float bw[3][8], tw[3][8];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                if (a.lb[i] && j < a.lr[i]) {   // uniform
+                    load8<FP32>(a.lb[i], ncol[i] * a.lr[i] + j, bw[i]);
+                    load8<true>(trow, a.loff[i] + j, tw[i]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) bw[i][e] = tw[i][e] = 0.0f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) u3[i] += tw[i][e] * bw[i][e];
+        }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) lpart[i][slice][col] = u3[i];
+        __syncthreads();
+        if (tid < D) {
+            float fixed[3];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                float u = lpart[i][0][tid];
+#pragma unroll
+                for (int s = 1; s < NS; ++s) u += lpart[i][s][tid];
+                const float delta = FP32 ? u * a.lscale[i] : round_bf16(round_bf16(u) * a.lscale[i]);
+                fixed[i] = a.lb[i] ? round_bf16(base3[i] + delta) : base3[i];
+            }
+            qs[tid] = fixed[0];
+            ks[tid] = fixed[1];
+            vs[tid] = fixed[2];
         }
         __syncthreads();
     }
@@ -381,23 +415,6 @@ struct LoraArgs {
     int32_t off[LORA_MAX_ADAPTERS + 1];  // first column of each adapter in t
     int32_t n, M, K;
 };
-
-template <bool FP32>
-__device__ __forceinline__ void load8(const void *base, long index, float (&f)[8]) {
-    if constexpr (FP32) {
-        const float4 a = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index);
-        const float4 b = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index + 4);
-        f[0] = a.x, f[1] = a.y, f[2] = a.z, f[3] = a.w, f[4] = b.x, f[5] = b.y, f[6] = b.z, f[7] = b.w;
-    } else {
-        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + index);
-        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
-            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
-        }
-    }
-}
 
 // Both kernels are written without data-dependent branches: rows beyond M repeat row M - 1
 // (clamped index), which costs arithmetic but keeps every load of a lane in flight at once.
