@@ -67,7 +67,10 @@ int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q
  *   vrl_lora_down_bf16:    t[m, off_i + j] = sum_k x[m,k] * A_i[j,k]         for every adapter i
  *   vrl_lora_up_add_bf16:  y_i[m,n] = bf16( y_i[m,n] + scaling_i * sum_j t[m, off_i + j] * B_i[n,j] )
  * with t a float32 [M, r_total] scratch buffer of the caller's, off_i the sum of the ranks before
- * adapter i.  Adapter weights are float32 (what PEFT keeps by default: everything in fp32, one
+ * adapter i.  The up-projection also takes t in pieces: float32 [M, t_parts, r_total] whose t_parts
+ * rows per m are summed in order first (1 <= t_parts <= 256; 1 for what vrl_lora_down_bf16 wrote):
+ * vrl_rope_attn_decode_lora_bf16 leaves the down-projection of its output in that form, one piece
+ * per head.  Adapter weights are float32 (what PEFT keeps by default: everything in fp32, one
  * rounding when the result returns to bf16) or bf16 (weights_fp32 = 0: t, the up-projection and its
  * scaled value are rounded to bf16 as the bf16 modules round them); one type per launch.
  * 1 <= n_adapters <= 4, r % 8 == 0, r <= 64, K % 8 == 0, pointers 16-byte aligned.
@@ -83,8 +86,8 @@ typedef struct vrl_lora_adapter {
 
 int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_adapter *adapters, int n_adapters,
                        float *t, void *hip_stream);
-int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
-                         void *hip_stream);
+int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vrl_lora_adapter *adapters,
+                         int n_adapters, void *hip_stream);
 
 /*
  * vrl_rope_attn_decode_bf16 with the up-projections of the q, k, v adapters added while the new
@@ -92,8 +95,14 @@ int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters
  * and the attention: q, k, v hold the base projections' outputs, `t` the down-projections of the
  * group (vrl_lora_down_bf16), and the kernel attends with (and appends to the cache)
  *   q' = bf16(q + scaling_q * t[:, off_q : off_q + r_q] . B_q^T), likewise k', v'
- * with the roundings described above.  A NULL B means the projection has no adapter; at least one
- * must be given.  q, k and v themselves are left as they are.
+ * with the roundings described above.  A NULL B means the projection has no adapter.  q, k and v
+ * themselves are left as they are.
+ * The adapter of the projection that consumes `out` (o_proj) can have its down-projection computed
+ * here as well, in place of a vrl_lora_down_bf16 launch after the attention: with o_A given, the
+ * workgroup of row m, head h writes
+ *   o_t[m, h, j] = sum_d out[m, h * D + d] * o_A[j, h * D + d]        (out as rounded to bf16)
+ * and vrl_lora_up_add_bf16(o_t, n_heads, ...) adds the up-projection of the heads' sum.
+ * At least one of q_B, k_B, v_B, o_A must be given; t may be NULL when only o_A is.
  */
 typedef struct vrl_attn_lora {
     const float *t;          /* [M, t_stride] float32, 16-byte aligned */
@@ -104,6 +113,10 @@ typedef struct vrl_attn_lora {
     int32_t offset[3];       /* first column of each adapter in t, a multiple of 4 */
     float scaling[3];
     int32_t reserved;
+    const void *o_A;         /* [o_r, n_heads * D] (type as weights_fp32 says), 16-byte aligned, or NULL */
+    float *o_t;              /* [M, n_heads, o_r] float32, 16-byte aligned */
+    int32_t o_r;             /* a multiple of 8 up to 64 */
+    int32_t reserved2;
 } vrl_attn_lora;
 
 int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,

@@ -224,6 +224,30 @@ def test_decode_layer_validation(lib):
     assert call(qs=128) == 1001          # rows narrower than the heads they hold
     assert call(ks=260) == 1001          # row stride must keep rows 16-byte aligned
     assert call(kc=p + 8) == 1002 and call(pos=p + 4) == 1002
+    # the adapter record of the second form
+    with_lora = lib.vrl_rope_attn_decode_lora_bf16
+    rec = _lib.AttnLora()
+
+    def call_lora(r):
+        a = ok
+        return with_lora(a["q"], a["k"], a["v"], a["qs"], a["ks"], a["kc"], a["vc"], a["cos"], a["sin"], a["mask"],
+                         a["pos"], a["out"], a["M"], a["H"], a["Hkv"], a["D"], a["L"], a["scale"],
+                         ctypes.byref(r) if r is not None else None, None)
+
+    assert call_lora(None) == 1003 and call_lora(rec) == 1003     # no record, a record without any adapter
+    rec.q_B, rec.r[0], rec.t_stride, rec.weights_fp32 = p, 8, 8, 1
+    assert call_lora(rec) == 1003                                 # q/k/v adapters read t
+    rec.t, rec.r[0] = p, 12
+    assert call_lora(rec) == 1001                                 # rank % 8
+    rec.r[0], rec.offset[0] = 8, 4
+    assert call_lora(rec) == 1001                                 # the adapter's columns must lie inside a row of t
+    rec.offset[0], rec.q_B = 0, None
+    rec.o_A, rec.o_r = p, 16
+    assert call_lora(rec) == 1003                                 # nowhere to leave the pieces
+    rec.o_t, rec.o_r = p, 72
+    assert call_lora(rec) == 1001
+    rec.o_r, rec.o_t = 16, p + 8
+    assert call_lora(rec) == 1002
 
 
 def test_lora_validation(lib):
@@ -233,7 +257,7 @@ def test_lora_validation(lib):
         ad.A, ad.B, ad.y, ad.N, ad.r, ad.scaling, ad.weights_fp32 = p, p, p, 64, 8, 2.0, 1
     down, up = lib.vrl_lora_down_bf16, lib.vrl_lora_up_add_bf16
     assert down(None, 1, 256, ads, 2, p, None) == 1003 and down(p, 1, 256, None, 2, p, None) == 1003
-    assert down(p, 1, 256, ads, 2, None, None) == 1003 and up(None, 1, ads, 2, None) == 1003
+    assert down(p, 1, 256, ads, 2, None, None) == 1003 and up(None, 1, 1, ads, 2, None) == 1003
     assert down(p, 0, 256, ads, 2, p, None) == 1001 and down(p, 33, 256, ads, 2, p, None) == 1001   # rows
     assert down(p, 1, 260, ads, 2, p, None) == 1001 and down(p, 1, 256, ads, 5, p, None) == 1001    # K % 8, adapters
     ads[1].r = 12
@@ -245,9 +269,11 @@ def test_lora_validation(lib):
     ads[1].weights_fp32, ads[1].A = 1, p + 8
     assert down(p, 1, 256, ads, 2, p, None) == 1002
     ads[1].A = p
-    assert down(p, 1, 256, ads, 2, p + 4, None) == 1002 and up(p + 4, 1, ads, 2, None) == 1002   # t is read 16 bytes at a time
+    assert down(p, 1, 256, ads, 2, p + 4, None) == 1002 and up(p + 4, 1, 1, ads, 2, None) == 1002   # t is read 16 bytes at a time
     ads[1].y = None
-    assert up(p, 1, ads, 2, None) == 1003                 # the up-projection needs somewhere to add to
+    assert up(p, 1, 1, ads, 2, None) == 1003              # the up-projection needs somewhere to add to
+    ads[1].y = p
+    assert up(p, 0, 1, ads, 2, None) == 1001 and up(p, 257, 1, ads, 2, None) == 1001   # pieces of t per row
 
 
 def test_cfg_sample_validation(lib):

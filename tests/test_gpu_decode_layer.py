@@ -336,6 +336,66 @@ def test_attention_adds_the_qkv_adapters_itself(ops_mod, M, H, Hkv, D, fp32, whi
         ops_mod.rope_attn_decode(q1, k1, v1, kc1, vc1, t["cos"], t["sin"], mask, pos, c["scaling"], lora=group)
 
 
+@pytest.mark.parametrize("M,H,Hkv,D,fp32,r,with_qkv", [(2, 16, 16, 128, True, 32, True), (32, 16, 16, 128, True, 32, False),
+                                                        (3, 8, 2, 64, False, 16, False), (5, 4, 4, 64, True, 64, True),
+                                                        (9, 16, 16, 128, False, 64, False), (4, 2, 1, 128, True, 8, False)])
+def test_attention_leaves_the_output_adapters_down_projection(ops_mod, M, H, Hkv, D, fp32, r, with_qkv):
+    """``rope_attn_decode(..., out_lora=group)``: the launch writes, per head, that head's share of
+    ``out . A^T``; the heads' sum is the down-projection of the whole row (float64 over the bf16 output),
+    the attention output itself is what the plain launch gives, and ``launch_up`` over the pieces equals the
+    oracle's adapter applied to that output."""
+    say("attention with output adapter", M, H, Hkv, D, fp32, r, with_qkv)
+    L, p, N, K = 96, 57, 200, 256
+    c = attn_case(500 + M, M, H, Hkv, D, L, p)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    t = {n: bits_to_bf16(c[n], DEV) for n in ("q", "k", "v", "cos", "sin")}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([p], dtype=torch.int64, device=DEV)
+    gen = torch.Generator().manual_seed(M + r)
+    A = (torch.randn(r, H * D, generator=gen) * (H * D) ** -0.5).to(dtype).to(DEV)
+    B = (torch.randn(N, r, generator=gen) * 0.2).to(dtype).to(DEV)
+    y0 = rand_bits(np.random.default_rng(M), (M, N))
+    y = bits_to_bf16(y0, DEV)
+    out = torch.empty((M, H * D), dtype=torch.bfloat16, device=DEV)
+    group = ops_mod.LoraAdd(out, [(A, B, 1.5, y)], parts=H)
+    qkv = None
+    if with_qkv:
+        x = bits_to_bf16(rand_bits(np.random.default_rng(M + 1), (M, K)), DEV)
+        Aq = (torch.randn(16, K, generator=gen) * K ** -0.5).to(dtype).to(DEV)
+        Bq = (torch.randn(H * D, 16, generator=gen) * 0.2).to(dtype).to(DEV)
+        qkv = ops_mod.LoraAdd(x, [(Aq, Bq, 2.0, t["q"])])
+        qkv.launch_down()
+    kc, vc = bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV)
+    got = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc, vc, t["cos"], t["sin"], mask, pos, c["scaling"],
+                                   out=out, lora=qkv, out_lora=group)
+    kc2, vc2 = bits_to_bf16(c["kc"], DEV), bits_to_bf16(c["vc"], DEV)
+    plain = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc2, vc2, t["cos"], t["sin"], mask, pos, c["scaling"],
+                                     lora=qkv)
+    torch.cuda.synchronize()
+    # another build of the same kernel body: the compiler may fuse a multiply-add differently
+    assert got.data_ptr() == out.data_ptr()
+    print("  outputs that differ from the plain launch:", (got != plain).float().mean().item(),
+          (got.float() - plain.float()).abs().max().item(), flush=True)
+    within_one_step_of(bf16_to_bits(got), bf16_to_bits(plain), bf16_to_bits(plain))
+    assert (got != plain).float().mean().item() < 0.01
+    # the pieces: [M, H, r], head h from columns h*D .. (h+1)*D of the output
+    o64 = out.float().cpu().numpy().astype(np.float64)
+    A64 = A.float().cpu().numpy().astype(np.float64)
+    pieces = group.t.cpu().numpy().astype(np.float64)
+    assert pieces.shape == (M, H, r)
+    want_pieces = np.einsum("mhd,jhd->mhj", o64.reshape(M, H, D), A64.reshape(r, H, D))
+    scale = np.abs(o64).max() * np.abs(A64).max() * D
+    assert np.abs(pieces - want_pieces).max() <= 2.0 ** -20 * scale
+    assert np.abs(pieces.sum(axis=1) - o64 @ A64.T).max() <= 2.0 ** -18 * scale * H
+    group.launch_up()
+    torch.cuda.synchronize()
+    want = d.lora_add(y0, bf16_to_bits(out), A.float().cpu().numpy(), B.float().cpu().numpy(), 1.5, fp32)
+    within_one_step_of(bf16_to_bits(y), want, y0)
+    with pytest.raises(ValueError):   # a group over another tensor than `out`
+        ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc2, vc2, t["cos"], t["sin"], mask, pos, c["scaling"],
+                                 out_lora=group)
+
+
 # ------------------------------------------------------------------ seeded random shapes through every decode-layer launch
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_shapes(ops_mod, seed):

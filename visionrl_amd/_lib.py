@@ -101,6 +101,10 @@ class AttnLora(ctypes.Structure):
         ("offset", ctypes.c_int32 * 3),
         ("scaling", ctypes.c_float * 3),
         ("reserved", ctypes.c_int32),
+        ("o_A", ctypes.c_void_p),
+        ("o_t", ctypes.c_void_p),
+        ("o_r", ctypes.c_int32),
+        ("reserved2", ctypes.c_int32),
     ]
 
 
@@ -160,7 +164,7 @@ def _bind(lib):
     lib.vrl_lora_down_bf16.restype = ci
     lib.vrl_lora_down_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
     lib.vrl_lora_up_add_bf16.restype = ci
-    lib.vrl_lora_up_add_bf16.argtypes = [vp, ci, ctypes.POINTER(LoraAdapter), ci, vp]
+    lib.vrl_lora_up_add_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp]
     lib.vrl_rope_attn_decode_bf16.restype = ci
     lib.vrl_rope_attn_decode_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                               ci, ci, ci, ci, ci, ctypes.c_float, vp]

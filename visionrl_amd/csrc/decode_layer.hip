@@ -119,6 +119,10 @@ struct AttnArgs {
     const void *lb[3];       // B [N, r] of the q, k, v adapter, nullptr for none
     int lr[3], loff[3];      // rank, first column in t
     float lscale[3];
+    // adapter on the projection that consumes `out`: this head's share of out . A^T goes to ot
+    const void *oa;          // A [orank, n_heads * D], nullptr for none
+    float *ot;               // [M, n_heads, orank]
+    int orank;
 };
 
 // Raw cache vectors: D / 16 bf16 values of one slot per lane (16 or 8 bytes).
@@ -225,6 +229,28 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         }
     };
     if (p > 0) request(0);
+
+    // The adapter of the projection that follows: thread (j, l16) holds the lane's VEC columns of row j
+    // of A (rows j, j + OJ, ... if the rank exceeds OJ; the first is requested here, ahead of its use).
+    constexpr int OJ = ATT_WAVES * WAVE / 16;
+    const int oj = tid >> 4;
+    float oaw[VEC];
+    auto request_oa = [&](int j) {
+        const long at = (long)j * a.n_heads * D + (long)h * D + l16 * VEC;
+        if constexpr (VEC == 8) {
+            load8<LORA == 1>(a.oa, at, oaw);
+        } else if constexpr (LORA == 1) {
+            const float4 w4 = *reinterpret_cast<const float4 *>(static_cast<const float *>(a.oa) + at);
+            oaw[0] = w4.x, oaw[1] = w4.y, oaw[2] = w4.z, oaw[3] = w4.w;
+        } else {
+            const uint2 w2 = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(a.oa) + at);
+            oaw[0] = bf16_to_f32(w2.x & 0xFFFFu), oaw[1] = bf16_to_f32(w2.x >> 16);
+            oaw[2] = bf16_to_f32(w2.y & 0xFFFFu), oaw[3] = bf16_to_f32(w2.y >> 16);
+        }
+    };
+    if constexpr (LORA != 0) {
+        if (a.oa && oj < a.orank) request_oa(oj);
+    }
 
     if constexpr (LORA != 0) {
         // q, k, v of this head with their adapters added: base + scaling * sum_j t[j] * B[n, j] with the
@@ -401,7 +427,25 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             }
             o /= sum;
         }
-        a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)f32_to_bf16_bits(o);
+        const uint32_t bits = f32_to_bf16_bits(o);
+        a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)bits;
+        if constexpr (LORA != 0) qs[tid] = bf16_to_f32(bits);  // what the next projection reads
+    }
+    if constexpr (LORA != 0) {
+        if (a.oa) {  // uniform
+            __syncthreads();
+            float ov[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) ov[i] = qs[l16 * VEC + i];
+            for (int j = oj; j < a.orank; j += OJ) {
+                if (j != oj) request_oa(j);
+                float part = 0.0f;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) part += ov[i] * oaw[i];
+                part = row16_sum(part);  // the sixteen lanes that share row j
+                if (l16 == 0) a.ot[((long)m * a.n_heads + h) * a.orank + j] = part;
+            }
+        }
     }
 }
 
@@ -484,7 +528,7 @@ __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__re
 constexpr int UP_THREADS = 64;
 constexpr int UP_ROWS = 8;
 template <bool FP32, int RB>
-__global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__restrict__ t, LoraArgs a) {
+__global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__restrict__ t, int parts, LoraArgs a) {
     extern __shared__ __align__(16) float ts[];  // UP_ROWS x r of this adapter
     const int i = blockIdx.y;
     vrl_lora_adapter ad = a.ad[0];
@@ -502,13 +546,24 @@ __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__
 #pragma unroll
     for (int d = 0; d < UP_ROWS; ++d)  // rows past the end repeat the last one and are not stored
         base[d] = y[(long)(m_lo + (d < rows ? d : rows - 1)) * ad.N + nn];
-    {   // t of this adapter: rows of r floats (r % 8 == 0), four at a time, requests issued together
+    {   // t of this adapter: rows of r floats (r % 8 == 0), four at a time; a row given as `parts`
+        // partial rows is their sum in order (a bf16 adapter's t is rounded once the sum is complete)
         const int r4 = r >> 2, count = rows * r4;
-#pragma unroll 4
         for (int idx = threadIdx.x; idx < count; idx += UP_THREADS) {
             const int m = idx / r4;
-            *reinterpret_cast<float4 *>(ts + 4 * idx) =
-                *reinterpret_cast<const float4 *>(t + (long)(m_lo + m) * total + first + 4 * (idx - m * r4));
+            const float *src = t + (long)(m_lo + m) * parts * total + first + 4 * (idx - m * r4);
+            float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int q0 = 0; q0 < parts; q0 += 16) {   // sixteen pieces requested together, added in order
+                float4 w[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                    w[u] = *reinterpret_cast<const float4 *>(src + (long)(q0 + u < parts ? q0 + u : parts - 1) * total);
+#pragma unroll
+                for (int u = 0; u < 16; ++u)
+                    if (q0 + u < parts) v.x += w[u].x, v.y += w[u].y, v.z += w[u].z, v.w += w[u].w;
+            }
+            if (!FP32) v.x = round_bf16(v.x), v.y = round_bf16(v.y), v.z = round_bf16(v.z), v.w = round_bf16(v.w);
+            *reinterpret_cast<float4 *>(ts + 4 * idx) = v;
         }
     }
     float bf[RB];
@@ -547,10 +602,10 @@ void launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_
 }
 
 template <bool FP32, int RB>
-void launch_lora_up(const float *t, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
+void launch_lora_up(const float *t, int parts, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
     hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>),
                        dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n, (a.M + UP_ROWS - 1) / UP_ROWS),
-                       dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, a);
+                       dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, parts, a);
 }
 
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
@@ -649,8 +704,6 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
         launch_attn<0>(a, M, D, stream);
         return (int)hipGetLastError();
     }
-    if (!lora->t) return VRL_INT4_ENULL;
-    if (misaligned(lora->t, 16) || lora->t_stride < 8 || lora->t_stride % 4 != 0) return VRL_INT4_ESHAPE;
     const void *bs[3] = {lora->q_B, lora->k_B, lora->v_B};
     bool any = false;
     for (int i = 0; i < 3; ++i) {
@@ -660,10 +713,21 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
         a.lscale[i] = lora->scaling[i];
         if (!bs[i]) continue;
         any = true;
+        if (!lora->t) return VRL_INT4_ENULL;
+        if (misaligned(lora->t, 16) || lora->t_stride < 8 || lora->t_stride % 4 != 0) return VRL_INT4_ESHAPE;
         if (lora->r[i] < 8 || lora->r[i] % 8 != 0 || lora->r[i] > LORA_MAX_RANK || lora->offset[i] < 0 ||
             lora->offset[i] % 4 != 0 || lora->offset[i] + lora->r[i] > lora->t_stride)
             return VRL_INT4_ESHAPE;
         if (misaligned(bs[i], 16)) return VRL_INT4_EALIGN;
+    }
+    if (lora->o_A) {
+        if (!lora->o_t) return VRL_INT4_ENULL;
+        if (lora->o_r < 8 || lora->o_r % 8 != 0 || lora->o_r > LORA_MAX_RANK) return VRL_INT4_ESHAPE;
+        if (misaligned(lora->o_A, 16) || misaligned(lora->o_t, 16)) return VRL_INT4_EALIGN;
+        a.oa = lora->o_A;
+        a.ot = lora->o_t;
+        a.orank = lora->o_r;
+        any = true;
     }
     if (!any) return VRL_INT4_ENULL;
     a.t = lora->t;
@@ -710,9 +774,10 @@ extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_ad
     return (int)hipGetLastError();
 }
 
-extern "C" int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapter *adapters, int n_adapters,
-                                    void *hip_stream) {
+extern "C" int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vrl_lora_adapter *adapters,
+                                    int n_adapters, void *hip_stream) {
     if (!t) return VRL_INT4_ENULL;
+    if (t_parts < 1 || t_parts > 256) return VRL_INT4_ESHAPE;
     if (misaligned(t, 16)) return VRL_INT4_EALIGN;
     LoraArgs a;
     memset(&a, 0, sizeof a);
@@ -725,9 +790,9 @@ extern "C" int vrl_lora_up_add_bf16(const float *t, int M, const vrl_lora_adapte
     }
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const bool fp32 = a.ad[0].weights_fp32 != 0;
-    if (fp32) max_r <= 32 ? launch_lora_up<true, 32>(t, a, max_n, max_r, stream)
-                          : launch_lora_up<true, 64>(t, a, max_n, max_r, stream);
-    else max_r <= 32 ? launch_lora_up<false, 32>(t, a, max_n, max_r, stream)
-                     : launch_lora_up<false, 64>(t, a, max_n, max_r, stream);
+    if (fp32) max_r <= 32 ? launch_lora_up<true, 32>(t, t_parts, a, max_n, max_r, stream)
+                          : launch_lora_up<true, 64>(t, t_parts, a, max_n, max_r, stream);
+    else max_r <= 32 ? launch_lora_up<false, 32>(t, t_parts, a, max_n, max_r, stream)
+                     : launch_lora_up<false, 64>(t, t_parts, a, max_n, max_r, stream);
     return (int)hipGetLastError();
 }

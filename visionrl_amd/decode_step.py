@@ -22,8 +22,9 @@ fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry 
 adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
 the norm as a launch of its own (the adapters read the normalised row), a down-projection launch
 for the q|k|v adapters (their up-projections are added by the attention launch as it reads q, k, v)
-and a down- and an up-projection launch for o_proj's: nine launches.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not qualify, and
-callers then keep the module path.
+and an up-projection launch for o_proj's (its down-projection is left behind by the attention launch,
+one piece per head): eight launches.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not
+qualify, and callers then keep the module path.
 """
 
 from __future__ import annotations
@@ -200,20 +201,22 @@ class NativeDecodeTrunk:
                               (launch.table, len(launch.table), ctypes.byref(launch.norm))))
             return launch.outputs
 
-        def lora(x, outs, adapters, up=True):
+        def lora(x, outs, adapters, up=True, parts=1):
             """outs[i] += adapter i applied to x, for the projections that carry one: a down-projection
-            launch and, unless the consumer adds the up-projection itself (``up=False``: the attention
+            launch (unless the producer of x leaves it in ``parts`` pieces: the attention does for its
+            output) and, unless the consumer adds the up-projection itself (``up=False``: the attention
             does for q, k, v), an up-projection launch.  Returns the group or ``None``."""
             todo = [(A, B, s, y) for y, ad in zip(outs, adapters) if ad is not None for A, B, s in [ad]]
             if not todo:
                 return None
-            launch = ops.LoraAdd(x, todo)
+            launch = ops.LoraAdd(x, todo, parts=parts)
             self._keep.append(launch)
             n = len(launch.table)
-            calls.append((lib.vrl_lora_down_bf16, (x.data_ptr(), rows, x.shape[1], launch.table, n,
-                                                   launch.t.data_ptr())))
+            if parts == 1:
+                calls.append((lib.vrl_lora_down_bf16, (x.data_ptr(), rows, x.shape[1], launch.table, n,
+                                                       launch.t.data_ptr())))
             if up:
-                calls.append((lib.vrl_lora_up_add_bf16, (launch.t.data_ptr(), rows, launch.table, n)))
+                calls.append((lib.vrl_lora_up_add_bf16, (launch.t.data_ptr(), parts, rows, launch.table, n)))
             return launch
 
         def normed_gemv(module, weights, fused, adapters=(), up=True):
@@ -249,13 +252,17 @@ class NativeDecodeTrunk:
             attn_args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), keys.data_ptr(),
                          values.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(), mask.data_ptr(),
                          slot.data_ptr(), self.attn.data_ptr(), rows, H, Hkv, D, self.max_len, float(attn.scaling))
-            if group is None:
-                calls.append((lib.vrl_rope_attn_decode_bf16, attn_args))
-            else:   # the attention adds the up-projections of the q, k, v adapters while it reads them
-                calls.append((lib.vrl_rope_attn_decode_lora_bf16,
-                              (*attn_args, ctypes.byref(group.attn_record(q, k, v)))))
+            # the attention adds the up-projections of the q, k, v adapters while it reads them, and leaves
+            # the down-projection of o_proj's adapter behind, one piece per head
+            record = group.attn_record(q, k, v) if group is not None else None
+            attn_at = len(calls)
+            calls.append(None)
             outs = gemv([(self.attn, proj["o_proj"][0], False)])
-            lora(self.attn, outs, [proj["o_proj"][1]])
+            o_group = lora(self.attn, outs, [proj["o_proj"][1]], parts=H)
+            if o_group is not None:
+                record = o_group.attn_output_record(record)
+            calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args) if record is None else \
+                (lib.vrl_rope_attn_decode_lora_bf16, (*attn_args, ctypes.byref(record)))
             (state["x"],) = outs
             (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
             (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])

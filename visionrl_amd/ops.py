@@ -566,7 +566,7 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: tor
 def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mask: torch.Tensor,
                      position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None,
-                     lora: "LoraAdd | None" = None) -> torch.Tensor:
+                     lora: "LoraAdd | None" = None, out_lora: "LoraAdd | None" = None) -> torch.Tensor:
     """Rotary embedding, cache append and attention for one new token per row, one launch.
 
     ``q [M, H*D]``, ``k, v [M, Hkv*D]`` bf16 (rows may be strided views of one buffer), caches
@@ -576,6 +576,8 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
     ``LlamaAttention.forward`` (reached from ``vrl/models/families/janus_pro/policy.py:673-678``).
     ``lora`` is a :class:`LoraAdd` over exactly the q, k, v outputs passed here whose down-projection
     was launched: the attention then adds the up-projections itself (q, k, v stay as they are).
+    ``out_lora`` is a :class:`LoraAdd` with one adapter over ``out`` built with ``parts = H``: the launch
+    leaves that adapter's down-projection in its ``t``, one piece per head, for its ``launch_up``.
     """
     dev = _require_device("k_cache", k_cache)
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.dtype != torch.bfloat16 or \
@@ -608,12 +610,16 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
     args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), k_cache.data_ptr(),
             v_cache.data_ptr(), cos.data_ptr(), sin.data_ptr(), mask.data_ptr(), position.data_ptr(),
             out.data_ptr(), M, H, Hkv, D, L, float(scaling))
+    record = lora.attn_record(q, k, v) if lora is not None else None
+    if out_lora is not None:
+        if out_lora.x.data_ptr() != out.data_ptr() or out_lora.parts != H:
+            raise ValueError("out_lora must be built over `out` with one part per head")
+        record = out_lora.attn_output_record(record)
     with _on(dev):
-        if lora is None:
+        if record is None:
             rc = _lib.load().vrl_rope_attn_decode_bf16(*args, _stream_handle(dev))
         else:
-            rc = _lib.load().vrl_rope_attn_decode_lora_bf16(*args, ctypes.byref(lora.attn_record(q, k, v)),
-                                                            _stream_handle(dev))
+            rc = _lib.load().vrl_rope_attn_decode_lora_bf16(*args, ctypes.byref(record), _stream_handle(dev))
     _lib.check(rc, "vrl_rope_attn_decode_bf16")
     return out
 
@@ -628,9 +634,13 @@ class LoraAdd:
     projection, updated in place: ``y += scaling * (x A^T) B^T`` with the roundings the wrapper's
     own forward applies (``vrl/models/families/janus_pro/policy.py:298-324`` attaches the adapters).
     ``x`` is the fixed bf16 ``[M <= 32, K]`` input buffer of the group.
+
+    ``parts > 1`` (one adapter only): the down-projection is left to the launch that produces ``x``, which
+    writes it as ``parts`` partial rows per activation row (the attention launch does, one per head:
+    :meth:`attn_output_record`); ``t`` is then ``[M, parts, r]`` and :meth:`launch_down` is not used.
     """
 
-    def __init__(self, x: torch.Tensor, adapters):
+    def __init__(self, x: torch.Tensor, adapters, parts: int = 1):
         if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_contiguous():
             raise ValueError("x must be contiguous bfloat16 [M, K]")
         dev = _require_device("x", x)
@@ -653,7 +663,10 @@ class LoraAdd:
             rec.A, rec.B, rec.y, rec.N, rec.r = A.data_ptr(), B.data_ptr(), y.data_ptr(), N, r
             rec.scaling, rec.weights_fp32 = float(scaling), int(A.dtype == torch.float32)
             total += r
-        self.t = torch.empty((M, total), dtype=torch.float32, device=dev)
+        if parts != 1 and (len(adapters) != 1 or not 1 < parts <= 256):
+            raise ValueError("a down-projection in parts: one adapter, 2 to 256 parts")
+        self.parts = int(parts)
+        self.t = torch.empty((M, total) if parts == 1 else (M, parts, total), dtype=torch.float32, device=dev)
         self.x, self.M, self.K, self.device = x, M, K, dev
         self._keep = list(adapters)
 
@@ -667,8 +680,8 @@ class LoraAdd:
     def launch_up(self):
         """``y_i += scaling_i * t_i . B_i^T`` for every adapter of the group."""
         with _on(self.device):
-            rc = _lib.load().vrl_lora_up_add_bf16(self.t.data_ptr(), self.M, self.table, len(self.table),
-                                                  _stream_handle(self.device))
+            rc = _lib.load().vrl_lora_up_add_bf16(self.t.data_ptr(), self.parts, self.M, self.table,
+                                                  len(self.table), _stream_handle(self.device))
         _lib.check(rc, "vrl_lora_up_add_bf16")
 
     def launch(self):
@@ -694,4 +707,18 @@ class LoraAdd:
         if not found:
             raise ValueError("no adapter")
         self._attn_record = rec   # kept alive for a launch that is only enqueued
+        return rec
+
+    def attn_output_record(self, rec=None):
+        """Adds this group (one adapter over the attention output, built with ``parts = n_heads``) to a
+        ``vrl_attn_lora`` record, or starts one: the attention launch then writes ``t`` itself."""
+        if rec is None:
+            rec = _lib.AttnLora()
+            rec.weights_fp32 = self.table[0].weights_fp32
+        elif rec.weights_fp32 != self.table[0].weights_fp32:
+            raise ValueError("the adapters of one attention launch must all be float32 or all bfloat16")
+        if len(self.table) != 1 or self.parts == 1 or self.K % self.parts != 0:
+            raise ValueError("needs one adapter whose down-projection is split into one part per head")
+        rec.o_A, rec.o_t, rec.o_r = self.table[0].A, self.t.data_ptr(), self.table[0].r
+        self._attn_record = rec
         return rec
