@@ -276,6 +276,30 @@ def test_lora_validation(lib):
     assert up(p, 0, 1, ads, 2, None) == 1001 and up(p, 257, 1, ads, 2, None) == 1001   # pieces of t per row
 
 
+def test_base_launch_with_down_projection_validation(lib):
+    keep, p = buf(1 << 16)
+    probs = (_lib.Problem * 2)()
+    for rec in probs:
+        rec.x = rec.qweight = rec.y = p
+        rec.M, rec.N, rec.K, rec.G, rec.prepacked = 2, 64, 256, 128, 1
+    ads = (_lib.LoraAdapter * 2)()
+    for ad in ads:
+        ad.A, ad.B, ad.y, ad.N, ad.r, ad.scaling, ad.weights_fp32 = p, p, p, 64, 8, 2.0, 1
+    f = lib.vrl_int4_gemv_prepacked_lora_bf16
+    assert f(probs, 2, None, 2, p, None) == 1003 and f(probs, 2, ads, 2, None, None) == 1003
+    assert f(probs, 2, ads, 2, p + 4, None) == 1002
+    assert f(probs, 2, ads, 0, p, None) == 1001 and f(probs, 2, ads, 5, p, None) == 1001
+    probs[1].x = p + 512
+    assert f(probs, 2, ads, 2, p, None) == 1001          # every problem reads the adapters' input
+    probs[1].x, probs[1].M = p, 1
+    assert f(probs, 2, ads, 2, p, None) == 1001
+    probs[1].M, probs[1].fused_gate_up = 2, 1
+    assert f(probs, 2, ads, 2, p, None) == 1001          # no fused gate|up problem beside adapters
+    probs[1].fused_gate_up = 0
+    ads[1].r = 12
+    assert f(probs, 2, ads, 2, p, None) == 1001
+
+
 def test_cfg_sample_validation(lib):
     keep, p = buf(4096)
     f = lib.vrl_cfg_sample_bf16

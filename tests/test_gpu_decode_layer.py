@@ -396,6 +396,43 @@ def test_attention_leaves_the_output_adapters_down_projection(ops_mod, M, H, Hkv
                                  out_lora=group)
 
 
+@pytest.mark.parametrize("M,K,Ns,ranks,fp32", [(2, 2048, (2048, 2048, 2048), (32, 32, 32), True),
+                                               (32, 2048, (2048, 2048, 2048), (32, 32, 32), True),
+                                               (7, 512, (96, 32), (8, 24), False), (16, 4096, (4096, 1024, 1024), (64, 16, 16), True),
+                                               (20, 5632, (2048,), (16,), False), (1, 256, (48,), (8,), True)])
+def test_down_projection_rides_with_the_base_launch(ops_mod, M, K, Ns, ranks, fp32):
+    """``DirectGemv.launch(lora_down=group)``: the base projections equal the plain launch's and ``t`` the
+    down-projection launch's, bit for bit (the same code, as extra workgroups of one launch)."""
+    from tests._util import to_device
+    say("base launch with down-projection", M, K, Ns, ranks, fp32)
+    rng = np.random.default_rng(M + K)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    x = bits_to_bf16(rand_bits(rng, (M, K)), DEV)
+    gen = torch.Generator().manual_seed(K + M)
+    packed, ads = [], []
+    for i, (N, r) in enumerate(zip(Ns, ranks)):
+        w = to_device(o.make_operands(900 + i, M, K, N, 128), DEV)
+        packed.append(ops_mod.int4_prepack(w["qweight"], w["scales"], w["qzeros"], 128))
+        A = (torch.randn(r, K, generator=gen) * K ** -0.5).to(dtype).to(DEV)
+        B = (torch.randn(N, r, generator=gen) * 0.2).to(dtype).to(DEV)
+        ads.append((A, B))
+    plain = ops_mod.DirectGemv([(x, pw, False) for pw in packed])
+    want_y = [y.clone() for y in plain.launch()]
+    alone = ops_mod.LoraAdd(x, [(A, B, 1.0, y) for (A, B), y in zip(ads, want_y)])
+    alone.launch_down()
+    both = ops_mod.DirectGemv([(x, pw, False) for pw in packed])
+    group = ops_mod.LoraAdd(x, [(A, B, 1.0, y) for (A, B), y in zip(ads, both.outputs)])
+    group.t.fill_(float("nan"))
+    got_y = both.launch(lora_down=group)
+    torch.cuda.synchronize()
+    for a, b in zip(got_y, want_y):
+        assert torch.equal(a, b)
+    assert torch.equal(group.t, alone.t)
+    t64 = x.float().cpu().numpy().astype(np.float64) @ np.concatenate(
+        [A.float().cpu().numpy().astype(np.float64) for A, _ in ads]).T
+    assert np.abs(group.t.cpu().numpy() - t64).max() <= (2.0 ** -7 if not fp32 else 2.0 ** -16) * max(1.0, np.abs(t64).max())
+
+
 # ------------------------------------------------------------------ seeded random shapes through every decode-layer launch
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_shapes(ops_mod, seed):

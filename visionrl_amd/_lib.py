@@ -34,6 +34,7 @@ SYMBOLS = (
     "vrl_rope_attn_decode_lora_bf16",
     "vrl_lora_down_bf16",
     "vrl_lora_up_add_bf16",
+    "vrl_int4_gemv_prepacked_lora_bf16",
 )
 
 
@@ -163,6 +164,8 @@ def _bind(lib):
                                                    ctypes.POINTER(AttnLora), vp]
     lib.vrl_lora_down_bf16.restype = ci
     lib.vrl_lora_down_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
+    lib.vrl_int4_gemv_prepacked_lora_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_lora_bf16.argtypes = [ctypes.POINTER(Problem), ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
     lib.vrl_lora_up_add_bf16.restype = ci
     lib.vrl_lora_up_add_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp]
     lib.vrl_rope_attn_decode_bf16.restype = ci

@@ -18,6 +18,7 @@
 
 #include "../../include/vrl_decode.h"
 #include "../../include/vrl_int4.h"
+#include "lora.hpp"
 #include "wave_reduce.hpp"
 
 namespace {
@@ -27,7 +28,6 @@ constexpr int THREADS = 256;
 constexpr int WAVES = THREADS / WAVE;
 constexpr int MAX_NORM_K = 16384;
 constexpr int MAX_CACHE_LEN = 8192;
-constexpr int LORA_MAX_RANK = 64;
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
 
@@ -162,24 +162,6 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
     for (int i = 0; i < VEC; ++i) a.acc[i] = a.acc[i] * c1 + acc2[i] * c2;
 }
 
-
-// eight consecutive adapter weights (float32 or bf16) as floats
-template <bool FP32>
-__device__ __forceinline__ void load8(const void *base, long index, float (&f)[8]) {
-    if constexpr (FP32) {
-        const float4 a = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index);
-        const float4 b = *reinterpret_cast<const float4 *>(static_cast<const float *>(base) + index + 4);
-        f[0] = a.x, f[1] = a.y, f[2] = a.z, f[3] = a.w, f[4] = b.x, f[5] = b.y, f[6] = b.z, f[7] = b.w;
-    } else {
-        const uint4 w = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(base) + index);
-        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bf16_to_f32(u[e] & 0xFFFFu);
-            f[2 * e + 1] = bf16_to_f32(u[e] >> 16);
-        }
-    }
-}
 
 // One workgroup of ATT_WAVES waves per (head, row): 16 when there are few workgroups (each should
 // keep many requests in flight), 8 when there are at least two per CU (several then share a CU
@@ -450,75 +432,13 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
 }
 
 // ---------------------------------------------------------------- LoRA adapters over an int4 projection
-constexpr int LORA_MAX_ADAPTERS = 4;
-constexpr int LORA_MAX_ROWS = 32;
-constexpr int LORA_MAX_TOTAL = 256;
-
-struct LoraArgs {
-    vrl_lora_adapter ad[LORA_MAX_ADAPTERS];
-    int32_t off[LORA_MAX_ADAPTERS + 1];  // first column of each adapter in t
-    int32_t n, M, K;
-};
-
-// Both kernels are written without data-dependent branches: rows beyond M repeat row M - 1
-// (clamped index), which costs arithmetic but keeps every load of a lane in flight at once.
-// MB is the number of rows a workgroup handles (8 or 16; blockIdx.y picks the row block); FP32 is the
-// adapters' weight type.
-
-// One workgroup per column of t (an adapter row j) and block of MB rows: its four waves take
-// interleaved 512-value pieces of K; a lane holds 8 values of the A row and requests the matching 8
-// values of all its activation rows at once, then every row's partial sum is reduced over the wave
-// and the four waves meet in LDS.
+// One workgroup per column of t (an adapter row) and block of MB rows (8 or 16; blockIdx.y picks the
+// block): lora_down_item.  FP32 is the adapters' weight type.
 template <bool FP32, int MB>
 __global__ __launch_bounds__(THREADS) void lora_down_kernel(const uint16_t *__restrict__ x, LoraArgs a,
                                                             float *__restrict__ t) {
-    __shared__ float part[WAVES][LORA_MAX_ROWS];
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int col = blockIdx.x;
-    const int total = a.off[a.n];
-    int i = 0;
-#pragma unroll
-    for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
-        if (k < a.n && a.off[k] <= col) i = k;
-    const void *A = a.ad[0].A;
-    int first = 0;
-#pragma unroll
-    for (int k = 1; k < LORA_MAX_ADAPTERS; ++k)
-        if (k == i) A = a.ad[k].A, first = a.off[k];   // scalar selects, no indexing of the argument block
-    const long arow = (long)(col - first) * a.K;
-    const int m_lo = blockIdx.y * MB, rows = min(MB, a.M - m_lo);
-    x += (long)m_lo * a.K;
-    float acc[MB];
-#pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
-    for (int k = (wave * WAVE + lane) * 8; k < a.K; k += THREADS * 8) {
-        float af[8];
-        load8<FP32>(A, arow + k, af);
-        uint4 xr[MB];
-#pragma unroll
-        for (int u = 0; u < MB; ++u) xr[u] = *reinterpret_cast<const uint4 *>(x + (long)(u < rows ? u : rows - 1) * a.K + k);
-        __builtin_amdgcn_sched_barrier(0);  // all requests before the first use
-#pragma unroll
-        for (int u = 0; u < MB; ++u) {
-            const uint32_t w[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                acc[u] += bf16_to_f32(w[e] & 0xFFFFu) * af[2 * e] + bf16_to_f32(w[e] >> 16) * af[2 * e + 1];
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-        const float v = wave_sum(acc[m]);
-        if (lane == 0) part[wave][m] = v;
-    }
-    __syncthreads();
-    if (threadIdx.x < rows) {
-        float v = part[0][threadIdx.x];
-#pragma unroll
-        for (int w = 1; w < WAVES; ++w) v += part[w][threadIdx.x];
-        if (!FP32) v = round_bf16(v);  // lora_A's output tensor is bf16 then
-        t[(long)(m_lo + threadIdx.x) * total + col] = v;
-    }
+    __shared__ float part[LORA_DOWN_WAVES * MB];
+    lora_down_item<FP32, MB>(x, a, t, true, blockIdx.x, blockIdx.y * MB, threadIdx.x / WAVE, threadIdx.x % WAVE, part);
 }
 
 // One thread per output column, 64 columns per workgroup, eight rows per workgroup (blockIdx.z): t of
@@ -611,27 +531,6 @@ void launch_lora_up(const float *t, int parts, const LoraArgs &a, int max_n, int
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 
-// host side: one argument block for both LoRA launches
-int lora_args(LoraArgs &a, int M, int K, const vrl_lora_adapter *adapters, int n, bool need_y) {
-    if (!adapters) return VRL_INT4_ENULL;
-    if (n < 1 || n > LORA_MAX_ADAPTERS || M < 1 || M > LORA_MAX_ROWS || K < 8 || K % 8 != 0) return VRL_INT4_ESHAPE;
-    a.n = n;
-    a.M = M;
-    a.K = K;
-    a.off[0] = 0;
-    for (int i = 0; i < n; ++i) {
-        const vrl_lora_adapter &ad = adapters[i];
-        if (!ad.A || !ad.B || (need_y && !ad.y)) return VRL_INT4_ENULL;
-        if (ad.r < 8 || ad.r % 8 != 0 || ad.r > LORA_MAX_RANK || ad.N < 1) return VRL_INT4_ESHAPE;
-        if (misaligned(ad.A, 16) || misaligned(ad.B, 16) || misaligned(ad.y, 2)) return VRL_INT4_EALIGN;
-        if ((ad.weights_fp32 != 0) != (adapters[0].weights_fp32 != 0)) return VRL_INT4_ESHAPE;  // one type per launch
-        a.ad[i] = ad;
-        a.off[i + 1] = a.off[i] + ad.r;
-    }
-    for (int i = n; i < LORA_MAX_ADAPTERS; ++i) a.off[i + 1] = a.off[n];
-    if (a.off[n] > LORA_MAX_TOTAL) return VRL_INT4_ESHAPE;
-    return VRL_INT4_OK;
-}
 }  // namespace
 
 extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const void *weight, void *h_out,

@@ -320,9 +320,9 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int KS, int TW, bool NORM, bool XG = false>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG = false, bool LD = false>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
-    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG>;
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG, LD>;
     if (lds > 64 * 1024) {
         // once per instantiation and device: the attribute belongs to the function on that device
         static std::atomic<uint64_t> raised{0};
@@ -353,6 +353,16 @@ int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int wor
     if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1, NORM>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2, NORM>(args, workgroups, lds, stream);
     if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1, NORM>(args, workgroups, lds, stream);
+    return VRL_INT4_EPLAN;
+}
+
+// with the adapters' down-projection as extra workgroups: plain (staged, unfused) problems only
+int launch_direct_lora(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
+    if (ks == 4 && tw == 1) return launch_direct<false, 4, 1, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 4) return launch_direct<false, 4, 4, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 1) return launch_direct<false, 8, 1, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 2) return launch_direct<false, 8, 2, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 16 && tw == 1) return launch_direct<false, 16, 1, false, false, true>(args, workgroups, lds, stream);
     return VRL_INT4_EPLAN;
 }
 
@@ -451,8 +461,14 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     return (int)hipGetLastError();
 }
 
+struct DirectLora {
+    const vrl_lora_adapter *adapters;
+    int n_adapters;
+    float *t;
+};
+
 static int direct_launch(const vrl_int4_problem *problems, int n_problems, const vrl_int4_norm *norm,
-                         void *hip_stream) {
+                         const DirectLora *lora, void *hip_stream) {
     if (!problems) return VRL_INT4_ENULL;
     if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
     bool fused_any = false;
@@ -476,7 +492,8 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // One super-chunk per wave: the waves can fetch their own activations, with nothing staged and one
     // tile per workgroup.  Long K always does; shorter K with 8+ rows does while the launch is small
     // (every tile then fetches its rows from L2 itself: for a wide matrix one staging per TW tiles wins).
-    const bool xg = !norm && max_nsc <= ks && (ks == 16 || (max_m >= 8 && slab_tiles <= 2L * device_cu_count()));
+    const bool xg = !norm && !lora && max_nsc <= ks &&
+                    (ks == 16 || (max_m >= 8 && slab_tiles <= 2L * device_cu_count()));
     const int tw = (max_m >= 8 && !xg) ? 16 / ks : 1;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
@@ -538,8 +555,25 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
             xz_bytes = std::max(xz_bytes, need);
         }
     }
-    const size_t lds = xg ? red : xz_bytes + red;
+    size_t lds = xg ? red : xz_bytes + red;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    if (lora) {
+        // the adapters read the input every problem of the launch reads
+        const vrl_int4_problem &q0 = problems[0];
+        if (fused_any || !lora->t) return fused_any ? VRL_INT4_ESHAPE : VRL_INT4_ENULL;
+        if (reinterpret_cast<uintptr_t>(lora->t) & 15u) return VRL_INT4_EALIGN;
+        for (int i = 1; i < n_problems; ++i)
+            if (problems[i].x != q0.x || problems[i].M != q0.M || problems[i].K != q0.K) return VRL_INT4_ESHAPE;
+        const int rc = lora_args(args.ld.a, q0.M, q0.K, lora->adapters, lora->n_adapters, false);
+        if (rc != VRL_INT4_OK) return rc;
+        args.ld.x = static_cast<const uint16_t *>(q0.x);
+        args.ld.t = lora->t;
+        args.ld.fp32 = args.ld.a.ad[0].weights_fp32 != 0;
+        args.ld.wg_begin = (int)workgroups;
+        workgroups += lora_down_workgroups(args.ld.a, ks * tw);
+        lds = std::max(lds, (size_t)ks * tw * 16 * sizeof(float));
+        return launch_direct_lora(args, ks, tw, (int)workgroups, lds, stream);
+    }
     if (norm)
         return fused_any ? launch_direct_shape<true, true>(args, ks, tw, false, (int)workgroups, lds, stream)
                          : launch_direct_shape<false, true>(args, ks, tw, false, (int)workgroups, lds, stream);
@@ -548,13 +582,21 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
 }
 
 int vrl_int4_gemv_prepacked_bf16(const vrl_int4_problem *problems, int n_problems, void *hip_stream) {
-    return direct_launch(problems, n_problems, nullptr, hip_stream);
+    return direct_launch(problems, n_problems, nullptr, nullptr, hip_stream);
+}
+
+int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_problems,
+                                      const vrl_lora_adapter *adapters, int n_adapters, float *t,
+                                      void *hip_stream) {
+    if (!adapters) return VRL_INT4_ENULL;
+    const DirectLora lora{adapters, n_adapters, t};
+    return direct_launch(problems, n_problems, nullptr, &lora, hip_stream);
 }
 
 int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_problems,
                                       const vrl_int4_norm *norm, void *hip_stream) {
     if (!norm) return VRL_INT4_ENULL;
-    return direct_launch(problems, n_problems, norm, hip_stream);
+    return direct_launch(problems, n_problems, norm, nullptr, hip_stream);
 }
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {

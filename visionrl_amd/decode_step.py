@@ -20,10 +20,10 @@ op in fp32, rounded to bf16); the attention keeps its probabilities in fp32.
 Needs a trunk whose projections were swapped for prepacked :class:`Int4Linear` modules with the
 fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry one active LoRA
 adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
-the norm as a launch of its own (the adapters read the normalised row), a down-projection launch
-for the q|k|v adapters (their up-projections are added by the attention launch as it reads q, k, v)
-and an up-projection launch for o_proj's (its down-projection is left behind by the attention launch,
-one piece per head): eight launches.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not
+the norm as a launch of its own (the adapters read the normalised row) and an up-projection launch for
+o_proj's adapter: seven launches.  The down-projections of the q|k|v adapters ride with the q|k|v
+launch as extra workgroups and their up-projections are added by the attention launch as it reads q, k,
+v; the attention launch also leaves o_proj's down-projection behind, one piece per head.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not
 qualify, and callers then keep the module path.
 """
 
@@ -201,18 +201,19 @@ class NativeDecodeTrunk:
                               (launch.table, len(launch.table), ctypes.byref(launch.norm))))
             return launch.outputs
 
-        def lora(x, outs, adapters, up=True, parts=1):
+        def lora(x, outs, adapters, up=True, down=True, parts=1):
             """outs[i] += adapter i applied to x, for the projections that carry one: a down-projection
-            launch (unless the producer of x leaves it in ``parts`` pieces: the attention does for its
-            output) and, unless the consumer adds the up-projection itself (``up=False``: the attention
-            does for q, k, v), an up-projection launch.  Returns the group or ``None``."""
+            launch (unless another launch computes it: ``down=False``, or the producer of x leaves it in
+            ``parts`` pieces, as the attention does for its output) and, unless the consumer adds the
+            up-projection itself (``up=False``: the attention does for q, k, v), an up-projection
+            launch.  Returns the group or ``None``."""
             todo = [(A, B, s, y) for y, ad in zip(outs, adapters) if ad is not None for A, B, s in [ad]]
             if not todo:
                 return None
             launch = ops.LoraAdd(x, todo, parts=parts)
             self._keep.append(launch)
             n = len(launch.table)
-            if parts == 1:
+            if down and parts == 1:
                 calls.append((lib.vrl_lora_down_bf16, (x.data_ptr(), rows, x.shape[1], launch.table, n,
                                                        launch.t.data_ptr())))
             if up:
@@ -231,8 +232,14 @@ class NativeDecodeTrunk:
                 calls.append((lib.vrl_add_rmsnorm_bf16,
                               (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,
                                w.data_ptr(), h_out.data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+                # the adapters read the normalised row, so it is written out; their down-projection and the
+                # base projections share one launch
+                launch_at = len(calls)
                 outs = gemv([(self.normed, pw, fused) for pw in weights])
-                group = lora(self.normed, outs, adapters, up)   # adapters read the normalised row, so it is written out
+                group = lora(self.normed, outs, adapters, up, down=fused)
+                if group is not None and not fused:
+                    calls[launch_at] = (lib.vrl_int4_gemv_prepacked_lora_bf16,
+                                        (*calls[launch_at][1], group.table, len(group.table), group.t.data_ptr()))
             state["res"] = h_out
             return outs, group
 

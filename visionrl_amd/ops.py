@@ -382,10 +382,18 @@ class DirectGemv:
         self.norm = rec
         self._keep.append((residual, weight, h_out))
 
-    def launch(self):
+    def launch(self, lora_down: "LoraAdd | None" = None):
+        """``lora_down``: a :class:`LoraAdd` over the input every problem of this launch reads; its
+        down-projection then runs in the same launch (in place of its ``launch_down``)."""
         lib = _lib.load()
         with _on(self.device):
-            if self.norm is not None:
+            if lora_down is not None:
+                if self.norm is not None or lora_down.parts != 1:
+                    raise ValueError("the adapters' down-projection joins a launch without a norm, in one piece")
+                rc = lib.vrl_int4_gemv_prepacked_lora_bf16(self.table, len(self.table), lora_down.table,
+                                                           len(lora_down.table), lora_down.t.data_ptr(),
+                                                           _stream_handle(self.device))
+            elif self.norm is not None:
                 rc = lib.vrl_int4_gemv_prepacked_norm_bf16(self.table, len(self.table), ctypes.byref(self.norm),
                                                            _stream_handle(self.device))
             else:
