@@ -95,7 +95,7 @@ int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vrl_lora_adap
  * vrl_int4_gemv_prepacked_bf16 and vrl_lora_down_bf16 of the same input in one launch: the base
  * projections of a group (q|k|v of one layer: the wrapper computes base_layer(x) and lora_A(x) from the
  * same x) and the down-projections of their adapters do not depend on each other, so the latter run
- * as extra workgroups behind the tiles'.  Every problem must read the same x [M, K] (M <= 32), none
+ * as extra workgroups of the same grid.  Every problem must read the same x [M, K] (M <= 32), none
  * may be a fused gate|up problem; `adapters`, `t` as for vrl_lora_down_bf16 (y and B are not used).
  */
 int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_problems,

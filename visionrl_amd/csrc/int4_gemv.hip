@@ -569,8 +569,8 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         args.ld.x = static_cast<const uint16_t *>(q0.x);
         args.ld.t = lora->t;
         args.ld.fp32 = args.ld.a.ad[0].weights_fp32 != 0;
-        args.ld.wg_begin = (int)workgroups;
-        workgroups += lora_down_workgroups(args.ld.a, ks * tw);
+        args.ld.wgs = lora_down_workgroups(args.ld.a, ks * tw);
+        workgroups += args.ld.wgs;
         lds = std::max(lds, (size_t)ks * tw * 16 * sizeof(float));
         return launch_direct_lora(args, ks, tw, (int)workgroups, lds, stream);
     }

@@ -625,12 +625,13 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
 // cuts activations of more than 16 rows, or too large for LDS, into row slabs, one record each.
 constexpr int DIRECT_MAX = 8;
 // LD instantiations carry the down-projection of LoRA adapters over the same input as extra
-// workgroups behind the tiles' (lora.hpp): the two are independent, so they share the launch.
+// workgroups (lora.hpp): the two are independent, so they share the launch.  The extra workgroups
+// come first in the grid: they run longer than a tile's and should start first.
 struct LoraDownArgs {
     LoraArgs a;
     const uint16_t *x;   // [a.M, a.K]: the input of the launch's problems
     float *t;            // [a.M, r_total]
-    int32_t wg_begin;    // first workgroup of the down-projection
+    int32_t wgs;         // workgroups of the down-projection: the first of the grid
     int32_t fp32;        // the adapters' weight type
 };
 struct DirectArgs {
@@ -644,13 +645,13 @@ struct DirectArgs {
 template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD>
 __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    const int g = blockIdx.x;
+    int g = blockIdx.x;
     if constexpr (LD) {
-        if (g >= a.ld.wg_begin) {  // uniform over the workgroup
-            lora_down_workgroup<KS * TW>(a.ld.x, a.ld.a, a.ld.t, a.ld.fp32 != 0, g - a.ld.wg_begin,
-                                         reinterpret_cast<float *>(smem));
+        if (g < a.ld.wgs) {  // uniform over the workgroup
+            lora_down_workgroup<KS * TW>(a.ld.x, a.ld.a, a.ld.t, a.ld.fp32 != 0, g, reinterpret_cast<float *>(smem));
             return;
         }
+        g -= a.ld.wgs;
     }
     DevProblem p = a.recs[0];
 #pragma unroll
