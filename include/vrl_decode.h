@@ -103,6 +103,17 @@ int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_pr
                                       void *hip_stream);
 
 /*
+ * vrl_int4_gemv_prepacked_bf16 of one problem and vrl_lora_up_add_bf16 of its adapter in one launch:
+ *   y[m,n] = bf16( bf16(x . W^T)[m,n] + scaling * sum_j t[m,j] * B[n,j] )
+ * with t [M, t_parts, r] as for vrl_lora_up_add_bf16 (the down-projection of the same x, e.g. the
+ * pieces vrl_rope_attn_decode_lora_bf16 left) and the adapter's N equal to the problem's; A and y
+ * of the adapter record are not used (the sum goes to the problem's y).  Not for a fused gate|up
+ * problem.
+ */
+int vrl_int4_gemv_prepacked_lora_up_bf16(const vrl_int4_problem *problem, const vrl_lora_adapter *adapter,
+                                         const float *t, int t_parts, void *hip_stream);
+
+/*
  * vrl_rope_attn_decode_bf16 with the up-projections of the q, k, v adapters added while the new
  * token's projections are read, in place of a vrl_lora_up_add_bf16 launch between the int4 launch
  * and the attention: q, k, v hold the base projections' outputs, `t` the down-projections of the

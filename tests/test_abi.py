@@ -300,6 +300,27 @@ def test_base_launch_with_down_projection_validation(lib):
     assert f(probs, 2, ads, 2, p, None) == 1001
 
 
+def test_base_launch_with_up_projection_validation(lib):
+    keep, p = buf(1 << 16)
+    prob = (_lib.Problem * 1)()
+    prob[0].x = prob[0].qweight = prob[0].y = p
+    prob[0].M, prob[0].N, prob[0].K, prob[0].G, prob[0].prepacked = 2, 64, 256, 128, 1
+    ad = (_lib.LoraAdapter * 1)()
+    ad[0].A, ad[0].B, ad[0].y, ad[0].N, ad[0].r, ad[0].scaling, ad[0].weights_fp32 = p, p, p, 64, 8, 2.0, 1
+    f = lib.vrl_int4_gemv_prepacked_lora_up_bf16
+    assert f(prob, None, p, 1, None) == 1003 and f(prob, ad, None, 1, None) == 1003 and f(None, ad, p, 1, None) == 1003
+    assert f(prob, ad, p + 4, 1, None) == 1002
+    assert f(prob, ad, p, 0, None) == 1001 and f(prob, ad, p, 257, None) == 1001
+    ad[0].N = 32
+    assert f(prob, ad, p, 1, None) == 1001               # the adapter's width is the problem's
+    ad[0].N, ad[0].r = 64, 12
+    assert f(prob, ad, p, 1, None) == 1001
+    ad[0].r, ad[0].B = 8, None
+    assert f(prob, ad, p, 1, None) == 1003
+    ad[0].B, prob[0].fused_gate_up, prob[0].N = p, 1, 64
+    assert f(prob, ad, p, 1, None) == 1001               # not beside a fused gate|up problem
+
+
 def test_cfg_sample_validation(lib):
     keep, p = buf(4096)
     f = lib.vrl_cfg_sample_bf16

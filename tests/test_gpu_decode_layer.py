@@ -433,6 +433,50 @@ def test_down_projection_rides_with_the_base_launch(ops_mod, M, K, Ns, ranks, fp
     assert np.abs(group.t.cpu().numpy() - t64).max() <= (2.0 ** -7 if not fp32 else 2.0 ** -16) * max(1.0, np.abs(t64).max())
 
 
+@pytest.mark.parametrize("M,K,N,r,parts,fp32", [(2, 2048, 2048, 32, 16, True), (32, 2048, 2048, 32, 16, True),
+                                                (7, 512, 100, 8, 1, False), (16, 4096, 4096, 64, 32, True),
+                                                (20, 5632, 2048, 16, 3, False), (1, 256, 48, 8, 1, True),
+                                                (32, 2048, 16384, 24, 2, True), (9, 11008, 64, 40, 1, False)])
+def test_up_projection_joins_the_base_launch(ops_mod, M, K, N, r, parts, fp32):
+    """``DirectGemv.launch(lora_up=group)`` against the two launches (base, then ``launch_up``) and
+    against the oracle's adapter applied to the base launch's output."""
+    from tests._util import to_device
+    say("base launch with up-projection", M, K, N, r, parts, fp32)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    w = to_device(o.make_operands(700 + M, M, K, N, 128), DEV)
+    x = w["x"]
+    packed = ops_mod.int4_prepack(w["qweight"], w["scales"], w["qzeros"], 128)
+    gen = torch.Generator().manual_seed(M + N)
+    A = (torch.randn(r, K, generator=gen) * K ** -0.5).to(dtype).to(DEV)
+    B = (torch.randn(N, r, generator=gen) * 0.2).to(dtype).to(DEV)
+    pieces = (torch.randn(M, parts, r, generator=gen) * 0.5).to(DEV)   # any split of t: only the sum matters
+    two = ops_mod.DirectGemv([(x, packed, False)])
+    base = two.launch()[0].clone()
+    g2 = ops_mod.LoraAdd(x, [(A, B, 1.5, two.outputs[0])], parts=parts)
+    g2.t.copy_(pieces if parts > 1 else pieces[:, 0])
+    g2.launch_up()
+    one = ops_mod.DirectGemv([(x, packed, False)])
+    g1 = ops_mod.LoraAdd(x, [(A, B, 1.5, one.outputs[0])], parts=parts)
+    g1.t.copy_(g2.t)
+    got = one.launch(lora_up=g1)[0]
+    torch.cuda.synchronize()
+    want = two.outputs[0]
+    print("  outputs that differ from the two launches:", (got != want).float().mean().item(), flush=True)
+    within_one_step_of(bf16_to_bits(got), bf16_to_bits(want), bf16_to_bits(base))
+    assert (got != want).float().mean().item() < 0.01
+    # against float64: base + 1.5 * (sum of the pieces, rounded for a bf16 adapter) . B^T
+    t64 = pieces.double().sum(dim=1).cpu().numpy()
+    if not fp32:
+        t64 = o.bf16_bits_to_f32(o.f32_to_bf16_bits(pieces.sum(dim=1).cpu().numpy())).astype(np.float64)
+    u = t64 @ B.double().cpu().numpy().T
+    delta = u * 1.5 if fp32 else o.bf16_bits_to_f32(o.f32_to_bf16_bits(
+        (o.bf16_bits_to_f32(o.f32_to_bf16_bits(u.astype(np.float32))) * np.float32(1.5)))).astype(np.float64)
+    exact = o.f32_to_bf16_bits((base.float().cpu().numpy().astype(np.float64) + delta).astype(np.float32))
+    within_one_step_of(bf16_to_bits(got), exact, bf16_to_bits(base))
+    with pytest.raises(ValueError):
+        one.launch(lora_up=g2)   # a group over another output
+
+
 # ------------------------------------------------------------------ seeded random shapes through every decode-layer launch
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_shapes(ops_mod, seed):

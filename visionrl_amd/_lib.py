@@ -35,6 +35,7 @@ SYMBOLS = (
     "vrl_lora_down_bf16",
     "vrl_lora_up_add_bf16",
     "vrl_int4_gemv_prepacked_lora_bf16",
+    "vrl_int4_gemv_prepacked_lora_up_bf16",
 )
 
 
@@ -166,6 +167,8 @@ def _bind(lib):
     lib.vrl_lora_down_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
     lib.vrl_int4_gemv_prepacked_lora_bf16.restype = ci
     lib.vrl_int4_gemv_prepacked_lora_bf16.argtypes = [ctypes.POINTER(Problem), ci, ctypes.POINTER(LoraAdapter), ci, vp, vp]
+    lib.vrl_int4_gemv_prepacked_lora_up_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_lora_up_bf16.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(LoraAdapter), vp, ci, vp]
     lib.vrl_lora_up_add_bf16.restype = ci
     lib.vrl_lora_up_add_bf16.argtypes = [vp, ci, ci, ctypes.POINTER(LoraAdapter), ci, vp]
     lib.vrl_rope_attn_decode_bf16.restype = ci

@@ -183,7 +183,7 @@ class StaticARSampler:
     (``cfg_weight``, ``temperature``, ``image_token_num``).  ``graph=False`` runs every step
     eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
     for the part after the head.  With ``native`` (the default) the trunk of a decode step runs as
-    :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (five launches per layer, seven with LoRA
+    :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (five launches per layer, six with LoRA
     adapters on the attention projections) when the policy went through ``apply_int4_to_policy``
     with its defaults; otherwise, and for the prompt pass, the trunk module itself is called.
     """

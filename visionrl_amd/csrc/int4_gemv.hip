@@ -320,9 +320,9 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int KS, int TW, bool NORM, bool XG = false, bool LD = false>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG = false, bool LD = false, bool UP = false>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
-    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG, LD>;
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG, LD, UP>;
     if (lds > 64 * 1024) {
         // once per instantiation and device: the attribute belongs to the function on that device
         static std::atomic<uint64_t> raised{0};
@@ -354,6 +354,16 @@ int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int wor
     if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2, NORM>(args, workgroups, lds, stream);
     if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1, NORM>(args, workgroups, lds, stream);
     return VRL_INT4_EPLAN;
+}
+
+// with an adapter's up-projection added before the store: one plain problem, one tile per workgroup
+int launch_direct_up(const DirectArgs &args, int ks, bool xg, int workgroups, size_t lds, hipStream_t stream) {
+    if (ks == 4) return xg ? launch_direct<false, 4, 1, false, true, false, true>(args, workgroups, lds, stream)
+                           : launch_direct<false, 4, 1, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 8) return xg ? launch_direct<false, 8, 1, false, true, false, true>(args, workgroups, lds, stream)
+                           : launch_direct<false, 8, 1, false, false, false, true>(args, workgroups, lds, stream);
+    return xg ? launch_direct<false, 16, 1, false, true, false, true>(args, workgroups, lds, stream)
+              : launch_direct<false, 16, 1, false, false, false, true>(args, workgroups, lds, stream);
 }
 
 // with the adapters' down-projection as extra workgroups: plain (staged, unfused) problems only
@@ -461,10 +471,12 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     return (int)hipGetLastError();
 }
 
-struct DirectLora {
+struct DirectLora {   // adapters joined to a plan-free launch: down-projections (up false) or one up-projection
     const vrl_lora_adapter *adapters;
     int n_adapters;
     float *t;
+    bool up;
+    int t_parts;
 };
 
 static int direct_launch(const vrl_int4_problem *problems, int n_problems, const vrl_int4_norm *norm,
@@ -492,9 +504,10 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // One super-chunk per wave: the waves can fetch their own activations, with nothing staged and one
     // tile per workgroup.  Long K always does; shorter K with 8+ rows does while the launch is small
     // (every tile then fetches its rows from L2 itself: for a wide matrix one staging per TW tiles wins).
-    const bool xg = !norm && !lora && max_nsc <= ks &&
+    const bool lora_up = lora && lora->up, lora_down = lora && !lora->up;
+    const bool xg = !norm && !lora_down && max_nsc <= ks &&
                     (ks == 16 || (max_m >= 8 && slab_tiles <= 2L * device_cu_count()));
-    const int tw = (max_m >= 8 && !xg) ? 16 / ks : 1;
+    const int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
@@ -557,7 +570,26 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     }
     size_t lds = xg ? red : xz_bytes + red;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    if (lora) {
+    if (lora_up) {
+        // the launch's one problem carries one adapter: y = base + scaling * t . B^T
+        const vrl_int4_problem &q0 = problems[0];
+        const vrl_lora_adapter &ad = lora->adapters[0];
+        if (!lora->t || !ad.B) return VRL_INT4_ENULL;
+        if (n_problems != 1 || lora->n_adapters != 1 || fused_any || ad.N != q0.N || ad.r < 8 || ad.r % 8 != 0 ||
+            ad.r > LORA_MAX_RANK || lora->t_parts < 1 || lora->t_parts > 256)
+            return VRL_INT4_ESHAPE;
+        if ((reinterpret_cast<uintptr_t>(lora->t) | reinterpret_cast<uintptr_t>(ad.B)) & 15u) return VRL_INT4_EALIGN;
+        args.up.t = lora->t;
+        args.up.B = ad.B;
+        args.up.x0 = static_cast<const uint16_t *>(q0.x);
+        args.up.parts = lora->t_parts;
+        args.up.r = ad.r;
+        args.up.fp32 = ad.weights_fp32 != 0;
+        args.up.scaling = ad.scaling;
+        lds += (size_t)(MAX_TILE_M + 16) * (ad.r + 4) * sizeof(float);
+        return launch_direct_up(args, ks, xg, (int)workgroups, lds, stream);
+    }
+    if (lora_down) {
         // the adapters read the input every problem of the launch reads
         const vrl_int4_problem &q0 = problems[0];
         if (fused_any || !lora->t) return fused_any ? VRL_INT4_ESHAPE : VRL_INT4_ENULL;
@@ -589,8 +621,15 @@ int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_pr
                                       const vrl_lora_adapter *adapters, int n_adapters, float *t,
                                       void *hip_stream) {
     if (!adapters) return VRL_INT4_ENULL;
-    const DirectLora lora{adapters, n_adapters, t};
+    const DirectLora lora{adapters, n_adapters, t, false, 1};
     return direct_launch(problems, n_problems, nullptr, &lora, hip_stream);
+}
+
+int vrl_int4_gemv_prepacked_lora_up_bf16(const vrl_int4_problem *problem, const vrl_lora_adapter *adapter,
+                                         const float *t, int t_parts, void *hip_stream) {
+    if (!adapter) return VRL_INT4_ENULL;
+    const DirectLora lora{adapter, 1, const_cast<float *>(t), true, t_parts};
+    return direct_launch(problem, 1, nullptr, &lora, hip_stream);
 }
 
 int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_problems,

@@ -517,11 +517,85 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // wave fetches its own A operand (16 rows x 512 k: sixteen 16-byte buffer loads per lane, zeros for
 // rows beyond M and k beyond K through the buffer's range check) while its weights arrive; LDS
 // holds only the partial tiles, and 16 rows per record fit whatever K is.
-template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG>
+// UP instantiations (plan-free launches of one problem) add a LoRA adapter's up-projection to the
+// tile before it is stored: y = bf16(bf16(x . W^T) + scaling * t . B^T), the second half of a PEFT
+// wrapper's forward (vrl/models/families/janus_pro/policy.py:298-324 attaches the adapters), with t
+// the adapter's down-projection of x, handed over in `parts` pieces per row that are summed in order.
+struct LoraUpArgs {
+    const float *t;      // [M, parts, r] float32
+    const void *B;       // [N, r], float32 or bf16
+    const uint16_t *x0;  // row 0 of the problem's x: a record's first row is (p.x - x0) / K
+    int32_t parts, r, fp32;
+    float scaling;
+};
+
+// t of the record's rows (pieces summed; rounded to bf16 for a bf16 adapter, whose lora_A output is a
+// bf16 tensor) and the rows of B for the workgroup's `cols` columns from `col0`, into LDS with row
+// stride r + 4 floats
+template <bool FP32>
+__device__ __forceinline__ void stage_lora_up(const DevProblem &p, const LoraUpArgs &u, int col0, int cols,
+                                              float *ts, float *bs, int nthreads) {
+    const int r = u.r, stride = r + 4, r4 = r >> 2, r8 = r >> 3;
+    const long m0 = (p.x - u.x0) / p.K;
+    for (int idx = threadIdx.x; idx < p.M * r4; idx += nthreads) {
+        const int m = idx / r4, j4 = idx - m * r4;
+        const float *src = u.t + (m0 + m) * u.parts * r + 4 * j4;
+        float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int q0 = 0; q0 < u.parts; q0 += 16) {   // sixteen pieces requested together, added in order
+            float4 w[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                w[k] = *reinterpret_cast<const float4 *>(src + (long)(q0 + k < u.parts ? q0 + k : u.parts - 1) * r);
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                if (q0 + k < u.parts) v.x += w[k].x, v.y += w[k].y, v.z += w[k].z, v.w += w[k].w;
+        }
+        if (!FP32) v.x = lora_round_bf16(v.x), v.y = lora_round_bf16(v.y), v.z = lora_round_bf16(v.z), v.w = lora_round_bf16(v.w);
+        *reinterpret_cast<float4 *>(ts + m * stride + 4 * j4) = v;
+    }
+    for (int idx = threadIdx.x; idx < cols * r8; idx += nthreads) {
+        const int c = idx / r8, j8 = idx - c * r8;
+        const int n = min(col0 + c, p.N - 1);   // columns past the end repeat the last one and are not stored
+        float f[8];
+        load8<FP32>(u.B, (long)n * r + 8 * j8, f);
+        *reinterpret_cast<float4 *>(bs + c * stride + 8 * j8) = float4{f[0], f[1], f[2], f[3]};
+        *reinterpret_cast<float4 *>(bs + c * stride + 8 * j8 + 4) = float4{f[4], f[5], f[6], f[7]};
+    }
+}
+
+// store_tile<1, false> with the adapter added; brow = the B row of the lane's column
+template <bool FP32>
+__device__ __forceinline__ void store_tile_lora(const DevProblem &p, int tile_local, const f32x4_t &acc,
+                                                const LoraUpArgs &u, const float *ts, const float *bs) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int col = tile_local * 16 + (lane & 15);
+    if (col >= p.N) return;
+    const int stride = u.r + 4;
+    const float *brow = bs + (lane & 15) * stride;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = 4 * (lane >> 4) + i;
+        if (m < p.M) {
+            const float *trow = ts + m * stride;
+            float s = 0.0f;
+            for (int j = 0; j < u.r; j += 4) {
+                const float4 tv = *reinterpret_cast<const float4 *>(trow + j);
+                const float4 bv = *reinterpret_cast<const float4 *>(brow + j);
+                s += tv.x * bv.x + tv.y * bv.y + tv.z * bv.z + tv.w * bv.w;
+            }
+            const float delta = FP32 ? s * u.scaling : lora_round_bf16(lora_round_bf16(s) * u.scaling);
+            const float base = bf16_bits_to_f32(pack_bf16_rne(acc[i], 0.0f) & 0xFFFFu);  // the base layer's bf16 output
+            as_global(p.y)[(long)m * p.N + col] = (uint16_t)(pack_bf16_rne(base + delta, 0.0f) & 0xFFFFu);
+        }
+    }
+}
+
+template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG, bool UP = false>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
-                                                 const NormArgs &norm) {
+                                                 const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{}) {
     constexpr int RS = FUSED ? 2 : 1;
     static_assert(!XG || (TW == 1 && !NORM), "register-fed activations: one tile per workgroup, no norm");
+    static_assert(!UP || (!FUSED && !NORM), "an adapter's up-projection joins a plain problem");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tw = wave / KS, kw = wave % KS;  // tile of the round, share of K
     const int lane = threadIdx.x & (WAVE - 1);
@@ -538,6 +612,15 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     bool work = sc0 < sc1 && tile < t1;  // wave-uniform
     PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, work ? tile : t0, sc0);
     if (work) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
+    // the adapter's operands sit behind every workgroup's partial tiles; the barrier before the
+    // partial tiles are read makes them visible
+    float *lora_ts = reinterpret_cast<float *>(smem + (size_t)xrows * xstride * 2) +
+                     TW * (KS - 1) * RS * WAVE * 4;
+    float *lora_bs = lora_ts + 16 * (UP ? up.r + 4 : 0);   // t of the record's (at most 16) rows, then B
+    if constexpr (UP) {
+        if (up.fp32) stage_lora_up<true>(p, up, t0 * 16, TW * 16, lora_ts, lora_bs, KS * TW * WAVE);
+        else stage_lora_up<false>(p, up, t0 * 16, TW * 16, lora_ts, lora_bs, KS * TW * WAVE);
+    }
     u32x4_t xpre[1][16];
     if constexpr (XG) {
         const int lc = lane & 15, kbase = sc0 * PP_SC + (lane >> 4) * 128;  // the lane's row and 128-k span
@@ -577,7 +660,13 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
             for (int w = 1; w < KS; ++w)
 #pragma unroll
                 for (int r = 0; r < RS; ++r) acc[r][0] += red[((w - 1) * RS + r) * WAVE + lane];
-            store_tile<1, FUSED>(p, tile, acc);
+            if constexpr (UP) {
+                const float *brows = lora_bs + (tile - t0) * 16 * (up.r + 4);
+                if (up.fp32) store_tile_lora<true>(p, tile, acc[0][0], up, lora_ts, brows);
+                else store_tile_lora<false>(p, tile, acc[0][0], up, lora_ts, brows);
+            } else {
+                store_tile<1, FUSED>(p, tile, acc);
+            }
         }
         work = work && next >= 0;
         if (base + TW < t1) __syncthreads();  // the partial tiles are read before they are rewritten
@@ -585,10 +674,14 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 }
 
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
-template <bool FUSED, int KS, int TW, bool NORM, bool XG>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool UP = false>
 __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem,
-                                               const NormArgs &norm) {
-    if (FUSED && p.fused) {
+                                               const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{}) {
+    if constexpr (UP) {
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, false, XG, true>(p, t0, t1, smem, norm, up);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, false, XG, true>(p, t0, t1, smem, norm, up);
+        else split_segment_pp<false, KS, TW, 4, false, XG, true>(p, t0, t1, smem, norm, up);
+    } else if (FUSED && p.fused) {
         if (p.G == 128) split_segment_pp<FUSED, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm);
         else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
         else split_segment_pp<FUSED, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
@@ -640,9 +733,10 @@ struct DirectArgs {
     DevProblem recs[DIRECT_MAX];  // tile_begin holds the record's first workgroup here
     NormArgs norm;                // read by the NORM instantiations only
     LoraDownArgs ld;              // read by the LD instantiations only
+    LoraUpArgs up;                // read by the UP instantiations only
 };
 
-template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD, bool UP>
 __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     int g = blockIdx.x;
@@ -659,7 +753,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
     const int t0 = (g - p.tile_begin) * TW;
-    split_by_group<FUSED, KS, TW, NORM, XG>(p, t0, min(tiles, t0 + TW), smem, a.norm);
+    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW), smem, a.norm, a.up);
 }
 
 }  // namespace

@@ -20,10 +20,11 @@ op in fp32, rounded to bf16); the attention keeps its probabilities in fp32.
 Needs a trunk whose projections were swapped for prepacked :class:`Int4Linear` modules with the
 fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry one active LoRA
 adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
-the norm as a launch of its own (the adapters read the normalised row) and an up-projection launch for
-o_proj's adapter: seven launches.  The down-projections of the q|k|v adapters ride with the q|k|v
-launch as extra workgroups and their up-projections are added by the attention launch as it reads q, k,
-v; the attention launch also leaves o_proj's down-projection behind, one piece per head.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not
+the norm as a launch of its own (the adapters read the normalised row): six launches.  The
+down-projections of the q|k|v adapters ride with the q|k|v launch as extra workgroups and their
+up-projections are added by the attention launch as it reads q, k, v; the attention launch also leaves
+o_proj's down-projection behind, one piece per head, and o_proj's launch adds the up-projection before
+it stores.  :meth:`NativeDecodeTrunk.unsupported` says why a trunk does not
 qualify, and callers then keep the module path.
 """
 
@@ -264,10 +265,13 @@ class NativeDecodeTrunk:
             record = group.attn_record(q, k, v) if group is not None else None
             attn_at = len(calls)
             calls.append(None)
+            launch_at = len(calls)
             outs = gemv([(self.attn, proj["o_proj"][0], False)])
-            o_group = lora(self.attn, outs, [proj["o_proj"][1]], parts=H)
-            if o_group is not None:
+            o_group = lora(self.attn, outs, [proj["o_proj"][1]], up=False, parts=H)
+            if o_group is not None:   # o_proj's launch adds the up-projection itself
                 record = o_group.attn_output_record(record)
+                calls[launch_at] = (lib.vrl_int4_gemv_prepacked_lora_up_bf16,
+                                    (calls[launch_at][1][0], o_group.table, o_group.t.data_ptr(), H))
             calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args) if record is None else \
                 (lib.vrl_rope_attn_decode_lora_bf16, (*attn_args, ctypes.byref(record)))
             (state["x"],) = outs

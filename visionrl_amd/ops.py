@@ -382,12 +382,20 @@ class DirectGemv:
         self.norm = rec
         self._keep.append((residual, weight, h_out))
 
-    def launch(self, lora_down: "LoraAdd | None" = None):
+    def launch(self, lora_down: "LoraAdd | None" = None, lora_up: "LoraAdd | None" = None):
         """``lora_down``: a :class:`LoraAdd` over the input every problem of this launch reads; its
-        down-projection then runs in the same launch (in place of its ``launch_down``)."""
+        down-projection then runs in the same launch (in place of its ``launch_down``).
+        ``lora_up``: a :class:`LoraAdd` with one adapter over this launch's one output, whose ``t`` is
+        ready; the launch adds its up-projection before it stores (in place of its ``launch_up``)."""
         lib = _lib.load()
         with _on(self.device):
-            if lora_down is not None:
+            if lora_up is not None:
+                if lora_down is not None or self.norm is not None or len(self.table) != 1 or \
+                        len(lora_up.table) != 1 or lora_up.table[0].y != self.table[0].y:
+                    raise ValueError("an up-projection joins the launch of the one problem whose output it adds to")
+                rc = lib.vrl_int4_gemv_prepacked_lora_up_bf16(self.table, lora_up.table, lora_up.t.data_ptr(),
+                                                              lora_up.parts, _stream_handle(self.device))
+            elif lora_down is not None:
                 if self.norm is not None or lora_down.parts != 1:
                     raise ValueError("the adapters' down-projection joins a launch without a norm, in one piece")
                 rc = lib.vrl_int4_gemv_prepacked_lora_bf16(self.table, len(self.table), lora_down.table,
