@@ -123,8 +123,10 @@ __device__ __forceinline__ void stage_x_natural(const DevProblem &p, int k0, int
 // the record's x points into `x0`, a sublayer output; what the tiles multiply is
 //   weight * bf16(h * rsqrt(mean(h^2) + eps)),  h = residual ? bf16(x + residual) : x
 // with the roundings LlamaDecoderLayer.forward / LlamaRMSNorm.forward apply to bf16 tensors.
-// Every workgroup normalises the rows it stages (one wave per row, the row kept in registers);
-// the first workgroup of a record flagged PP_WRITE_H also writes h to `h_out`.
+// Every workgroup normalises the rows it stages (the row kept in registers: one wave per row, or,
+// when there are fewer rows than waves, `split` waves per row whose sums of squares meet in LDS: a
+// single wave issues too slowly to hide a row's arithmetic); the first workgroup of a record flagged
+// PP_WRITE_H also writes h to `h_out`.
 struct NormArgs {
     const uint16_t *x0;        // base of the activation tensor the records' x point into
     const uint16_t *residual;  // same shape as x0, or nullptr
@@ -136,9 +138,12 @@ struct NormArgs {
 constexpr int PP_WRITE_H = 4;       // DevProblem::prepacked bit
 constexpr int NORM_MAX_K = 4096;    // eight 16-byte words per lane hold a row
 
-template <int NW>  // 16-byte words per lane that hold a row: K <= NW * 512
+// NW: 16-byte words per lane that hold a wave's share of a row (K <= NW * split * 512); `scratch`:
+// one float per wave, used when split > 1 (then M * split <= nwaves: one pass)
+template <int NW>
 __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
-                                                  int xstride, int nwaves, bool write_h) {
+                                                  int xstride, int nwaves, bool write_h, int split,
+                                                  float *scratch) {
     typedef __attribute__((address_space(1))) u32x4_t *gptr_w4;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & (WAVE - 1);
@@ -155,15 +160,18 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
             *reinterpret_cast<u32x4_t *>(xs + p.M * xstride + (j << 3)) = zero;
     const long base = p.x - n.x0;
     const float inv_k = 1.0f / (float)p.K;
-    for (int m = wave; m < p.M; m += nwaves) {
+    const int per_pass = nwaves / split, part = wave % split;
+    for (int m0 = 0; m0 < p.M; m0 += per_pass) {
+        const int m = m0 + wave / split;
+        const bool live = m < p.M;  // wave-uniform
         const long row = base + (long)m * p.K;
         u32x4_t h[NW], rv[NW], wv[NW];
         // one memory round trip: the row, its residual and the norm weight are requested together
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
-            const int k = (i * WAVE + lane) << 3;
+            const int k = ((part * NW + i) * WAVE + lane) << 3;
             h[i] = rv[i] = wv[i] = zero;
-            if (k < p.K) {
+            if (live && k < p.K) {
                 h[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.x0 + row + k));
                 if (n.residual) rv[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.residual + row + k));
                 wv[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.weight + k));
@@ -172,8 +180,8 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
         float ss = 0.0f;
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
-            const int k = (i * WAVE + lane) << 3;
-            if (k < p.K) {
+            const int k = ((part * NW + i) * WAVE + lane) << 3;
+            if (live && k < p.K) {
                 if (n.residual) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
@@ -191,11 +199,17 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
             }
         }
         ss = wave_sum(ss);
+        if (split > 1) {  // uniform; the row's waves add their shares in one order
+            if (lane == 0) scratch[wave] = ss;
+            __syncthreads();
+            ss = 0.0f;
+            for (int q = 0; q < split; ++q) ss += scratch[wave - part + q];
+        }
         const float r = rsqrtf(ss * inv_k + n.eps);
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
-            const int k = (i * WAVE + lane) << 3;
-            if (k < p.K) {
+            const int k = ((part * NW + i) * WAVE + lane) << 3;
+            if (live && k < p.K) {
                 u32x4_t y;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -211,10 +225,17 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
 }
 
 __device__ __forceinline__ void stage_x_norm(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
-                                             int xstride, int nwaves, bool write_h) {
+                                             int xstride, int nwaves, bool write_h, float *scratch) {
     // rows up to 2048 wide keep half the registers (the 16-wave workgroups have 128 per lane)
-    if (p.K <= NORM_MAX_K / 2) stage_x_norm_rows<NORM_MAX_K / (16 * WAVE)>(p, n, kext, xs, xstride, nwaves, write_h);
-    else stage_x_norm_rows<NORM_MAX_K / (8 * WAVE)>(p, n, kext, xs, xstride, nwaves, write_h);
+    const int words = p.K <= NORM_MAX_K / 2 ? NORM_MAX_K / (16 * WAVE) : NORM_MAX_K / (8 * WAVE);
+    int split = 1;
+    while (2 * split * p.M <= nwaves && 2 * split <= words) split *= 2;
+    switch (words / split) {
+        case 8: stage_x_norm_rows<8>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
+        case 4: stage_x_norm_rows<4>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
+        case 2: stage_x_norm_rows<2>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
+        default: stage_x_norm_rows<1>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
+    }
 }
 
 struct PPGroup {
@@ -632,7 +653,8 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
         __syncthreads();
         if constexpr (NORM)
             stage_x_norm(p, norm, nsc * PP_SC, xs, xstride, KS * TW,
-                         t0 == 0 && (p.prepacked & PP_WRITE_H) && norm.h_out != nullptr);
+                         t0 == 0 && (p.prepacked & PP_WRITE_H) && norm.h_out != nullptr,
+                         reinterpret_cast<float *>(smem + (size_t)xrows * xstride * 2));  // the partial tiles' space, still free
         else
             stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, KS * TW * WAVE);
         __syncthreads();
