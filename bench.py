@@ -399,7 +399,7 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
     ``reference_style`` is the loop of vrl/models/families/janus_pro/policy.py:624-731 with the trunk's
     dynamic cache and the torch formulas for the tail, without its per-row cache copies and host
     read-backs (so a lower bound for the reference); ``static_*`` is visionrl_amd.ar_decode over the
-    trunk module, ``native_*`` the same with the trunk as visionrl_amd.decode_step (7 launches per layer).
+    trunk module, ``native_*`` the same with the trunk as visionrl_amd.decode_step (5 launches per layer, 6 with adapters).
     """
     import types
 
