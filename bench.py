@@ -392,7 +392,8 @@ def decode_tail(device, steps: int):
     return out
 
 
-def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16), prompt: int = 304):
+def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16), prompt: int = 304,
+                   shape=(HIDDEN, INTER, LAYERS, 16)):
     """ms per decode step of the image-token loop on a Janus-Pro-1B shaped policy (random weights), at
     cache lengths around the middle of a 576-token image (a 304-token context, then 48 tokens).
 
@@ -403,6 +404,8 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
     """
     import types
 
+    hidden, inter, layers, heads = shape   # Janus-Pro-1B by default; (4096, 11008, 30, 32) is the 7B-class trunk
+
     import torch.nn.functional as F
     from torch import nn
     from transformers import LlamaConfig, LlamaModel
@@ -410,16 +413,16 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
     from visionrl_amd.ar_decode import StaticARSampler
     from visionrl_amd.policy_glue import apply_int4_to_policy
 
-    cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=LAYERS,
-                      num_attention_heads=16, num_key_value_heads=16, vocab_size=128,
+    cfg = LlamaConfig(hidden_size=hidden, intermediate_size=inter, num_hidden_layers=layers,
+                      num_attention_heads=heads, num_key_value_heads=heads, vocab_size=128,
                       max_position_embeddings=1024)
 
     class MMGPT(nn.Module):
         def __init__(self):
             super().__init__()
             self.language_model = types.SimpleNamespace(model=LlamaModel(cfg).to(torch.bfloat16).eval())
-            self.gen_head = nn.Linear(HIDDEN, HEAD, bias=False).to(torch.bfloat16)
-            self.gen_embed = nn.Embedding(HEAD, HIDDEN).to(torch.bfloat16)
+            self.gen_head = nn.Linear(hidden, HEAD, bias=False).to(torch.bfloat16)
+            self.gen_embed = nn.Embedding(HEAD, hidden).to(torch.bfloat16)
 
         def prepare_gen_img_embeds(self, ids):
             return self.gen_embed(ids)
@@ -469,7 +472,7 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
         return (timed(tokens) - min(timed(1), timed(1))) / (tokens - 1)
 
     out = {"tokens_per_call": tokens, "prompt_tokens": prompt,
-           "model": "LlamaModel 24 x (2048, 5632), 16 heads, head 2048->16384, random weights"}
+           "model": f"LlamaModel {layers} x ({hidden}, {inter}), {heads} heads, head {hidden}->{HEAD}, random weights"}
     with torch.device(device):
         torch.manual_seed(0)
         policy = Policy()
@@ -478,8 +481,8 @@ def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1
     inputs = {}
     for B in batches:
         g = torch.Generator(device=device).manual_seed(7000 + B)
-        inputs[B] = (torch.randn((B, prompt, HIDDEN), generator=g, device=device).to(torch.bfloat16),
-                     torch.randn((B, prompt, HIDDEN), generator=g, device=device).to(torch.bfloat16),
+        inputs[B] = (torch.randn((B, prompt, hidden), generator=g, device=device).to(torch.bfloat16),
+                     torch.randn((B, prompt, hidden), generator=g, device=device).to(torch.bfloat16),
                      torch.ones((B, prompt), dtype=torch.long, device=device),
                      torch.ones((B, prompt), dtype=torch.long, device=device))
     for B in batches if only is None else ():
@@ -627,6 +630,8 @@ def main():
     ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
     ap.add_argument("--ar-decode", type=int, default=0, metavar="B",
                     help="run only the recorded decode loop at batch B on the int4 policy and exit (for profilers)")
+    ap.add_argument("--trunk-7b", action="store_true",
+                    help="with --ar-decode: the 7B-class trunk (30 x (4096, 11008), 32 heads) instead of the 1B one")
     ap.add_argument("--attn-decode", type=int, default=0, metavar="ROWS",
                     help="run 8 attention decode launches (16 heads x 128, slot 330 of 384) over distinct caches "
                          "at ROWS rows and exit (for counter runs)")
@@ -667,7 +672,8 @@ def main():
         return
     if args.ar_decode:
         which = "int4_lora_native_hip_graph" if args.lora else "int4_native_hip_graph"
-        print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,))))
+        shape = (4096, 11008, 30, 32) if args.trunk_7b else (HIDDEN, INTER, LAYERS, 16)
+        print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,), shape=shape)))
         return
     if args.single_calls:
         for M in (1, 32):

@@ -570,6 +570,24 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     }
     size_t lds = xg ? red : xz_bytes + red;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    // More workgroups than the device holds at once (16 waves and 160 KB of LDS per CU) would run in
+    // waves of workgroups, each staging x and ramping up again: a workgroup then walks several sets of
+    // TW tiles, the next set's first loads issued under the current one's last.
+    args.rounds = 1;
+    if (!lora_up) {
+        const long per_cu = std::max<long>(1, std::min<long>(16 / (ks * tw), (long)(160 * 1024 / std::max<size_t>(lds, 1024))));
+        const long capacity = per_cu * device_cu_count();
+        args.rounds = (int)std::min<long>(8, (workgroups + capacity - 1) / capacity);
+        if (args.rounds > 1) {
+            workgroups = 0;
+            for (int i = 0; i < args.n; ++i) {
+                DevProblem &p = args.recs[i];
+                const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
+                p.tile_begin = (int)workgroups;
+                workgroups += (tiles + tw * args.rounds - 1) / (tw * args.rounds);
+            }
+        }
+    }
     if (lora_up) {
         // the launch's one problem carries one adapter: y = base + scaling * t . B^T
         const vrl_int4_problem &q0 = problems[0];

@@ -735,7 +735,9 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_split_kernel(const DevProblem 
 
 // The same latency mode without a plan in device memory: up to DIRECT_MAX records travel
 // as kernel arguments (no dependent loads before the first weight request).  Workgroup g of
-// the launch takes the TW tiles (g - first workgroup of its record) * TW ... of that record.
+// the launch takes the TW * rounds tiles from (g - first workgroup of its record) * TW * rounds of
+// that record, TW at a time (rounds > 1 when the launch would otherwise have more workgroups than
+// the device holds at once: a second wave of workgroups would stage x and ramp up all over again).
 // This is the single-call path of a prepacked weight (and of q|k|v, gate|up groups); the host
 // cuts activations of more than 16 rows, or too large for LDS, into row slabs, one record each.
 constexpr int DIRECT_MAX = 8;
@@ -751,7 +753,7 @@ struct LoraDownArgs {
 };
 struct DirectArgs {
     int32_t n;
-    int32_t pad;
+    int32_t rounds;               // sets of TW tiles a workgroup walks, one after the other
     DevProblem recs[DIRECT_MAX];  // tile_begin holds the record's first workgroup here
     NormArgs norm;                // read by the NORM instantiations only
     LoraDownArgs ld;              // read by the LD instantiations only
@@ -774,8 +776,8 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
     for (int k = 1; k < DIRECT_MAX; ++k)
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
-    const int t0 = (g - p.tile_begin) * TW;
-    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW), smem, a.norm, a.up);
+    const int t0 = (g - p.tile_begin) * TW * a.rounds;
+    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW * a.rounds), smem, a.norm, a.up);
 }
 
 }  // namespace
