@@ -143,7 +143,8 @@ typedef struct vrl_int4_plan_info {
  * the records travel as kernel arguments, the waves of a workgroup split K of a 16-column
  * tile.  Meant for decode and rollout batches (the launch is one memory round trip).  Every
  * problem must have prepacked = 1; activations are taken in slabs of at most 16 rows (fewer
- * for K > 8192, where a slab must fit LDS), and all slabs of a call together may number at
+ * where a slab is staged in LDS and does not fit it: K > 16384, or K > 4096 with adapters'
+ * down-projections in the launch), and all slabs of a call together may number at
  * most 8 (for K = 2048: three problems of 32 rows), else VRL_INT4_ESHAPE and the caller uses
  * a grouped plan or vrl_int4_gemv_bf16.  scales and qzeros of the records are ignored.
  */

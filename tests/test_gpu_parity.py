@@ -496,6 +496,9 @@ DIRECT_SHAPES = [
     # more than one slab of rows, several tiles per workgroup, a ragged last workgroup
     (32, 2048, 2048, False), (17, 2048, 100, False), (32, 5632, 208, False), (9, 1024, 80, False),
     (32, 11008, 48, False), (32, 2048, 2 * 720, True), (20, 4096, 2 * 112, True), (16, 2048, 2064, False),
+    # long K with register-fed activations: two super-chunks per wave (ragged share, full share), and more
+    # tiles than the device holds workgroups (a workgroup walks two sets)
+    (12, 8704, 64, False), (16, 16384, 32, False), (4, 11008, 4352, False), (2, 4096, 2 * 8256, True),
 ]
 
 
@@ -567,9 +570,10 @@ def test_direct_rejects_what_it_cannot_take(ops_mod):
         ops_mod.DirectGemv([(d["x"], pw, False)])            # 33 rows
     with pytest.raises(ValueError):
         ops_mod.DirectGemv([(d["x"][:1], pw, False)] * 9)    # nine problems
-    big = o.make_operands(9301, 32, 11008, 16, G)            # LDS holds 6 such rows: 6 slabs per problem
+    big = o.make_operands(9301, 32, 11008, 16, G)            # two 16-row slabs per problem, eight per launch
     db = to_device(big, DEV)
     pwb = ops_mod.int4_prepack(db["qweight"], db["scales"], db["qzeros"], G)
-    assert pwb.direct_slab_rows() == 6
+    assert pwb.direct_slab_rows() == 6                       # the staged form's bound (what LDS holds of such rows)
+    ops_mod.DirectGemv([(db["x"], pwb, False)] * 4).launch()
     with pytest.raises(ValueError):
-        ops_mod.DirectGemv([(db["x"], pwb, False)] * 2).launch()
+        ops_mod.DirectGemv([(db["x"], pwb, False)] * 5).launch()

@@ -501,12 +501,18 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // KS waves split K of a tile (one super-chunk each where K allows); with 8 or more
     // activation rows a workgroup carries several tiles so that one staging of x serves them
     const int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
-    // One super-chunk per wave: the waves can fetch their own activations, with nothing staged and one
-    // tile per workgroup.  Long K always does; shorter K with 8+ rows does while the launch is small
-    // (every tile then fetches its rows from L2 itself: for a wide matrix one staging per TW tiles wins).
+    // The waves can fetch their own activations, with nothing staged and one tile per workgroup.  Long K
+    // does with one super-chunk per wave, and with two when staging would need more than one slab of
+    // rows (the second fetch waits for the first super-chunk's arithmetic); shorter K with 8+ rows and one
+    // super-chunk per wave does while the launch is small (every tile then fetches its rows from L2
+    // itself: for a wide matrix one staging per TW tiles wins).
     const bool lora_up = lora && lora->up, lora_down = lora && !lora->up;
-    const bool xg = !norm && !lora_down && max_nsc <= ks &&
-                    (ks == 16 || (max_m >= 8 && slab_tiles <= 2L * device_cu_count()));
+    // rows of the longest K that LDS holds beside a 16-wave workgroup's partial tiles
+    const long staged_rows = (long)((DIRECT_LDS_CAP - (size_t)15 * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t)) /
+                                    ((size_t)(max_nsc * PP_SC + XPAD) * 2));
+    const bool xg = !norm && !lora_down &&
+                    (ks == 16 ? max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows)
+                              : max_nsc <= ks && max_m >= 8 && slab_tiles <= 2L * device_cu_count());
     const int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab

@@ -342,14 +342,16 @@ __device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t,
 // for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
 // if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
 // never runs dry between tiles.
-// XG: the A operand of the one super-chunk the call covers (sc1 == sc0 + 1) was fetched into registers by
-// the caller (xpre[b][4 * d + dd]) instead of being staged in LDS.
+// XG: the A operand is not staged in LDS: xpre[b][4 * d + dd] holds it for super-chunk `xpre_sc`
+// (fetched by the caller) and is fetched again through `xr`, a range-checked resource over the
+// record's x, whenever the walk reaches another super-chunk.
 template <int MB, bool FUSED, int GQ, bool XG = false>
 __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
                                                int next_tile, const uint16_t *xs, int xstride,
                                                int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
                                                f32x4_t (&acc)[FUSED ? 2 : 1][MB],
-                                               const u32x4_t (*xpre)[16] = nullptr) {
+                                               u32x4_t (*xpre)[16] = nullptr, int *xpre_sc = nullptr,
+                                               const rsrc_t *xr = nullptr) {
     constexpr int RS = FUSED ? 2 : 1;
     const int lane = threadIdx.x & (WAVE - 1);
     const int lc = lane & 15;
@@ -437,6 +439,15 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
     const uint32_t voff = lane * 16u;
     for (int sc = sc0; sc < sc1; ++sc) {
         const bool last = sc + 1 == sc1;
+        if constexpr (XG) {
+            if (*xpre_sc != sc) {  // wave-uniform; never with one super-chunk per wave
+                const int kb = sc * PP_SC + kq * 128;
+                const uint32_t vo = (lc < p.M && kb < p.K) ? (uint32_t)(lc * p.K + kb) * 2u : PP_OUT_OF_RANGE;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) xpre[0][i] = __builtin_amdgcn_raw_buffer_load_b128(*xr, vo + 16u * i, 0, 0);
+                *xpre_sc = sc;
+            }
+        }
         uint32_t rw[RS], rm[RS];
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
@@ -533,11 +544,12 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
 // o_proj, ...).  A workgroup carries TW such tiles at once (KS * TW waves), so that one
 // staging of the activations serves TW tiles: that matters once x is tens of KB (8+ rows).
 // LDS: staged activations, then TW x (KS - 1) x RS partial tiles.
-// XG (plan-free launches of long K, one super-chunk per wave): no staging at all.  With K split over
-// the waves and one tile per workgroup every activation value is used by exactly one wave, so each
-// wave fetches its own A operand (16 rows x 512 k: sixteen 16-byte buffer loads per lane, zeros for
-// rows beyond M and k beyond K through the buffer's range check) while its weights arrive; LDS
-// holds only the partial tiles, and 16 rows per record fit whatever K is.
+// XG (plan-free launches of long K): no staging at all.  With K split over the waves and one tile
+// per workgroup every activation value is used by exactly one wave, so each wave fetches its own A
+// operand (16 rows x 512 k: sixteen 16-byte buffer loads per lane, zeros for rows beyond M and k
+// beyond K through the buffer's range check) while its weights arrive, and again for every further
+// super-chunk of its share (K > 8192: two per wave); LDS holds only the partial tiles, and 16 rows
+// per record fit whatever K is.
 // UP instantiations (plan-free launches of one problem) add a LoRA adapter's up-projection to the
 // tile before it is stored: y = bf16(bf16(x . W^T) + scaling * t . B^T), the second half of a PEFT
 // wrapper's forward (vrl/models/families/janus_pro/policy.py:298-324 attaches the adapters), with t
@@ -643,9 +655,11 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
         else stage_lora_up<false>(p, up, t0 * 16, TW * 16, lora_ts, lora_bs, KS * TW * WAVE);
     }
     u32x4_t xpre[1][16];
+    int xpre_sc = sc0;
+    rsrc_t xr = rsrc;  // replaced below for XG
     if constexpr (XG) {
         const int lc = lane & 15, kbase = sc0 * PP_SC + (lane >> 4) * 128;  // the lane's row and 128-k span
-        const rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.x), 0, p.M * p.K * 2, 0x00020000);
+        xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(p.x), 0, p.M * p.K * 2, 0x00020000);
         const uint32_t voff = (work && lc < p.M && kbase < p.K) ? (uint32_t)(lc * p.K + kbase) * 2u : PP_OUT_OF_RANGE;
 #pragma unroll
         for (int i = 0; i < 16; ++i) xpre[0][i] = __builtin_amdgcn_raw_buffer_load_b128(xr, voff + 16u * i, 0, 0);
@@ -667,7 +681,7 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
         for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if (work) {
             if constexpr (XG)
-                stream_rows_pp<1, FUSED, GQ, true>(p, rsrc, cur, next, nullptr, 0, sc0, sc1, ring, acc, xpre);
+                stream_rows_pp<1, FUSED, GQ, true>(p, rsrc, cur, next, nullptr, 0, sc0, sc1, ring, acc, xpre, &xpre_sc, &xr);
             else
                 stream_rows_pp<1, FUSED, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
             if (next >= 0) cur = pp_tile_ptr<FUSED>(p, next, sc0);
