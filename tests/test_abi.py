@@ -164,7 +164,7 @@ def test_direct_prepacked_validation(lib):
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
     probs[1].G, probs[1].y = 128, p + 2          # misaligned output
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1002
-    probs[1].y, probs[1].M, probs[1].K = p, 32, 16384  # LDS holds 4 such rows: 8 slabs, 9 with the first problem
+    probs[1].y, probs[1].M, probs[1].K = p, 32, 16896  # beyond the register-fed form; LDS holds 4 such rows: 8 slabs, 9 with the first problem
     assert lib.vrl_int4_gemv_prepacked_bf16(probs, 2, None) == 1001
 
 
