@@ -625,6 +625,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true",
                     help="run just the grouped decode-step launches (for profilers)")
+    ap.add_argument("--rows", type=int, default=1, choices=(1, 32),
+                    help="with --only-headline: 1 = the M=1 set (default), 32 = the rollout-batch set plus the "
+                         "image-token head")
     ap.add_argument("--single-calls", action="store_true",
                     help="loop single-GEMV launches over distinct weights per shape and exit (for profilers)")
     ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
@@ -693,13 +696,18 @@ def main():
         print(json.dumps({"single_calls": "done"}))
         return
 
-    items = build_set(2, 1, device, with_head=False)
+    if args.only_headline and args.rows == 32:
+        items = build_set(3, 32, device, with_head=True)
+    else:
+        items = build_set(2, 1, device, with_head=False)
     torch.cuda.synchronize()
 
     if args.only_headline:
         grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items])
         ms = time_region(grouped.launch, args.steps, args.warmup)
-        print(json.dumps({"ms_per_step": ms}))
+        nbytes = sum(it["bytes"] for it in items)
+        print(json.dumps({"rows": args.rows, "ms_per_step": ms, "algorithmic_bytes_per_step": nbytes,
+                          "GBps": nbytes / (ms * 1e-3) / 1e9}))
         return
 
     strat, total_bytes, grouped = measure_set(items, args.steps, args.warmup)

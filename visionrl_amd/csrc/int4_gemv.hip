@@ -842,9 +842,12 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             const int out_cols = p.fused ? p.N / 2 : p.N;
             const int nt = (out_cols + 15) / 16;
             const double c = (double)p.K * (p.fused ? 2 : 1) + 512.0;
+            // a record walked in staged passes deals its tiles to the waves in lock-step, one per
+            // wave at a time: a range inside it is cut at a multiple of the workgroup's waves
+            const int cut = (p.prepacked && p.kc < pp_nsc(p.K) * PP_SC) ? wpb : 1;
             for (int t = 0; t < nt; ++t) {
                 // tile (p.tile_begin + t) starts block b+1 once the blocks so far hold their share
-                while (b + 1 < grid && acc_cost >= total_cost * (b + 1) / (double)grid) {
+                while (b + 1 < grid && t % cut == 0 && acc_cost >= total_cost * (b + 1) / (double)grid) {
                     ++b;
                     block_begin[b] = p.tile_begin + t;
                 }

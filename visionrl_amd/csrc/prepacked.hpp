@@ -340,8 +340,11 @@ __device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t,
 
 // acc += x[:, 512*sc0 : 512*sc1) . W[tile rows, same k]^T from a prepacked blob; xs holds x
 // for exactly that k range.  On entry the ring holds super-chunk sc0 of this tile (pp_prime);
-// if next_tile >= 0 the ring holds that tile's super-chunk sc0 on return, so that the wave
-// never runs dry between tiles.
+// if next_tile >= 0 the ring holds that tile's super-chunk sc0 (next_sc0, if given) on return,
+// so that the wave never runs dry between tiles.
+// prio >= 0: the wave's issue priority rotates with every super-chunk, starting at prio (walks
+// in lock-step between barriers, where the hardware's preference for the oldest wave of a SIMD
+// would make the whole workgroup wait for the youngest).
 // XG: the A operand is not staged in LDS: xpre[b][4 * d + dd] holds it for super-chunk `xpre_sc`
 // (fetched by the caller) and is fetched again through `xr`, a range-checked resource over the
 // record's x, whenever the walk reaches another super-chunk.
@@ -351,7 +354,8 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                                                int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
                                                f32x4_t (&acc)[FUSED ? 2 : 1][MB],
                                                u32x4_t (*xpre)[16] = nullptr, int *xpre_sc = nullptr,
-                                               const rsrc_t *xr = nullptr) {
+                                               const rsrc_t *xr = nullptr, int next_sc0 = -1,
+                                               int prio = -1) {
     constexpr int RS = FUSED ? 2 : 1;
     const int lane = threadIdx.x & (WAVE - 1);
     const int lc = lane & 15;
@@ -435,10 +439,18 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
     // the blob: the buffer range check answers such a load with zeros without touching
     // memory, and the loop body exists once and has no branch.
     const bool has_next = next_tile >= 0;
-    const PPTilePtr<FUSED> nxt = pp_tile_ptr<FUSED>(p, has_next ? next_tile : 0, sc0);
+    const PPTilePtr<FUSED> nxt = pp_tile_ptr<FUSED>(p, has_next ? next_tile : 0, next_sc0 < 0 ? sc0 : next_sc0);
     const uint32_t voff = lane * 16u;
     for (int sc = sc0; sc < sc1; ++sc) {
         const bool last = sc + 1 == sc1;
+        if (prio >= 0) {  // wave-uniform
+            switch ((prio + sc) & 3) {
+                case 0: __builtin_amdgcn_s_setprio(0); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                default: __builtin_amdgcn_s_setprio(3); break;
+            }
+        }
         if constexpr (XG) {
             if (*xpre_sc != sc) {  // wave-uniform; never with one super-chunk per wave
                 const int kb = sc * PP_SC + kq * 128;
@@ -502,8 +514,13 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
     } else if constexpr (PASSES) {
         // activations do not fit: K is walked in staged passes, and every wave carries T tiles
         // through a pass so that one staging serves T * WPB tiles
+        // The ring runs through the whole segment: the last super-chunk of a (tile, pass) step
+        // pulls in the first of the wave's next step (its next tile of this pass, else its first
+        // tile of the next pass, else of the next round), also across the barriers of a staging.
         constexpr int T = FUSED ? 1 : (MB == 2 ? 2 : 4);
         const rsrc_t rsrc = pp_blob_rsrc(p);
+        PPRing<RS, GQ> ring;
+        if (t0 + wave < t1) pp_prime<FUSED, GQ>(rsrc, pp_tile_ptr<FUSED>(p, t0 + wave, 0), ring);
         for (int round = t0; round < t1; round += WPB * T) {
             f32x4_t acc[T][RS][MB];
 #pragma unroll
@@ -521,12 +538,25 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
                 for (int i = 0; i < T; ++i) {
                     const int tile = round + i * WPB + wave;  // neighbouring waves, neighbouring tiles
                     if (tile < t1) {
-                        PPRing<RS, GQ> ring;
                         const PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile, sc0);
-                        pp_prime<FUSED, GQ>(rsrc, cur, ring);
-                        stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, -1, xs, xstride, sc0, sc1, ring, acc[i]);
+                        int ntile = -1, nsc0 = sc0;
+                        if (i + 1 < T && tile + WPB < t1) {
+                            ntile = tile + WPB;
+                        } else if (sc1 < nsc) {
+                            ntile = round + wave;
+                            nsc0 = sc1;
+                        } else if (round + WPB * T + wave < t1) {
+                            ntile = round + WPB * T + wave;
+                            nsc0 = 0;
+                        }
+                        // waves w, w + 4, w + 8, w + 12 share a SIMD: each starts the pass at
+                        // another priority and moves on with every super-chunk
+                        const int prio = (wave >> 2) + i * (sc1 - sc0);
+                        stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, ntile, xs, xstride, sc0, sc1, ring, acc[i],
+                                                      nullptr, nullptr, nullptr, nsc0, prio);
                     }
                 }
+                __builtin_amdgcn_s_setprio(0);
             }
 #pragma unroll
             for (int i = 0; i < T; ++i) {
