@@ -517,7 +517,7 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
         // The ring runs through the whole segment: the last super-chunk of a (tile, pass) step
         // pulls in the first of the wave's next step (its next tile of this pass, else its first
         // tile of the next pass, else of the next round), also across the barriers of a staging.
-        constexpr int T = FUSED ? 1 : (MB == 2 ? 2 : 4);
+        constexpr int T = FUSED ? 1 : 4;
         const rsrc_t rsrc = pp_blob_rsrc(p);
         PPRing<RS, GQ> ring;
         if (t0 + wave < t1) pp_prime<FUSED, GQ>(rsrc, pp_tile_ptr<FUSED>(p, t0 + wave, 0), ring);
