@@ -711,7 +711,6 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         const long nt = (out_cols + 15) / 16;
         tiles += nt;
         if (tiles >= (1L << 30)) return VRL_INT4_ESHAPE;
-        total_cost += (double)nt * ((double)p.K * (p.fused ? 2 : 1) + 512.0);
         const int kfull = p.prepacked ? pp_nsc(p.K) * PP_SC : p.K;
         const size_t need = (size_t)p.M * (kfull + XPAD) * 2;
         if (need > x_need) x_need = need;
@@ -834,6 +833,19 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
         }
     } else
     {
+        // what a tile costs: its k extent plus a fixed part; a record walked in staged passes
+        // pays for its stagings and barriers on top (measured: the workgroups that hold such tiles
+        // ended 28 % after the others at equal weight; 1.45 is the best of a sweep from 1.0 to 2.4 on
+        // the 1B set at 32 rows, and is worth 7-8 % on the 7B-class sets at 8 and 16 rows)
+        const double pass_factor = 1.45;
+        auto tile_cost = [&](const DevProblem &p) {
+            const bool passes = p.prepacked && p.kc < pp_nsc(p.K) * PP_SC;
+            return ((double)p.K * (p.fused ? 2 : 1) + 512.0) * (passes ? pass_factor : 1.0);
+        };
+        for (int i = 0; i < n_problems; ++i) {
+            const DevProblem &p = recs[i];
+            total_cost += (double)(((p.fused ? p.N / 2 : p.N) + 15) / 16) * tile_cost(p);
+        }
         int b = 0;
         double acc_cost = 0.0;
         block_begin[0] = 0;
@@ -841,7 +853,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             const DevProblem &p = recs[i];
             const int out_cols = p.fused ? p.N / 2 : p.N;
             const int nt = (out_cols + 15) / 16;
-            const double c = (double)p.K * (p.fused ? 2 : 1) + 512.0;
+            const double c = tile_cost(p);
             // a record walked in staged passes deals its tiles to the waves in lock-step, one per
             // wave at a time: a range inside it is cut at a multiple of the workgroup's waves
             const int cut = (p.prepacked && p.kc < pp_nsc(p.K) * PP_SC) ? wpb : 1;
