@@ -321,6 +321,29 @@ def test_prepacked_grouped_parity(ops_mod, M, K, N, fused):
     assert (np.abs(got - ref_op) <= tol).all()
 
 
+@pytest.mark.parametrize("M,K,N", [(32, 1024, 144), (1, 512, 80), (16, 2048, 112)])
+def test_prepacked_records_sharing_activations(ops_mod, M, K, N):
+    """Records side by side that read the same x (q|k|v, gate|up) keep it staged; a record
+    with another x between them, or after them, stages its own.  Few tiles per record, so that
+    every workgroup's range runs over several records."""
+    say("shared x", M, K, N)
+    G = 128
+    sets = [o.make_operands(6500 + 10 * i + M, M, K, N, G) for i in range(6)]
+    x1 = bits_to_bf16(sets[0]["x_bits"], DEV)
+    x2 = bits_to_bf16(sets[2]["x_bits"], DEV)
+    which = [0, 0, 2, 0, 0, 2]                       # whose activations record i multiplies
+    problems = []
+    for i, ops in enumerate(sets):
+        d = to_device(ops, DEV)
+        pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+        problems.append(((x1, x2)[which[i] // 2], pw, False))
+    _, ys = run_grouped(ops_mod, problems)
+    for i, (ops, y) in enumerate(zip(sets, ys)):
+        ref = dict(ops)
+        ref["x_bits"] = sets[which[i]]["x_bits"]
+        assert_gemv_close(bf16_to_bits(y), ref, G, f"record {i} of 6, M{M} K{K} N{N}")
+
+
 @pytest.mark.parametrize("M,K,N", [(1, 512, 32), (4, 1024, 48), (16, 640, 16)])
 def test_prepacked_one_hot_is_the_exact_weight_column(ops_mod, M, K, N):
     """The matrix-core dequant of the prepacked path reproduces the canonical tile bit for bit."""

@@ -55,15 +55,17 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
     const int t_end = block_tab[blockIdx.x + 1].x;
     if (t >= t_end) return;  // block-uniform
     const int lo = entry.y;
+    StagedX staged;
     for (int pi = lo; t < t_end && pi < n_problems; ++pi) {
         const DevProblem p = plan[pi];
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
         if (PP && (!CANON || p.prepacked)) {
-            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES, GQ>(p, a, b, smem);
-            else stream_segment_pp<MB, false, WPB, PASSES, GQ>(p, a, b, smem);
+            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES, GQ>(p, a, b, smem, staged);
+            else stream_segment_pp<MB, false, WPB, PASSES, GQ>(p, a, b, smem, staged);
         } else if (CANON) {
+            staged.x = nullptr;  // the canonical walk stages in its own order
             if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
             else stream_segment<MB, false, WPB>(p, a, b, smem);
         }

@@ -473,8 +473,16 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
     }
 }
 
+// What a workgroup's LDS holds of staged activations, so that a segment over the same x as the one
+// before it (q|k|v or gate|up of a layer: records side by side in a plan) does not stage it again.
+struct StagedX {
+    const uint16_t *x = nullptr;  // nullptr: nothing whole
+    int M = 0, K = 0, kc = 0, zero_row = 0;
+};
+
 template <int MB, bool FUSED, int WPB, bool PASSES, int GQ>
-__device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem) {
+__device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
+                                                  StagedX &staged) {
     constexpr int RS = FUSED ? 2 : 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile offsets stay scalar
     uint16_t *xs = reinterpret_cast<uint16_t *>(smem);
@@ -493,10 +501,18 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
         const rsrc_t rsrc = pp_blob_rsrc(p);
         PPTilePtr<FUSED> cur = pp_tile_ptr<FUSED>(p, tile < t1 ? tile : t0, 0);
         if (tile < t1) pp_prime<FUSED, GQ>(rsrc, cur, ring);  // weights are on their way while x is staged
+        const int zero_row = p.prepacked & PP_ZERO_ROW;
+        const bool resident = staged.x == p.x && staged.M == p.M && staged.K == p.K && staged.kc == p.kc &&
+                              staged.zero_row == zero_row;  // block-uniform
         __syncthreads();
         if (threadIdx.x == 0) next_tile = t0 + WPB;
-        stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
+        if (!resident) stage_x_natural(p, 0, nsc * PP_SC, xs, xstride, WPB * WAVE);
         __syncthreads();
+        staged.x = p.x;
+        staged.M = p.M;
+        staged.K = p.K;
+        staged.kc = p.kc;
+        staged.zero_row = zero_row;
         while (tile < t1) {
             int nt = 0;
             if ((threadIdx.x & (WAVE - 1)) == 0) nt = atomicAdd(&next_tile, 1);
@@ -518,6 +534,7 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
         // pulls in the first of the wave's next step (its next tile of this pass, else its first
         // tile of the next pass, else of the next round), also across the barriers of a staging.
         constexpr int T = FUSED ? 1 : 4;
+        staged.x = nullptr;  // the passes leave a part of K behind
         const rsrc_t rsrc = pp_blob_rsrc(p);
         PPRing<RS, GQ> ring;
         if (t0 + wave < t1) pp_prime<FUSED, GQ>(rsrc, pp_tile_ptr<FUSED>(p, t0 + wave, 0), ring);
