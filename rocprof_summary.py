@@ -5,7 +5,7 @@ release write a SQLite database (``*_results.db``).  This prints, per kernel who
 name contains one of the given substrings, the call count and average duration
 (kernel trace) or the average counter value per dispatch (PMC run):
 
-    python -m visionrl_amd.rocprof_summary prof_trace/headline_results.db gemv prepack
+    python rocprof_summary.py prof_trace/headline_results.db gemv prepack
 """
 
 from __future__ import annotations

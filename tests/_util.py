@@ -28,16 +28,19 @@ def to_device(ops: dict, device) -> dict:
     }
 
 
-def assert_gemv_close(y_bits: np.ndarray, ops: dict, G: int, what: str = ""):
-    """The operator tolerance, stated once.
+# what: [outputs checked, outputs that are cancelled, of those: outputs beyond the strict bound]
+TOLERANCE_LOG: dict = {}
 
-    |y - y_ref| <= max(1 bf16 ulp at y_ref, 1e-2 |y_ref|) + 2^-18 sum|x w|, with
-    y_ref the float64 product over the canonical (bit-exact) bf16 weights.
-    Returns the worst backward error |y - y_ref| / sum|x w| for reporting.
+
+def check_gemv(y: np.ndarray, y_ref: np.ndarray, a_ref: np.ndarray, what: str = "") -> float:
+    """The operator tolerance, stated once (``oracle.gemv_tolerance``).
+
+    |y - y_ref| <= max(1 bf16 ulp at y_ref, 1e-2 |y_ref|) for every output with
+    |y_ref| >= 2^-6 sum|x w|; outputs that cancel below that may carry 2^-18 sum|x w| of fp32
+    reassociation noise on top.  y_ref is the float64 product over the canonical (bit-exact) bf16
+    weights.  How many outputs needed the extra term is counted per ``what`` in ``TOLERANCE_LOG``
+    and printed.  Returns the worst backward error |y - y_ref| / sum|x w|.
     """
-    y = oracle.bf16_bits_to_f32(y_bits).astype(np.float64)
-    y_ref = oracle.gemv_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
-    a_ref = oracle.gemv_abs_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
     assert y.shape == y_ref.shape, f"{what}: shape {y.shape} vs {y_ref.shape}"
     err = np.abs(y - y_ref)
     tol = oracle.gemv_tolerance(y_ref, a_ref)
@@ -46,4 +49,27 @@ def assert_gemv_close(y_bits: np.ndarray, ops: dict, G: int, what: str = ""):
         f"{what}: {int(bad.sum())} of {bad.size} outputs out of tolerance; worst at "
         f"{np.unravel_index(np.argmax(err - tol), err.shape)}: got {y.flat[np.argmax(err - tol)]!r} "
         f"ref {y_ref.flat[np.argmax(err - tol)]!r}")
+    cancelled = oracle.gemv_cancelled(y_ref, a_ref)
+    needed = cancelled & (err > oracle.gemv_strict_tolerance(y_ref))
+    key = what.split(":")[0] if what else "gemv"
+    log = TOLERANCE_LOG.setdefault(key, [0, 0, 0])
+    log[0] += err.size
+    log[1] += int(cancelled.sum())
+    log[2] += int(needed.sum())
     return float((err / np.maximum(a_ref, 1e-300)).max())
+
+
+def report_tolerance(key: str) -> None:
+    import sys
+
+    n, cancelled, needed = TOLERANCE_LOG.get(key, (0, 0, 0))
+    print(f"[tolerance] {key}: {n} outputs, {cancelled} cancelled below 2^-6 sum|x w|, "
+          f"{needed} of them beyond max(1 ulp, 1e-2 |y_ref|) (passed on the 2^-18 sum|x w| term)",
+          file=sys.stderr, flush=True)
+
+
+def assert_gemv_close(y_bits: np.ndarray, ops: dict, G: int, what: str = ""):
+    """``check_gemv`` of a device result (bf16 bit patterns) against the oracle's float64 product."""
+    y = oracle.bf16_bits_to_f32(y_bits).astype(np.float64)
+    y_ref, a_ref = oracle.gemv_and_abs_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    return check_gemv(y, y_ref, a_ref, what)

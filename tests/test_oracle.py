@@ -378,3 +378,29 @@ def test_make_operands_is_seeded_and_in_range():
     lg = o.make_operands(44, 1, 256, 64, 32, scale_mode="loguniform")
     s = o.bf16_bits_to_f32(lg["scales_bits"])
     assert s.min() >= 0.99e-4 and s.max() <= 1.01e-1
+
+
+def test_tolerance_rule_is_strict_unless_the_output_cancels():
+    """max(1 ulp, 1e-2 |y|) as stated wherever |y_ref| >= 2^-6 sum|x w|; 2^-18 sum|x w| on top below that."""
+    y_ref = np.array([1.0, 1.0, 0.0, 3.0e-3, -2.5], dtype=np.float64)
+    a_ref = np.array([2.0, 128.0, 5.0, 1.0, 100.0], dtype=np.float64)
+    cancelled = o.gemv_cancelled(y_ref, a_ref)
+    assert cancelled.tolist() == [False, True, True, True, False]
+    strict = o.gemv_strict_tolerance(y_ref)
+    assert strict[0] == 1e-2 and strict[4] == 2.5e-2              # 1e-2 |y| above one bf16 step (2^-7, 2^-6)
+    assert strict[2] == 2.0 ** -133                                # a bf16 subnormal step at zero
+    tol = o.gemv_tolerance(y_ref, a_ref)
+    assert (tol[~cancelled] == strict[~cancelled]).all()
+    assert np.allclose(tol[cancelled] - strict[cancelled], 2.0 ** -18 * a_ref[cancelled], rtol=1e-12)
+
+
+def test_fp32_accumulation_in_numpy_order_passes_the_rule_and_rarely_needs_the_slack():
+    ops = o.make_operands(31, 4, 2048, 512, 128)
+    args = (ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], 128)
+    y = o.bf16_bits_to_f32(o.gemv_bf16(*args)).astype(np.float64)
+    y_ref, a_ref = o.gemv_and_abs_f64(*args)
+    assert (y_ref == o.gemv_f64(*args)).all() and (a_ref == o.gemv_abs_f64(*args)).all()
+    err = np.abs(y - y_ref)
+    assert (err <= o.gemv_tolerance(y_ref, a_ref)).all()
+    needed = o.gemv_cancelled(y_ref, a_ref) & (err > o.gemv_strict_tolerance(y_ref))
+    assert needed.mean() < 0.02      # the extra term is for the few outputs that cancel to almost nothing
