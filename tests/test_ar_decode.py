@@ -55,15 +55,25 @@ class StubPolicy:
         return self.mmgpt.language_model.model
 
 
-def make_inputs(B, n_text, dtype, device, seed=3, hidden=HIDDEN):
+def make_inputs(B, n_text, dtype, device, seed=3, hidden=HIDDEN, side="left"):
+    """Prompt embeddings and masks of a chunk.  ``side="left"``: left padding of different lengths.
+    ``side="right"``: what the reference's executor hands over (``_tokenize_prompts`` pads to
+    ``max_text_length`` on the right, vrl/models/families/janus_pro/executor.py:439-462, and
+    ``align_pair`` right-pads, vrl/engine/ar/executor_base.py:166-195): ones, then zeros, the last
+    prompt slot a padding slot, and the unconditional "" prompt of row 0 almost all padding; the image
+    tokens' ones follow the zeros, so the mask has a hole in the middle."""
     g = torch.Generator().manual_seed(seed)
     cond = torch.randn(B, n_text, hidden, generator=g).to(dtype).to(device)
     uncond = torch.randn(B, n_text, hidden, generator=g).to(dtype).to(device)
     cmask = torch.ones(B, n_text, dtype=torch.long)
     umask = torch.ones(B, n_text, dtype=torch.long)
-    for b in range(B):   # left padding of different lengths, as the tokenizer produces
-        cmask[b, :b % 3] = 0
-        umask[b, :(b + 2) % 4] = 0
+    for b in range(B):
+        if side == "left":
+            cmask[b, :b % 3] = 0
+            umask[b, :(b + 2) % 4] = 0
+        else:
+            cmask[b, n_text - 1 - b % 3:] = 0
+            umask[b, (1 if b == 0 else n_text - 1 - (b + 2) % 4):] = 0
     return cond, uncond, cmask.to(device), umask.to(device)
 
 
@@ -90,9 +100,11 @@ def reference_loop(policy, cond, uncond, cmask, umask, cfg_weight, temperature, 
 
 
 # ------------------------------------------------------------------ CPU: the static-cache logic
-def test_static_cache_loop_samples_what_the_reference_loop_samples():
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_static_cache_loop_samples_what_the_reference_loop_samples(side):
     policy = StubPolicy()
-    cond, uncond, cmask, umask = make_inputs(3, 7, torch.float32, "cpu")
+    cond, uncond, cmask, umask = make_inputs(3, 7, torch.float32, "cpu", side=side)
+    assert side == "left" or (int(umask[0].sum()) == 1 and not cmask[:, -1].any())
     torch.manual_seed(11)
     want_t, want_lp = reference_loop(policy, cond, uncond, cmask, umask, 5.0, 1.0, 12)
     sampler = StaticARSampler(policy, graph=False, fused_tail=False)
@@ -104,7 +116,7 @@ def test_static_cache_loop_samples_what_the_reference_loop_samples():
     assert len(want_t.unique()) > 6   # the draw is not degenerate
 
     # a second call reuses the buffers (other prompts, other length inside the same bucket, other seed)
-    cond2, uncond2, cmask2, umask2 = make_inputs(3, 9, torch.float32, "cpu", seed=4)
+    cond2, uncond2, cmask2, umask2 = make_inputs(3, 9, torch.float32, "cpu", seed=4, side=side)
     torch.manual_seed(12)
     want_t2, want_lp2 = reference_loop(policy, cond2, uncond2, cmask2, umask2, 5.0, 1.0, 10)
     torch.manual_seed(12)
@@ -298,13 +310,14 @@ def test_graph_replays_equal_eager_steps(int4_policy, native):
 
 
 @pytest.mark.gpu
-def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy):
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy, side):
     """Same int4 policy through the reference loop (dynamic cache, torch formulas for the tail):
     same tokens under the same seed; log-probabilities within a bf16 rounding of the log-softmax.
     The trunk stays the module here (``native=False``): the native trunk agrees with it to bf16
     roundings only, which the tests below bound."""
     print("ar decode: static fused vs reference loop", flush=True)
-    cond, uncond, cmask, umask = make_inputs(3, 7, torch.bfloat16, "cuda:0")
+    cond, uncond, cmask, umask = make_inputs(3, 7, torch.bfloat16, "cuda:0", side=side)
     torch.manual_seed(31)
     want_t, want_lp = reference_loop(int4_policy, cond, uncond, cmask, umask, 5.0, 1.0, 16)
     for graph in (False, True):
@@ -317,12 +330,13 @@ def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy):
 
 
 @pytest.mark.gpu
-def test_native_trunk_tracks_the_module_trunk(int4_policy):
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_native_trunk_tracks_the_module_trunk(int4_policy, side):
     """Teacher-forced: both trunks consume the same inputs step after step, each over its own cache;
     hidden states and appended cache rows stay within bf16 roundings of each other."""
     print("ar decode: native trunk vs module trunk", flush=True)
     rows, n_text, steps = 6, 7, 12
-    cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=41)
+    cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=41, side=side)
     sessions = []
     for native in (True, False):
         sampler = StaticARSampler(int4_policy, graph=False, native=native)

@@ -407,3 +407,98 @@ def test_gradient_reaches_the_input_of_a_quantised_layer():
         assert torch.equal(x.grad, ref.grad)
         with torch.no_grad():
             assert not q(x).requires_grad and not gu(x).requires_grad
+
+
+def test_a_prepacked_copy_knows_when_its_source_changed():
+    """The canonical buffers are the module's state; the prepacked copy is derived from them and is
+    stale after an in-place write (``load_state_dict``), a replaced buffer (``.to()``) or when torch
+    keeps no modification counter for a buffer (inference tensors cannot be told apart)."""
+    from visionrl_amd.linear import _source_changed, _source_state
+
+    a, b = torch.zeros(4), torch.ones(4)
+    state = _source_state(a, b)
+    assert not _source_changed(state, a, b)
+    b.add_(1)
+    assert _source_changed(state, a, b)
+    state = _source_state(a, b)
+    assert _source_changed(state, a.clone(), b)
+    with torch.inference_mode():
+        c = torch.zeros(4)
+    assert _source_changed(_source_state(c), c)
+    mod = Int4Linear(128, 16, 128)
+    assert not mod.packed_is_stale()                 # nothing prepacked
+    mod._packed, mod._packed_from = object(), _source_state(mod.qweight, mod.scales, mod.qzeros)
+    assert not mod.packed_is_stale()
+    mod.load_state_dict({k: v.clone() + 1 for k, v in mod.state_dict().items()})
+    assert mod.packed_is_stale()
+    assert mod._fresh_packed() is None               # made again: on the CPU there is no prepacked form
+
+
+@pytest.mark.gpu
+def test_hand_over_is_void_once_the_input_was_written_or_the_leader_ran_again():
+    """A persistent input buffer rewritten in place between q_proj(x) and k_proj(x), and a k_proj call
+    that follows a step in which it was skipped: the sibling computes from what x holds now."""
+    dev = "cuda:0"
+    torch.manual_seed(8)
+    mods = [Int4Linear.from_linear(nn.Linear(512, n, bias=False).to(torch.bfloat16).to(dev), 128).prepack_()
+            for n in (128, 96, 64)]
+    alone = [Int4Linear.from_packed(m.qweight, m.scales, m.qzeros, 128).prepack_() for m in mods]
+    q, k, v = mods
+    q.group_with(k, v)
+    x = torch.randn(2, 1, 512, device=dev).to(torch.bfloat16)
+    first = [m(x) for m in alone]
+    q(x)
+    assert k._handed is not None
+    x.mul_(-3)                                           # the same tensor object, other contents
+    now = [m(x) for m in alone]
+    assert torch.equal(k(x), now[1]) and not torch.equal(now[1], first[1])
+    assert torch.equal(v(x), now[2])
+    # step 1 hands over, k is skipped; step 2 reuses the buffer: the leader's new call voids the old results
+    q(x)
+    x.copy_(torch.randn_like(x))
+    assert torch.equal(q(x), alone[0](x)) and torch.equal(k(x), alone[1](x)) and torch.equal(v(x), alone[2](x))
+    # a leader call that takes another route (too many rows for the grouped launch) leaves nothing behind
+    q(x)
+    big = torch.randn(40, 512, device=dev).to(torch.bfloat16)
+    q(big)
+    assert k._handed is None and v._handed is None
+    # inputs without a modification counter are never handed over
+    with torch.inference_mode():
+        xi = torch.randn(2, 512, device=dev).to(torch.bfloat16)
+        yq = q(xi)
+        assert k._handed is None and torch.equal(yq, alone[0](xi)) and torch.equal(k(xi), alone[1](xi))
+
+
+@pytest.mark.gpu
+def test_loading_a_state_dict_into_a_prepacked_module_refreshes_the_decode_path():
+    """Decode-sized calls stream the prepacked copy, prompt-sized ones and dequantize() the canonical
+    buffers: after ``load_state_dict`` both must follow the new weights."""
+    dev = "cuda:0"
+    torch.manual_seed(9)
+    old = Int4Linear.from_linear(nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev), 128).prepack_()
+    new = Int4Linear.from_linear(nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev), 128).prepack_()
+    x = torch.randn(3, 512, device=dev).to(torch.bfloat16)
+    before, want = old(x), new(x)
+    assert not torch.equal(before, want)
+    blob = old._packed
+    old.load_state_dict(new.state_dict())
+    assert old.packed_is_stale()
+    assert torch.equal(old(x), want) and old._packed is not blob and not old.packed_is_stale()
+    gu_old = Int4GateUpSiLU(Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128),
+                            Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128)).prepack_()
+    gu_new = Int4GateUpSiLU(Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128),
+                            Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128)).prepack_()
+    want = gu_new(x)
+    gu_old.load_state_dict(gu_new.state_dict())
+    assert torch.equal(gu_old(x), want)
+    # a grouped leader notices a stale sibling and a refreshed sibling rebuilds the group's launch
+    q = Int4Linear.from_linear(nn.Linear(512, 128, bias=False).to(torch.bfloat16).to(dev), 128).prepack_()
+    q.group_with(old)
+    old.load_state_dict(Int4Linear.from_linear(nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev), 128).state_dict())
+    fresh = Int4Linear.from_packed(old.qweight, old.scales, old.qzeros, 128).prepack_()
+    x3 = x.reshape(1, 3, 512)
+    q(x3)
+    assert old._handed is None                           # the sibling's copy was stale: no hand-over
+    assert torch.equal(old(x3), fresh(x3))
+    q(x3)
+    assert old._handed is not None and torch.equal(old(x3), fresh(x3))

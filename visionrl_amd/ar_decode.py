@@ -38,6 +38,7 @@ from __future__ import annotations
 
 import dataclasses
 import types
+import weakref
 from typing import Any
 
 import torch
@@ -80,13 +81,29 @@ class StaticARState:
     reference: Any = None          # the policy's own (init_ar_state, step_ar, finalize_ar_state), if it has them
     delegate: Any = None           # their state, once a partial batch sent the generation their way
 
+    released: bool = False         # finalized: the session's buffers may serve another generation
+    final: Any = None              # (token ids, log-probabilities) as finalize_ar_state returned them
+
+    @property
+    def finished(self) -> bool:
+        return self.position >= self.image_token_num
+
     @property
     def token_ids(self) -> torch.Tensor:
-        return self.session.tokens[:, :self.image_token_num]
+        """Tokens sampled so far (columns from ``position`` on are not yet written).  A view of the
+        session's buffer while the generation runs, a copy once it has finished: the buffer is
+        rewritten by the next generation of this shape."""
+        if self.released:
+            return self.final[0]
+        view = self.session.tokens[:, :self.image_token_num]
+        return view.clone() if self.finished else view
 
     @property
     def logprobs(self) -> torch.Tensor:
-        return self.session.logprobs[:, :self.image_token_num]
+        if self.released:
+            return self.final[1]
+        view = self.session.logprobs[:, :self.image_token_num]
+        return view.clone() if self.finished else view
 
 
 class _Session:
@@ -111,6 +128,7 @@ class _Session:
         self.slot = torch.zeros(1, dtype=torch.long, device=device)   # cache slot of the next new token
         self.native = None     # NativeDecodeTrunk once the cache exists, False if the trunk does not qualify
         self.graph = None
+        self.owner = None      # weak reference to the state whose generation the buffers hold
         self.signature = None  # of the trunk's modules and adapter state the launch list / graph were made for
 
     # -- one call of sample_image_tokens starts here
@@ -215,7 +233,15 @@ class StaticARSampler:
         return float(cfg), float(temp), int(n_img)
 
     def _session(self, key, make):
+        """The cached session of this shape if no live generation holds it, else a new one (which
+        takes its place in the cache; the busy one stays with its state until that is finalized or
+        dropped).  The reference's states are independent objects (``policy.py:114-130``); here two
+        states of one shape must not share cache, token and log-probability buffers."""
         sess = self._sessions.pop(key, None)
+        if sess is not None and sess.owner is not None:
+            holder = sess.owner()
+            if holder is not None and not holder.released:
+                sess = None
         if sess is None:
             while len(self._sessions) >= self.max_sessions:   # oldest first: caches are GBs at 1B scale
                 self._sessions.pop(next(iter(self._sessions)))
@@ -241,13 +267,17 @@ class StaticARSampler:
         key = (2 * B, hidden, max_len, dtype, device, cfg, temp, cond_attention_mask.dtype)
         sess = self._session(key, lambda: _Session(self, 2 * B, hidden, max_len, dtype, device, cfg, temp,
                                                    cond_attention_mask.dtype))
-        return StaticARState(session=sess, inputs=(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
-                                                   uncond_attention_mask),
-                             cfg_weight=cfg, temperature=temp, image_token_num=n_img, batch_size=B)
+        state = StaticARState(session=sess, inputs=(cond_inputs_embeds, uncond_inputs_embeds, cond_attention_mask,
+                                                    uncond_attention_mask),
+                              cfg_weight=cfg, temperature=temp, image_token_num=n_img, batch_size=B)
+        sess.owner = weakref.ref(state)
+        return state
 
     def _advance(self, state: "StaticARState") -> None:
         """One token for every row: the prompt pass first, then eager / recorded decode steps."""
         sess = state.session
+        if state.released:
+            raise ValueError("the state was finalized")
         if state.position >= state.image_token_num:
             raise ValueError("the generation has already finished sampling")
         if state.position == 0:
@@ -309,8 +339,12 @@ class StaticARSampler:
         """``(image_token_ids, logprobs)`` of the rows sampled so far up to ``image_token_num``."""
         if state.delegate is not None:
             return state.reference[2](state.delegate)
+        if state.released:
+            raise ValueError("the state was finalized before")
         n = state.image_token_num
-        return state.session.tokens[:, :n].clone(), state.session.logprobs[:, :n].clone()
+        out = state.session.tokens[:, :n].clone(), state.session.logprobs[:, :n].clone()
+        state.final, state.released = out, True    # the session may serve the next generation of this shape
+        return out
 
     @torch.no_grad()
     def sample_image_tokens(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,

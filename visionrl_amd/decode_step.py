@@ -112,8 +112,21 @@ def trunk_signature(trunk) -> tuple:
                 scaling = getattr(mod, "scaling", None)
                 scaling = tuple(sorted(scaling.items())) if hasattr(scaling, "items") else scaling
                 sig.append((id(mod), bool(getattr(mod, "merged", False)),
-                            bool(getattr(mod, "disable_adapters", False)), active, scaling))
+                            bool(getattr(mod, "disable_adapters", False)), active, scaling, _packed_ids(mod)))
     return tuple(sig)
+
+
+def _packed_ids(mod) -> tuple:
+    """The prepacked copies a projection (or fused MLP) streams from, made again first where the canonical
+    buffers changed since (``load_state_dict`` into a prepacked module): a launch list holds blob
+    addresses, so a new copy is a new signature."""
+    inner = getattr(mod, "base_layer", mod)
+    parts = (inner.gate_up, inner.down_proj) if isinstance(inner, Int4LlamaMLP) else (inner,)
+    out = []
+    for part in parts:
+        fresh = getattr(part, "_fresh_packed", None)
+        out.append(id(fresh()) if fresh is not None else None)
+    return tuple(out)
 
 
 class NativeDecodeTrunk:

@@ -12,6 +12,8 @@ the dequantised weight through the library GEMM, so the gradient reaches the inp
 
 from __future__ import annotations
 
+import weakref
+
 import torch
 import torch.nn.functional as F
 from torch import nn
@@ -27,6 +29,23 @@ GEMM_ROWS = 32
 def _wants_grad(x: torch.Tensor) -> bool:
     """The HIP launches are not recorded by autograd: such calls take the dequant + GEMM route."""
     return torch.is_grad_enabled() and x.requires_grad
+
+
+def _version(t: torch.Tensor):
+    """The tensor's in-place modification counter, or ``None`` where torch keeps none (inference tensors)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
+def _source_state(*tensors):
+    """Identity and modification counters of the tensors a prepacked copy was made from."""
+    return tuple((t, _version(t)) for t in tensors)
+
+
+def _source_changed(state, *tensors) -> bool:
+    return any(t is not t0 or v0 is None or _version(t) != v0 for t, (t0, v0) in zip(tensors, state))
 
 
 def _rows(x: torch.Tensor, in_features: int) -> torch.Tensor:
@@ -96,12 +115,34 @@ class Int4Linear(nn.Module):
         if self.qweight.is_cuda and ops.PrepackedWeight.supported(self.out_features, self.in_features,
                                                                   self.group_size):
             self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
+            self._packed_from = _source_state(self.qweight, self.scales, self.qzeros)
             self._direct_rows = self._packed.direct_rows()
             self._call = ops.DirectCall([self._packed])
         group = getattr(self, "_group", None)
         if group is not None:  # rebuild the group's launch over the new copies
             self.group_with(*group[1:])
+        leader = getattr(self, "_leader", None)
+        leader = leader() if leader is not None else None   # the module whose launch computes this one's output too
+        if leader is not None and leader is not self and getattr(leader, "_group", None) is not None:
+            leader.group_with(*leader._group[1:])
         return self
+
+    def packed_is_stale(self) -> bool:
+        """True when the canonical buffers were written (``load_state_dict``, an in-place edit) or
+        replaced (``.to()``) after :meth:`prepack_` copied them."""
+        return getattr(self, "_packed", None) is not None and \
+            _source_changed(self._packed_from, self.qweight, self.scales, self.qzeros)
+
+    def _fresh_packed(self):
+        """The prepacked copy, made again first if the canonical buffers changed under it."""
+        packed = getattr(self, "_packed", None)
+        if packed is not None and _source_changed(self._packed_from, self.qweight, self.scales, self.qzeros):
+            if self.qweight.is_cuda and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("the int4 weight changed after prepack_(): call prepack_() again before "
+                                   "recording a graph over this module")
+            self.prepack_()
+            packed = self._packed
+        return packed
 
     def group_with(self, *others: "Int4Linear") -> "Int4Linear":
         """Launch ``others`` together with this module whenever it is called (q|k|v of one layer).
@@ -118,6 +159,8 @@ class Int4Linear(nn.Module):
         if any(o.in_features != self.in_features for o in others):
             raise ValueError("grouped modules take the same input")
         self._group = (self, *others)
+        for m in others:
+            m._leader = weakref.ref(self)
         self._group_call = None
         if all(getattr(m, "_packed", None) is not None for m in self._group):
             self._group_call = ops.DirectCall([m._packed for m in self._group])
@@ -132,21 +175,28 @@ class Int4Linear(nn.Module):
         handed = getattr(self, "_handed", None)
         if handed is not None:
             self._handed = None
+        group = getattr(self, "_group", None)
+        if group is not None:   # a new call of the leader: whatever it handed over before is void
+            for m in group[1:]:
+                m._handed = None
         if torch.compiler.is_compiling():
             y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         elif _wants_grad(x):
             y = F.linear(rows, self.dequantize())
-        elif handed is not None and handed[0] is x:  # computed by the group leader's launch
-            y = handed[1]
+        elif handed is not None and handed[0] is x and handed[1] == _version(x):
+            y = handed[2]   # computed by the group leader's launch from this very tensor, unchanged since
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
-            packed = getattr(self, "_packed", None)
+            packed = self._fresh_packed()
             M = rows.shape[0]
             if packed is not None and packed.blob.device == rows.device:
                 call = getattr(self, "_group_call", None)
-                if call is not None and M <= call.max_rows:
+                version = _version(x) if call is not None else None
+                if call is not None and M <= call.max_rows and version is not None and \
+                        not any(m.packed_is_stale() for m in group[1:]):
+                    # (an input without a modification counter cannot be recognised later: no hand-over)
                     ys = call(rows)
-                    for m, ym in zip(self._group[1:], ys[1:]):
-                        m._handed = (x, ym)
+                    for m, ym in zip(group[1:], ys[1:]):
+                        m._handed = (x, version, ym)
                     y = ys[0]
                 elif M <= self._direct_rows:
                     y = self._call(rows)[0]
@@ -192,13 +242,17 @@ class Int4GateUpSiLU(nn.Module):
         if self.qweight.is_cuda and self.intermediate_size % 16 == 0 and \
                 ops.PrepackedWeight.supported(2 * self.intermediate_size, self.in_features, self.group_size):
             self._packed = ops.int4_prepack(self.qweight, self.scales, self.qzeros, self.group_size)
+            self._packed_from = _source_state(self.qweight, self.scales, self.qzeros)
             self._direct_rows = self._packed.direct_rows(fused=True)
             self._call = ops.DirectCall([self._packed], fused=True)
         return self
 
+    packed_is_stale = Int4Linear.packed_is_stale
+    _fresh_packed = Int4Linear._fresh_packed
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
-        packed = getattr(self, "_packed", None)
+        packed = None if torch.compiler.is_compiling() else self._fresh_packed()
         grad = _wants_grad(x) and not torch.compiler.is_compiling()
         if packed is not None and not grad and not torch.compiler.is_compiling() \
                 and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
