@@ -29,6 +29,8 @@ SYMBOLS = (
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
     "vrl_cfg_sample_bf16",
+    "vrl_int4_head_sample_workspace_bytes",
+    "vrl_int4_head_sample_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
     "vrl_rope_attn_decode_lora_bf16",
@@ -157,6 +159,11 @@ def _bind(lib):
     lib.vrl_int4_gemv_grouped_bf16.argtypes = [vp, ctypes.POINTER(PlanInfo), vp]
     lib.vrl_cfg_sample_bf16.restype = ci
     lib.vrl_cfg_sample_bf16.argtypes = [vp, vp, vp, vp, ci, ci, ctypes.c_float, ctypes.c_float, vp]
+    lib.vrl_int4_head_sample_workspace_bytes.restype = ctypes.c_size_t
+    lib.vrl_int4_head_sample_workspace_bytes.argtypes = [ci, ci]
+    lib.vrl_int4_head_sample_bf16.restype = ci
+    lib.vrl_int4_head_sample_bf16.argtypes = [ctypes.POINTER(Problem), vp, vp, vp, ci, ctypes.c_float,
+                                              ctypes.c_float, vp, ctypes.c_size_t, vp]
     lib.vrl_add_rmsnorm_bf16.restype = ci
     lib.vrl_add_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_float, vp]
     lib.vrl_rope_attn_decode_lora_bf16.restype = ci

@@ -46,6 +46,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .decode_step import NativeDecodeTrunk, trunk_signature
+from .linear import Int4Linear
 
 __all__ = ["StaticARSampler", "StaticARState", "StaticARStepResult", "install_static_ar_sampler"]
 
@@ -129,11 +130,20 @@ class _Session:
         self.native = None     # NativeDecodeTrunk once the cache exists, False if the trunk does not qualify
         self.graph = None
         self.owner = None      # weak reference to the state whose generation the buffers hold
+        self.head_workspace = None   # of the fused head + tail launch
         self.signature = None  # of the trunk's modules and adapter state the launch list / graph were made for
+
+    def _head_packed(self):
+        """The prepacked weight of a bare, bias-free int4 ``gen_head`` (made again first if its canonical
+        buffers changed), else ``None``."""
+        head = getattr(self.sampler.base, "gen_head", None)
+        if isinstance(head, Int4Linear) and head.bias is None:
+            return head._fresh_packed()
+        return None
 
     # -- one call of sample_image_tokens starts here
     def begin(self, mask: torch.Tensor) -> None:
-        signature = trunk_signature(self.sampler.trunk)
+        signature = (trunk_signature(self.sampler.trunk), id(self._head_packed()))
         if signature != self.signature:   # modules swapped, adapters merged / disabled / switched: start over
             self.signature, self.native, self.graph = signature, None, None
         self.cache.reset()
@@ -146,8 +156,20 @@ class _Session:
     def tail(self, hidden: torch.Tensor) -> None:
         """Head, guided draw, log-probability, bookkeeping, next input (``policy.py:684-700``)."""
         s = self.sampler
-        logits = s.base.gen_head(hidden).squeeze(1)
-        if s.fused_tail and logits.dtype == torch.bfloat16 and logits.is_cuda:
+        packed = self._head_packed() if s.fused_tail and s.fused_head else None
+        if packed is not None and hidden.dtype == torch.bfloat16 and hidden.is_cuda and \
+                ops.head_sample_supported(self.rows2, packed):
+            # head and tail in one launch: the logits never reach memory
+            if self.head_workspace is None:
+                self.head_workspace = ops.head_sample_workspace(self.rows2 // 2, packed.N, hidden.device)
+            sampled, lp = ops.head_sample(hidden.reshape(self.rows2, -1), packed, self.cfg_weight, self.temperature,
+                                          workspace=self.head_workspace)
+            logits = None
+        else:
+            logits = s.base.gen_head(hidden).squeeze(1)
+        if logits is None:
+            pass
+        elif s.fused_tail and logits.dtype == torch.bfloat16 and logits.is_cuda:
             sampled, lp = ops.cfg_sample(logits.contiguous(), self.cfg_weight, self.temperature)
         else:
             cond, uncond = logits.chunk(2, dim=0)
@@ -200,14 +222,16 @@ class StaticARSampler:
     ``prepare_gen_img_embeds`` (``policy.py:226-238``), ``config`` the defaults
     (``cfg_weight``, ``temperature``, ``image_token_num``).  ``graph=False`` runs every step
     eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
-    for the part after the head.  With ``native`` (the default) the trunk of a decode step runs as
+    for the part after the head; ``fused_head=False`` keeps the head a launch of its own in front of
+    the fused tail (with it, a prepacked int4 ``gen_head`` and the tail are one launch and the logits
+    are never written).  With ``native`` (the default) the trunk of a decode step runs as
     :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (five launches per layer, six with LoRA
     adapters on the attention projections) when the policy went through ``apply_int4_to_policy``
     with its defaults; otherwise, and for the prompt pass, the trunk module itself is called.
     """
 
     def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True, native: bool = True,
-                 length_bucket: int = 64, max_sessions: int = 2):
+                 fused_head: bool = True, length_bucket: int = 64, max_sessions: int = 2):
         self.policy = policy
         self.trunk = policy._lm_trunk()
         self.base = policy._base()
@@ -216,6 +240,7 @@ class StaticARSampler:
                 raise TypeError(f"policy._base() has no {name}")
         self.graph = bool(graph)
         self.fused_tail = bool(fused_tail)
+        self.fused_head = bool(fused_head)
         self.native = bool(native)
         self.length_bucket = int(length_bucket)
         self.max_sessions = int(max_sessions)

@@ -21,7 +21,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_NAME = "libvrl_int4.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
 BENCH_LIB_PATH = os.path.join(CSRC, "libvrl_bench.so")
-SOURCES = ["int4_gemv.hip", "cfg_sample.hip", "decode_layer.hip"]
+SOURCES = ["int4_gemv.hip", "cfg_sample.hip", "decode_layer.hip", "head_sample.hip"]
 BENCH_SOURCES = ["bench_kernels.hip"]
 
 HIPCC_FLAGS = [

@@ -60,6 +60,7 @@ int vrl_bench_stream_read(const void *buf, size_t bytes, void *sink, int waves_p
     const uint32_t waves = (uint32_t)cus * (uint32_t)waves_per_cu / 4u * 4u;
     uint64_t per_wave = (bytes + waves - 1) / waves;
     per_wave = (per_wave + 4095) / 4096 * 4096;
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(stream_read_kernel<4>, dim3(waves / 4), dim3(4 * WAVE), 0,
                        reinterpret_cast<hipStream_t>(hip_stream), buf, (uint32_t)bytes, (uint32_t)per_wave,
                        static_cast<uint32_t *>(sink));

@@ -517,12 +517,14 @@ __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__
 
 template <bool FP32, int MB>
 void launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_t stream) {
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL((lora_down_kernel<FP32, MB>), dim3(a.off[a.n], (a.M + MB - 1) / MB), dim3(THREADS), 0, stream,
                        x, a, t);
 }
 
 template <bool FP32, int RB>
 void launch_lora_up(const float *t, int parts, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>),
                        dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n, (a.M + UP_ROWS - 1) / UP_ROWS),
                        dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, parts, a);
@@ -547,6 +549,7 @@ extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const v
     auto ws = static_cast<const uint16_t *>(weight);
     auto hs = static_cast<uint16_t *>(h_out);
     auto ys = static_cast<uint16_t *>(y);
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     if (residual)
         hipLaunchKernelGGL(add_rmsnorm_kernel<true>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
     else

@@ -168,6 +168,7 @@ int launch_tile(const DevProblem &p, hipStream_t stream) {
     const int cols_per_tile = p.fused ? 16 * (R / 2) : 16 * R;
     const int tiles = (out_cols + cols_per_tile - 1) / cols_per_tile;
     const size_t smem = tile_smem_bytes<R, MB>(p.M, p.kc);
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL((gemv_tile_kernel<R, MB, TILE_WPB>), dim3(tiles), dim3(TILE_WPB * WAVE), smem,
                        stream, p);
     return (int)hipGetLastError();
@@ -178,6 +179,7 @@ int launch_problem(DevProblem p, hipStream_t stream) {
     if (!tile_path_ok(p)) {
         // the generic kernel walks activation rows itself, any M
         const int waves = 4;
+        (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
         hipLaunchKernelGGL(gemv_generic_kernel, dim3((out_cols + waves - 1) / waves),
                            dim3(waves * WAVE), 0, stream, p);
         return (int)hipGetLastError();
@@ -238,9 +240,18 @@ int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *
                   hipStream_t stream) {
     auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ>;
     if (info->lds_bytes > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, info->lds_bytes);
-        if (e != hipSuccess) return (int)e;
+        // once per instantiation and device (the attribute belongs to the function on that device), at the
+        // largest size a plan may ask for: no runtime call in a timed or captured launch after the first
+        static std::atomic<uint64_t> raised{0};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(raised.load(std::memory_order_relaxed) & bit)) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_PER_CU);
+            if (e != hipSuccess) return (int)e;
+            raised.fetch_or(bit, std::memory_order_relaxed);
+        }
     }
     if (!recs) {
         int per_cu = 0;
@@ -250,6 +261,7 @@ int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *
         info->grid = per_cu;
         return VRL_INT4_OK;
     }
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes,
                        stream, recs, block_begin, info->n_problems);
     return (int)hipGetLastError();
@@ -310,6 +322,7 @@ int launch_split(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *b
         info->grid = per_cu;
         return VRL_INT4_OK;
     }
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes, stream, recs,
                        block_tab, info->n_problems);
     return (int)hipGetLastError();
@@ -338,6 +351,7 @@ int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_
             raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
     return (int)hipGetLastError();
 }
@@ -445,6 +459,7 @@ int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *q
     long blocks = (total + 255) / 256;
     const long cap = (long)device_cu_count() * 32;
     if (blocks > cap) blocks = cap;
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
@@ -466,6 +481,7 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     long blocks = (total + 255) / 256;
     const long cap = (long)device_cu_count() * 32;
     if (blocks > cap) blocks = cap;
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
     hipLaunchKernelGGL(prepack_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),

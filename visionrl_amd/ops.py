@@ -25,7 +25,8 @@ from .int4_format import check_packed
 
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
-           "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "add_rmsnorm",
+           "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "head_sample", "head_sample_supported",
+           "head_sample_workspace", "add_rmsnorm",
            "rope_attn_decode", "LoraAdd"]
 
 
@@ -489,6 +490,77 @@ def cfg_sample(logits: torch.Tensor, cfg_weight: float, temperature: float, *,
                                              logprob.data_ptr(), B, V, float(cfg_weight), float(temperature),
                                              _stream_handle(dev))
     _lib.check(rc, "vrl_cfg_sample_bf16")
+    return sampled, logprob
+
+
+def head_sample_supported(rows: int, head: PrepackedWeight) -> bool:
+    """Whether :func:`head_sample` takes ``rows = 2B`` activation rows for this head: the library's own
+    rule (B <= 16, V a multiple of 16 up to 65536, the rows fit a workgroup's LDS beside the partial tiles)."""
+    if rows < 2 or rows % 2 or rows > 32 or head.N < 16 or head.N > 65536 or head.N % 16:
+        return False
+    nsc = (head.K + 511) // 512
+    if nsc > 16:
+        return False
+    ks = 16 if nsc > 8 else (8 if nsc > 4 else 4)
+    tw = 16 // ks if rows >= 8 else 1
+    lds = rows * (nsc * 512 + 8) * 2 + tw * (ks - 1) * (2 if rows > 16 else 1) * 64 * 16
+    return lds <= 160 * 1024 - 64
+
+
+def head_sample_workspace(B: int, V: int, device) -> torch.Tensor:
+    """A zeroed workspace for :func:`head_sample` at batch ``B`` and vocabulary ``V`` (reusable by
+    calls that do not overlap in time)."""
+    nbytes = _lib.load().vrl_int4_head_sample_workspace_bytes(int(B), int(V))
+    if nbytes == 0:
+        raise ValueError(f"head_sample takes 1 <= B <= 16 and V a multiple of 16 up to 65536, got B={B}, V={V}")
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device)
+
+
+def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, temperature: float, *,
+                generator: torch.Generator | None = None, noise: torch.Tensor | None = None,
+                logits_out: torch.Tensor | None = None, workspace: torch.Tensor | None = None):
+    """The image-token head and the sampling tail of a decode step in one launch.
+
+    Stands for ``vrl/models/families/janus_pro/policy.py:684-693``: ``x`` is the bf16 ``[2B, K]``
+    last hidden state (conditional rows first), ``head`` the prepacked ``gen_head`` weight
+    ``[V, K]``; returns ``(sampled int64 [B], logprob float32 [B])`` like :func:`cfg_sample` over the
+    head's logits, which are written to ``logits_out`` (bf16 ``[2B, V]``) only if that is given.
+    The draw consumes the random stream as ``torch.multinomial(probs, 1)`` does; ``workspace`` is a
+    tensor from :func:`head_sample_workspace` (made per call if omitted: pass one in a decode loop).
+    Raises ``ValueError`` for shapes the launch does not take (:func:`head_sample_supported`).
+    """
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[0] % 2 != 0 or x.shape[0] < 2 or x.shape[1] != head.K:
+        raise ValueError(f"x must be bfloat16 [2B, {head.K}]: conditional rows, then unconditional rows")
+    if not temperature > 0:
+        raise ValueError("temperature must be positive")
+    dev = _require_device("x", x)
+    _require_device("prepacked blob", head.blob, dev)
+    B, V = x.shape[0] // 2, head.N
+    if not head_sample_supported(x.shape[0], head):
+        raise ValueError(f"head_sample does not take {x.shape[0]} rows of K={head.K} for a head of {V} entries")
+    if noise is None:
+        noise = torch.empty((B, V), dtype=torch.bfloat16, device=dev).exponential_(1.0, generator=generator)
+    elif noise.dtype != torch.bfloat16 or tuple(noise.shape) != (B, V):
+        raise ValueError(f"noise must be bfloat16 [{B}, {V}]")
+    _require_device("noise", noise, dev)
+    if logits_out is not None:
+        if logits_out.dtype != torch.bfloat16 or tuple(logits_out.shape) != (2 * B, V):
+            raise ValueError(f"logits_out must be bfloat16 [{2 * B}, {V}]")
+        _require_device("logits_out", logits_out, dev)
+    if workspace is None:
+        workspace = head_sample_workspace(B, V, dev)
+    elif workspace.dtype != torch.uint8 or workspace.device != dev or not workspace.is_contiguous():
+        raise ValueError("workspace must be a contiguous uint8 tensor on the device of x")
+    sampled = torch.empty(B, dtype=torch.int64, device=dev)
+    logprob = torch.empty(B, dtype=torch.float32, device=dev)
+    rec = _lib.Problem()
+    rec.x, rec.qweight, rec.y = x.data_ptr(), head.blob.data_ptr(), (logits_out.data_ptr() if logits_out is not None else None)
+    rec.M, rec.N, rec.K, rec.G, rec.prepacked = 2 * B, V, head.K, head.group_size, 1
+    with _on(dev):
+        rc = _lib.load().vrl_int4_head_sample_bf16(ctypes.byref(rec), noise.data_ptr(), sampled.data_ptr(),
+                                                   logprob.data_ptr(), B, float(cfg_weight), float(temperature),
+                                                   workspace.data_ptr(), workspace.numel(), _stream_handle(dev))
+    _lib.check(rc, "vrl_int4_head_sample_bf16")
     return sampled, logprob
 
 
