@@ -206,13 +206,12 @@ int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_t *sampled,
  *   guided, probs, sampled, logprob                  as vrl_cfg_sample_bf16 states them
  * `head` is one prepacked problem: x bf16 [2B, K] (M = 2B), qweight the blob of the [V, K] head,
  * y NULL (the logits are not wanted: they never reach memory) or bf16 [2B, V]; noise bf16 [B, V];
- * sampled int64 [B]; logprob float [B].  The tiles of the head leave per-tile softmax partials, the
- * scaled rows and a mask of the entries that can still win the draw in `workspace`; the workgroup that
- * finishes last completes the rows, with the arithmetic of vrl_cfg_sample_bf16 (the softmax sums are
- * added up in another, fixed order).
+ * sampled int64 [B]; logprob float [B].  Two kernels are enqueued: the tiles of the head leave
+ * per-tile softmax partials, the scaled rows and a mask of the entries that can still win the draw in
+ * `workspace`; a small second kernel (one workgroup per batch row) completes the rows from them, with
+ * the arithmetic of vrl_cfg_sample_bf16 (the softmax sums are added up in another, fixed order).
  * workspace: device memory of at least vrl_int4_head_sample_workspace_bytes(B, V) bytes, 256-byte
- * aligned, whose first 256 bytes are zero before the first call; a call leaves them zero again.  Two
- * calls that overlap in time must not share a workspace.
+ * aligned, contents irrelevant on entry.  Two calls that overlap in time must not share a workspace.
  * Preconditions beyond the library's: 1 <= B <= 16, 16 <= V <= 65536 with V % 16 == 0, temperature > 0,
  * G in {32, 64, 128}, and the 2B activation rows fit the LDS of a workgroup beside the kernel's partial
  * tiles (for example K = 2048 at up to 32 rows, K = 4096 at up to 16, K = 8192 at up to 8): else

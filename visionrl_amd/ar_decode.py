@@ -162,7 +162,7 @@ class _Session:
             # head and tail in one launch: the logits never reach memory
             if self.head_workspace is None:
                 self.head_workspace = ops.head_sample_workspace(self.rows2 // 2, packed.N, hidden.device)
-            sampled, lp = ops.head_sample(hidden.reshape(self.rows2, -1), packed, self.cfg_weight, self.temperature,
+            sampled, lp = ops.head_sample(hidden.reshape(self.rows2, -1).contiguous(), packed, self.cfg_weight, self.temperature,
                                           workspace=self.head_workspace)
             logits = None
         else:

@@ -13,17 +13,21 @@
 // Every workgroup computes 16-column tiles of the head exactly as the plan-free launch of prepacked.hpp
 // does (waves split K of a tile, partial tiles meet in LDS).  The wave that holds a finished tile rounds
 // the logits to bf16, forms guided / T and cond / T for its B x 16 entries and leaves in a workspace:
-//   gt, ct   [B, V] bf16    the two scaled rows (read back only where a draw can win)
-//   part     [B, tiles]     {max, sum exp(. - max)} of the tile's 16 entries, for both rows
-//   mask     [B, tiles]     which of the 16 entries can still win the draw: those whose
-//                           exp(gt - tile max) / q lies within 2^-5 of the tile's largest.  The final
-//                           ratio bf16(bf16(exp(gt - max) / sum) / q) is that quantity times one
-//                           factor per row, through two monotone roundings of relative size 2^-8 each,
-//                           so an entry further below its tile's best than that can neither win nor tie.
-// The last workgroup to finish (a counter in the workspace) then takes one wave per batch row: the row's
-// maxima and sums from the tile partials in a fixed order, the ratio of every marked entry with exactly
-// the arithmetic of cfg_sample.hip, the lowest index among equal maxima, and the log-probability.
-// No workgroup waits for another: the last one is whichever increments the counter last.
+//   gt, ct   [B, V] bf16    the two scaled rows (read back only for the rare second candidates of a tile)
+//   rec      [B, tiles]     32 bytes per tile: {max, sum exp(. - max)} of the tile's 16 entries for both
+//                           rows; the entry with the tile's largest exp(gt - tile max) / q (its gt, q, ct
+//                           and column), which is the tile's first candidate for the draw; and a mask of
+//                           the entries within 2^-5 of that largest.  The final ratio
+//                           bf16(bf16(exp(gt - max) / sum) / q) is that quantity times one factor per
+//                           row, through two monotone roundings of relative size 2^-8 each, so an entry
+//                           further below its tile's best than that can neither win nor tie.
+// A second, small launch of the same call (one workgroup per batch row, a thread per tile) then finishes
+// the rows: the row's maxima and sums from the tile partials in a fixed order, the ratio of the marked
+// entries with exactly the arithmetic of cfg_sample.hip, the lowest index among equal maxima, and the
+// log-probability.  (Finishing the rows inside the first launch, by whichever workgroup counts itself
+// last, was built and measured: the device-wide visibility it needs within one launch - a release
+// fence per workgroup, or written-through stores and uncached reads - and the registers the last
+// workgroup's part adds to every wave cost more than the second launch's 2 us.)
 
 #include <atomic>
 
@@ -36,9 +40,8 @@ struct HeadArgs {
     const uint16_t *noise;   // [B, V] bf16, strictly positive
     long long *sampled;      // [B]
     float *logprob;          // [B]
-    uint32_t *counter;       // zero between launches
-    f32x4_t *part;           // [B, tiles]: {max gt, sum exp(gt - max), max ct, sum exp(ct - max)}
-    uint16_t *mask;          // [B, tiles]
+    u32x4_t *rec;            // [B, tiles][2]: {max gt, sum exp(gt - max), max ct, sum exp(ct - max)} as float bits,
+                             // then {gt | q << 16, ct | mask << 16, column, 0} of the tile's first candidate
     uint16_t *gt;            // [B, V]
     uint16_t *ct;            // [B, V]
     int32_t B, tiles, rounds, reserved;
@@ -73,93 +76,201 @@ constexpr float HS_MARGIN = 1.0f - 0.03125f;   // 2^-5 below the tile's best: ou
 // The wave that holds tile `tile` ([2B rows] x 16 columns, accumulators in the MFMA layout: lane % 16 =
 // column, rows 16 b + 4 (lane / 16) + i): logits to bf16, scaled rows, tile partials and draw mask.
 // `tb` is the wave's own [16 * MB][16] floats of LDS.
+// The wave that summed up tile `tile` ([2B rows] x 16 columns, accumulators in the MFMA layout: lane % 16 =
+// column, rows 16 b + 4 (lane / 16) + i) leaves the logits, rounded to bf16 as the head's output tensor
+// holds them, in the tile's [16 * MB][16] floats of LDS.
 template <int MB>
-__device__ __forceinline__ void head_epilogue(const HeadArgs &a, int tile, const f32x4_t (&acc)[1][MB], float *tb) {
+__device__ __forceinline__ void head_tile_logits(const f32x4_t (&acc)[1][MB], float *tb) {
     const int lane = threadIdx.x & (WAVE - 1);
     const int col = lane & 15, rg = lane >> 4;
-    const int B = a.B, V = a.p.N;
 #pragma unroll
     for (int b = 0; b < MB; ++b)
 #pragma unroll
         for (int i = 0; i < 4; ++i) tb[(16 * b + 4 * rg + i) * 16 + col] = hs_round_bf16(acc[0][b][i]);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// the draw of the lane's entry: batch row lane / 16 + 4 j, column lane % 16 of the tile
+__device__ __forceinline__ uint16_t head_noise(const HeadArgs &a, int tile, int j) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int b = (lane >> 4) + 4 * j;
+    return as_global(a.noise)[(long)(b < a.B ? b : 0) * a.p.N + min(tile * 16 + (lane & 15), a.p.N - 1)];
+}
+
+// Wave j of the tile's waves takes the batch rows lane / 16 + 4 j (one per DPP row of 16 lanes, a lane per
+// column): scaled rows, tile partials, first candidate and draw mask.  q16: head_noise(tile, j), requested
+// before the tile's weights were streamed.
+__device__ __forceinline__ void head_epilogue(const HeadArgs &a, int tile, const float *tb, int j, uint16_t q16) {
+    typedef __attribute__((address_space(1))) u32x4_t *gptr_w4;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int col = lane & 15, rg = lane >> 4;
+    const int B = a.B, V = a.p.N;
     const int n = tile * 16 + col;
     const bool col_ok = n < V;
-#pragma unroll
-    for (int j = 0; j < 2 * MB; ++j) {
-        const int b = rg + 4 * j;                 // uniform over the 16 lanes of a DPP row
-        const bool ok = b < B && col_ok;
-        const int bb = b < B ? b : 0;
-        float gtv, ctv;
-        hs_scaled_pair(tb[bb * 16 + col], tb[(B + bb) * 16 + col], a.w, a.inv_t, gtv, ctv);
-        const long at = (long)bb * V + (col_ok ? n : 0);
-        const float q = bf16_bits_to_f32(as_global(a.noise)[at]);
-        if (ok) {
-            as_global(a.gt)[at] = hs_bf16_bits(gtv);
-            as_global(a.ct)[at] = hs_bf16_bits(ctv);
-        }
-        const float gm = row16_max(ok ? gtv : -INFINITY), cm = row16_max(ok ? ctv : -INFINITY);
-        const float eg = ok ? expf(gtv - gm) : 0.0f, ec = ok ? expf(ctv - cm) : 0.0f;
-        const float gs = row16_sum(eg), cs = row16_sum(ec);
-        // which entries can still win the draw (a NaN or an infinity compares in their favour)
-        const float e = eg / q;
-        const float eb = row16_max(e == e ? e : INFINITY);
-        const bool cand = ok && !(e < eb * HS_MARGIN);
-        const uint64_t votes = __ballot(cand);
-        if (col == 0 && b < B) {
-            typedef __attribute__((address_space(1))) f32x4_t *gptr_f4;
-            *(gptr_f4)(uintptr_t)(a.part + (long)b * a.tiles + tile) = f32x4_t{gm, gs, cm, cs};
-            as_global(a.mask)[(long)b * a.tiles + tile] = (uint16_t)((votes >> (16 * rg)) & 0xFFFFu);
-        }
+    const int b = rg + 4 * j;                 // uniform over the 16 lanes of a DPP row
+    const bool ok = b < B && col_ok;
+    const int bb = b < B ? b : 0;
+    float gtv, ctv;
+    hs_scaled_pair(tb[bb * 16 + col], tb[(B + bb) * 16 + col], a.w, a.inv_t, gtv, ctv);
+    const long at = (long)bb * V + (col_ok ? n : 0);
+    const float q = bf16_bits_to_f32(q16);
+    if (ok) {
+        as_global(a.gt)[at] = hs_bf16_bits(gtv);
+        as_global(a.ct)[at] = hs_bf16_bits(ctv);
+    }
+    const float gm = row16_max(ok ? gtv : -INFINITY), cm = row16_max(ok ? ctv : -INFINITY);
+    const float eg = ok ? expf(gtv - gm) : 0.0f, ec = ok ? expf(ctv - cm) : 0.0f;
+    const float gs = row16_sum(eg), cs = row16_sum(ec);
+    // which entries can still win the draw (a NaN or an infinity compares in their favour), and the first of them
+    float e = eg / q;
+    e = e == e ? e : INFINITY;
+    e = ok ? e : -INFINITY;
+    const float eb = row16_max(e);
+    const bool cand = ok && !(e < eb * HS_MARGIN);
+    const uint32_t votes = (uint32_t)((__ballot(cand) >> (16 * rg)) & 0xFFFFu);
+    const uint32_t bests = (uint32_t)((__ballot(ok && e == eb) >> (16 * rg)) & 0xFFFFu);
+    const int best_col = bests ? __builtin_ctz(bests) : 0;
+    const int from = 16 * rg + best_col;
+    const uint32_t g_b = __shfl((int)hs_bf16_bits(gtv), from, WAVE) & 0xFFFFu;
+    const uint32_t q_b = __shfl((int)q16, from, WAVE) & 0xFFFFu;
+    const uint32_t c_b = __shfl((int)hs_bf16_bits(ctv), from, WAVE) & 0xFFFFu;
+    if (col == 0 && b < B) {
+        gptr_w4 dst = (gptr_w4)(uintptr_t)(a.rec + 2 * ((long)b * a.tiles + tile));
+        dst[0] = __builtin_bit_cast(u32x4_t, f32x4_t{gm, gs, cm, cs});
+        dst[1] = u32x4_t{g_b | (q_b << 16), c_b | (votes << 16), (uint32_t)best_col, 0u};
     }
 }
 
-// One wave finishes batch row b from what every tile left behind.
-__device__ __forceinline__ void head_final_row(const HeadArgs &a, int b) {
-    typedef const __attribute__((address_space(1))) f32x4_t *gptr_cf4;
-    const int lane = threadIdx.x & (WAVE - 1);
+// the same with the entry's cond / T riding along (the log-probability needs it for the winner)
+__device__ __forceinline__ void hs_take_better(float &bv, int &bi, float &bc, float ov, int oi, float oc) {
+    const bool other_nan = ov != ov, mine_nan = bv != bv;
+    const bool take = mine_nan ? (other_nan && oi < bi) : (other_nan || ov > bv || (ov == bv && oi < bi));
+    if (take) {
+        bv = ov;
+        bi = oi;
+        bc = oc;
+    }
+}
+
+// One workgroup finishes batch row blockIdx.x from what every tile left behind: TPT tiles per thread,
+// their records requested as one batch.  The tile's first candidate is evaluated from the record; the
+// other marked entries (rare) only if their tile's first comes within 2^-4 of the best ratio of the row
+// (an entry the tile ranks below its first can exceed that first's ratio by rounding only: two
+// roundings of 2^-8), and those are read from the scaled rows.
+constexpr int MERGE_THREADS = 256;
+template <int TPT>
+__global__ __launch_bounds__(MERGE_THREADS) void head_merge_kernel(HeadArgs a) {
+    typedef const __attribute__((address_space(1))) u32x4_t *gptr_cw4;
+    constexpr int WAVES = MERGE_THREADS / WAVE;
+    __shared__ float red_f[4][WAVES];
+    __shared__ int red_i[WAVES];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int wave = tid / WAVE, lane = tid % WAVE;
     const int tiles = a.tiles, V = a.p.N;
-    gptr_cf4 part = (gptr_cf4)(uintptr_t)(a.part + (long)b * tiles);
+    gptr_cw4 rec = (gptr_cw4)(uintptr_t)(a.rec + 2 * (long)b * tiles);
+    gptr_cu16 gtp = as_global(a.gt + (long)b * V), ctp = as_global(a.ct + (long)b * V);
+    gptr_cu16 qp = as_global(a.noise + (long)b * V);
+    f32x4_t pt[TPT];
+    u32x4_t first_of[TPT];
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+        const int tt = min(MERGE_THREADS * k + tid, tiles - 1);
+        pt[k] = __builtin_bit_cast(f32x4_t, rec[2 * tt]);
+        first_of[k] = rec[2 * tt + 1];
+    }
+    auto block_all = [&](float &v0, float &v1, bool is_max) {   // every thread ends with the block's two results
+        v0 = is_max ? wave_max(v0) : wave_sum(v0);
+        v1 = is_max ? wave_max(v1) : wave_sum(v1);
+        __syncthreads();   // the buffer may still be read from the previous reduction
+        if (lane == 0) {
+            red_f[0][wave] = v0;
+            red_f[1][wave] = v1;
+        }
+        __syncthreads();
+        v0 = red_f[0][0];
+        v1 = red_f[1][0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) {   // one order in every thread
+            v0 = is_max ? fmaxf(v0, red_f[0][w]) : v0 + red_f[0][w];
+            v1 = is_max ? fmaxf(v1, red_f[1][w]) : v1 + red_f[1][w];
+        }
+    };
     float gm = -INFINITY, cm = -INFINITY;
-    for (int t = lane; t < tiles; t += WAVE) {
-        const f32x4_t pt = part[t];
-        gm = fmaxf(gm, pt[0]);
-        cm = fmaxf(cm, pt[2]);
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+        const bool in = MERGE_THREADS * k + tid < tiles;
+        gm = fmaxf(gm, in ? pt[k][0] : -INFINITY);
+        cm = fmaxf(cm, in ? pt[k][2] : -INFINITY);
     }
-    gm = wave_max(gm);
-    cm = wave_max(cm);
+    block_all(gm, cm, true);
     float gs = 0.0f, cs = 0.0f;
-    for (int t = lane; t < tiles; t += WAVE) {     // a fixed order: the same sums whichever workgroup is last
-        const f32x4_t pt = part[t];
-        gs += pt[1] * expf(pt[0] - gm);
-        cs += pt[3] * expf(pt[2] - cm);
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {   // a fixed order of the sums
+        const bool in = MERGE_THREADS * k + tid < tiles;
+        gs += in ? pt[k][1] * expf(pt[k][0] - gm) : 0.0f;
+        cs += in ? pt[k][3] * expf(pt[k][2] - cm) : 0.0f;
     }
-    gs = wave_sum(gs);
-    cs = wave_sum(cs);
-    float bv = -INFINITY;
+    block_all(gs, cs, false);
+
+    float bv = -INFINITY, bc = 0.0f;
     int bi = 0x7FFFFFFF;
-    for (int t = lane; t < tiles; t += WAVE) {
-        uint32_t m = as_global(a.mask)[(long)b * tiles + t];
-        while (m) {
-            const int bit = __builtin_ctz(m);
-            m &= m - 1;
-            const int idx = 16 * t + bit;
-            const float gt = bf16_bits_to_f32(as_global(a.gt)[(long)b * V + idx]);
-            const float q = bf16_bits_to_f32(as_global(a.noise)[(long)b * V + idx]);
-            const float p = hs_round_bf16(expf(gt - gm) / gs);
-            hs_take_better(bv, bi, hs_round_bf16(p / q), idx);
+    float first[TPT];
+    uint32_t m[TPT];
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+        const int t = MERGE_THREADS * k + tid;
+        const uint32_t col = first_of[k][2] & 15u;
+        const float p = hs_round_bf16(expf(bf16_bits_to_f32(first_of[k][0] & 0xFFFFu) - gm) / gs);
+        first[k] = hs_round_bf16(p / bf16_bits_to_f32(first_of[k][0] >> 16));
+        m[k] = t < tiles ? (first_of[k][1] >> 16) & ~(1u << col) : 0u;
+        if (t < tiles) hs_take_better(bv, bi, bc, first[k], 16 * t + (int)col, bf16_bits_to_f32(first_of[k][1] & 0xFFFFu));
+    }
+    // the other marked entries of the tiles that are still in the race
+    float seen = bv == bv ? bv : INFINITY, unused = 0.0f;
+    block_all(seen, unused, true);
+    const float floor_ratio = seen * 0.9375f;
+    int more = 0;
+#pragma unroll
+    for (int k = 0; k < TPT; ++k) {
+        if (!(first[k] >= floor_ratio) && first[k] == first[k]) m[k] = 0u;   // a NaN keeps its tile in
+        more |= m[k] != 0u;
+    }
+    while (__syncthreads_or(more)) {   // block-uniform
+        uint16_t g16[TPT], q16[TPT], c16[TPT];
+#pragma unroll
+        for (int k = 0; k < TPT; ++k) {
+            const int idx = 16 * min(MERGE_THREADS * k + tid, tiles - 1) + (m[k] ? __builtin_ctz(m[k]) : 0);
+            g16[k] = gtp[idx];
+            q16[k] = qp[idx];
+            c16[k] = ctp[idx];
+        }
+        more = 0;
+#pragma unroll
+        for (int k = 0; k < TPT; ++k) {
+            const int idx = 16 * min(MERGE_THREADS * k + tid, tiles - 1) + (m[k] ? __builtin_ctz(m[k]) : 0);
+            const float p = hs_round_bf16(expf(bf16_bits_to_f32(g16[k]) - gm) / gs);
+            if (m[k]) hs_take_better(bv, bi, bc, hs_round_bf16(p / bf16_bits_to_f32(q16[k])), idx, bf16_bits_to_f32(c16[k]));
+            m[k] &= m[k] - 1;
+            more |= m[k] != 0u;
         }
     }
 #pragma unroll
     for (int off = WAVE / 2; off > 0; off >>= 1)
-        hs_take_better(bv, bi, __shfl_xor(bv, off, WAVE), __shfl_xor(bi, off, WAVE));
+        hs_take_better(bv, bi, bc, __shfl_xor(bv, off, WAVE), __shfl_xor(bi, off, WAVE), __shfl_xor(bc, off, WAVE));
+    __syncthreads();
     if (lane == 0) {
-        if (bi >= V) bi = 0;   // only if no entry was marked at all: cannot happen for finite logits
-        const float ct = bf16_bits_to_f32(as_global(a.ct)[(long)b * V + bi]);
+        red_f[2][wave] = bv;
+        red_f[3][wave] = bc;
+        red_i[wave] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < WAVES; ++w) hs_take_better(bv, bi, bc, red_f[2][w], red_i[w], red_f[3][w]);
+        if (bi >= V) {   // no tile at all: cannot happen (V >= 16)
+            bi = 0;
+            bc = bf16_bits_to_f32(ctp[0]);
+        }
         a.sampled[b] = bi;
-        a.logprob[b] = hs_round_bf16(ct - cm - logf(cs));
+        a.logprob[b] = hs_round_bf16(bc - cm - logf(cs));
     }
 }
 
@@ -168,7 +279,6 @@ __device__ __forceinline__ void head_final_row(const HeadArgs &a, int b) {
 template <int KS, int TW, int GQ, int MB>
 __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    __shared__ int is_last;
     const DevProblem &p = a.p;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tw = wave / KS, kw = wave % KS;
@@ -177,10 +287,11 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
     const int xstride = p.kc + XPAD;
     uint8_t *after_x = smem + (size_t)p.M * xstride * 2;
     f32x4_t *red = reinterpret_cast<f32x4_t *>(after_x) + tw * (KS - 1) * MB * WAVE;
-    // the logit tile takes the place of the tile's partial sums once they are added up (2 KiB per row block
-    // in at least 3 KiB): between two barriers only the wave that finishes the tile touches that space
+    // the logit tile takes the place of the tile's partial sums once they are added up (1 KiB per row block
+    // in at least 3 KiB): written by the wave that adds them up, read by the tile's waves after a barrier
     float *tb = reinterpret_cast<float *>(red);
     static_assert((KS - 1) * WAVE * sizeof(f32x4_t) >= 16 * 16 * sizeof(float), "the logit tile fits the partial tiles");
+    static_assert(KS >= 2 * MB, "a wave per group of four batch rows");
     const int nsc = pp_nsc(p.K);
     const int per = (nsc + KS - 1) / KS;
     const int sc0 = min(nsc, kw * per), sc1 = min(nsc, sc0 + per);
@@ -199,6 +310,8 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
         f32x4_t acc[1][MB];
 #pragma unroll
         for (int b = 0; b < MB; ++b) acc[0][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        uint16_t q16 = 0;
+        if (kw < 2 * MB && tile < t1) q16 = head_noise(a, tile, kw);   // the tile's draws arrive while its weights stream
         if (work) {
             stream_rows_pp<MB, false, GQ>(p, rsrc, cur, next, xs + sc0 * PP_SC, xstride, sc0, sc1, ring, acc);
             if (next >= 0) cur = pp_tile_ptr<false>(p, next, sc0);
@@ -214,42 +327,29 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
 #pragma unroll
                 for (int b = 0; b < MB; ++b) acc[0][b] += red[((w - 1) * MB + b) * WAVE + lane];
             if (p.y) store_tile<MB, false>(p, tile, acc);
-            head_epilogue<MB>(a, tile, acc, tb);
+            head_tile_logits<MB>(acc, tb);
         }
+        __syncthreads();   // the logits of the round's tiles are in LDS: the tile's waves share its batch rows
+        if (kw < 2 * MB && tile < t1) head_epilogue(a, tile, tb, kw, q16);
         work = work && next >= 0;
         if (base + TW < t1) __syncthreads();   // the partial tiles are read before they are rewritten
     }
-    // whoever arrives last finishes the rows; what the others wrote is visible to it: every workgroup
-    // releases its stores before it counts itself, the last one acquires after it saw the count
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t seen = atomicAdd(a.counter, 1u);
-        is_last = seen == gridDim.x - 1;
-    }
-    __syncthreads();
-    if (!is_last) return;   // block-uniform
-    __threadfence();
-    for (int b = wave; b < a.B; b += KS * TW) head_final_row(a, b);
-    if (threadIdx.x == 0) *a.counter = 0u;   // the next launch starts from zero again
 }
 
 constexpr int HS_MAX_B = 16;
-constexpr size_t HS_LDS_CAP = 160 * 1024 - 64;   // what a workgroup can have, less the kernel's static word
-constexpr size_t HS_COUNTER_BYTES = 256;
+constexpr size_t HS_LDS_CAP = 160 * 1024;   // what a workgroup can have
 
 size_t hs_align(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct HeadLayout {
-    size_t part, mask, gt, ct, total;
+    size_t rec, gt, ct, total;
 };
 
 HeadLayout head_layout(int B, int V) {
     const size_t tiles = ((size_t)V + 15) / 16;
     HeadLayout l;
-    l.part = HS_COUNTER_BYTES;
-    l.mask = l.part + hs_align((size_t)B * tiles * sizeof(f32x4_t));
-    l.gt = l.mask + hs_align((size_t)B * tiles * sizeof(uint16_t));
+    l.rec = 0;
+    l.gt = l.rec + hs_align((size_t)B * tiles * 32);
     l.ct = l.gt + hs_align((size_t)B * V * sizeof(uint16_t));
     l.total = l.ct + hs_align((size_t)B * V * sizeof(uint16_t));
     return l;
@@ -333,9 +433,7 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
     args.noise = static_cast<const uint16_t *>(noise);
     args.sampled = reinterpret_cast<long long *>(sampled);
     args.logprob = logprob;
-    args.counter = reinterpret_cast<uint32_t *>(ws);
-    args.part = reinterpret_cast<f32x4_t *>(ws + lay.part);
-    args.mask = reinterpret_cast<uint16_t *>(ws + lay.mask);
+    args.rec = reinterpret_cast<u32x4_t *>(ws + lay.rec);
     args.gt = reinterpret_cast<uint16_t *>(ws + lay.gt);
     args.ct = reinterpret_cast<uint16_t *>(ws + lay.ct);
     args.B = B;
@@ -349,16 +447,26 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
     args.rounds = (int)std::min<long>(16, (workgroups + capacity - 1) / capacity);
     workgroups = (args.tiles + tw * args.rounds - 1) / (tw * args.rounds);
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    int rc;
     if (mb == 1) {
-        if (ks == 4 && tw == 1) return launch_head_group<4, 1, 1>(args, (int)workgroups, lds, stream);
-        if (ks == 4 && tw == 4) return launch_head_group<4, 4, 1>(args, (int)workgroups, lds, stream);
-        if (ks == 8 && tw == 1) return launch_head_group<8, 1, 1>(args, (int)workgroups, lds, stream);
-        if (ks == 8 && tw == 2) return launch_head_group<8, 2, 1>(args, (int)workgroups, lds, stream);
-        return launch_head_group<16, 1, 1>(args, (int)workgroups, lds, stream);
+        if (ks == 4 && tw == 1) rc = launch_head_group<4, 1, 1>(args, (int)workgroups, lds, stream);
+        else if (ks == 4 && tw == 4) rc = launch_head_group<4, 4, 1>(args, (int)workgroups, lds, stream);
+        else if (ks == 8 && tw == 1) rc = launch_head_group<8, 1, 1>(args, (int)workgroups, lds, stream);
+        else if (ks == 8 && tw == 2) rc = launch_head_group<8, 2, 1>(args, (int)workgroups, lds, stream);
+        else rc = launch_head_group<16, 1, 1>(args, (int)workgroups, lds, stream);
+    } else {
+        if (ks == 4) rc = launch_head_group<4, 4, 2>(args, (int)workgroups, lds, stream);
+        else if (ks == 8) rc = launch_head_group<8, 2, 2>(args, (int)workgroups, lds, stream);
+        else rc = launch_head_group<16, 1, 2>(args, (int)workgroups, lds, stream);
     }
-    if (ks == 4) return launch_head_group<4, 4, 2>(args, (int)workgroups, lds, stream);
-    if (ks == 8) return launch_head_group<8, 2, 2>(args, (int)workgroups, lds, stream);
-    return launch_head_group<16, 1, 2>(args, (int)workgroups, lds, stream);
+    if (rc != VRL_INT4_OK) return rc;
+    // the rows: one workgroup each
+    (void)hipGetLastError();
+    if (args.tiles <= 4 * MERGE_THREADS)
+        hipLaunchKernelGGL(head_merge_kernel<4>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
+    else
+        hipLaunchKernelGGL(head_merge_kernel<16>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
+    return (int)hipGetLastError();
 }
 
 }  // namespace

@@ -87,6 +87,7 @@ struct StreamShape { int wpb; int per_cu; size_t lds; };
 // resident, LDS the shape may use}
 constexpr StreamShape STREAM_SHAPES[3] = {{4, 15, 32 * 1024}, {8, 2, 72 * 1024}, {16, 1, 144 * 1024}};
 constexpr size_t LDS_PER_CU = 160 * 1024;
+constexpr size_t STREAM_LDS_CAP = LDS_PER_CU - 1024;   // dynamic LDS a grouped launch may ask for (the kernels hold a few static words)
 constexpr size_t DIRECT_LDS_CAP = 150 * 1024;   // plan-free launches: staged activations + partial tiles
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -248,7 +249,7 @@ int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *
         const uint64_t bit = 1ull << (dev & 63);
         if (!(raised.load(std::memory_order_relaxed) & bit)) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_PER_CU);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)STREAM_LDS_CAP);
             if (e != hipSuccess) return (int)e;
             raised.fetch_or(bit, std::memory_order_relaxed);
         }
@@ -915,7 +916,7 @@ int vrl_int4_gemv_grouped_bf16(const void *plan_dev, const vrl_int4_plan_info *i
                                void *hip_stream) {
     if (!plan_dev || !info) return VRL_INT4_ENULL;
     if (info->n_problems < 1 || info->total_tiles < 1 || info->grid < 1 ||
-        info->grid > MAX_PLAN_GRID || info->lds_bytes < 0 || (size_t)info->lds_bytes > LDS_PER_CU ||
+        info->grid > MAX_PLAN_GRID || info->lds_bytes < 0 || (size_t)info->lds_bytes > STREAM_LDS_CAP ||
         !aligned16(plan_dev))
         return VRL_INT4_EPLAN;
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);

@@ -508,17 +508,17 @@ def head_sample_supported(rows: int, head: PrepackedWeight) -> bool:
 
 
 def head_sample_workspace(B: int, V: int, device) -> torch.Tensor:
-    """A zeroed workspace for :func:`head_sample` at batch ``B`` and vocabulary ``V`` (reusable by
-    calls that do not overlap in time)."""
+    """A workspace for :func:`head_sample` at batch ``B`` and vocabulary ``V`` (reusable by calls that
+    do not overlap in time)."""
     nbytes = _lib.load().vrl_int4_head_sample_workspace_bytes(int(B), int(V))
     if nbytes == 0:
         raise ValueError(f"head_sample takes 1 <= B <= 16 and V a multiple of 16 up to 65536, got B={B}, V={V}")
-    return torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
 def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, temperature: float, *,
                 generator: torch.Generator | None = None, noise: torch.Tensor | None = None,
-                logits_out: torch.Tensor | None = None, workspace: torch.Tensor | None = None):
+                logits_out: torch.Tensor | None = None, workspace: torch.Tensor | None = None, out=None):
     """The image-token head and the sampling tail of a decode step in one launch.
 
     Stands for ``vrl/models/families/janus_pro/policy.py:684-693``: ``x`` is the bf16 ``[2B, K]``
@@ -526,7 +526,8 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     ``[V, K]``; returns ``(sampled int64 [B], logprob float32 [B])`` like :func:`cfg_sample` over the
     head's logits, which are written to ``logits_out`` (bf16 ``[2B, V]``) only if that is given.
     The draw consumes the random stream as ``torch.multinomial(probs, 1)`` does; ``workspace`` is a
-    tensor from :func:`head_sample_workspace` (made per call if omitted: pass one in a decode loop).
+    tensor from :func:`head_sample_workspace` (made per call if omitted: pass one in a decode loop);
+    ``out = (sampled, logprob)`` reuses output tensors.
     Raises ``ValueError`` for shapes the launch does not take (:func:`head_sample_supported`).
     """
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[0] % 2 != 0 or x.shape[0] < 2 or x.shape[1] != head.K:
@@ -551,8 +552,14 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
         workspace = head_sample_workspace(B, V, dev)
     elif workspace.dtype != torch.uint8 or workspace.device != dev or not workspace.is_contiguous():
         raise ValueError("workspace must be a contiguous uint8 tensor on the device of x")
-    sampled = torch.empty(B, dtype=torch.int64, device=dev)
-    logprob = torch.empty(B, dtype=torch.float32, device=dev)
+    if out is None:
+        out = (torch.empty(B, dtype=torch.int64, device=dev), torch.empty(B, dtype=torch.float32, device=dev))
+    sampled, logprob = out
+    if sampled.dtype != torch.int64 or logprob.dtype != torch.float32 or tuple(sampled.shape) != (B,) or \
+            tuple(logprob.shape) != (B,):
+        raise ValueError(f"out must be (int64 [{B}], float32 [{B}])")
+    _require_device("sampled", sampled, dev)
+    _require_device("logprob", logprob, dev)
     rec = _lib.Problem()
     rec.x, rec.qweight, rec.y = x.data_ptr(), head.blob.data_ptr(), (logits_out.data_ptr() if logits_out is not None else None)
     rec.M, rec.N, rec.K, rec.G, rec.prepacked = 2 * B, V, head.K, head.group_size, 1
