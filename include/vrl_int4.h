@@ -47,6 +47,7 @@ extern "C" {
 #define VRL_INT4_EALIGN 1002  /* a pointer is not 16-byte aligned */
 #define VRL_INT4_ENULL 1003   /* a required pointer is NULL */
 #define VRL_INT4_EPLAN 1004   /* malformed or undersized grouped plan */
+#define VRL_INT4_ELIMIT 1005  /* beyond the fixed size of the library's own scratch memory */
 
 int vrl_int4_abi_version(void);
 
@@ -221,6 +222,21 @@ size_t vrl_int4_head_sample_workspace_bytes(int B, int V);
 int vrl_int4_head_sample_bf16(const vrl_int4_problem *head, const void *noise, int64_t *sampled,
                               float *logprob, int B, float cfg_weight, float temperature,
                               void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
+ * vrl_int4_head_sample_bf16 without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no
+ * counterpart in the reference.  The partials, masks and scaled rows go to a fixed array that the
+ * library holds in the memory of every GPU it runs on (1,572,864 bytes, kept until the process ends),
+ * so the call allocates nothing.  Limits: B <= 16 and V <= 16384, else VRL_INT4_ELIMIT (nothing is
+ * enqueued); everything else as vrl_int4_head_sample_bf16.  Every call on a GPU uses that GPU's one
+ * array: calls that overlap in time on one GPU (two streams, two threads) race and must be ordered by
+ * the caller.  The first call on a device looks the array's address up (no allocation, but make it
+ * outside a stream capture).
+ */
+int vrl_int4_head_sample_static_bf16(const vrl_int4_problem *head, const void *noise, int64_t *sampled,
+                                     float *logprob, int B, float cfg_weight, float temperature,
+                                     void *hip_stream);
 
 #ifdef __cplusplus
 }

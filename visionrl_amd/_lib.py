@@ -31,6 +31,7 @@ SYMBOLS = (
     "vrl_cfg_sample_bf16",
     "vrl_int4_head_sample_workspace_bytes",
     "vrl_int4_head_sample_bf16",
+    "vrl_int4_head_sample_static_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
     "vrl_rope_attn_decode_lora_bf16",
@@ -164,6 +165,9 @@ def _bind(lib):
     lib.vrl_int4_head_sample_bf16.restype = ci
     lib.vrl_int4_head_sample_bf16.argtypes = [ctypes.POINTER(Problem), vp, vp, vp, ci, ctypes.c_float,
                                               ctypes.c_float, vp, ctypes.c_size_t, vp]
+    lib.vrl_int4_head_sample_static_bf16.restype = ci
+    lib.vrl_int4_head_sample_static_bf16.argtypes = [ctypes.POINTER(Problem), vp, vp, vp, ci, ctypes.c_float,
+                                                     ctypes.c_float, vp]
     lib.vrl_add_rmsnorm_bf16.restype = ci
     lib.vrl_add_rmsnorm_bf16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ctypes.c_float, vp]
     lib.vrl_rope_attn_decode_lora_bf16.restype = ci

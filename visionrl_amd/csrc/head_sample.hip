@@ -469,9 +469,52 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same launches for callers that cannot bring a workspace along: the library's own scratch.
+// One array per GPU, in that GPU's memory from the moment the code object is loaded there until
+// the process ends; its address is asked for once per device (the array's name in host code is a
+// handle for that query, not a device address).
+constexpr int HS_STATIC_MAX_V = 16384;
+constexpr size_t HS_STATIC_BYTES = (size_t)HS_MAX_B * (HS_STATIC_MAX_V / 16) * 32 +
+                                   2 * (size_t)HS_MAX_B * HS_STATIC_MAX_V * 2;   // 1,572,864 bytes
+static __device__ __align__(256) unsigned char scratch[HS_STATIC_BYTES];
+
+constexpr int HS_MAX_DEVICES = 64;
+
+// the current device's copy of `scratch`
+int scratch_address(void **out) {
+    static std::atomic<void *> known[HS_MAX_DEVICES];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= HS_MAX_DEVICES) return VRL_INT4_ESHAPE;
+    void *ptr = known[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return (int)hipErrorInvalidSymbol;
+        known[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return VRL_INT4_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int vrl_int4_head_sample_static_bf16(const vrl_int4_problem *head, const void *noise, int64_t *sampled,
+                                     float *logprob, int B, float cfg_weight, float temperature,
+                                     void *hip_stream) {
+    if (!head) return VRL_INT4_ENULL;
+    if (B < 1 || B > HS_MAX_B || head->N > HS_STATIC_MAX_V) return VRL_INT4_ELIMIT;
+    void *ptr = nullptr;
+    const int rc = scratch_address(&ptr);
+    if (rc != VRL_INT4_OK) return rc;
+    static_assert(HS_STATIC_BYTES % 256 == 0, "whole 256-byte lines");
+    return head_sample_launch(head, noise, sampled, logprob, B, cfg_weight, temperature, ptr, HS_STATIC_BYTES,
+                              hip_stream);
+}
 
 size_t vrl_int4_head_sample_workspace_bytes(int B, int V) {
     if (B < 1 || B > HS_MAX_B || V < 16 || V > 65536 || V % 16 != 0) return 0;

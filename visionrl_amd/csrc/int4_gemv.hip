@@ -434,6 +434,7 @@ const char *vrl_int4_error_string(int code) {
         case VRL_INT4_EALIGN: return "pointer is not 16-byte aligned";
         case VRL_INT4_ENULL: return "required pointer is NULL";
         case VRL_INT4_EPLAN: return "malformed or undersized grouped plan";
+        case VRL_INT4_ELIMIT: return "beyond the fixed size of the library's own scratch memory";
         default: break;
     }
     if (code > 0 && code < 1000) return hipGetErrorString(static_cast<hipError_t>(code));

@@ -518,7 +518,7 @@ def head_sample_workspace(B: int, V: int, device) -> torch.Tensor:
 
 def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, temperature: float, *,
                 generator: torch.Generator | None = None, noise: torch.Tensor | None = None,
-                logits_out: torch.Tensor | None = None, workspace: torch.Tensor | None = None, out=None):
+                logits_out: torch.Tensor | None = None, workspace: "torch.Tensor | str | None" = None, out=None):
     """The image-token head and the sampling tail of a decode step in one launch.
 
     Stands for ``vrl/models/families/janus_pro/policy.py:684-693``: ``x`` is the bf16 ``[2B, K]``
@@ -526,8 +526,10 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     ``[V, K]``; returns ``(sampled int64 [B], logprob float32 [B])`` like :func:`cfg_sample` over the
     head's logits, which are written to ``logits_out`` (bf16 ``[2B, V]``) only if that is given.
     The draw consumes the random stream as ``torch.multinomial(probs, 1)`` does; ``workspace`` is a
-    tensor from :func:`head_sample_workspace` (made per call if omitted: pass one in a decode loop);
-    ``out = (sampled, logprob)`` reuses output tensors.
+    tensor from :func:`head_sample_workspace` (made per call if omitted: pass one in a decode loop), or
+    the string ``"static"`` for the library's own fixed scratch (``vrl_int4_head_sample_static_bf16``:
+    B <= 16, V <= 16384, one call at a time per GPU); with ``noise`` and ``out = (sampled, logprob)``
+    given as well, the call then allocates nothing.
     Raises ``ValueError`` for shapes the launch does not take (:func:`head_sample_supported`).
     """
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[0] % 2 != 0 or x.shape[0] < 2 or x.shape[1] != head.K:
@@ -548,9 +550,10 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
         if logits_out.dtype != torch.bfloat16 or tuple(logits_out.shape) != (2 * B, V):
             raise ValueError(f"logits_out must be bfloat16 [{2 * B}, {V}]")
         _require_device("logits_out", logits_out, dev)
+    static = isinstance(workspace, str) and workspace == "static"
     if workspace is None:
         workspace = head_sample_workspace(B, V, dev)
-    elif workspace.dtype != torch.uint8 or workspace.device != dev or not workspace.is_contiguous():
+    elif not static and (workspace.dtype != torch.uint8 or workspace.device != dev or not workspace.is_contiguous()):
         raise ValueError("workspace must be a contiguous uint8 tensor on the device of x")
     if out is None:
         out = (torch.empty(B, dtype=torch.int64, device=dev), torch.empty(B, dtype=torch.float32, device=dev))
@@ -564,9 +567,14 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     rec.x, rec.qweight, rec.y = x.data_ptr(), head.blob.data_ptr(), (logits_out.data_ptr() if logits_out is not None else None)
     rec.M, rec.N, rec.K, rec.G, rec.prepacked = 2 * B, V, head.K, head.group_size, 1
     with _on(dev):
-        rc = _lib.load().vrl_int4_head_sample_bf16(ctypes.byref(rec), noise.data_ptr(), sampled.data_ptr(),
-                                                   logprob.data_ptr(), B, float(cfg_weight), float(temperature),
-                                                   workspace.data_ptr(), workspace.numel(), _stream_handle(dev))
+        if static:   # the library's own scratch: the call allocates nothing
+            rc = _lib.load().vrl_int4_head_sample_static_bf16(ctypes.byref(rec), noise.data_ptr(), sampled.data_ptr(),
+                                                              logprob.data_ptr(), B, float(cfg_weight),
+                                                              float(temperature), _stream_handle(dev))
+        else:
+            rc = _lib.load().vrl_int4_head_sample_bf16(ctypes.byref(rec), noise.data_ptr(), sampled.data_ptr(),
+                                                       logprob.data_ptr(), B, float(cfg_weight), float(temperature),
+                                                       workspace.data_ptr(), workspace.numel(), _stream_handle(dev))
     _lib.check(rc, "vrl_int4_head_sample_bf16")
     return sampled, logprob
 
