@@ -196,6 +196,16 @@ def measure_set(items, steps: int, warmup: int):
     # the launch that was just timed, every output of every record
     out["grouped_1_launch_worst_backward_error"] = check_outputs(items, grouped.outputs, "grouped launch")
 
+    # the comparison build whose dot product runs on the vector unit (v_dot2_f32_bf16) instead of the matrix
+    # cores: same blob, same dequantisation, same stream (one activation row only)
+    if all(it["x"].shape[0] == 1 for it in items):
+        vdot = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items], valu_dot=True)
+        ms_v, blocks_v = time_blocks(vdot.launch, steps, warmup, blocks=5, min_warm_ms=100.0)
+        record("grouped_1_launch_valu_dot", ms_v, 1)
+        out["grouped_1_launch_valu_dot_blocks_ms"] = blocks_v
+        check_outputs(items, vdot.outputs, "grouped launch, vector-unit dot product")
+        del vdot
+
     # the same launch over the canonical layout (no load-time repack)
     canon = ops.GroupedGemv([(it["x"], it["qweight"], it["scales"], it["qzeros"], GROUP, False)
                              for it in items])
@@ -759,6 +769,8 @@ def main():
     ap.add_argument("--rows", type=int, default=1, choices=(1, 32),
                     help="with --only-headline: 1 = the M=1 set (default), 32 = the rollout-batch set plus the "
                          "image-token head")
+    ap.add_argument("--valu-dot", action="store_true",
+                    help="with --only-headline (M=1): the comparison build whose dot product runs on the vector unit")
     ap.add_argument("--single-calls", action="store_true",
                     help="loop single-GEMV launches over distinct weights per shape and exit (for profilers)")
     ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
@@ -840,11 +852,11 @@ def main():
     torch.cuda.synchronize()
 
     if args.only_headline:
-        grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items])
+        grouped = ops.GroupedGemv([(it["x"], it["prepacked"], False) for it in items], valu_dot=args.valu_dot)
         ms, per_block = time_blocks(grouped.launch, args.steps, args.warmup)
         nbytes = sum(it["bytes"] for it in items)
         worst = check_outputs(items, grouped.outputs, "grouped launch")
-        print(json.dumps({"rows": args.rows, "ms_per_step": ms, "blocks_ms": per_block,
+        print(json.dumps({"rows": args.rows, "valu_dot": bool(args.valu_dot), "ms_per_step": ms, "blocks_ms": per_block,
                           "algorithmic_bytes_per_step": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9,
                           "outputs_checked": len(items), "worst_backward_error": worst}))
         return

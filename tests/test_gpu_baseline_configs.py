@@ -118,3 +118,34 @@ def test_whole_decode_step_in_one_launch(ops_mod):
     grouped.launch()
     torch.cuda.synchronize()
     assert all(torch.equal(a, b) for a, b in zip(first, grouped.outputs))
+
+
+def test_vector_unit_dot_build_of_the_grouped_launch(ops_mod):
+    """The comparison build (dot product by v_dot2_f32_bf16 instead of the matrix cores): the same
+    dequantised weights bit for bit (one-hot activations return a column of the tile) and outputs
+    within the operator tolerance, over a plan with more tiles than the device has workgroup slots."""
+    say("grouped launch, vector-unit dot product")
+    shapes = [(2048, 2048)] * 4 + [(2048, 5632)] * 2 + [(5632, 2048)]
+    problems, checks = [], []
+    for layer in range(6):
+        for j, (K, N) in enumerate(shapes):
+            ops = o.make_operands(2300 + 10 * layer + j, 1, K, N, 128)
+            if layer == 0:                       # x = e_k: the output row is column k of the dequantised tile
+                k = (37 * j + 5) % K
+                ops["x_bits"] = np.zeros((1, K), dtype=np.uint16)
+                ops["x_bits"][0, k] = 0x3F80
+            d = to_device(ops, DEV)
+            problems.append((d["x"], ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], 128), False))
+            checks.append((ops, (37 * j + 5) % K if layer == 0 else None))
+    grouped = ops_mod.GroupedGemv(problems, valu_dot=True)
+    assert grouped.info.variant & 256 and not grouped.info.variant & 32      # the stream build, vector-unit dot
+    outs = grouped.launch()
+    torch.cuda.synchronize()
+    for y, (ops, k) in zip(outs, checks):
+        assert_gemv_close(bf16_to_bits(y), ops, 128, "vector-unit dot")
+        if k is not None:
+            w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], 128)
+            assert (bf16_to_bits(y)[0] == w[:, k]).all()
+    with pytest.raises(ValueError):             # one activation row only
+        x2 = torch.zeros((2, 2048), dtype=torch.bfloat16, device=DEV)
+        ops_mod.GroupedGemv([(x2, problems[0][1], False)] * 600, valu_dot=True)

@@ -44,7 +44,9 @@ namespace {
 // record with two A operands per weight tile (weights streamed once); PASSES adds the
 // path for prepacked records whose activations do not fit LDS whole (it carries several
 // accumulator tiles, so plans that do not need it run a build without it).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ>
+// VDOT: the comparison build whose dot product runs on the vector unit (one activation row, plain prepacked
+// records of group size 128 only).
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ, bool VDOT = false>
 __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
                                                                 const int2 *__restrict__ block_tab,
                                                                 int n_problems) {
@@ -63,7 +65,7 @@ __global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem
         const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
         if (PP && (!CANON || p.prepacked)) {
             if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES, GQ>(p, a, b, smem, staged);
-            else stream_segment_pp<MB, false, WPB, PASSES, GQ>(p, a, b, smem, staged);
+            else stream_segment_pp<MB, false, WPB, PASSES, GQ, VDOT>(p, a, b, smem, staged);
         } else if (CANON) {
             staged.x = nullptr;  // the canonical walk stages in its own order
             if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
@@ -232,14 +234,14 @@ static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
 constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16,
-              VARIANT_SPLIT = 32, VARIANT_G64 = 64, VARIANT_G32 = 128;
+              VARIANT_SPLIT = 32, VARIANT_G64 = 64, VARIANT_G32 = 128, VARIANT_VDOT = 256;
 
 // With recs == nullptr nothing is launched: info->grid receives the number of workgroups of
 // this build that one CU holds at info->lds_bytes (the plan builder sizes the grid with it).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ = 1>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ = 1, bool VDOT = false>
 int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
                   hipStream_t stream) {
-    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ>;
+    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ, VDOT>;
     if (info->lds_bytes > 64 * 1024) {
         // once per instantiation and device (the attribute belongs to the function on that device), at the
         // largest size a plan may ask for: no runtime call in a timed or captured launch after the first
@@ -300,6 +302,13 @@ int launch_stream_variant(vrl_int4_plan_info *info, const DevProblem *recs, cons
     const bool passes = (info->variant & VARIANT_PASSES) != 0;
     // prepacked-only plans hold one group size (the kernel build is specialised for it)
     const int gq = (info->variant & VARIANT_G32) ? 4 : ((info->variant & VARIANT_G64) ? 2 : 1);
+    if (info->variant & VARIANT_VDOT) {
+        if constexpr (WPB == 4 && MB == 1) {
+            if (v == VARIANT_PP && !passes && gq == 1)
+                return launch_stream<4, 1, false, true, false, false, 1, true>(info, recs, bb, stream);
+        }
+        return VRL_INT4_EPLAN;
+    }
     if (v == VARIANT_PP || v == (VARIANT_PP | VARIANT_FUSED)) {
         return launch_stream_pp<WPB, MB>(info, recs, bb, stream, (v & VARIANT_FUSED) != 0, passes, gq);
     }
@@ -699,6 +708,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     long tiles = 0;
     double total_cost = 0.0;
     int variant = 0;
+    bool valu_dot = false, valu_dot_ok = true;   // a problem asks for the vector-unit dot product (reserved[0] == 1); all do and qualify
     int pp_group_size = 0;      // group size of the prepacked records, -1 if they differ
     size_t x_need = 0;  // bytes the largest activation matrix needs if staged whole
     for (int i = 0; i < n_problems; ++i) {
@@ -726,6 +736,8 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             return VRL_INT4_ESHAPE;
         if (p.prepacked) pp_group_size = (pp_group_size == 0 || pp_group_size == p.G) ? p.G : -1;
         if (p.M > MAX_TILE_M) variant |= VARIANT_MB2;
+        valu_dot = valu_dot || q.reserved[0] == 1;
+        valu_dot_ok = valu_dot_ok && q.reserved[0] == 1 && q.prepacked && !q.fused_gate_up && q.M == 1 && q.G == 128;
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const long nt = (out_cols + 15) / 16;
@@ -792,7 +804,12 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     // As many waves share a tile as it has super-chunks (4, 8 or 16), fewer if the plan would
     // not fit the device at that width.
     size_t red_bytes = 0;
-    if (shape == 0 && !(variant & (VARIANT_CANON | VARIANT_MB2 | VARIANT_PASSES))) {
+    if (valu_dot) {
+        // the comparison build is the 4-wave one over plain prepacked problems of one activation row
+        if (!valu_dot_ok || shape != 0 || (variant & VARIANT_PASSES)) return VRL_INT4_ESHAPE;
+        variant |= VARIANT_VDOT;
+    }
+    if (shape == 0 && !(variant & (VARIANT_CANON | VARIANT_MB2 | VARIANT_PASSES | VARIANT_VDOT))) {
         int max_nsc = 1;
         for (int i = 0; i < n_problems; ++i) max_nsc = std::max(max_nsc, pp_nsc(recs[i].K));
         variant |= VARIANT_SPLIT;

@@ -348,7 +348,12 @@ __device__ __forceinline__ void pp_prime(rsrc_t rsrc, const PPTilePtr<FUSED> &t,
 // XG: the A operand is not staged in LDS: xpre[b][4 * d + dd] holds it for super-chunk `xpre_sc`
 // (fetched by the caller) and is fetched again through `xr`, a range-checked resource over the
 // record's x, whenever the walk reaches another super-chunk.
-template <int MB, bool FUSED, int GQ, bool XG = false>
+// VDOT (one activation row, kept for the comparison the roofline asks for): the dot product on the
+// vector unit instead of the 16x16x32 matrix instruction.  A lane multiplies the eight weights it just
+// rebuilt (its row, eight consecutive k) with the matching activations (one LDS read, the same address for
+// the 16 lanes of a k quarter) in four v_dot2_f32_bf16 and keeps one running sum, in acc[r][0][0]; the
+// four k quarters of a row meet when the tile is stored (store_tile_vdot).
+template <int MB, bool FUSED, int GQ, bool XG = false, bool VDOT = false>
 __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc, const PPTilePtr<FUSED> &cur,
                                                int next_tile, const uint16_t *xs, int xstride,
                                                int sc0, int sc1, PPRing<FUSED ? 2 : 1, GQ> &ring,
@@ -398,8 +403,10 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
 #pragma unroll
             for (int dd = 0; dd < 4; ++dd) {
                 bf16x8_t xa[MB];
+                u32x4_t xrow;   // VDOT: the activation row's eight values
+                if constexpr (VDOT) xrow = *reinterpret_cast<const u32x4_t *>(xs + kloc + 8 * dd);
 #pragma unroll
-                for (int b = 0; b < MB; ++b) {
+                for (int b = 0; b < (VDOT ? 0 : MB); ++b) {
                     if constexpr (XG) {
                         xa[b] = __builtin_bit_cast(bf16x8_t, xpre[b][4 * d + dd]);
                     } else {
@@ -423,9 +430,23 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
                     const u32x4_t wv = {pack_bf16_rne(d0[0], d0[1]), pack_bf16_rne(d0[2], d0[3]),
                                         pack_bf16_rne(d1[0], d1[1]), pack_bf16_rne(d1[2], d1[3])};
                     const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, wv);
+                    if constexpr (VDOT) {
+                        // Four running sums, so that no dot instruction accumulates onto the result of one of the
+                        // three before it (the hardware does not interlock a DOT result read that early).  Inline
+                        // assembly: this toolchain drops all but the first of several independent
+                        // __builtin_amdgcn_fdot2_f32_bf16 chains.
+                        asm volatile("v_dot2_f32_bf16 %0, %4, %8, %0\n\t"
+                                     "v_dot2_f32_bf16 %1, %5, %9, %1\n\t"
+                                     "v_dot2_f32_bf16 %2, %6, %10, %2\n\t"
+                                     "v_dot2_f32_bf16 %3, %7, %11, %3"
+                                     : "+v"(acc[r][0][0]), "+v"(acc[r][0][1]), "+v"(acc[r][0][2]), "+v"(acc[r][0][3])
+                                     : "v"(wv[0]), "v"(wv[1]), "v"(wv[2]), "v"(wv[3]), "v"(xrow[0]), "v"(xrow[1]),
+                                       "v"(xrow[2]), "v"(xrow[3]));
+                    } else {
 #pragma unroll
-                    for (int b = 0; b < MB; ++b)
-                        acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
+                        for (int b = 0; b < MB; ++b)
+                            acc[r][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[b], bop, acc[r][b], 0, 0, 0);
+                    }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -480,7 +501,15 @@ struct StagedX {
     int M = 0, K = 0, kc = 0, zero_row = 0;
 };
 
-template <int MB, bool FUSED, int WPB, bool PASSES, int GQ>
+// the four k quarters of each of the tile's 16 rows (lanes l, l + 16, l + 32, l + 48) added up and stored
+__device__ __forceinline__ void store_tile_vdot(const DevProblem &p, int tile_local, float part) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    part = row16_sum_quarters(part);
+    const int col = tile_local * 16 + lane;
+    if (lane < 16 && col < p.N) as_global(p.y)[col] = (uint16_t)(pack_bf16_rne(part, 0.0f) & 0xFFFFu);
+}
+
+template <int MB, bool FUSED, int WPB, bool PASSES, int GQ, bool VDOT = false>
 __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
                                                   StagedX &staged) {
     constexpr int RS = FUSED ? 2 : 1;
@@ -522,8 +551,12 @@ __device__ __forceinline__ void stream_segment_pp(const DevProblem &p, int t0, i
             for (int r = 0; r < RS; ++r)
 #pragma unroll
                 for (int b = 0; b < MB; ++b) acc[r][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            stream_rows_pp<MB, FUSED, GQ>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
-            store_tile<MB, FUSED>(p, tile, acc);
+            stream_rows_pp<MB, FUSED, GQ, false, VDOT>(p, rsrc, cur, nt < t1 ? nt : -1, xs, xstride, 0, nsc, ring, acc);
+            if constexpr (VDOT) {
+                asm volatile("s_nop 2" ::: "memory");   // the last dot results are read next
+                store_tile_vdot(p, tile, (acc[0][0][0] + acc[0][0][1]) + (acc[0][0][2] + acc[0][0][3]));
+            }
+            else store_tile<MB, FUSED>(p, tile, acc);
             tile = nt;
             if (tile < t1) cur = pp_tile_ptr<FUSED>(p, tile, 0);
         }

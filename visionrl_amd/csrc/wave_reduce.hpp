@@ -34,6 +34,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     v = row16_sum(v);
     return (lane_of(v, 0) + lane_of(v, 16)) + (lane_of(v, 32) + lane_of(v, 48));
 }
+// lanes l, l + 16, l + 32, l + 48 added up in that order; lanes 0..15 hold the results
+__device__ __forceinline__ float row16_sum_quarters(float v) {
+    const float q1 = __shfl_down(v, 16, 64), q2 = __shfl_down(v, 32, 64), q3 = __shfl_down(v, 48, 64);
+    return ((v + q1) + q2) + q3;
+}
 __device__ __forceinline__ float wave_max(float v) {
     v = row16_max(v);
     return fmaxf(fmaxf(lane_of(v, 0), lane_of(v, 16)), fmaxf(lane_of(v, 32), lane_of(v, 48)));
