@@ -55,7 +55,7 @@ def test_apply_swaps_every_decode_linear():
     summary = apply_int4_to_policy(policy, group_size=128)
     # nothing is prepacked on the CPU: the MFMA-shaped copies are made only for weights on a GPU
     assert summary == {"linears": 7 * LAYERS, "fused_mlps": LAYERS, "head_linears": 1, "group_size": 128,
-                       "prepacked": 0, "qkv_groups": 0}
+                       "prepacked": 0, "dense_kept": 0, "qkv_groups": 0}
     for layer in policy._lm_trunk().layers:
         for name in ("q_proj", "k_proj", "v_proj", "o_proj"):
             mod = getattr(layer.self_attn, name)
@@ -375,6 +375,52 @@ def test_prompt_sized_calls_go_through_the_library_gemm():
         # and it stays within a bf16 rounding or two of the fused decode kernel's fp32 epilogue
         small = gu(x[:1, :8])
         assert (small.float() - got[:1, :8].float()).abs().max().item() <= 2.0 ** -6 * max(1.0, got.abs().max().item())
+
+
+@pytest.mark.gpu
+def test_kept_dense_weight_serves_prompt_sized_calls_until_the_source_changes():
+    """``keep_dense_()``: prompt-sized and gradient-carrying calls multiply by one kept bf16 tensor (the
+    same results, no dequantisation per call); a write to the canonical buffers makes the next call
+    rebuild it; ``keep_dense_(False)`` drops it."""
+    import torch.nn.functional as F
+
+    dev = "cuda:0"
+    torch.manual_seed(14)
+    q = Int4Linear.from_linear(nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev), 128).prepack_()
+    gu = Int4GateUpSiLU(Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128),
+                        Int4Linear.from_linear(nn.Linear(512, 64, bias=False).to(torch.bfloat16).to(dev), 128)).prepack_()
+    x = torch.randn(80, 512, device=dev).to(torch.bfloat16)
+    want_q, want_gu = q(x), gu(x)
+    q.keep_dense_(), gu.keep_dense_()
+    assert torch.equal(q(x), want_q) and torch.equal(gu(x), want_gu)
+    kept = q._dense[1]
+    assert torch.equal(kept, q.dequantize())
+    assert torch.equal(q(x), want_q) and q._dense[1] is kept          # the second call reuses the tensor
+    xg = x.clone().requires_grad_(True)
+    q(xg).float().sum().backward()                                     # and so does the replay's route
+    assert q._dense[1] is kept and xg.grad is not None
+    small = x[:2]
+    assert torch.equal(q(small), Int4Linear.from_packed(q.qweight, q.scales, q.qzeros, 128).prepack_()(small))
+    # a new weight: the kept tensor and the prepacked copy are both rebuilt on the next call
+    other = Int4Linear.from_linear(nn.Linear(512, 96, bias=False).to(torch.bfloat16).to(dev), 128)
+    q.load_state_dict(other.state_dict())
+    assert torch.equal(q(x), F.linear(x, other.dequantize())) and q._dense[1] is not kept
+    q.keep_dense_(False)
+    assert q._dense is None and torch.equal(q(x), F.linear(x, other.dequantize())) and q._dense is None
+
+
+def test_keep_dense_option_reaches_every_quantised_module():
+    from visionrl_amd.policy_glue import apply_int4_to_policy, int4_options_from_spec
+
+    policy = StubPolicy()
+    summary = apply_int4_to_policy(policy, prepack=False, keep_dense=True)
+    assert summary["dense_kept"] == 6 * LAYERS + 1      # q, k, v, o, gate|up, down per layer, and the head
+    kinds = (Int4Linear, Int4GateUpSiLU)
+    assert all(getattr(m, "_keep_dense", False) for m in policy.mmgpt.modules() if isinstance(m, kinds))
+
+    class Spec:
+        extra = {"int4": {"keep_dense": True}}
+    assert int4_options_from_spec(Spec())["keep_dense"] is True
 
 
 @pytest.mark.gpu

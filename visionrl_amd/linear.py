@@ -170,6 +170,26 @@ class Int4Linear(nn.Module):
         """The canonical bf16 weight ``[N, K]`` (bit-exact tile), e.g. for the train-time replay."""
         return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
 
+    def keep_dense_(self, keep: bool = True) -> "Int4Linear":
+        """Keep the dequantised bf16 weight between calls (2 bytes per weight beside the 0.56 of the int4
+        buffers): prompt-sized calls and the train-time replay (``policy.py:419-424``: one forward per
+        micro-batch) then multiply by the kept tensor instead of rebuilding it every call.  It is rebuilt
+        when the canonical buffers were written or replaced since; ``keep=False`` drops it."""
+        self._keep_dense = bool(keep)
+        self._dense = None
+        return self
+
+    def _dense_weight(self) -> torch.Tensor:
+        """The bf16 weight for a library GEMM: the kept copy if there is one and it is current."""
+        if not getattr(self, "_keep_dense", False):
+            return ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
+        kept = getattr(self, "_dense", None)
+        if kept is None or _source_changed(kept[0], self.qweight, self.scales, self.qzeros):
+            kept = (_source_state(self.qweight, self.scales, self.qzeros),
+                    ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size))
+            self._dense = kept
+        return kept[1]
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
         handed = getattr(self, "_handed", None)
@@ -182,7 +202,7 @@ class Int4Linear(nn.Module):
         if torch.compiler.is_compiling():
             y = ops.int4_gemv(rows, self.qweight, self.scales, self.qzeros, self.group_size)
         elif _wants_grad(x):
-            y = F.linear(rows, self.dequantize())
+            y = F.linear(rows, self._dense_weight())
         elif handed is not None and handed[0] is x and handed[1] == _version(x):
             y = handed[2]   # computed by the group leader's launch from this very tensor, unchanged since
         else:  # eager decode: skip the operator dispatcher, it costs more than the kernel
@@ -206,7 +226,7 @@ class Int4Linear(nn.Module):
                 packed = None
             if packed is None and M > GEMM_ROWS:
                 # prompt-sized call: the GEMV kernels would stream the weight once per 16 rows
-                y = F.linear(rows, self.dequantize())
+                y = F.linear(rows, self._dense_weight())
             elif packed is None:
                 y = torch.empty((M, self.out_features), dtype=torch.bfloat16, device=rows.device)
                 ops.int4_gemv_into(y, rows, self.qweight, self.scales, self.qzeros, self.group_size)
@@ -249,6 +269,8 @@ class Int4GateUpSiLU(nn.Module):
 
     packed_is_stale = Int4Linear.packed_is_stale
     _fresh_packed = Int4Linear._fresh_packed
+    keep_dense_ = Int4Linear.keep_dense_
+    _dense_weight = Int4Linear._dense_weight
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         rows = _rows(x, self.in_features)
@@ -258,8 +280,7 @@ class Int4GateUpSiLU(nn.Module):
                 and rows.shape[0] <= self._direct_rows and packed.blob.device == rows.device:
             y = self._call(rows)[0]
         elif (grad or rows.shape[0] > GEMM_ROWS) and not torch.compiler.is_compiling():
-            w = ops.int4_dequant(self.qweight, self.scales, self.qzeros, self.group_size)
-            gate, up = F.linear(rows, w).chunk(2, dim=-1)   # prompt-sized call: one library GEMM
+            gate, up = F.linear(rows, self._dense_weight()).chunk(2, dim=-1)   # prompt-sized call: one library GEMM
             y = F.silu(gate) * up
         else:
             y = ops.int4_gate_up_silu(rows, self.qweight, self.scales, self.qzeros, self.group_size)
@@ -286,6 +307,11 @@ class Int4LlamaMLP(nn.Module):
     def prepack_(self) -> "Int4LlamaMLP":
         self.gate_up.prepack_()
         self.down_proj.prepack_()
+        return self
+
+    def keep_dense_(self, keep: bool = True) -> "Int4LlamaMLP":
+        self.gate_up.keep_dense_(keep)
+        self.down_proj.keep_dense_(keep)
         return self
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -13,7 +13,7 @@ Hook points in the reference (all under ``vrl/models/families/janus_pro/``):
 * ``builder.py:11-33``, ``:77-113`` and ``vrl/distributed/ray/rollout/worker.py:143-163``:
   rollout workers build the policy from a ``RuntimeBuildSpec`` whose ``extra``
   dict is the only channel for new scalar options; ``extra["int4"]`` carries
-  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true,
+  ``{"group_size": 128, "targets": [...], "fuse_mlp": true, "head": true, "prepack": true, "group_qkv": true, "keep_dense": false,
   "static_sampler": true}`` (the last one routes ``sample_image_tokens`` and the step API through
   :mod:`visionrl_amd.ar_decode`).
 
@@ -98,7 +98,8 @@ def _swap_all_linears(module: nn.Module, group_size: int) -> int:
 
 def apply_int4_to_policy(policy: Any, group_size: int = 128,
                          targets: Iterable[str] = DEFAULT_TARGETS, fuse_mlp: bool = True,
-                         head: bool = True, prepack: bool = True, group_qkv: bool = True) -> dict:
+                         head: bool = True, prepack: bool = True, group_qkv: bool = True,
+                         keep_dense: bool = False) -> dict:
     """Quantise the decode linears of ``policy`` in place; returns a count summary.
 
     ``fuse_mlp`` replaces a whole MLP block by :class:`Int4LlamaMLP` (gate||up with
@@ -107,6 +108,9 @@ def apply_int4_to_policy(policy: Any, group_size: int = 128,
     of every quantised weight that lives on a GPU, which decode-sized calls (up to 32
     activation rows) stream through the plan-free launch; with ``group_qkv`` the three
     projections of an attention block then share one launch per decode step.
+    ``keep_dense`` also keeps the dequantised bf16 weight of every quantised module (four times
+    the int4 bytes) so that prompt passes and the train-time replay's micro-batches stop rebuilding
+    it on every call.
     """
     targets = tuple(targets)
     unknown = set(targets) - set(DEFAULT_TARGETS)
@@ -148,6 +152,14 @@ def apply_int4_to_policy(policy: Any, group_size: int = 128,
                 if isinstance(mod, (Int4Linear, Int4GateUpSiLU)):
                     mod.prepack_()
                     summary["prepacked"] += int(getattr(mod, "_packed", None) is not None)
+    summary["dense_kept"] = 0
+    if keep_dense:
+        roots = [trunk] + ([owner.gen_head] if head and owner is not None else [])
+        for root in roots:
+            for mod in root.modules():
+                if isinstance(mod, (Int4Linear, Int4GateUpSiLU)):
+                    mod.keep_dense_()
+                    summary["dense_kept"] += 1
     summary["qkv_groups"] = 0
     if prepack and group_qkv:
         for layer in trunk.layers:
@@ -173,7 +185,7 @@ def int4_options_from_spec(spec: Any) -> dict | None:
         opt = {}
     if not isinstance(opt, dict):
         raise TypeError('RuntimeBuildSpec.extra["int4"] must be true or a dict of options')
-    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack", "group_qkv", "static_sampler"}
+    allowed = {"group_size", "targets", "fuse_mlp", "head", "prepack", "group_qkv", "keep_dense", "static_sampler"}
     unknown = set(opt) - allowed
     if unknown:
         raise ValueError(f'unknown keys in extra["int4"]: {sorted(unknown)}')
@@ -183,6 +195,7 @@ def int4_options_from_spec(spec: Any) -> dict | None:
             "head": bool(opt.get("head", True)),
             "prepack": bool(opt.get("prepack", True)),
             "group_qkv": bool(opt.get("group_qkv", True)),
+            "keep_dense": bool(opt.get("keep_dense", False)),
             "static_sampler": bool(opt.get("static_sampler", True))}
 
 
