@@ -466,6 +466,52 @@ def decode_tail(device, steps: int):
     return out
 
 
+def decode_head_and_tail(device, steps: int, heads: int = 16):
+    """The image-token head (2048 -> 16384, int4) and the sampling tail per decode step: the plan-free head launch
+    followed by the tail launch, against the one call that does both (vrl_int4_head_sample_bf16).  One HIP graph
+    per form holds ``heads`` calls, each over a head of its own (16 x 18.6 MB: the weights do not stay in the
+    L2 caches between calls); microseconds per call."""
+    from visionrl_amd import ops
+
+    packed = []
+    for i in range(heads):
+        qw, sc, qz = make_weights(7000 + i, HIDDEN, HEAD, 128, device)
+        packed.append(ops.int4_prepack(qw, sc, qz, 128))
+        del qw, sc, qz
+    out = {"heads": heads, "shape": f"{HIDDEN}->{HEAD}, G=128"}
+    for B in (1, 4, 16):
+        x = (make_x(7100 + B, 2 * B, HIDDEN, device).float() * 0.5).to(torch.bfloat16)
+        noise = torch.empty((B, HEAD), dtype=torch.bfloat16, device=device).exponential_(1.0)
+        ws = ops.head_sample_workspace(B, HEAD, device)
+        res = (torch.empty(B, dtype=torch.int64, device=device), torch.empty(B, dtype=torch.float32, device=device))
+        launches = [ops.DirectGemv([(x, pw, False)]) for pw in packed]
+
+        def one_call():
+            for pw in packed:
+                ops.head_sample(x, pw, 5.0, 1.0, noise=noise, workspace=ws, out=res)
+
+        def head_then_tail():
+            for launch in launches:
+                (logits,) = launch.launch()
+                ops.cfg_sample(logits, 5.0, 1.0, noise=noise)
+
+        def head_only():
+            for launch in launches:
+                launch.launch()
+
+        entry = {}
+        for name, fn in (("one_call", one_call), ("head_then_tail", head_then_tail), ("head_only", head_only)):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            entry[f"{name}_us"] = time_region(graph.replay, max(20, steps // 5), 5) / heads * 1e3
+            del graph
+        out[f"B{B}"] = entry
+    return out
+
+
 def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16), prompt: int = 304,
                    shape=(HIDDEN, INTER, LAYERS, 16)):
     """ms per decode step of the image-token loop on a Janus-Pro-1B shaped policy (random weights), at
@@ -781,6 +827,8 @@ def main():
     ap.add_argument("--attn-decode", type=int, default=0, metavar="ROWS",
                     help="run 8 attention decode launches (16 heads x 128, slot 330 of 384) over distinct caches "
                          "at ROWS rows and exit (for counter runs)")
+    ap.add_argument("--head-sample", action="store_true",
+                    help="only the head + sampling tail of a decode step: two launches against the one call")
     ap.add_argument("--stream-read", action="store_true",
                     help="time the plain streaming read of 642.5 MB and exit (for profilers)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -841,6 +889,10 @@ def main():
         print(json.dumps({"single_calls": "done"}))
         return
 
+    if args.head_sample:
+        print(json.dumps({"decode_head_and_tail": decode_head_and_tail(device, args.steps)}))
+        return
+
     if args.stream_read:
         print(json.dumps({"stream_read": stream_read(device, 642_539_520, args.steps, args.warmup)}))
         return
@@ -889,6 +941,10 @@ def main():
         tail = decode_tail(device, args.steps)
     except Exception as exc:
         tail = {"error": repr(exc)[:300]}
+    try:
+        head_tail = decode_head_and_tail(device, args.steps)
+    except Exception as exc:
+        head_tail = {"error": repr(exc)[:300]}
     best = max(strat["GBps"], key=lambda k: strat["GBps"][k])
 
     del items, grouped
@@ -973,7 +1029,8 @@ def main():
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency, "stream_read": read,
                    "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
-                   "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "ar_decode_loop_1b": ar_loop,
+                   "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "decode_head_and_tail": head_tail,
+                   "ar_decode_loop_1b": ar_loop,
                    "other_configs": others},
     }
     print(json.dumps(result))
