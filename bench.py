@@ -431,6 +431,44 @@ def module_path(items, steps: int):
     return out
 
 
+def prompt_pass_linears(device, steps: int):
+    """The linears of the prompt pass (vrl/models/families/janus_pro/policy.py:523, iteration 0: 2B x 256 rows)
+    through the int4 modules: every module dequantises its weight (bit-exact tile) and calls the library GEMM;
+    with ``keep_dense_()`` the bf16 tile is kept between calls.  Four layers' modules, milliseconds per
+    24-layer pass (the measured four scaled by six), at 2 x 256 and 32 x 256 rows."""
+    from visionrl_amd.linear import Int4GateUpSiLU, Int4Linear
+
+    layers = []
+    for layer in range(4):
+        mods = {}
+        for proj, (K, N) in (("q", (HIDDEN, HIDDEN)), ("k", (HIDDEN, HIDDEN)), ("v", (HIDDEN, HIDDEN)),
+                             ("o", (HIDDEN, HIDDEN)), ("gate", (HIDDEN, INTER)), ("up", (HIDDEN, INTER)),
+                             ("down", (INTER, HIDDEN))):
+            qw, sc, qz = make_weights(8000 + 10 * layer + len(mods), K, N, GROUP, device)
+            mods[proj] = Int4Linear.from_packed(qw, sc, qz, GROUP)
+        layers.append((mods["q"], mods["k"], mods["v"], mods["o"], Int4GateUpSiLU(mods["gate"], mods["up"]), mods["down"]))
+    out = {}
+    for rows in (512, 8192):
+        x = make_x(8100, rows, HIDDEN, device)
+        entry = {}
+        for keep in (False, True):
+            for mods in layers:
+                for m in mods:
+                    m.keep_dense_(keep)
+
+            def run():
+                for q, k, v, o, gate_up, down in layers:
+                    q(x), k(x), v(x)
+                    o(x)
+                    down(gate_up(x))
+
+            with torch.no_grad():
+                ms = time_region(run, max(5, steps // 40), 2)
+            entry["kept_dense_ms" if keep else "dequant_per_call_ms"] = ms * LAYERS / len(layers)
+        out[f"rows{rows}"] = entry
+    return out
+
+
 def decode_tail(device, steps: int):
     """CFG + softmax + draw + log-probability over [2B, 16384] logits: fused launch vs the tensor ops."""
     import torch.nn.functional as F
@@ -453,14 +491,18 @@ def decode_tail(device, steps: int):
         def fused():
             return ops.cfg_sample(logits, w, T)
 
-        entry = {}
+        # per call from a graph of 16 calls: a graph of one call is dominated by what launching a graph
+        # costs (about 10 us), which a decode step pays once for all of its launches
+        calls = 16
+        entry = {"calls_per_graph": calls}
         for name, fn in (("torch_ops", torch_ops), ("fused", fused)):
             entry[f"{name}_eager_us"] = time_region(fn, max(20, steps // 5), 5) * 1e3
             graph = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
             with torch.cuda.graph(graph):
-                fn()
-            entry[f"{name}_hip_graph_us"] = time_region(graph.replay, max(20, steps // 5), 5) * 1e3
+                for _ in range(calls):
+                    fn()
+            entry[f"{name}_hip_graph_us"] = time_region(graph.replay, max(20, steps // 5), 5) / calls * 1e3
             del graph
         out[f"B{B}"] = entry
     return out
@@ -890,7 +932,9 @@ def main():
         return
 
     if args.head_sample:
-        print(json.dumps({"decode_head_and_tail": decode_head_and_tail(device, args.steps)}))
+        print(json.dumps({"decode_head_and_tail": decode_head_and_tail(device, args.steps),
+                          "decode_tail_cfg_sample": decode_tail(device, args.steps),
+                          "prompt_pass_linears": prompt_pass_linears(device, args.steps)}))
         return
 
     if args.stream_read:
@@ -941,6 +985,10 @@ def main():
         tail = decode_tail(device, args.steps)
     except Exception as exc:
         tail = {"error": repr(exc)[:300]}
+    try:
+        prompt = prompt_pass_linears(device, args.steps)
+    except Exception as exc:
+        prompt = {"error": repr(exc)[:300]}
     try:
         head_tail = decode_head_and_tail(device, args.steps)
     except Exception as exc:
@@ -1030,6 +1078,7 @@ def main():
         "detail": {"m1": strat, "m1_best_strategy": best, "m1_us_per_call": latency, "stream_read": read,
                    "m32_plus_head": strat32, "m32_algorithmic_bytes_per_step": bytes32,
                    "m1_through_modules": modules, "decode_tail_cfg_sample": tail, "decode_head_and_tail": head_tail,
+                   "prompt_pass_linears": prompt,
                    "ar_decode_loop_1b": ar_loop,
                    "other_configs": others},
     }
