@@ -162,6 +162,10 @@ NORM_FUSED_CASES = [
     (32, 2048, [2048, 2048, 2048], False, True), (2, 2048, [2 * 5632], True, True), (32, 2048, [2 * 704], True, True),
     (3, 4096, [256], False, False), (5, 640, [48, 80], False, True), (16, 1536, [64], False, True),
     (9, 2048, [100], False, False),
+    # rows wider than 2048 with one wave per row (eight words per lane: the residual and the norm weight pass
+    # through the registers in halves), incl. a K that is no multiple of 512 and the 7B-class shapes
+    (16, 4096, [256, 128], False, True), (32, 4096, [2 * 1024], True, True), (5, 3072, [64], False, True),
+    (7, 2560, [48], False, False), (32, 4096, [4096], False, True),
 ]
 
 

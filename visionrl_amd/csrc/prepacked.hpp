@@ -224,6 +224,102 @@ __device__ __forceinline__ void stage_x_norm_rows(const DevProblem &p, const Nor
     }
 }
 
+// The same for a wave that holds a whole row of 2049 to 4096 values (eight words per lane, one wave per
+// row): the row stays packed in registers, the residual and the norm weight pass through four registers'
+// worth of words at a time (the second half of the residual and both halves of the weight are requested when
+// their registers are free: round trips into cache beyond the first).  Row, residual and weight held
+// together are 96 registers, which made every build of the kernel that contains this path allocate 154 to
+// 177 and the 16-wave builds spill.
+__device__ __forceinline__ void stage_x_norm_rows_wide(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
+                                                       int xstride, int nwaves, bool write_h) {
+    typedef __attribute__((address_space(1))) u32x4_t *gptr_w4;
+    constexpr int NW = 8, CH = 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int nthreads = nwaves * WAVE;
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+    const int padw = (kext - p.K) >> 3;
+    for (int idx = threadIdx.x; idx < p.M * padw; idx += nthreads) {
+        const int m = idx / padw;
+        *reinterpret_cast<u32x4_t *>(xs + m * xstride + p.K + ((idx - m * padw) << 3)) = zero;
+    }
+    if (p.prepacked & PP_ZERO_ROW)
+        for (int j = threadIdx.x; j < (kext >> 3); j += nthreads)
+            *reinterpret_cast<u32x4_t *>(xs + p.M * xstride + (j << 3)) = zero;
+    const long base = p.x - n.x0;
+    const float inv_k = 1.0f / (float)p.K;
+    for (int m0 = 0; m0 < p.M; m0 += nwaves) {
+        const int m = m0 + wave;
+        const bool live = m < p.M;  // wave-uniform
+        const long row = base + (long)m * p.K;
+        u32x4_t h[NW], t[CH];
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            const int k = (i * WAVE + lane) << 3;
+            h[i] = zero;
+            if (live && k < p.K) h[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.x0 + row + k));
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NW; c += CH) {
+            if (n.residual) {
+#pragma unroll
+                for (int i = 0; i < CH; ++i) {
+                    const int k = ((c + i) * WAVE + lane) << 3;
+                    t[i] = zero;
+                    if (live && k < p.K) t[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.residual + row + k));
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const int k = ((c + i) * WAVE + lane) << 3;
+                if (live && k < p.K) {
+                    if (n.residual) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            h[c + i][e] = pack_bf16_rne(
+                                bf16_bits_to_f32(t[i][e] & 0xFFFFu) + bf16_bits_to_f32(h[c + i][e] & 0xFFFFu),
+                                bf16_bits_to_f32(t[i][e] >> 16) + bf16_bits_to_f32(h[c + i][e] >> 16));
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float lo = bf16_bits_to_f32(h[c + i][e] & 0xFFFFu), hi = bf16_bits_to_f32(h[c + i][e] >> 16);
+                        ss += lo * lo;
+                        ss += hi * hi;
+                    }
+                    if (write_h) *(gptr_w4)(uintptr_t)(n.h_out + row + k) = h[c + i];
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        const float r = rsqrtf(ss * inv_k + n.eps);
+#pragma unroll
+        for (int c = 0; c < NW; c += CH) {
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const int k = ((c + i) * WAVE + lane) << 3;
+                t[i] = zero;
+                if (live && k < p.K) t[i] = *as_global(reinterpret_cast<const u32x4_t *>(n.weight + k));
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const int k = ((c + i) * WAVE + lane) << 3;
+                if (live && k < p.K) {
+                    u32x4_t y;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t xn = pack_bf16_rne(bf16_bits_to_f32(h[c + i][e] & 0xFFFFu) * r,
+                                                          bf16_bits_to_f32(h[c + i][e] >> 16) * r);
+                        y[e] = pack_bf16_rne(bf16_bits_to_f32(t[i][e] & 0xFFFFu) * bf16_bits_to_f32(xn & 0xFFFFu),
+                                             bf16_bits_to_f32(t[i][e] >> 16) * bf16_bits_to_f32(xn >> 16));
+                    }
+                    *reinterpret_cast<u32x4_t *>(xs + m * xstride + k) = y;
+                }
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ void stage_x_norm(const DevProblem &p, const NormArgs &n, int kext, uint16_t *xs,
                                              int xstride, int nwaves, bool write_h, float *scratch) {
     // rows up to 2048 wide keep half the registers (the 16-wave workgroups have 128 per lane)
@@ -231,7 +327,7 @@ __device__ __forceinline__ void stage_x_norm(const DevProblem &p, const NormArgs
     int split = 1;
     while (2 * split * p.M <= nwaves && 2 * split <= words) split *= 2;
     switch (words / split) {
-        case 8: stage_x_norm_rows<8>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
+        case 8: stage_x_norm_rows_wide(p, n, kext, xs, xstride, nwaves, write_h); break;  // split == 1 here
         case 4: stage_x_norm_rows<4>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
         case 2: stage_x_norm_rows<2>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
         default: stage_x_norm_rows<1>(p, n, kext, xs, xstride, nwaves, write_h, split, scratch); break;
