@@ -556,8 +556,9 @@ def decode_head_and_tail(device, steps: int, heads: int = 16):
 
 def ar_decode_loop(device, tokens: int = 48, only: str | None = None, batches=(1, 16), prompt: int = 304,
                    shape=(HIDDEN, INTER, LAYERS, 16)):
-    """ms per decode step of the image-token loop on a Janus-Pro-1B shaped policy (random weights), at
-    cache lengths around the middle of a 576-token image (a 304-token context, then 48 tokens).
+    """ms per decode step of the image-token loop on a Janus-Pro-1B shaped policy (random weights) after a
+    context of ``prompt`` tokens (304 by default, then 48 generated tokens: where a generation over a
+    256-slot prompt starts; its middle is at 544 slots, its end at 832).
 
     ``reference_style`` is the loop of vrl/models/families/janus_pro/policy.py:624-731 with the trunk's
     dynamic cache and the torch formulas for the tail, without its per-row cache copies and host
@@ -1010,6 +1011,17 @@ def main():
     except Exception as exc:
         ar_loop = {"error": repr(exc)[:300]}
     torch.cuda.empty_cache()
+    # the same step where a generation over a prompt padded to 256 slots spends its time: around slot
+    # 256 + 288 (its middle) and around slot 800 (its end)
+    for name, ctx in (("B1_at_544_slots", 520), ("B1_at_808_slots", 784)):
+        try:
+            long_run = ar_decode_loop(device, only="int4_native_hip_graph", batches=(1,), prompt=ctx)
+            if isinstance(ar_loop, dict):
+                ar_loop[name] = long_run["B1"]
+        except Exception as exc:
+            if isinstance(ar_loop, dict):
+                ar_loop[name] = {"error": repr(exc)[:300]}
+        torch.cuda.empty_cache()
 
     try:
         others = other_configs(device, args.steps, args.warmup)
@@ -1028,6 +1040,11 @@ def main():
             chain = {"what": "one decode step of a Janus-Pro-1B shaped policy at B=1 (2 rows): 24 dependent layers "
                              "(five launches each), head and sampling tail, replayed from one HIP graph",
                      "ms_per_step": step_ms, "GBps_of_int4_weights": step_bytes / (step_ms * 1e-3) / 1e9,
+                     "cache_slots": "304 + 48 (the start of a generation); ms_per_step_at_544_slots: its middle",
+                     "ms_per_step_at_544_slots": (ar_loop.get("B1_at_544_slots") or {}).get(
+                         "int4_native_hip_graph_ms_per_token"),
+                     "ms_per_step_at_808_slots": (ar_loop.get("B1_at_808_slots") or {}).get(
+                         "int4_native_hip_graph_ms_per_token"),
                      "linears_only_4_launches_per_layer_hip_graph_ms": strat["ms_per_step"].get(
                          "per_layer_4_launches_hip_graph")}
 

@@ -20,6 +20,7 @@
 #ifndef VRL_DECODE_H
 #define VRL_DECODE_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #include "vrl_int4.h"
@@ -59,6 +60,24 @@ int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q
                               const void *mask, const int64_t *position, void *out,
                               int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
                               void *hip_stream);
+
+/*
+ * The same launch for few (row, head) pairs (M * n_heads <= 128; above that it is the launch above): the
+ * cached slots of a pair are divided over 8, 4 or 2 workgroups (for up to 32, 64, 128 pairs), so that
+ * a long cache is read by many compute units instead of one per pair; each leaves its running softmax
+ * state in `workspace`, and whichever finishes last merges them in index order and writes `out`
+ * (deterministic; no workgroup waits for another).  Results equal the launch above up to the order of
+ * the fp32 sums.  `workspace`: vrl_rope_attn_decode_split_workspace_bytes(M, n_heads, D) bytes of device
+ * memory, 256-byte aligned, whose first M * n_heads * 4 bytes are zero before the first launch (every
+ * launch leaves them zero again); launches that share a workspace must be ordered by the stream.
+ * No counterpart in the reference (its attention is the library's, policy.py:673-678).
+ */
+size_t vrl_rope_attn_decode_split_workspace_bytes(int M, int n_heads, int D);
+int vrl_rope_attn_decode_split_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                    void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                    const void *mask, const int64_t *position, void *out,
+                                    int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                    void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
  * LoRA adapters on top of an int4 projection, for the decode step of a policy whose attention

@@ -287,11 +287,15 @@ def int4_policy():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("native", [False, True])
-def test_graph_replays_equal_eager_steps(int4_policy, native):
+@pytest.mark.parametrize("native", [False, True, "split"])
+def test_graph_replays_equal_eager_steps(int4_policy, native, monkeypatch):
     """Every replayed step against the same step run eagerly: tokens and log-probabilities bit for bit,
     over two calls (the second reuses the recorded graph) with eager work and syncs in between."""
     print("ar decode: graph vs eager, native trunk", native, flush=True)
+    if native == "split":   # the attention's split form whatever the cache length
+        from visionrl_amd.decode_step import NativeDecodeTrunk
+        monkeypatch.setattr(NativeDecodeTrunk, "SPLIT_ATTENTION_FROM", 0)
+        native = True
     eager = StaticARSampler(int4_policy, graph=False, native=native)
     graphed = StaticARSampler(int4_policy, graph=True, native=native)
     for call, (n_text, n_img, seed) in enumerate(((7, 24, 21), (11, 20, 22), (7, 24, 21))):
@@ -330,11 +334,15 @@ def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy, 
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("side", ["left", "right"])
-def test_native_trunk_tracks_the_module_trunk(int4_policy, side):
+@pytest.mark.parametrize("side,split", [("left", False), ("right", False), ("left", True)])
+def test_native_trunk_tracks_the_module_trunk(int4_policy, side, split, monkeypatch):
     """Teacher-forced: both trunks consume the same inputs step after step, each over its own cache;
-    hidden states and appended cache rows stay within bf16 roundings of each other."""
+    hidden states and appended cache rows stay within bf16 roundings of each other (also with the
+    attention in its split form, which long caches of few rows take)."""
     print("ar decode: native trunk vs module trunk", flush=True)
+    if split:
+        from visionrl_amd.decode_step import NativeDecodeTrunk
+        monkeypatch.setattr(NativeDecodeTrunk, "SPLIT_ATTENTION_FROM", 0)
     rows, n_text, steps = 6, 7, 12
     cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=41, side=side)
     sessions = []

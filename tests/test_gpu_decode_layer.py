@@ -95,6 +95,128 @@ def test_rope_attn_decode_parity(ops_mod, M, H, Hkv, D, L, p):
     assert (np.abs(got - want) <= tol).all(), np.abs(got - want).max()
 
 
+SPLIT_CASES = [
+    # M, H, Hkv, D, L, p: 8 workgroups per pair up to 32 pairs, 4 up to 64, 2 up to 128; ranges of multiples of 64
+    # slots: empty ranges, one partly filled range, exact multiples, a long cache
+    (2, 16, 16, 128, 896, 0), (2, 16, 16, 128, 896, 1), (2, 16, 16, 128, 896, 63), (2, 16, 16, 128, 896, 64),
+    (2, 16, 16, 128, 896, 65), (2, 16, 16, 128, 896, 330), (2, 16, 16, 128, 896, 512), (2, 16, 16, 128, 896, 830),
+    (2, 16, 16, 128, 896, 895), (4, 16, 16, 128, 384, 300), (8, 16, 16, 128, 384, 383), (1, 6, 3, 64, 48, 47),
+    (2, 8, 2, 128, 2048, 2000), (3, 4, 4, 64, 8192, 5000),
+]
+
+
+def run_attn_split(ops_mod, c, ws, out=None):
+    t = {k: bits_to_bf16(c[k], DEV) for k in ("q", "k", "v", "kc", "vc", "cos", "sin")}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([c["p"]], dtype=torch.int64, device=DEV)
+    out = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], t["kc"], t["vc"], t["cos"], t["sin"], mask, pos,
+                                   c["scaling"], split_workspace=ws, out=out)
+    return out, t["kc"], t["vc"]
+
+
+@pytest.mark.parametrize("M,H,Hkv,D,L,p", SPLIT_CASES)
+def test_split_rope_attn_decode_parity(ops_mod, M, H, Hkv, D, L, p):
+    """The slots of a (row, head) pair divided over several workgroups, merged by the last to finish:
+    same oracle, same bound, same cache update as the one-workgroup form; counters back at zero."""
+    say("rope_attn split", M, H, Hkv, D, L, p)
+    c = attn_case(3000 + p + L, M, H, Hkv, D, L, p)
+    want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
+                                                c["mask"], p, H, Hkv, c["scaling"])
+    ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV)
+    out, kc, vc = run_attn_split(ops_mod, c, ws)
+    torch.cuda.synchronize()
+    assert (bf16_to_bits(kc) == kc_want).all() and (bf16_to_bits(vc) == vc_want).all()
+    got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)
+    tol = 0.51 * o.bf16_ulp(want.astype(np.float32)) + 2e-5 * np.abs(want).max()
+    assert (np.abs(got - want) <= tol).all(), np.abs(got - want).max()
+    assert int(ws[: M * H * 4].view(torch.int32).abs().sum()) == 0          # ready for the next launch
+    # the one-workgroup launch over the same inputs: equal up to the order of the fp32 sums
+    plain, _, _ = run_attn(ops_mod, c)
+    dist = ulp_distance(bf16_to_bits(out), bf16_to_bits(plain))
+    assert dist.max() <= 1 and (dist > 0).mean() < 0.02
+
+
+def test_split_rope_attn_launches_share_one_workspace(ops_mod):
+    """Forty launches back to back over one workspace, every one with other inputs, positions and masks,
+    checked afterwards: a launch must read what its own workgroups wrote, never what an earlier launch
+    left in the workspace or in a cache; masked slots and an all-masked row included."""
+    say("rope_attn split, repeated launches")
+    M, H, D, L = 2, 16, 128, 640
+    ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV)
+    rng = np.random.default_rng(77)
+    runs = []
+    for i in range(40):
+        p = int(rng.integers(0, L))
+        c = attn_case(4000 + i, M, H, H, D, L, p)
+        if i % 5 == 1:
+            c["mask"][0, : max(1, p // 2)] = 0
+        if i % 7 == 3:
+            c["mask"][1, :] = 0
+        runs.append((c, run_attn_split(ops_mod, c, ws)))                  # enqueued, not yet checked
+    torch.cuda.synchronize()
+    for c, (out, kc, vc) in runs:
+        want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
+                                                    c["mask"], c["p"], H, H, c["scaling"])
+        assert (bf16_to_bits(kc) == kc_want).all() and (bf16_to_bits(vc) == vc_want).all()
+        got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)
+        dead = ~c["mask"][:, : c["p"] + 1].any(axis=1)        # nothing attendable: the launch writes zeros
+        assert (got[dead] == 0).all()
+        want, got = want[~dead], got[~dead]
+        tol = 0.51 * o.bf16_ulp(want.astype(np.float32)) + 2e-5 * np.abs(want).max()
+        assert (np.abs(got - want) <= tol).all(), (c["p"], np.abs(got - want).max())
+
+
+def test_split_rope_attn_in_a_graph_equals_eager(ops_mod):
+    """Recorded once, replayed with eager launches and synchronisations between the replays, the position
+    advancing as in a decode loop: every replay equals the eager launch bit for bit (the merge runs in
+    index order whichever workgroup arrives last)."""
+    say("rope_attn split, graph replay")
+    M, H, D, L = 2, 16, 128, 512
+    c = attn_case(4100, M, H, H, D, L, 200)
+    t = {k: bits_to_bf16(c[k], DEV) for k in ("q", "k", "v", "kc", "vc", "cos", "sin")}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([200], dtype=torch.int64, device=DEV)
+    ws, ws_eager = (ops_mod.rope_attn_split_workspace(M, H, D, DEV) for _ in range(2))
+    out = torch.empty((M, H * D), dtype=torch.bfloat16, device=DEV)
+    call = lambda kc, vc, w, o_: ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc, vc, t["cos"], t["sin"], mask,
+                                                           pos, c["scaling"], split_workspace=w, out=o_)
+    kc_g, vc_g = t["kc"].clone(), t["vc"].clone()
+    call(kc_g, vc_g, ws, out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(kc_g, vc_g, ws, out)
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    kc_e, vc_e = kc_g.clone(), vc_g.clone()
+    for step in range(6):
+        pos.fill_(201 + 37 * step)
+        for name in ("q", "k", "v"):
+            t[name].copy_((torch.randn(t[name].shape, generator=gen, device=DEV) * 0.7).to(torch.bfloat16))
+        want = call(kc_e, vc_e, ws_eager, None)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(kc_g, kc_e) and torch.equal(vc_g, vc_e)
+
+
+def test_split_rope_attn_refuses_what_it_does_not_take(ops_mod):
+    c = attn_case(4200, 2, 4, 4, 64, 32, 5)
+    t = [bits_to_bf16(c[n], DEV) for n in ("q", "k", "v", "kc", "vc", "cos", "sin")]
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.tensor([5], dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(*t, mask, pos, 0.125, split_workspace=torch.zeros(64, dtype=torch.uint8, device=DEV))
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(*t, mask, pos, 0.125,
+                                 split_workspace=ops_mod.rope_attn_split_workspace(2, 4, 64, DEV).float())
+    # more pairs than the split form is for: the same entry point runs the one-workgroup launch
+    big = attn_case(4201, 16, 16, 16, 64, 32, 7)
+    ws = ops_mod.rope_attn_split_workspace(16, 16, 64, DEV)
+    out, _, _ = run_attn_split(ops_mod, big, ws)
+    plain, _, _ = run_attn(ops_mod, big)
+    assert torch.equal(out, plain)
+
+
 def test_rope_attn_masks_and_strided_inputs(ops_mod):
     say("rope_attn masks, fused qkv buffer")
     M, H, D, L, p = 2, 4, 64, 32, 20

@@ -34,6 +34,8 @@ SYMBOLS = (
     "vrl_int4_head_sample_static_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
+    "vrl_rope_attn_decode_split_workspace_bytes",
+    "vrl_rope_attn_decode_split_bf16",
     "vrl_rope_attn_decode_lora_bf16",
     "vrl_lora_down_bf16",
     "vrl_lora_up_add_bf16",
@@ -185,6 +187,11 @@ def _bind(lib):
     lib.vrl_rope_attn_decode_bf16.restype = ci
     lib.vrl_rope_attn_decode_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                               ci, ci, ci, ci, ci, ctypes.c_float, vp]
+    lib.vrl_rope_attn_decode_split_workspace_bytes.restype = ctypes.c_size_t
+    lib.vrl_rope_attn_decode_split_workspace_bytes.argtypes = [ci, ci, ci]
+    lib.vrl_rope_attn_decode_split_bf16.restype = ci
+    lib.vrl_rope_attn_decode_split_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
+                                                    ci, ci, ci, ci, ci, ctypes.c_float, vp, ctypes.c_size_t, vp]
 
 
 def load():

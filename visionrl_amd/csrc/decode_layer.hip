@@ -103,6 +103,8 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_kernel(const uint16_t *x,
 }
 
 // ---------------------------------------------------------------- rotary + cache append + attention
+constexpr int ATTN_MAX_SPLITS = 8;   // workgroups that share the cached slots of one (row, head) in the split form
+
 struct AttnArgs {
     const uint16_t *q, *k, *v;
     uint16_t *k_cache, *v_cache;
@@ -123,6 +125,9 @@ struct AttnArgs {
     const void *oa;          // A [orank, n_heads * D], nullptr for none
     float *ot;               // [M, n_heads, orank]
     int orank;
+    // SPLIT instantiations: the cached slots of a (row, head) are divided over gridDim.z workgroups
+    uint32_t *arrived;       // [M, n_heads] counters, zero between launches
+    float *partials;         // [M, n_heads, gridDim.z, D + 2]: unnormalised output, maximum, sum
 };
 
 // Raw cache vectors: D / 16 bf16 values of one slot per lane (16 or 8 bytes).
@@ -182,8 +187,18 @@ __device__ __forceinline__ void merge(Partial<VEC> &a, float m2, float l2, const
 // the groups, the waves and the new token's own slot are merged at the end.
 // ATT_UNROLL: slots per 16-lane group in flight (keys and values: 2 * ATT_UNROLL vector loads per lane)
 // LORA: 0 none, 1 float32 adapter weights, 2 bf16 adapter weights
-template <int D, int ATT_WAVES, int ATT_UNROLL, int LORA, bool STREAMED>
+// SPLIT: with few (row, head) pairs a workgroup's compute unit becomes the limit (its vector memory path
+// moves 64 bytes per cycle: 128 KB of keys and values per 256 slots take 2.9 us, and a cache of 830
+// slots four such trips), so gridDim.z workgroups share the slots of a pair, a contiguous range each.
+// Each leaves its running softmax state (unnormalised output, maximum, sum) in `partials` and counts
+// itself in `arrived`; whichever counts last merges the states in index order (the same sums
+// whatever the order of arrival), writes the output and clears the counter.  Nobody waits for anybody.
+// The states and the counter are exchanged through device-scope atomic stores, loads and adds (they
+// bypass the per-XCD caches), and a workgroup counts itself only when its stores have completed, so
+// no cache write-back or invalidate is needed.
+template <int D, int ATT_WAVES, int ATT_UNROLL, int LORA, bool STREAMED, bool SPLIT = false>
 __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnArgs a) {
+    static_assert(!SPLIT || LORA == 0, "the split form carries no adapters");
     constexpr int VEC = D / 16;
     __shared__ float qs[D];                 // rotated query
     __shared__ float ks[D];                 // rotated key of the new token
@@ -191,6 +206,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     __shared__ float pm[ATT_WAVES], pl[ATT_WAVES];
     __shared__ float pacc[ATT_WAVES][D];
     __shared__ float s_new;                 // score of the new token's own slot
+    __shared__ uint32_t s_before;           // SPLIT: workgroups of the pair that had arrived before this one
 
     const long long p64 = *a.position;
     if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the grid
@@ -205,22 +221,31 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
     const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
     constexpr int STEP = 4 * ATT_WAVES * ATT_UNROLL;  // slots the workgroup visits per batch
+    // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
+    // multiple of 64 slots (what the workgroup's waves visit together)
+    const int n_split = SPLIT ? (int)gridDim.z : 1, split = SPLIT ? (int)blockIdx.z : 0;
+    int j_lo = 0, j_hi = p;
+    if constexpr (SPLIT) {
+        const int share = ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
+        j_lo = min(p, split * share);
+        j_hi = min(p, j_lo + share);
+    }
 
     // The cached slots do not depend on the new token: the first batch of keys and values is
     // requested before anything else and arrives while the query is rotated.
     RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
     bool live[ATT_UNROLL];
-    auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs p >= 1
+    auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs j_hi > j_lo
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             const int j = j0 + u * 4 * ATT_WAVES + wave * 4 + sub;
-            const int jj = j < p ? j : p - 1;  // slots past the end repeat the last one and are not counted
+            const int jj = j < j_hi ? j : j_hi - 1;  // slots past the end repeat the last one and are not counted
             kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
             vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
-            live[u] = j < p && mask[jj] != 0;
+            live[u] = j < j_hi && mask[jj] != 0;
         }
     };
-    if (p > 0) request(0);
+    if (j_hi > j_lo) request(j_lo);
 
     // The adapter of the projection that follows: thread (j, l16) holds the lane's VEC columns of row j
     // of A (rows j, j + OJ, ... if the rank exceeds OJ; the first is requested here, ahead of its use).
@@ -321,7 +346,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         qs[tid] = qe;
         ks[tid] = ke;
         vs[tid] = v_own;
-        if (h % group == 0) {  // one workgroup per kv head appends; readers of slot p use their own copy
+        if (h % group == 0 && split == 0) {  // one workgroup per kv head appends; readers of slot p use their own copy
             a.k_cache[cache_base + (long)p * D + tid] = (uint16_t)f32_to_bf16_bits(ke);
             a.v_cache[cache_base + (long)p * D + tid] = (uint16_t)f32_to_bf16_bits(v_own);
         }
@@ -341,7 +366,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         float dot = 0.0f;
         for (int d = lane; d < D; d += WAVE) dot += qs[d] * ks[d];
         dot = wave_sum(dot);
-        if (lane == 0) s_new = mask[p] ? dot * a.scaling : -INFINITY;
+        if (lane == 0) s_new = (mask[p] && split == 0) ? dot * a.scaling : -INFINITY;  // one workgroup of a pair counts it
     }
 
     Partial<VEC> st;
@@ -353,8 +378,8 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     // cached slots 0..p-1, a batch per trip; the batch of the first trip is already on its way.
     // The running softmax is rescaled once per batch: one maximum over the batch's scores and the
     // state, one exponential per score and one for the state.
-    for (int j0 = 0; j0 < p; j0 += STEP) {
-        if (j0 > 0) request(j0);
+    for (int j0 = j_lo; j0 < j_hi; j0 += STEP) {
+        if (j0 > j_lo) request(j0);
         float sc[ATT_UNROLL];
         float mx = st.m;
 #pragma unroll
@@ -417,11 +442,59 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
                 o += c * pacc[w][tid];
                 sum += c * pl[w];
             }
-            o /= sum;
+            if constexpr (!SPLIT) o /= sum;
         }
-        const uint32_t bits = f32_to_bf16_bits(o);
-        a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)bits;
-        if constexpr (LORA != 0) qs[tid] = bf16_to_f32(bits);  // what the next projection reads
+        if constexpr (SPLIT) {
+            // this workgroup's state: o and sum relative to mx (zeros and -inf if it saw nothing attendable)
+            float *mine = a.partials + (((long)m * a.n_heads + h) * n_split + split) * (D + 2);
+            __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) {
+                __hip_atomic_store(mine + D, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(mine + D + 1, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have completed before the workgroup counts itself
+        } else {
+            const uint32_t bits = f32_to_bf16_bits(o);
+            a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)bits;
+            if constexpr (LORA != 0) qs[tid] = bf16_to_f32(bits);  // what the next projection reads
+        }
+    }
+    if constexpr (SPLIT) {
+        uint32_t *count = a.arrived + (long)m * a.n_heads + h;
+        __syncthreads();
+        if (tid == 0) s_before = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_before != (uint32_t)(n_split - 1)) return;  // uniform: somebody else arrives last
+        if (tid < D) {
+            const float *all = a.partials + ((long)m * a.n_heads + h) * n_split * (D + 2);
+            // every state is requested before any is used: one memory round trip
+            float pm_[ATTN_MAX_SPLITS], ps_[ATTN_MAX_SPLITS], po_[ATTN_MAX_SPLITS];
+#pragma unroll
+            for (int z = 0; z < ATTN_MAX_SPLITS; ++z) {
+                pm_[z] = -INFINITY, ps_[z] = 0.0f, po_[z] = 0.0f;
+                if (z < n_split) {
+                    const float *part = all + z * (D + 2);
+                    pm_[z] = __hip_atomic_load(part + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ps_[z] = __hip_atomic_load(part + D + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    po_[z] = __hip_atomic_load(part + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int z = 0; z < ATTN_MAX_SPLITS; ++z) mx = fmaxf(mx, pm_[z]);
+            float o = 0.0f, sum = 0.0f;
+            if (mx != -INFINITY) {
+#pragma unroll
+                for (int z = 0; z < ATTN_MAX_SPLITS; ++z) {   // index order: the same sums whoever merges
+                    const float c = __expf(pm_[z] - mx);
+                    o += c * po_[z];
+                    sum += c * ps_[z];
+                }
+                o /= sum;
+            }
+            a.out[((long)m * a.n_heads + h) * D + tid] = (uint16_t)f32_to_bf16_bits(o);
+        }
+        if (tid == 0) __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     }
     if constexpr (LORA != 0) {
         if (a.oa) {  // uniform
@@ -588,9 +661,30 @@ void launch_attn_build(const AttnArgs &a, int M, int D, hipStream_t stream) {
 // layers together then exceed the memory-side cache, and nothing of them survives to the next step
 constexpr long STREAMED_CACHE_BYTES = 10L << 20;
 
+// the split form: `splits` workgroups of 16 waves per (row, head)
+int attn_splits(long pairs) { return pairs <= 32 ? 8 : (pairs <= 64 ? 4 : (pairs <= 128 ? 2 : 1)); }
+size_t attn_counter_bytes(long pairs) { return (size_t)(pairs * sizeof(uint32_t) + 255) / 256 * 256; }
+
+template <bool STREAMED>
+void launch_attn_split(const AttnArgs &a, int M, int D, int splits, hipStream_t stream) {
+    const dim3 grid(a.n_heads, M, splits);
+    if (D == 128)
+        hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4, 0, STREAMED, true>), grid, dim3(16 * WAVE), 0, stream, a);
+    else
+        hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4, 0, STREAMED, true>), grid, dim3(16 * WAVE), 0, stream, a);
+}
+
 template <int LORA>
 void launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
     const long cache_bytes = (long)M * a.n_kv_heads * a.L_max * D * 2 * 2;
+    if constexpr (LORA == 0) {
+        const int splits = a.partials ? attn_splits((long)a.n_heads * M) : 1;
+        if (splits > 1) {
+            if (cache_bytes > STREAMED_CACHE_BYTES) launch_attn_split<true>(a, M, D, splits, stream);
+            else launch_attn_split<false>(a, M, D, splits, stream);
+            return;
+        }
+    }
     if (cache_bytes > STREAMED_CACHE_BYTES) launch_attn_build<LORA, true>(a, M, D, stream);
     else launch_attn_build<LORA, false>(a, M, D, stream);
 }
@@ -598,7 +692,7 @@ void launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
 int attn_decode(const void *q, const void *k, const void *v, int q_stride, int kv_stride, void *k_cache,
                 void *v_cache, const void *cos, const void *sin, const void *mask, const int64_t *position,
                 void *out, int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
-                const vrl_attn_lora *lora, void *hip_stream) {
+                const vrl_attn_lora *lora, void *hip_stream, void *workspace = nullptr, size_t workspace_bytes = 0) {
     if (!q || !k || !v || !k_cache || !v_cache || !cos || !sin || !mask || !position || !out) return VRL_INT4_ENULL;
     if (M < 1 || M > 65535 || n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || n_heads > 65535 ||
         (D != 64 && D != 128) || L_max < 1 || L_max > MAX_CACHE_LEN || q_stride < n_heads * D ||
@@ -627,6 +721,15 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
     a.L_max = L_max;
     a.scaling = scaling;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    if (workspace) {
+        const long pairs = (long)n_heads * M;
+        const size_t need = attn_counter_bytes(pairs) + (size_t)pairs * ATTN_MAX_SPLITS * (D + 2) * sizeof(float);
+        if (lora) return VRL_INT4_ESHAPE;
+        if (workspace_bytes < need) return VRL_INT4_EPLAN;
+        if (misaligned(workspace, 256)) return VRL_INT4_EALIGN;
+        a.arrived = static_cast<uint32_t *>(workspace);
+        a.partials = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + attn_counter_bytes(pairs));
+    }
     if (!lora) {
         launch_attn<0>(a, M, D, stream);
         return (int)hipGetLastError();
@@ -672,6 +775,22 @@ extern "C" int vrl_rope_attn_decode_bf16(const void *q, const void *k, const voi
                                          void *hip_stream) {
     return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, position, out, M, n_heads,
                        n_kv_heads, D, L_max, scaling, nullptr, hip_stream);
+}
+
+extern "C" size_t vrl_rope_attn_decode_split_workspace_bytes(int M, int n_heads, int D) {
+    if (M < 1 || n_heads < 1 || (D != 64 && D != 128) || (long)M * n_heads > (1L << 24)) return 0;
+    const long pairs = (long)n_heads * M;
+    return attn_counter_bytes(pairs) + (size_t)pairs * ATTN_MAX_SPLITS * (D + 2) * sizeof(float);
+}
+
+extern "C" int vrl_rope_attn_decode_split_bf16(const void *q, const void *k, const void *v, int q_stride,
+                                               int kv_stride, void *k_cache, void *v_cache, const void *cos,
+                                               const void *sin, const void *mask, const int64_t *position, void *out,
+                                               int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                               void *workspace, size_t workspace_bytes, void *hip_stream) {
+    if (!workspace) return VRL_INT4_ENULL;
+    return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, position, out, M, n_heads,
+                       n_kv_heads, D, L_max, scaling, nullptr, hip_stream, workspace, workspace_bytes);
 }
 
 extern "C" int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, int q_stride,

@@ -138,6 +138,8 @@ class NativeDecodeTrunk:
     scalar holding the cache slot the new token takes; :meth:`run` leaves ``slot`` untouched.
     """
 
+    SPLIT_ATTENTION_FROM = 512   # cache slots from which the attention of few rows runs in its split form
+
     @staticmethod
     def unsupported(trunk, rows: int, max_len: int) -> str | None:
         """Why this trunk cannot run natively at ``rows`` rows, or ``None`` if it can."""
@@ -195,6 +197,13 @@ class NativeDecodeTrunk:
         self._keep = [cache, cur, mask, slot, streams]
         lib = _lib.load()
         fuse_norm = hidden <= 4096   # the linears normalise their input while staging it
+        # With few (row, head) pairs and a cache that grows long the attention divides a pair's cached slots
+        # over several workgroups (one workspace for all layers: the launches are ordered by the stream).
+        # Its exchange costs about 1.5 us per launch, which pays from about 400 cached slots on (at 2 rows
+        # a step takes 0.87 / 0.89 / 0.90 ms at 330 / 590 / 830 slots against 0.84 / 0.94 / 1.02 ms).
+        split_ws = ops.rope_attn_split_workspace(rows, H, D, dev) \
+            if rows * H <= 128 and self.max_len >= self.SPLIT_ATTENTION_FROM else None
+        self._keep.append(split_ws)
         calls = []       # (function, argument tuple without the stream)
         state = {"x": cur.view(rows, hidden), "res": None, "flip": 0}   # x: sublayer output not yet added to res
 
@@ -285,8 +294,13 @@ class NativeDecodeTrunk:
                 record = o_group.attn_output_record(record)
                 calls[launch_at] = (lib.vrl_int4_gemv_prepacked_lora_up_bf16,
                                     (calls[launch_at][1][0], o_group.table, o_group.t.data_ptr(), H))
-            calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args) if record is None else \
-                (lib.vrl_rope_attn_decode_lora_bf16, (*attn_args, ctypes.byref(record)))
+            if record is not None:
+                calls[attn_at] = (lib.vrl_rope_attn_decode_lora_bf16, (*attn_args, ctypes.byref(record)))
+            elif split_ws is not None:
+                calls[attn_at] = (lib.vrl_rope_attn_decode_split_bf16,
+                                  (*attn_args, split_ws.data_ptr(), split_ws.numel()))
+            else:
+                calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args)
             (state["x"],) = outs
             (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
             (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])

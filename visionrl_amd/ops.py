@@ -26,7 +26,7 @@ from .int4_format import check_packed
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
            "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "head_sample", "head_sample_supported",
-           "head_sample_workspace", "add_rmsnorm",
+           "head_sample_workspace", "add_rmsnorm", "rope_attn_split_workspace",
            "rope_attn_decode", "LoraAdd"]
 
 
@@ -672,7 +672,8 @@ def add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: tor
 def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
                      v_cache: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mask: torch.Tensor,
                      position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None,
-                     lora: "LoraAdd | None" = None, out_lora: "LoraAdd | None" = None) -> torch.Tensor:
+                     lora: "LoraAdd | None" = None, out_lora: "LoraAdd | None" = None,
+                     split_workspace: torch.Tensor | None = None) -> torch.Tensor:
     """Rotary embedding, cache append and attention for one new token per row, one launch.
 
     ``q [M, H*D]``, ``k, v [M, Hkv*D]`` bf16 (rows may be strided views of one buffer), caches
@@ -684,6 +685,9 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
     was launched: the attention then adds the up-projections itself (q, k, v stay as they are).
     ``out_lora`` is a :class:`LoraAdd` with one adapter over ``out`` built with ``parts = H``: the launch
     leaves that adapter's down-projection in its ``t``, one piece per head, for its ``launch_up``.
+    ``split_workspace`` (from :func:`rope_attn_split_workspace`, without adapters): with at most 128
+    (row, head) pairs several workgroups share the cached slots of a pair and the last one to finish
+    merges their results (``vrl_rope_attn_decode_split_bf16``); launches over one workspace must not overlap.
     """
     dev = _require_device("k_cache", k_cache)
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.dtype != torch.bfloat16 or \
@@ -721,13 +725,32 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
         if out_lora.x.data_ptr() != out.data_ptr() or out_lora.parts != H:
             raise ValueError("out_lora must be built over `out` with one part per head")
         record = out_lora.attn_output_record(record)
+    if split_workspace is not None:
+        if record is not None:
+            raise ValueError("the split form of the attention carries no adapters")
+        need = _lib.load().vrl_rope_attn_decode_split_workspace_bytes(M, H, D)
+        if split_workspace.dtype != torch.uint8 or split_workspace.numel() < need or \
+                not split_workspace.is_contiguous() or split_workspace.device != dev:
+            raise ValueError(f"split_workspace must be a contiguous uint8 tensor of {need} bytes on {dev}")
     with _on(dev):
-        if record is None:
+        if split_workspace is not None:
+            rc = _lib.load().vrl_rope_attn_decode_split_bf16(*args, split_workspace.data_ptr(),
+                                                             split_workspace.numel(), _stream_handle(dev))
+        elif record is None:
             rc = _lib.load().vrl_rope_attn_decode_bf16(*args, _stream_handle(dev))
         else:
             rc = _lib.load().vrl_rope_attn_decode_lora_bf16(*args, ctypes.byref(record), _stream_handle(dev))
     _lib.check(rc, "vrl_rope_attn_decode_bf16")
     return out
+
+
+def rope_attn_split_workspace(M: int, H: int, D: int, device) -> torch.Tensor:
+    """Zeroed scratch memory for the split form of :func:`rope_attn_decode` (counters, which every launch
+    leaves at zero again, and the workgroups' partial results); one per stream of launches."""
+    nbytes = _lib.load().vrl_rope_attn_decode_split_workspace_bytes(int(M), int(H), int(D))
+    if nbytes == 0:
+        raise ValueError("no split form for this shape")
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device)
 
 
 class LoraAdd:
