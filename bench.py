@@ -865,6 +865,9 @@ def main():
     ap.add_argument("--lora", action="store_true", help="with --ar-decode: LoRA adapters on q/k/v/o_proj")
     ap.add_argument("--ar-decode", type=int, default=0, metavar="B",
                     help="run only the recorded decode loop at batch B on the int4 policy and exit (for profilers)")
+    ap.add_argument("--context", type=int, default=304, metavar="SLOTS",
+                    help="with --ar-decode: tokens in the cache before the timed steps (304: the start of a "
+                         "generation, 520: its middle, 784: its end)")
     ap.add_argument("--trunk-7b", action="store_true",
                     help="with --ar-decode: the 7B-class trunk (30 x (4096, 11008), 32 heads) instead of the 1B one")
     ap.add_argument("--attn-decode", type=int, default=0, metavar="ROWS",
@@ -912,7 +915,8 @@ def main():
     if args.ar_decode:
         which = "int4_lora_native_hip_graph" if args.lora else "int4_native_hip_graph"
         shape = (4096, 11008, 30, 32) if args.trunk_7b else (HIDDEN, INTER, LAYERS, 16)
-        print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,), shape=shape)))
+        print(json.dumps(ar_decode_loop(device, only=which, batches=(args.ar_decode,), shape=shape,
+                                        prompt=args.context)))
         return
     if args.single_calls:
         for M in (1, 32):
