@@ -132,8 +132,9 @@ def test_split_rope_attn_decode_parity(ops_mod, M, H, Hkv, D, L, p):
     assert int(ws[: M * H * 4].view(torch.int32).abs().sum()) == 0          # ready for the next launch
     # the one-workgroup launch over the same inputs: equal up to the order of the fp32 sums
     plain, _, _ = run_attn(ops_mod, c)
-    dist = ulp_distance(bf16_to_bits(out), bf16_to_bits(plain))
-    assert dist.max() <= 1 and (dist > 0).mean() < 0.02
+    fa, fb = out.float(), plain.float()
+    assert bool(((fa - fb).abs() <= fb.abs() * 2.0 ** -7 + 4e-5 * fb.abs().max()).all())
+    assert float((out != plain).float().mean()) < 0.02
 
 
 def test_split_rope_attn_launches_share_one_workspace(ops_mod):
@@ -164,6 +165,43 @@ def test_split_rope_attn_launches_share_one_workspace(ops_mod):
         want, got = want[~dead], got[~dead]
         tol = 0.51 * o.bf16_ulp(want.astype(np.float32)) + 2e-5 * np.abs(want).max()
         assert (np.abs(got - want) <= tol).all(), (c["p"], np.abs(got - want).max())
+
+
+def test_split_rope_attn_tracks_the_one_workgroup_form_over_many_launches(ops_mod):
+    """Three hundred launches of both forms over one set of buffers, the position walking through a long cache
+    and the new token changing every time, results compared on the device: within one bf16 step of each other
+    (or, where an output cancels to almost nothing, within the fp32 noise of its terms), and different at all in
+    fewer than 2 % of the outputs (the forms differ in the order of their fp32 sums only); a state left over from an earlier launch
+    or a merge that ran before a state had arrived would be off by far more."""
+    say("rope_attn split vs one-workgroup form, 300 launches")
+    M, H, D, L = 2, 16, 128, 896
+    c = attn_case(4300, M, H, H, D, L, 0)
+    t = {k: bits_to_bf16(c[k], DEV) for k in ("q", "k", "v", "kc", "vc", "cos", "sin")}
+    kc2, vc2 = t["kc"].clone(), t["vc"].clone()
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    pos = torch.zeros(1, dtype=torch.int64, device=DEV)
+    ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV)
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    outs = []
+    for step in range(300):
+        pos.fill_((step * 37) % L)
+        for name in ("q", "k", "v"):
+            t[name].copy_((torch.randn(t[name].shape, generator=gen, device=DEV) * 0.7).to(torch.bfloat16))
+        a = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], t["kc"], t["vc"], t["cos"], t["sin"], mask, pos,
+                                     c["scaling"], split_workspace=ws)
+        b = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc2, vc2, t["cos"], t["sin"], mask, pos, c["scaling"])
+        outs.append((a, b))
+    torch.cuda.synchronize()
+    assert torch.equal(t["kc"], kc2) and torch.equal(t["vc"], vc2)
+    differing = 0.0
+    for a, b in outs:
+        fa, fb = a.float(), b.float()
+        # one bf16 step of the value, or for outputs that cancel to almost nothing the fp32 noise of O(1) terms
+        tol = fb.abs() * 2.0 ** -7 + 4e-5 * fb.abs().max()
+        assert bool(((fa - fb).abs() <= tol).all()), float((fa - fb).abs().max())
+        differing += float((a != b).float().mean())
+    assert differing / len(outs) < 0.02, differing / len(outs)
+    assert int(ws[: M * H * 4].view(torch.int32).abs().sum()) == 0
 
 
 def test_split_rope_attn_in_a_graph_equals_eager(ops_mod):
