@@ -139,6 +139,7 @@ class NativeDecodeTrunk:
     """
 
     SPLIT_ATTENTION_FROM = 512   # cache slots from which the attention of few rows runs in its split form
+    SPLIT_ATTENTION_PAIRS = 128  # (row, head) pairs up to which the library splits a pair's slots
 
     @staticmethod
     def unsupported(trunk, rows: int, max_len: int) -> str | None:
@@ -202,7 +203,7 @@ class NativeDecodeTrunk:
         # Its exchange costs about 1.5 us per launch, which pays from about 400 cached slots on (at 2 rows
         # a step takes 0.87 / 0.89 / 0.90 ms at 330 / 590 / 830 slots against 0.84 / 0.94 / 1.02 ms).
         split_ws = ops.rope_attn_split_workspace(rows, H, D, dev) \
-            if rows * H <= 128 and self.max_len >= self.SPLIT_ATTENTION_FROM else None
+            if rows * H <= self.SPLIT_ATTENTION_PAIRS and self.max_len >= self.SPLIT_ATTENTION_FROM else None
         self._keep.append(split_ws)
         calls = []       # (function, argument tuple without the stream)
         state = {"x": cur.view(rows, hidden), "res": None, "flip": 0}   # x: sublayer output not yet added to res
