@@ -156,8 +156,9 @@ def test_split_rope_attn_launches_share_one_workspace(ops_mod):
         runs.append((c, run_attn_split(ops_mod, c, ws)))                  # enqueued, not yet checked
     torch.cuda.synchronize()
     for c, (out, kc, vc) in runs:
-        want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
-                                                    c["mask"], c["p"], H, H, c["scaling"])
+        with np.errstate(invalid="ignore"):   # the oracle's softmax of a row with nothing attendable is NaN
+            want, kc_want, vc_want = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"],
+                                                        c["mask"], c["p"], H, H, c["scaling"])
         assert (bf16_to_bits(kc) == kc_want).all() and (bf16_to_bits(vc) == vc_want).all()
         got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)
         dead = ~c["mask"][:, : c["p"] + 1].any(axis=1)        # nothing attendable: the launch writes zeros
