@@ -125,9 +125,7 @@ typedef struct vrl_int4_problem {
     int32_t M, N, K, G;
     int32_t fused_gate_up; /* 0: y[M,N]; 1: rows are gate||up, y[M,N/2] with the SiLU epilogue */
     int32_t prepacked;     /* 1: qweight is a blob made by vrl_int4_prepack(); scales/qzeros unused */
-    int32_t reserved[2];   /* 0.  (reserved[0] = 1 on every problem of a grouped plan of plain prepacked M = 1,
-                              G = 128 problems selects the comparison build whose dot product runs on the
-                              vector unit instead of the matrix cores; it is slower and exists to be measured) */
+    int32_t reserved[2];   /* 0 */
 } vrl_int4_problem;
 
 typedef struct vrl_int4_plan_info {

@@ -30,6 +30,10 @@ def to_device(ops: dict, device) -> dict:
 
 # what: [outputs checked, outputs that are cancelled, of those: outputs beyond the strict bound]
 TOLERANCE_LOG: dict = {}
+# the share of a large plan's outputs that may need the extra term of the rule: about one in 10^5 cancel far
+# enough for fp32 reassociation noise to exceed a bf16 step of the result (tests/test_oracle.py shows a plain
+# fp32 sum on the CPU doing the same); a kernel that needs it more often has lost accuracy somewhere
+MAX_FRACTION_BEYOND_STRICT = 2e-5
 
 
 def check_gemv(y: np.ndarray, y_ref: np.ndarray, a_ref: np.ndarray, what: str = "") -> float:
@@ -59,10 +63,15 @@ def check_gemv(y: np.ndarray, y_ref: np.ndarray, a_ref: np.ndarray, what: str = 
     return float((err / np.maximum(a_ref, 1e-300)).max())
 
 
-def report_tolerance(key: str) -> None:
+def report_tolerance(key: str, cap: bool = False) -> None:
+    """Print the counts of ``key``; with ``cap``, fail if more than ``MAX_FRACTION_BEYOND_STRICT`` of the
+    outputs passed on the extra term only (``check_gemv`` has already refused any that is not cancelled)."""
     import sys
 
     n, cancelled, needed = TOLERANCE_LOG.get(key, (0, 0, 0))
+    if cap:
+        assert n > 0 and needed <= MAX_FRACTION_BEYOND_STRICT * n, (
+            f"{key}: {needed} of {n} outputs need the 2^-18 sum|x w| term, more than {MAX_FRACTION_BEYOND_STRICT:g} of them")
     print(f"[tolerance] {key}: {n} outputs, {cancelled} cancelled below 2^-6 sum|x w|, "
           f"{needed} of them beyond max(1 ulp, 1e-2 |y_ref|) (passed on the 2^-18 sum|x w| term)",
           file=sys.stderr, flush=True)

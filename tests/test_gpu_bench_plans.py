@@ -4,7 +4,9 @@
 activation tensor per distinct input of a decoder layer), ``ops.GroupedGemv`` builds the plan the
 benchmark launches (168 records at M = 1; 169 with the head at M = 32, walked in staged passes; 211
 for the 7B-class shapes at M = 1, 8, 16), and every output of every record is compared with
-``oracle.gemv_and_abs_f64`` under the operator tolerance, one matrix at a time.
+``oracle.gemv_and_abs_f64`` under the operator tolerance, one matrix at a time.  Per plan the number of
+outputs that pass only on the rule's extra term for cancelled sums is printed and capped
+(``tests._util.MAX_FRACTION_BEYOND_STRICT``); no output at or above 2^-6 sum|x w| may need it at all.
 """
 
 import sys
@@ -53,7 +55,7 @@ def run_and_check(items_by_rows, label):
             y = o.bf16_bits_to_f32(bf16_to_bits(plans[M].outputs[i])).astype(np.float64)
             check_gemv(y, x @ w.T, np.abs(x) @ np.abs(w).T, f"{label} M={M}: {it['name']}")
     for M in rows:
-        report_tolerance(f"{label} M={M}")
+        report_tolerance(f"{label} M={M}", cap=True)
 
 
 def test_janus_1b_step_m1():

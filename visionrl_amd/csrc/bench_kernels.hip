@@ -6,16 +6,16 @@
 // non-temporal 16-byte loads per lane (one contiguous KiB per wave load, four in flight per lane: the
 // access shape of the prepacked weight stream), folds what it reads into one word and writes that
 // word only if it equals a value the data never produces, so nothing is stored.
+//
+// vrl_bench_gemv_grouped_valu_dot_bf16: the grouped launch of the product library over a plan it built,
+// by the comparison build of its throughput kernel whose dot product runs on the vector unit
+// (v_dot2_f32_bf16) instead of the matrix cores.  It is slower and exists to be measured.
 
-#include <hip/hip_runtime.h>
-#include <stdint.h>
+#include "stream_kernel.hpp"
 
 namespace {
 
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-constexpr int WAVE = 64;
-constexpr int NT = 2;  // cache-policy bit: non-temporal
+constexpr int NT = BUFFER_NT;  // cache-policy bit: non-temporal
 
 // each wave reads `per_wave` bytes (a multiple of 4 KiB) from its own offset; waves past the end read
 // nothing (the buffer range check answers with zeros)
@@ -64,6 +64,26 @@ int vrl_bench_stream_read(const void *buf, size_t bytes, void *sink, int waves_p
     hipLaunchKernelGGL(stream_read_kernel<4>, dim3(waves / 4), dim3(4 * WAVE), 0,
                        reinterpret_cast<hipStream_t>(hip_stream), buf, (uint32_t)bytes, (uint32_t)per_wave,
                        static_cast<uint32_t *>(sink));
+    return (int)hipGetLastError();
+}
+
+// One grouped launch over `plan_dev` (the device copy of a plan made by vrl_int4_grouped_plan_build of the
+// product library) with the vector-unit dot product.  The plan must be the four-wave throughput form over
+// plain prepacked records of group size 128 (variant = prepacked only), and every record must carry one
+// activation row: the caller knows the records, this function sees only the descriptor.  Returns 0, a
+// VRL_INT4_E* code or a hipError_t value.
+int vrl_bench_gemv_grouped_valu_dot_bf16(const void *plan_dev, const vrl_int4_plan_info *info, void *hip_stream) {
+    if (!plan_dev || !info) return VRL_INT4_ENULL;
+    if (info->variant != VARIANT_PP || info->block_threads != 4 * WAVE || info->n_problems < 1 || info->grid < 1 ||
+        info->lds_bytes < 0 || info->lds_bytes > 64 * 1024 || (reinterpret_cast<uintptr_t>(plan_dev) & 15u))
+        return VRL_INT4_EPLAN;
+    const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
+    const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + 16);   // behind the plan's 16-byte header
+    const int2 *block_tab = reinterpret_cast<const int2 *>(recs + info->n_problems);
+    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
+    hipLaunchKernelGGL((gemv_stream_kernel<4, 1, false, true, false, false, 1, true>), dim3(info->grid),
+                       dim3(4 * WAVE), (size_t)info->lds_bytes, reinterpret_cast<hipStream_t>(hip_stream), recs,
+                       block_tab, info->n_problems);
     return (int)hipGetLastError();
 }
 

@@ -28,52 +28,15 @@
 // v_cvt_pk_bf16_f32 applies the one round-to-nearest-even the contract asks for.
 //
 // Source layout: common.hpp (types, bf16 helpers, the problem record), canonical.hpp (kernels over the
-// canonical triple), prepacked.hpp (repack, stream and latency kernels over the MFMA-shaped blob), this file
-// (the grouped stream kernel that dispatches to both halves, plan building, launchers, the C ABI).
+// canonical triple), prepacked.hpp (repack, stream and latency kernels over the MFMA-shaped blob),
+// stream_kernel.hpp (the grouped stream kernel that dispatches to both halves), this file (plan building,
+// launchers, the C ABI).
 
 #include <atomic>
 
-#include "prepacked.hpp"
+#include "stream_kernel.hpp"
 
 namespace {
-
-// CANON / PP / FUSED say which kinds of record the plan holds, so that a plan of
-// plain prepacked GEMVs runs the variant with the smallest register footprint.
-// WPB (waves per workgroup) grows with the LDS the staged activations need, so that
-// about 16 waves stay resident per CU; MB = 2 carries up to 32 activation rows per
-// record with two A operands per weight tile (weights streamed once); PASSES adds the
-// path for prepacked records whose activations do not fit LDS whole (it carries several
-// accumulator tiles, so plans that do not need it run a build without it).
-// VDOT: the comparison build whose dot product runs on the vector unit (one activation row, plain prepacked
-// records of group size 128 only).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ, bool VDOT = false>
-__global__ __launch_bounds__(WPB *WAVE) void gemv_stream_kernel(const DevProblem *__restrict__ plan,
-                                                                const int2 *__restrict__ block_tab,
-                                                                int n_problems) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    // block_tab[b] = {first tile of workgroup b, record that tile belongs to}
-    const int2 entry = block_tab[blockIdx.x];
-    int t = entry.x;
-    const int t_end = block_tab[blockIdx.x + 1].x;
-    if (t >= t_end) return;  // block-uniform
-    const int lo = entry.y;
-    StagedX staged;
-    for (int pi = lo; t < t_end && pi < n_problems; ++pi) {
-        const DevProblem p = plan[pi];
-        const int out_cols = p.fused ? p.N / 2 : p.N;
-        const int seg_end = min(t_end, p.tile_begin + (out_cols + 15) / 16);
-        const int a = t - p.tile_begin, b = seg_end - p.tile_begin;
-        if (PP && (!CANON || p.prepacked)) {
-            if (FUSED && p.fused) stream_segment_pp<MB, FUSED, WPB, PASSES, GQ>(p, a, b, smem, staged);
-            else stream_segment_pp<MB, false, WPB, PASSES, GQ, VDOT>(p, a, b, smem, staged);
-        } else if (CANON) {
-            staged.x = nullptr;  // the canonical walk stages in its own order
-            if (FUSED && p.fused) stream_segment<MB, FUSED, WPB>(p, a, b, smem);
-            else stream_segment<MB, false, WPB>(p, a, b, smem);
-        }
-        t = seg_end;
-    }
-}
 
 // -------------------------------------------------------------------------
 // host side
@@ -233,15 +196,13 @@ struct PlanHeader {
 static_assert(sizeof(PlanHeader) == 16, "plan header is 16 bytes");
 constexpr uint32_t PLAN_MAGIC = 0x34544956u;  // "VIT4"
 constexpr int MAX_PLAN_GRID = 4096;
-constexpr int VARIANT_CANON = 1, VARIANT_PP = 2, VARIANT_FUSED = 4, VARIANT_MB2 = 8, VARIANT_PASSES = 16,
-              VARIANT_SPLIT = 32, VARIANT_G64 = 64, VARIANT_G32 = 128, VARIANT_VDOT = 256;
 
 // With recs == nullptr nothing is launched: info->grid receives the number of workgroups of
 // this build that one CU holds at info->lds_bytes (the plan builder sizes the grid with it).
-template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ = 1, bool VDOT = false>
+template <int WPB, int MB, bool CANON, bool PP, bool FUSED, bool PASSES, int GQ = 1>
 int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_begin,
                   hipStream_t stream) {
-    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ, VDOT>;
+    auto kernel = &gemv_stream_kernel<WPB, MB, CANON, PP, FUSED, PASSES, GQ>;
     if (info->lds_bytes > 64 * 1024) {
         // once per instantiation and device (the attribute belongs to the function on that device), at the
         // largest size a plan may ask for: no runtime call in a timed or captured launch after the first
@@ -302,13 +263,6 @@ int launch_stream_variant(vrl_int4_plan_info *info, const DevProblem *recs, cons
     const bool passes = (info->variant & VARIANT_PASSES) != 0;
     // prepacked-only plans hold one group size (the kernel build is specialised for it)
     const int gq = (info->variant & VARIANT_G32) ? 4 : ((info->variant & VARIANT_G64) ? 2 : 1);
-    if (info->variant & VARIANT_VDOT) {
-        if constexpr (WPB == 4 && MB == 1) {
-            if (v == VARIANT_PP && !passes && gq == 1)
-                return launch_stream<4, 1, false, true, false, false, 1, true>(info, recs, bb, stream);
-        }
-        return VRL_INT4_EPLAN;
-    }
     if (v == VARIANT_PP || v == (VARIANT_PP | VARIANT_FUSED)) {
         return launch_stream_pp<WPB, MB>(info, recs, bb, stream, (v & VARIANT_FUSED) != 0, passes, gq);
     }
@@ -708,7 +662,6 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     long tiles = 0;
     double total_cost = 0.0;
     int variant = 0;
-    bool valu_dot = false, valu_dot_ok = true;   // a problem asks for the vector-unit dot product (reserved[0] == 1); all do and qualify
     int pp_group_size = 0;      // group size of the prepacked records, -1 if they differ
     size_t x_need = 0;  // bytes the largest activation matrix needs if staged whole
     for (int i = 0; i < n_problems; ++i) {
@@ -736,8 +689,6 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
             return VRL_INT4_ESHAPE;
         if (p.prepacked) pp_group_size = (pp_group_size == 0 || pp_group_size == p.G) ? p.G : -1;
         if (p.M > MAX_TILE_M) variant |= VARIANT_MB2;
-        valu_dot = valu_dot || q.reserved[0] == 1;
-        valu_dot_ok = valu_dot_ok && q.reserved[0] == 1 && q.prepacked && !q.fused_gate_up && q.M == 1 && q.G == 128;
         p.tile_begin = (int)tiles;
         const int out_cols = p.fused ? p.N / 2 : p.N;
         const long nt = (out_cols + 15) / 16;
@@ -804,12 +755,7 @@ int vrl_int4_grouped_plan_build(const vrl_int4_problem *problems, int n_problems
     // As many waves share a tile as it has super-chunks (4, 8 or 16), fewer if the plan would
     // not fit the device at that width.
     size_t red_bytes = 0;
-    if (valu_dot) {
-        // the comparison build is the 4-wave one over plain prepacked problems of one activation row
-        if (!valu_dot_ok || shape != 0 || (variant & VARIANT_PASSES)) return VRL_INT4_ESHAPE;
-        variant |= VARIANT_VDOT;
-    }
-    if (shape == 0 && !(variant & (VARIANT_CANON | VARIANT_MB2 | VARIANT_PASSES | VARIANT_VDOT))) {
+    if (shape == 0 && !(variant & (VARIANT_CANON | VARIANT_MB2 | VARIANT_PASSES))) {
         int max_nsc = 1;
         for (int i = 0; i < n_problems; ++i) max_nsc = std::max(max_nsc, pp_nsc(recs[i].K));
         variant |= VARIANT_SPLIT;

@@ -238,9 +238,7 @@ class GroupedGemv:
     MAX_ROWS = 16            # activation rows one canonical record of the plan may carry
     MAX_ROWS_PREPACKED = 32  # ... and one prepacked record (two MFMA row blocks per weight tile)
 
-    def __init__(self, problems, valu_dot: bool = False):
-        """``valu_dot``: the comparison build of the launch whose dot product runs on the vector unit
-        (``v_dot2_f32_bf16``) instead of the matrix cores; plain prepacked M = 1, group-128 problems only."""
+    def __init__(self, problems):
         if not problems:
             raise ValueError("GroupedGemv needs at least one problem")
         lib = _lib.load()
@@ -287,7 +285,6 @@ class GroupedGemv:
         for rec, vals in zip(table, records):
             (rec.x, rec.qweight, rec.scales, rec.qzeros, rec.y,
              rec.M, rec.N, rec.K, rec.G, rec.fused_gate_up, rec.prepacked) = vals
-            rec.reserved[0] = 1 if valu_dot else 0
         size = lib.vrl_int4_grouped_plan_size(n)
         host = torch.empty(size, dtype=torch.uint8)
         self.info = _lib.PlanInfo()
