@@ -174,6 +174,29 @@ typedef struct vrl_int4_norm {
 int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_problems,
                                       const vrl_int4_norm *norm, void *hip_stream);
 
+/*
+ * The plan-free launch of ONE plain prepacked problem with the linear's bias and a following activation
+ * applied to each tile before it is stored:
+ *   y = act(bf16(bf16(x . W^T) + bias))
+ * i.e. the roundings of a bf16 module that adds its bias to its output tensor and whose activation is a
+ * tensor op of its own.  This is the first half of a two-layer image-token head (Linear, GELU, Linear:
+ * what `gen_head` is in the Janus-Pro checkpoints, called at policy.py:138-160) and any biased linear.
+ * `norm` may be NULL; when given, the residual add and RMSNorm of vrl_int4_gemv_prepacked_norm_bf16 are
+ * applied to the activations on their way in (the trunk's final norm in front of the head).
+ * bias: bf16 [N] or NULL.  activation: VRL_INT4_ACT_NONE, or VRL_INT4_ACT_GELU for
+ * x / 2 * (1 + erf(x / sqrt(2))) evaluated in fp32 on the bf16 value and rounded to bf16 (torch.nn.GELU()).
+ */
+#define VRL_INT4_ACT_NONE 0
+#define VRL_INT4_ACT_GELU 1
+typedef struct vrl_int4_epilogue {
+    const void *bias;
+    int32_t activation;
+    int32_t reserved;   /* 0 */
+} vrl_int4_epilogue;
+
+int vrl_int4_gemv_prepacked_epilogue_bf16(const vrl_int4_problem *problem, const vrl_int4_norm *norm,
+                                          const vrl_int4_epilogue *epilogue, void *hip_stream);
+
 size_t vrl_int4_grouped_plan_size(int n_problems);
 
 /* Fills plan_host (plan_bytes >= vrl_int4_grouped_plan_size(n_problems)) and *info. */
@@ -224,10 +247,39 @@ int vrl_int4_head_sample_bf16(const vrl_int4_problem *head, const void *noise, i
                               void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
+ * vrl_int4_head_sample_bf16 with the parts of the decode step that surround it (each optional):
+ *   bias         bf16 [V] of a biased head: logits = bf16(bf16(x . W^T) + bias), the roundings of a bf16 module
+ *                that adds its bias to its output tensor (the last linear of Janus' two-layer head has one)
+ *   position     device scalar p (0 <= p < token_stride): tokens[b, p] = sampled[b], logprobs[b, p] = logprob[b]
+ *                (policy.py:695-696), then p + 1 is stored back; slot, if given, is incremented as well (the
+ *                cache slot counter of a static decode loop)
+ *   embed_table  bf16 [V, embed_dim], row t the input embedding of image token t (what
+ *                prepare_gen_img_embeds returns for it, policy.py:698-700): rows b and B + b of next_embeds
+ *                (bf16 [2B, embed_dim]) receive row sampled[b]; embed_dim a multiple of 8, 16-byte aligned rows
+ * All of it is done by the call's second kernel, one workgroup per batch row.  workspace as for
+ * vrl_int4_head_sample_bf16.
+ */
+typedef struct vrl_int4_head_extras {
+    const void *bias;
+    const void *embed_table;
+    void *next_embeds;
+    int64_t *tokens;
+    float *logprobs;
+    int64_t *position;
+    int64_t *slot;
+    int32_t embed_dim;
+    int32_t token_stride;
+} vrl_int4_head_extras;
+
+int vrl_int4_head_sample_ex_bf16(const vrl_int4_problem *head, const vrl_int4_head_extras *extras, const void *noise,
+                                 int64_t *sampled, float *logprob, int B, float cfg_weight, float temperature,
+                                 void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
  * vrl_int4_head_sample_bf16 without a workspace argument, for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no
  * counterpart in the reference.  The partials, masks and scaled rows go to a fixed array that the
- * library holds in the memory of every GPU it runs on (1,572,864 bytes, kept until the process ends),
+ * library holds in the memory of every GPU it runs on (1,573,120 bytes, kept until the process ends),
  * so the call allocates nothing.  Limits: B <= 16 and V <= 16384, else VRL_INT4_ELIMIT (nothing is
  * enqueued); everything else as vrl_int4_head_sample_bf16.  Every call on a GPU uses that GPU's one
  * array: calls that overlap in time on one GPU (two streams, two threads) race and must be ordered by

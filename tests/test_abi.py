@@ -332,3 +332,49 @@ def test_cfg_sample_validation(lib):
     assert f(p, p, p, p, 1, 16, 1.0, float("nan"), None) == 1001
     assert f(p + 1, p, p, p, 1, 16, 1.0, 1.0, None) == 1002
     assert f(p, p, p + 4, p, 1, 16, 1.0, 1.0, None) == 1002      # int64 output
+
+
+def test_epilogue_launch_validation(lib):
+    keep, p = buf(1 << 16)
+    prob = (_lib.Problem * 1)()
+    prob[0].x = prob[0].qweight = prob[0].y = p
+    prob[0].M, prob[0].N, prob[0].K, prob[0].G, prob[0].prepacked = 2, 64, 256, 128, 1
+    epi = _lib.Epilogue()
+    epi.bias, epi.activation = p, _lib.ACT_GELU
+    f = lib.vrl_int4_gemv_prepacked_epilogue_bf16
+    assert f(prob, None, None, None) == 1003 and f(None, None, ctypes.byref(epi), None) == 1003
+    epi.activation = 7
+    assert f(prob, None, ctypes.byref(epi), None) == 1001          # an activation the library does not know
+    epi.activation, epi.bias = _lib.ACT_GELU, p + 1
+    assert f(prob, None, ctypes.byref(epi), None) == 1002
+    epi.bias, prob[0].fused_gate_up = p, 1
+    assert f(prob, None, ctypes.byref(epi), None) == 1001          # a plain problem only
+    prob[0].fused_gate_up, prob[0].prepacked = 0, 0
+    assert f(prob, None, ctypes.byref(epi), None) == 1001
+
+
+def test_head_sample_extras_validation(lib):
+    keep, p = buf(1 << 20)
+    p = (p + 255) & ~255
+    head = _lib.Problem()
+    head.x = head.qweight = p
+    head.M, head.N, head.K, head.G, head.prepacked = 2, 64, 256, 128, 1
+    need = lib.vrl_int4_head_sample_workspace_bytes(1, 64)
+    assert need > 0 and need % 256 == 0
+    f = lib.vrl_int4_head_sample_ex_bf16
+    ex = _lib.HeadExtras()
+    assert f(ctypes.byref(head), None, p, p, p, 1, 5.0, 1.0, p, need, None) == 1003
+    ex.embed_table = p
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1003   # no destination
+    ex.next_embeds, ex.embed_dim = p, 12
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1001   # 16-byte rows
+    ex.embed_dim, ex.next_embeds = 16, p + 2
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1002
+    ex.next_embeds, ex.tokens = p, p
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1003   # tokens need a position
+    ex.position, ex.token_stride = p, 0
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1001
+    ex.token_stride, ex.position = 8, p + 4
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1002
+    ex.position = p
+    assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need - 256, None) == 1001  # workspace too small

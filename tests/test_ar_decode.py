@@ -608,3 +608,134 @@ def test_adapter_state_changes_invalidate_the_recorded_step():
     want = StaticARSampler(policy, graph=False, native=False).sample_image_tokens(*inputs, image_token_num=8)
     assert torch.equal(without[0], want[0]) and torch.equal(without[1], want[1])
     assert not torch.equal(without[1], with_adapters[1])
+
+
+# ------------------------------------------------------------------ the checkpoints' two-layer head and aligner
+class VisionHead(nn.Module):
+    """``gen_head`` as the Janus-Pro checkpoints hold it (the ``vision_head`` class of the upstream package, which
+    ``vrl/models/families/janus_pro/policy.py:803-842`` loads and ``policy.py:138-160`` calls): Linear, GELU,
+    Linear, both linears with a bias."""
+
+    def __init__(self, hidden, vocab):
+        super().__init__()
+        self.output_mlp_projector = nn.Linear(hidden, hidden)
+        self.vision_activation = nn.GELU()
+        self.vision_head = nn.Linear(hidden, vocab)
+
+    def forward(self, x):
+        return self.vision_head(self.vision_activation(self.output_mlp_projector(x)))
+
+
+class JanusShapedMMGPT(StubMMGPT):
+    """The stub with the checkpoints' head and input path of image tokens: ``gen_embed`` (8 values per token)
+    and the two-layer ``gen_aligner`` behind ``prepare_gen_img_embeds``."""
+
+    def __init__(self, dtype, aligner=True, **shape):
+        super().__init__(dtype, **shape)
+        hidden, vocab = shape.get("hidden", HIDDEN), shape.get("vocab", VOCAB_IMG)
+        torch.manual_seed(5)
+        self.gen_head = VisionHead(hidden, vocab).to(dtype)
+        with torch.no_grad():
+            self.gen_head.vision_head.weight.mul_(24.0)
+            self.gen_head.vision_head.bias.normal_(0.0, 1.0)
+            self.gen_head.output_mlp_projector.bias.normal_(0.0, 0.5)
+        if aligner:
+            self.gen_embed = nn.Embedding(vocab, 8).to(dtype)
+            self.gen_aligner = nn.Sequential(nn.Linear(8, hidden), nn.GELU(), nn.Linear(hidden, hidden)).to(dtype)
+
+    def prepare_gen_img_embeds(self, ids):
+        embeds = self.gen_embed(ids)
+        return self.gen_aligner(embeds) if hasattr(self, "gen_aligner") else embeds
+
+
+def janus_shaped_policy(aligner=True):
+    from visionrl_amd.policy_glue import apply_int4_to_policy
+
+    policy = StubPolicy(torch.bfloat16, "cuda:0")
+    policy.mmgpt = JanusShapedMMGPT(torch.bfloat16, aligner=aligner)
+    policy.mmgpt.language_model.model.to("cuda:0")
+    policy.mmgpt.to("cuda:0")
+    summary = apply_int4_to_policy(policy, group_size=128)
+    assert summary["head_linears"] == 2          # both linears of the head, found below its attributes
+    head = policy.mmgpt.gen_head
+    assert head.vision_head._packed is not None and head.output_mlp_projector._packed is not None
+    assert head.vision_head.bias is not None and head.output_mlp_projector.bias is not None
+    return policy
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("aligner", [False, True])
+def test_two_layer_head_runs_as_two_launches_and_samples_what_the_module_head_samples(aligner):
+    """The checkpoints' head through ``apply_int4_to_policy`` and the static sampler: its front is one launch
+    (final norm while staging, bias, GELU), its last linear and the tail one call; tokens under one seed equal
+    those of the same sampler with the head as modules followed by ``cfg_sample`` (and of eager steps), the
+    log-probabilities agree to a bf16 step."""
+    print("ar decode: two-layer head, aligner", aligner, flush=True)
+    policy = janus_shaped_policy(aligner)
+    cond, uncond, cmask, umask = make_inputs(3, 7, torch.bfloat16, "cuda:0", seed=61)
+    runs = {}
+    for name, opts in (("fused", {}), ("fused_eager", {"graph": False}), ("modules", {"fused_head": False}),
+                       ("no_table", {"embed_table": False})):
+        sampler = StaticARSampler(policy, **opts)
+        torch.manual_seed(62)
+        runs[name] = sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=24)
+        torch.cuda.synchronize()
+        (sess,) = sampler._sessions.values()
+        assert sess.native, name
+        if name == "fused":
+            assert sess.front_call is not None and sess.native.final is not None and sess.graph is not None
+            assert sess.native.launches == 5 * LAYERS        # the last norm went into the head's front launch
+            if not aligner:
+                assert sampler._table is not None            # a plain embedding tabulates exactly
+        if name == "modules":
+            assert sess.front_call is None and sess.native.launches == 5 * LAYERS + 1
+        if name == "no_table":
+            assert sampler._table is None
+    want_t, want_lp = runs["modules"]
+    assert len(want_t.unique()) > 12
+    for name in ("fused", "fused_eager", "no_table"):
+        got_t, got_lp = runs[name]
+        assert torch.equal(got_t, want_t), (name, got_t, want_t)
+        torch.testing.assert_close(got_lp, want_lp, rtol=2 ** -7, atol=2 ** -7)
+    assert torch.equal(runs["fused"][1], runs["fused_eager"][1])
+
+
+@pytest.mark.gpu
+def test_two_layer_head_logits_against_the_oracle():
+    """The head's two launches against the oracle's arithmetic on the same operands: front = GELU(bf16(x . W1^T)
+    + b1) with the stated roundings, logits = bf16(front . W2^T) + b2."""
+    import numpy as np
+
+    from oracle import int4_oracle as o
+    from tests._util import bf16_to_bits
+
+    print("ar decode: two-layer head against the oracle", flush=True)
+    policy = janus_shaped_policy(False)
+    head = policy.mmgpt.gen_head
+    from visionrl_amd import ops
+
+    x = torch.randn((6, HIDDEN), device="cuda:0").to(torch.bfloat16)
+    front = ops.EpilogueGemv(x, head.output_mlp_projector._packed, head.output_mlp_projector.bias, gelu=True).launch()
+    logits = torch.empty((6, VOCAB_IMG), dtype=torch.bfloat16, device="cuda:0")
+    ops.head_sample(front, head.vision_head._packed, 5.0, 1.0, logits_out=logits, bias=head.vision_head.bias)
+    torch.cuda.synchronize()
+    assert torch.equal(logits.view(6, 1, -1), head(x.view(6, 1, -1)))          # the module path, bit for bit
+
+    def lin(mod, xin_bits):
+        args = (xin_bits, mod.qweight.cpu().numpy(), bf16_to_bits(mod.scales), mod.qzeros.cpu().numpy(), 128)
+        y_ref, a_ref = o.gemv_and_abs_f64(*args)
+        return y_ref, a_ref, o.bf16_bits_to_f32(bf16_to_bits(mod.bias)).astype(np.float64)
+
+    y1, a1, b1 = lin(head.output_mlp_projector, bf16_to_bits(x))
+    pre = o.bf16_bits_to_f32(o.f32_to_bf16_bits((o.bf16_bits_to_f32(o.f32_to_bf16_bits(y1.astype(np.float32))) + b1).astype(np.float32)))
+    from math import erf
+    gelu = np.vectorize(lambda v: 0.5 * v * (1.0 + erf(v / np.sqrt(2.0))))
+    # the front launch within the linear's tolerance carried through bias and GELU (slope at most 1.13)
+    got_front = o.bf16_bits_to_f32(bf16_to_bits(front)).astype(np.float64)
+    tol = 1.13 * o.gemv_tolerance(y1, a1) + 2.0 ** -7 * np.abs(gelu(y1 + b1)) + 2.0 ** -8 * np.abs(y1 + b1) + 1e-30
+    assert (np.abs(got_front - gelu(y1 + b1)) <= tol).all()
+    # the last linear over the launch's own front output
+    y2, a2, b2 = lin(head.vision_head, bf16_to_bits(front))
+    got = o.bf16_bits_to_f32(bf16_to_bits(logits)).astype(np.float64)
+    # the linear's tolerance, and one more bf16 rounding for the sum with the bias
+    assert (np.abs(got - (y2 + b2)) <= o.gemv_tolerance(y2, a2) + o.bf16_ulp(y2 + b2)).all()

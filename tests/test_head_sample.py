@@ -158,3 +158,81 @@ def test_head_sample_refuses_what_it_does_not_take(ops_mod):
     db = to_device(big, DEV)
     wide = ops_mod.int4_prepack(db["qweight"], db["scales"], db["qzeros"], 128)
     assert not ops_mod.head_sample_supported(32, wide) and ops_mod.head_sample_supported(16, wide)
+
+
+@pytest.mark.parametrize("B,K,V", [(1, 2048, 16384), (16, 2048, 16384), (5, 1024, 4096)])
+def test_head_sample_with_bias_bookkeeping_and_next_embeddings(ops_mod, B, K, V):
+    """``vrl_int4_head_sample_ex_bf16``: the biased logits are the plain launch's plus the bias with the module's
+    two roundings; the draw over them is the oracle's; token and log-probability land at the device-side
+    position of the step's buffers, position and slot move on by one, and rows b and B + b of the next input
+    are the table's row of the sampled token.  Two calls in a row over one workspace."""
+    print(f"[case] head_sample extras B={B} K={K} V={V}", flush=True)
+    G, w, T, H, L = 128, 5.0, 1.0, 256, 40
+    ops, nb = make_head(900 + B + K, B, K, V, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    rng = np.random.default_rng(B)
+    bias_bits = o.f32_to_bf16_bits(rng.normal(0.0, 2.0, size=V).astype(np.float32))
+    bias = bits_to_bf16(bias_bits, DEV)
+    table = torch.randn((V, H), device=DEV).to(torch.bfloat16)
+    nxt = torch.zeros((2 * B, 1, H), dtype=torch.bfloat16, device=DEV)
+    tokens = torch.full((B, L), -1, dtype=torch.int64, device=DEV)
+    lps = torch.full((B, L), 7.0, dtype=torch.float32, device=DEV)
+    position = torch.tensor([17], dtype=torch.int64, device=DEV)
+    slot = torch.tensor([300], dtype=torch.int64, device=DEV)
+    ws = ops_mod.head_sample_workspace(B, V, DEV)
+    plain = torch.empty((2 * B, V), dtype=torch.bfloat16, device=DEV)
+    ops_mod.head_sample(d["x"], pw, w, T, noise=bits_to_bf16(nb, DEV), logits_out=plain, workspace=ws)
+    logits = torch.empty_like(plain)
+    for call in range(2):
+        n = o.f32_to_bf16_bits(rng.exponential(1.0, size=(B, V)).astype(np.float32))
+        n[n == 0] = 1
+        sampled, lp = ops_mod.head_sample(d["x"], pw, w, T, noise=bits_to_bf16(n, DEV), logits_out=logits,
+                                          workspace=ws, bias=bias, bookkeeping=(tokens, lps, position, slot),
+                                          embedding=(table, nxt))
+        torch.cuda.synchronize()
+        assert torch.equal(logits, plain + bias)                  # bf16(bf16(x . W^T) + bias), as the module adds it
+        assert check_against_oracle(sampled, lp, bf16_to_bits(logits), n, w, T) >= B - max(1, B // 8)
+        assert int(position) == 18 + call and int(slot) == 301 + call
+        assert torch.equal(tokens[:, 17 + call], sampled) and torch.equal(lps[:, 17 + call], lp)
+        assert torch.equal(nxt[:B, 0], table[sampled]) and torch.equal(nxt[B:, 0], table[sampled])
+    assert int((tokens != -1).sum()) == 2 * B and int((lps != 7.0).sum()) == 2 * B
+    # without a slot the cache counter stays; a position past the buffers writes nothing
+    position.fill_(L)
+    ops_mod.head_sample(d["x"], pw, w, T, workspace=ws, bookkeeping=(tokens, lps, position, None))
+    torch.cuda.synchronize()
+    assert int(position) == L + 1 and int(slot) == 302 and int((tokens != -1).sum()) == 2 * B
+
+
+@pytest.mark.parametrize("M,K,N,G,norm", [(2, 2048, 2048, 128, False), (2, 2048, 2048, 128, True),
+                                          (32, 2048, 2048, 128, True), (8, 4096, 4096, 128, True),
+                                          (5, 1024, 1536, 64, False)])
+def test_linear_with_bias_and_gelu_in_one_launch(ops_mod, M, K, N, G, norm):
+    """``vrl_int4_gemv_prepacked_epilogue_bf16`` (the front of a two-layer head): bit for bit what the plain
+    launch followed by the tensor ops gives (bias added to the bf16 output, exact GELU in fp32 on the bf16
+    value), and the linear itself against the oracle; with the trunk's last norm folded in, against the
+    normalising launch."""
+    print(f"[case] epilogue launch M={M} K={K} N={N} G={G} norm={norm}", flush=True)
+    ops = o.make_operands(1200 + M + K + N, M, K, N, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    gen = torch.Generator(device=DEV).manual_seed(M + K)
+    bias = torch.randn(N, generator=gen, device=DEV).to(torch.bfloat16)
+    norm_args = None
+    if norm:
+        res = torch.randn((M, K), generator=gen, device=DEV).to(torch.bfloat16)
+        nw = (1.0 + 0.1 * torch.randn(K, generator=gen, device=DEV)).to(torch.bfloat16)
+        norm_args = (res, nw, 1e-6)
+        (base,) = ops_mod.DirectGemv([(d["x"], pw, False)], norm=(res, nw, 1e-6, None)).launch()
+    else:
+        (base,) = ops_mod.DirectGemv([(d["x"], pw, False)]).launch()
+        torch.cuda.synchronize()
+        assert_gemv_close(bf16_to_bits(base), ops, G, f"epilogue base M{M} K{K} N{N}")
+    for b, gelu in ((bias, True), (bias, False), (None, True)):
+        got = ops_mod.EpilogueGemv(d["x"], pw, b, gelu=gelu, norm=norm_args).launch()
+        want = base if b is None else base + b
+        want = torch.nn.functional.gelu(want) if gelu else want
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (b is not None, gelu, (got.float() - want.float()).abs().max().item())
+    with pytest.raises(ValueError):
+        ops_mod.EpilogueGemv(d["x"], pw, bias[:-1].contiguous())

@@ -457,8 +457,9 @@ def test_gradient_reaches_the_input_of_a_quantised_layer():
 
 def test_a_prepacked_copy_knows_when_its_source_changed():
     """The canonical buffers are the module's state; the prepacked copy is derived from them and is
-    stale after an in-place write (``load_state_dict``), a replaced buffer (``.to()``) or when torch
-    keeps no modification counter for a buffer (inference tensors cannot be told apart)."""
+    stale after an in-place write (``load_state_dict``) or a replaced buffer (``.to()``).  Where torch keeps
+    no modification counter for a buffer (an inference tensor) the copy is tied to the tensor object, its
+    address and shape: such a module does not repack on every call, and ``prepack_()`` follows an edit."""
     from visionrl_amd.linear import _source_changed, _source_state
 
     a, b = torch.zeros(4), torch.ones(4)
@@ -470,7 +471,14 @@ def test_a_prepacked_copy_knows_when_its_source_changed():
     assert _source_changed(state, a.clone(), b)
     with torch.inference_mode():
         c = torch.zeros(4)
-    assert _source_changed(_source_state(c), c)
+        d = torch.zeros(4)
+    state = _source_state(c)
+    assert not _source_changed(state, c)        # the same object in the same place: not stale
+    assert _source_changed(state, d)            # another tensor
+    del d
+    state = _source_state(a)
+    del a                                       # the source is gone: whatever stands in its place is new
+    assert _source_changed(state, torch.zeros(4))
     mod = Int4Linear(128, 16, 128)
     assert not mod.packed_is_stale()                 # nothing prepacked
     mod._packed, mod._packed_from = object(), _source_state(mod.qweight, mod.scales, mod.qzeros)

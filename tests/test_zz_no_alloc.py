@@ -79,8 +79,9 @@ def test_static_scratch_entry_point_equals_the_workspace_one():
     want = ops.head_sample(d["x"], pw, 5.0, 1.0, noise=noise)
     out = (torch.empty(2, dtype=torch.int64, device=DEV), torch.empty(2, dtype=torch.float32, device=DEV))
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    allocations = lambda: torch.cuda.memory_stats()["allocation.all.allocated"]   # requests served so far
+    before = allocations()
     got = ops.head_sample(d["x"], pw, 5.0, 1.0, noise=noise, workspace="static", out=out)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before and got[0] is out[0]
+    assert allocations() == before and got[0] is out[0]
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])

@@ -25,12 +25,14 @@ SYMBOLS = (
     "vrl_int4_prepack",
     "vrl_int4_gemv_prepacked_bf16",
     "vrl_int4_gemv_prepacked_norm_bf16",
+    "vrl_int4_gemv_prepacked_epilogue_bf16",
     "vrl_int4_grouped_plan_size",
     "vrl_int4_grouped_plan_build",
     "vrl_int4_gemv_grouped_bf16",
     "vrl_cfg_sample_bf16",
     "vrl_int4_head_sample_workspace_bytes",
     "vrl_int4_head_sample_bf16",
+    "vrl_int4_head_sample_ex_bf16",
     "vrl_int4_head_sample_static_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
@@ -77,6 +79,35 @@ class Norm(ctypes.Structure):
         ("h_out", ctypes.c_void_p),
         ("eps", ctypes.c_float),
         ("reserved", ctypes.c_int32),
+    ]
+
+
+class Epilogue(ctypes.Structure):
+    """Mirror of ``vrl_int4_epilogue``."""
+
+    _fields_ = [
+        ("bias", ctypes.c_void_p),
+        ("activation", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+ACT_NONE, ACT_GELU = 0, 1
+
+
+class HeadExtras(ctypes.Structure):
+    """Mirror of ``vrl_int4_head_extras``."""
+
+    _fields_ = [
+        ("bias", ctypes.c_void_p),
+        ("embed_table", ctypes.c_void_p),
+        ("next_embeds", ctypes.c_void_p),
+        ("tokens", ctypes.c_void_p),
+        ("logprobs", ctypes.c_void_p),
+        ("position", ctypes.c_void_p),
+        ("slot", ctypes.c_void_p),
+        ("embed_dim", ctypes.c_int32),
+        ("token_stride", ctypes.c_int32),
     ]
 
 
@@ -167,6 +198,12 @@ def _bind(lib):
     lib.vrl_int4_head_sample_bf16.restype = ci
     lib.vrl_int4_head_sample_bf16.argtypes = [ctypes.POINTER(Problem), vp, vp, vp, ci, ctypes.c_float,
                                               ctypes.c_float, vp, ctypes.c_size_t, vp]
+    lib.vrl_int4_head_sample_ex_bf16.restype = ci
+    lib.vrl_int4_head_sample_ex_bf16.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(HeadExtras), vp, vp, vp, ci,
+                                                 ctypes.c_float, ctypes.c_float, vp, ctypes.c_size_t, vp]
+    lib.vrl_int4_gemv_prepacked_epilogue_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_epilogue_bf16.argtypes = [ctypes.POINTER(Problem), ctypes.POINTER(Norm),
+                                                          ctypes.POINTER(Epilogue), vp]
     lib.vrl_int4_head_sample_static_bf16.restype = ci
     lib.vrl_int4_head_sample_static_bf16.argtypes = [ctypes.POINTER(Problem), vp, vp, vp, ci, ctypes.c_float,
                                                      ctypes.c_float, vp]

@@ -44,9 +44,11 @@ from typing import Any
 import torch
 import torch.nn.functional as F
 
+from torch import nn
+
 from . import ops
 from .decode_step import NativeDecodeTrunk, trunk_signature
-from .linear import Int4Linear
+from .linear import Int4Linear, _source_changed, _source_state
 
 __all__ = ["StaticARSampler", "StaticARState", "StaticARStepResult", "install_static_ar_sampler"]
 
@@ -132,20 +134,50 @@ class _Session:
         self.owner = None      # weak reference to the state whose generation the buffers hold
         self.head_workspace = None   # of the fused head + tail launch
         self.signature = None  # of the trunk's modules and adapter state the launch list / graph were made for
+        self.head_verified = None    # the signature under which the head's split into (front, last linear) was checked
+        self.front_call = None       # the front of a two-layer head as one launch over the native trunk's output
+        self.sampled = torch.zeros(rows2 // 2, dtype=torch.long, device=device)
+        self.lp = torch.zeros(rows2 // 2, dtype=torch.float32, device=device)
+
+    def _head_parts(self):
+        """``(front modules, last linear)`` when ``gen_head`` is an int4 linear, an ``nn.Sequential`` that ends
+        in one, or a module shaped like the checkpoints' ``vision_head`` (``output_mlp_projector``,
+        ``vision_activation``, ``vision_head``, applied in that order: Linear, GELU, Linear); else ``None``."""
+        head = getattr(self.sampler.base, "gen_head", None)
+        if isinstance(head, Int4Linear):
+            return [], head
+        if isinstance(head, nn.Sequential) and len(head) >= 1 and isinstance(head[-1], Int4Linear):
+            return list(head)[:-1], head[-1]
+        names = ("output_mlp_projector", "vision_activation", "vision_head")
+        if all(isinstance(getattr(head, n, None), nn.Module) for n in names) and \
+                isinstance(head.vision_head, Int4Linear):
+            return [head.output_mlp_projector, head.vision_activation], head.vision_head
+        return None
 
     def _head_packed(self):
-        """The prepacked weight of a bare, bias-free int4 ``gen_head`` (made again first if its canonical
-        buffers changed), else ``None``."""
-        head = getattr(self.sampler.base, "gen_head", None)
-        if isinstance(head, Int4Linear) and head.bias is None:
-            return head._fresh_packed()
+        """The prepacked weight of the head's last int4 linear (made again first if its canonical buffers
+        changed), else ``None``."""
+        parts = self._head_parts()
+        return parts[1]._fresh_packed() if parts is not None else None
+
+    def _front_packed(self):
+        """The prepacked weight of the front of a two-layer head when that front is an int4 linear followed by
+        an exact GELU (one launch with the epilogue), else ``None``."""
+        parts = self._head_parts()
+        if parts is None or len(parts[0]) != 2:
+            return None
+        lin, act = parts[0]
+        if isinstance(lin, Int4Linear) and isinstance(act, nn.GELU) and getattr(act, "approximate", "none") == "none":
+            return lin._fresh_packed()
         return None
 
     # -- one call of sample_image_tokens starts here
     def begin(self, mask: torch.Tensor) -> None:
-        signature = (trunk_signature(self.sampler.trunk), id(self._head_packed()))
+        signature = (trunk_signature(self.sampler.trunk), id(self._head_packed()), id(self._front_packed()))
         if signature != self.signature:   # modules swapped, adapters merged / disabled / switched: start over
             self.signature, self.native, self.graph = signature, None, None
+            self.head_workspace = None    # sized for the head it was made for
+            self.front_call = None
         self.cache.reset()
         self.mask.fill_(1)
         self.mask[:, :mask.shape[1]].copy_(mask)
@@ -153,23 +185,58 @@ class _Session:
         self.slot.fill_(mask.shape[1])
         self.img_pos.zero_()
 
-    def tail(self, hidden: torch.Tensor) -> None:
-        """Head, guided draw, log-probability, bookkeeping, next input (``policy.py:684-700``)."""
+    def _front(self, parts, hidden: torch.Tensor) -> torch.Tensor:
+        """The modules of the head in front of its last linear, applied to ``[rows, 1, hidden]``."""
+        for module in parts[0]:
+            hidden = module(hidden)
+        return hidden
+
+    def _head_split_ok(self, parts, hidden: torch.Tensor) -> bool:
+        """Whether the head's last linear over its front is the head: checked once per set of modules, eagerly, on
+        the prompt pass's hidden state (an unknown ``forward`` could do more than the three attributes say)."""
+        if not parts[0] or self.head_verified == self.signature:
+            return True
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        same = torch.equal(self.sampler.base.gen_head(hidden), parts[1](self._front(parts, hidden)))
+        if same:
+            self.head_verified = self.signature
+        return same
+
+    def tail(self, hidden, advance_slot: bool = False) -> None:
+        """Head, guided draw, log-probability, bookkeeping, next input (``policy.py:684-700``).  ``hidden`` is
+        the trunk's ``[rows, 1, hidden]`` output, or ``None`` when the native trunk left its last norm to the
+        head's front launch.  ``advance_slot``: a decode step, after which the cache slot moves on."""
         s = self.sampler
-        packed = self._head_packed() if s.fused_tail and s.fused_head else None
-        if packed is not None and hidden.dtype == torch.bfloat16 and hidden.is_cuda and \
-                ops.head_sample_supported(self.rows2, packed):
-            # head and tail in one launch: the logits never reach memory
+        parts = self._head_parts() if s.fused_tail and s.fused_head else None
+        packed = parts[1]._fresh_packed() if parts is not None else None
+        fused = packed is not None and self.cur.dtype == torch.bfloat16 and self.cur.is_cuda and \
+            ops.head_sample_supported(self.rows2, packed) and (hidden is None or self._head_split_ok(parts, hidden))
+        if hidden is None and not fused:
+            raise RuntimeError("the trunk left its last norm to a head launch that does not exist")
+        if fused:
+            # head and tail in one call: the logits never reach memory, and the call writes token and
+            # log-probability at the position, moves the counters on and looks the next input up
+            if hidden is None:
+                rows = self.front_call.launch()
+            elif parts[0] and self.front_call is not None and self.native and self.native.normed is not None and \
+                    hidden.data_ptr() == self.native.normed.data_ptr():
+                rows = self.front_call.launch()
+            else:
+                rows = self._front(parts, hidden).reshape(self.rows2, -1).contiguous()
             if self.head_workspace is None:
-                self.head_workspace = ops.head_sample_workspace(self.rows2 // 2, packed.N, hidden.device)
-            sampled, lp = ops.head_sample(hidden.reshape(self.rows2, -1).contiguous(), packed, self.cfg_weight, self.temperature,
-                                          workspace=self.head_workspace)
-            logits = None
-        else:
-            logits = s.base.gen_head(hidden).squeeze(1)
-        if logits is None:
-            pass
-        elif s.fused_tail and logits.dtype == torch.bfloat16 and logits.is_cuda:
+                self.head_workspace = ops.head_sample_workspace(self.rows2 // 2, packed.N, rows.device)
+            table = s.embedding_table(packed.N, self.cur)
+            ops.head_sample(rows, packed, self.cfg_weight, self.temperature, workspace=self.head_workspace,
+                            out=(self.sampled, self.lp), bias=parts[1].bias,
+                            bookkeeping=(self.tokens, self.logprobs, self.img_pos, self.slot if advance_slot else None),
+                            embedding=None if table is None else (table, self.cur))
+            if table is None:
+                nxt = s.base.prepare_gen_img_embeds(torch.cat([self.sampled, self.sampled], dim=0).unsqueeze(-1))
+                self.cur.copy_(nxt.reshape(self.cur.shape))
+            return
+        logits = s.base.gen_head(hidden).squeeze(1)
+        if s.fused_tail and logits.dtype == torch.bfloat16 and logits.is_cuda:
             sampled, lp = ops.cfg_sample(logits.contiguous(), self.cfg_weight, self.temperature)
         else:
             cond, uncond = logits.chunk(2, dim=0)
@@ -182,6 +249,8 @@ class _Session:
         self.img_pos.add_(1)
         nxt = s.base.prepare_gen_img_embeds(torch.cat([sampled, sampled], dim=0).unsqueeze(-1))
         self.cur.copy_(nxt.reshape(self.cur.shape))
+        if advance_slot:
+            self.slot.add_(1)
 
     def prefill(self, embeds: torch.Tensor) -> None:
         out = self.sampler.trunk(inputs_embeds=embeds, attention_mask=self.mask, use_cache=True,
@@ -192,20 +261,32 @@ class _Session:
             s = self.sampler
             if s.native and self.cur.is_cuda and self.cur.dtype == torch.bfloat16 and \
                     NativeDecodeTrunk.unsupported(s.trunk, self.rows2, self.max_len) is None:
+                # a two-layer head whose front is one launch takes the trunk's last norm along
+                front = self._front_packed() if s.fused_tail and s.fused_head and \
+                    self.head_verified == self.signature and \
+                    ops.head_sample_supported(self.rows2, self._head_packed()) else None
                 try:
-                    self.native = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot)
+                    self.native = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot,
+                                                    final_norm=front is None)
+                    if front is not None:
+                        bias = self._head_parts()[0][0].bias
+                        if self.native.final is not None:
+                            x, res, w, eps = self.native.final
+                            self.front_call = ops.EpilogueGemv(x, front, bias, gelu=True, norm=(res, w, eps))
+                        else:
+                            self.front_call = ops.EpilogueGemv(self.native.normed, front, bias, gelu=True)
                 except (TypeError, ValueError):   # something the native launches do not take: module path
-                    self.native = False
+                    self.native, self.front_call = False, None
 
     def step(self) -> None:
         if self.native:
-            hidden = self.native.run().view(self.rows2, 1, -1)
+            hidden = self.native.run()
+            hidden = hidden.view(self.rows2, 1, -1) if hidden is not None else None
         else:
             out = self.sampler.trunk(inputs_embeds=self.cur, attention_mask=self.mask, use_cache=True,
                                      past_key_values=self.cache)
             hidden = out.last_hidden_state[:, -1:, :]
-        self.tail(hidden)
-        self.slot.add_(1)
+        self.tail(hidden, advance_slot=True)
 
     def capture(self) -> None:
         graph = torch.cuda.CUDAGraph()
@@ -224,14 +305,16 @@ class StaticARSampler:
     eagerly (same arithmetic, same random stream); ``fused_tail=False`` keeps the torch formulas
     for the part after the head; ``fused_head=False`` keeps the head a launch of its own in front of
     the fused tail (with it, a prepacked int4 ``gen_head`` and the tail are one launch and the logits
-    are never written).  With ``native`` (the default) the trunk of a decode step runs as
+    are never written; a two-layer head runs its front as one launch with bias and GELU and its last linear
+    in that call); ``embed_table`` see :meth:`embedding_table`.  With ``native`` (the default) the trunk of a decode step runs as
     :class:`visionrl_amd.decode_step.NativeDecodeTrunk` (five launches per layer, six with LoRA
     adapters on the attention projections) when the policy went through ``apply_int4_to_policy``
     with its defaults; otherwise, and for the prompt pass, the trunk module itself is called.
     """
 
     def __init__(self, policy: Any, *, graph: bool = True, fused_tail: bool = True, native: bool = True,
-                 fused_head: bool = True, length_bucket: int = 64, max_sessions: int = 2):
+                 fused_head: bool = True, embed_table: "bool | str" = "auto", length_bucket: int = 64,
+                 max_sessions: int = 2):
         self.policy = policy
         self.trunk = policy._lm_trunk()
         self.base = policy._base()
@@ -242,9 +325,67 @@ class StaticARSampler:
         self.fused_tail = bool(fused_tail)
         self.fused_head = bool(fused_head)
         self.native = bool(native)
+        if embed_table not in (True, False, "auto"):
+            raise ValueError('embed_table is True, False or "auto"')
+        self.embed_table = embed_table
+        self._table = None          # (tensor, state of the parameters it was made from) once built
+        self._table_refused = None  # the parameter state under which tabulating was tried and dropped
         self.length_bucket = int(length_bucket)
         self.max_sessions = int(max_sessions)
         self._sessions: dict = {}
+
+    def _embedding_params(self):
+        """The parameters ``prepare_gen_img_embeds`` reads in the checkpoints' layout (``gen_embed``, then
+        ``gen_aligner``; ``policy.py:698-700`` calls it), or ``None`` when the base holds neither."""
+        mods = [m for m in (getattr(self.base, n, None) for n in ("gen_embed", "gen_aligner")) if isinstance(m, nn.Module)]
+        if not mods:
+            return None
+        return [p for m in mods for p in list(m.parameters()) + list(m.buffers())]
+
+    def embedding_table(self, V: int, cur: torch.Tensor):
+        """``prepare_gen_img_embeds`` tabulated over the ``V`` image tokens (bf16 ``[V, hidden]``: the next input
+        is a function of the sampled token alone), for the head launch to look the next input up itself; ``None``
+        where that is switched off or would not be the module's own result.
+
+        ``"auto"``: built when the base holds ``gen_embed`` / ``gen_aligner`` (their parameters' modification
+        counters say when to build it again, in place) and a handful of tokens evaluated at the step's own batch
+        size give the tabulated rows bit for bit (a GEMM library may round a 16384-row product differently
+        from a two-row one: then the modules keep running every step).  ``True`` skips both conditions."""
+        if self.embed_table is False or not cur.is_cuda or cur.dtype != torch.bfloat16:
+            return None
+        params = self._embedding_params()
+        if params is None and self.embed_table != True:   # noqa: E712 ("auto" is truthy)
+            return None
+        if self._table is not None and (params is None or not _source_changed(self._table[1], *params)) and \
+                self._table[0].shape[0] == V:
+            return self._table[0]
+        if self._table_refused is not None and params is not None and \
+                not _source_changed(self._table_refused, *params):
+            return None
+        if torch.cuda.is_current_stream_capturing():
+            return self._table[0] if self._table is not None else None
+        ids = torch.arange(V, device=cur.device)
+        try:
+            table = self.base.prepare_gen_img_embeds(ids.unsqueeze(-1)).reshape(V, -1)
+        except (RuntimeError, IndexError):   # the embedding holds fewer tokens than the head
+            table = None
+        rows2 = cur.shape[0]
+        ok = table is not None and table.dtype == torch.bfloat16 and table.shape[1] == cur.shape[-1] and \
+            table.shape[1] % 8 == 0
+        if ok and self.embed_table == "auto":
+            probe = (torch.arange(rows2, device=cur.device) * 2654435761 + 12345) % V
+            probe[0], probe[-1] = 0, V - 1
+            ok = torch.equal(self.base.prepare_gen_img_embeds(probe.unsqueeze(-1)).reshape(rows2, -1), table[probe])
+        state = _source_state(*params) if params is not None else ()
+        if not ok:
+            self._table, self._table_refused = None, state
+            return None
+        if self._table is not None and self._table[0].shape == table.shape:
+            self._table[0].copy_(table)      # in place: recorded steps hold its address
+            self._table = (self._table[0], state)
+        else:
+            self._table = (table.contiguous(), state)
+        return self._table[0]
 
     def _defaults(self, cfg_weight, temperature, image_token_num):
         conf = getattr(self.policy, "config", None)
@@ -365,11 +506,12 @@ class StaticARSampler:
         if state.delegate is not None:
             return state.reference[2](state.delegate)
         if state.released:
-            raise ValueError("the state was finalized before")
+            return state.final     # like the reference's (``policy.py:616-622``), a second call returns the same
         n = state.image_token_num
         out = state.session.tokens[:, :n].clone(), state.session.logprobs[:, :n].clone()
-        state.final, state.released = out, True    # the session may serve the next generation of this shape
-        return out
+        if state.finished:         # the session may serve the next generation of this shape
+            state.final, state.released = out, True
+        return out                 # of an unfinished generation: a copy, and stepping stays legal
 
     @torch.no_grad()
     def sample_image_tokens(self, cond_inputs_embeds: torch.Tensor, uncond_inputs_embeds: torch.Tensor,

@@ -21,6 +21,13 @@
 #include "lora.hpp"
 #include "wave_reduce.hpp"
 
+// The split form of the attention hands partial results from workgroup to workgroup through device-scope
+// stores, a wait on the store counter and a relaxed counter increment (see the comment at the hand-over):
+// an argument about this architecture's caches, not one the language's memory model makes for every target.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "decode_layer.hip: the split attention's hand-over is written for gfx950; revisit it before building for another target"
+#endif
+
 namespace {
 
 constexpr int WAVE = 64;
@@ -452,6 +459,15 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
                 __hip_atomic_store(mine + D, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(mine + D + 1, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+            // Ordering of the hand-over, stated at the level it rests on (the gfx950 memory system, which the
+            // guard at the top of this file pins): the state goes out as device-scope stores, which are written
+            // through to the level every compute die shares; s_waitcnt vmcnt(0) returns when they have been
+            // acknowledged there, so the counter increment below, issued after it, is performed after the
+            // state is in place; the workgroup that reads n_split - 1 from the counter therefore finds every
+            // state with device-scope loads, which do not read the per-die caches (and it drops what those
+            // caches may hold with an acquire fence first, below).  A release on the increment would express
+            // the same in the language's memory model, and costs a write-back of the die's whole L2 per
+            // workgroup.
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have completed before the workgroup counts itself
         } else {
             const uint32_t bits = f32_to_bf16_bits(o);
@@ -465,6 +481,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         if (tid == 0) s_before = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (s_before != (uint32_t)(n_split - 1)) return;  // uniform: somebody else arrives last
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // only the merging workgroup pays for it, once per pair
         if (tid < D) {
             const float *all = a.partials + ((long)m * a.n_heads + h) * n_split * (D + 2);
             // every state is requested before any is used: one memory round trip

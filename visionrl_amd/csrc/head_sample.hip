@@ -46,6 +46,16 @@ struct HeadArgs {
     uint16_t *ct;            // [B, V]
     int32_t B, tiles, rounds, reserved;
     float w, inv_t;
+    // optional parts (vrl_int4_head_extras): each pointer may be null
+    const uint16_t *bias;         // [V]: logits = bf16(bf16(x . W^T) + bias)
+    const uint16_t *embed_table;  // [V, embed_dim]
+    uint16_t *next_embeds;        // [2B, embed_dim]
+    long long *tokens;            // [B, token_stride]
+    float *logprobs;              // [B, token_stride]
+    long long *position;          // device scalar: column of tokens / logprobs, incremented by the call
+    long long *slot;              // device scalar incremented by the call
+    long long *position_seen;     // in the workspace: the position as the first kernel found it
+    int32_t embed_dim, token_stride;
 };
 
 __device__ __forceinline__ float hs_round_bf16(float v) {
@@ -270,7 +280,34 @@ __global__ __launch_bounds__(MERGE_THREADS) void head_merge_kernel(HeadArgs a) {
             bc = bf16_bits_to_f32(ctp[0]);
         }
         a.sampled[b] = bi;
-        a.logprob[b] = hs_round_bf16(bc - cm - logf(cs));
+        const float lp = hs_round_bf16(bc - cm - logf(cs));
+        a.logprob[b] = lp;
+        if (a.position) {   // the step's bookkeeping (policy.py:695-696): token and log-probability at the position
+            const long long pos = *a.position_seen;
+            if (pos >= 0 && pos < a.token_stride) {
+                if (a.tokens) a.tokens[(long)b * a.token_stride + pos] = bi;
+                if (a.logprobs) a.logprobs[(long)b * a.token_stride + pos] = lp;
+            }
+            if (b == 0) {
+                *a.position = pos + 1;
+                if (a.slot) *a.slot += 1;
+            }
+        }
+        red_i[0] = bi;
+    }
+    if (a.embed_table) {   // uniform: the next input of both rows of the pair (policy.py:698-700)
+        __syncthreads();
+        const int token = red_i[0];
+        const int words = a.embed_dim >> 3;   // 16-byte words per row
+        gptr_cw4 src = (gptr_cw4)(uintptr_t)(a.embed_table + (long)token * a.embed_dim);
+        typedef __attribute__((address_space(1))) u32x4_t *gptr_w4;
+        gptr_w4 dst_c = (gptr_w4)(uintptr_t)(a.next_embeds + (long)b * a.embed_dim);
+        gptr_w4 dst_u = (gptr_w4)(uintptr_t)(a.next_embeds + (long)(a.B + b) * a.embed_dim);
+        for (int j = tid; j < words; j += MERGE_THREADS) {
+            const u32x4_t v = src[j];
+            dst_c[j] = v;
+            dst_u[j] = v;
+        }
     }
 }
 
@@ -297,6 +334,8 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
     const int sc0 = min(nsc, kw * per), sc1 = min(nsc, sc0 + per);
     const rsrc_t rsrc = pp_blob_rsrc(p);
     const int t0 = blockIdx.x * TW * a.rounds, t1 = min(a.tiles, t0 + TW * a.rounds);
+    // the second kernel's workgroups all need the position this call writes at, and one of them moves it on
+    if (a.position && blockIdx.x == 0 && threadIdx.x == 0) *a.position_seen = *a.position;
     PPRing<1, GQ> ring;
     int tile = t0 + tw;
     bool work = sc0 < sc1 && tile < t1;   // wave-uniform
@@ -326,6 +365,13 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
             for (int w = 1; w < KS; ++w)
 #pragma unroll
                 for (int b = 0; b < MB; ++b) acc[0][b] += red[((w - 1) * MB + b) * WAVE + lane];
+            if (a.bias) {   // uniform: the module adds its bias to its bf16 output tensor
+                const float bias = bf16_bits_to_f32(as_global(a.bias)[min(tile * 16 + (lane & 15), p.N - 1)]);
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[0][b][i] = hs_round_bf16(hs_round_bf16(acc[0][b][i]) + bias);
+            }
             if (p.y) store_tile<MB, false>(p, tile, acc);
             head_tile_logits<MB>(acc, tb);
         }
@@ -342,7 +388,7 @@ constexpr size_t HS_LDS_CAP = 160 * 1024;   // what a workgroup can have
 size_t hs_align(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct HeadLayout {
-    size_t rec, gt, ct, total;
+    size_t rec, gt, ct, pos, total;
 };
 
 HeadLayout head_layout(int B, int V) {
@@ -351,7 +397,8 @@ HeadLayout head_layout(int B, int V) {
     l.rec = 0;
     l.gt = l.rec + hs_align((size_t)B * tiles * 32);
     l.ct = l.gt + hs_align((size_t)B * V * sizeof(uint16_t));
-    l.total = l.ct + hs_align((size_t)B * V * sizeof(uint16_t));
+    l.pos = l.ct + hs_align((size_t)B * V * sizeof(uint16_t));
+    l.total = l.pos + 256;
     return l;
 }
 
@@ -393,7 +440,7 @@ int cu_count() {
 
 int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t *sampled, float *logprob, int B,
                        float cfg_weight, float temperature, void *workspace, size_t workspace_bytes,
-                       void *hip_stream) {
+                       void *hip_stream, const vrl_int4_head_extras *extras = nullptr) {
     if (!head || !noise || !sampled || !logprob || !workspace) return VRL_INT4_ENULL;
     if (!head->x || !head->qweight) return VRL_INT4_ENULL;
     if (!head->prepacked || head->fused_gate_up) return VRL_INT4_ESHAPE;
@@ -440,6 +487,31 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
     args.tiles = V / 16;
     args.w = cfg_weight;
     args.inv_t = 1.0f / temperature;
+    if (extras) {
+        const vrl_int4_head_extras &e = *extras;
+        if (e.embed_table || e.next_embeds) {
+            if (!e.embed_table || !e.next_embeds) return VRL_INT4_ENULL;
+            if (e.embed_dim < 8 || e.embed_dim % 8 != 0) return VRL_INT4_ESHAPE;
+            if ((reinterpret_cast<uintptr_t>(e.embed_table) | reinterpret_cast<uintptr_t>(e.next_embeds)) & 15u)
+                return VRL_INT4_EALIGN;
+        }
+        if ((e.tokens || e.logprobs || e.slot) && !e.position) return VRL_INT4_ENULL;
+        if (e.position && e.token_stride < 1) return VRL_INT4_ESHAPE;
+        if ((reinterpret_cast<uintptr_t>(e.bias) & 1u) || (reinterpret_cast<uintptr_t>(e.tokens) & 7u) ||
+            (reinterpret_cast<uintptr_t>(e.logprobs) & 3u) || (reinterpret_cast<uintptr_t>(e.position) & 7u) ||
+            (reinterpret_cast<uintptr_t>(e.slot) & 7u))
+            return VRL_INT4_EALIGN;
+        args.bias = static_cast<const uint16_t *>(e.bias);
+        args.embed_table = static_cast<const uint16_t *>(e.embed_table);
+        args.next_embeds = static_cast<uint16_t *>(e.next_embeds);
+        args.tokens = reinterpret_cast<long long *>(e.tokens);
+        args.logprobs = e.logprobs;
+        args.position = reinterpret_cast<long long *>(e.position);
+        args.slot = reinterpret_cast<long long *>(e.slot);
+        args.position_seen = reinterpret_cast<long long *>(ws + lay.pos);
+        args.embed_dim = e.embed_dim;
+        args.token_stride = e.token_stride;
+    }
     // as many workgroups as the device holds at once: a second round of workgroups would stage x again
     const long per_cu = std::max<long>(1, std::min<long>(16 / (ks * tw), (long)(160 * 1024 / std::max<size_t>(lds, 1024))));
     const long capacity = per_cu * cu_count();
@@ -476,7 +548,7 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
 // handle for that query, not a device address).
 constexpr int HS_STATIC_MAX_V = 16384;
 constexpr size_t HS_STATIC_BYTES = (size_t)HS_MAX_B * (HS_STATIC_MAX_V / 16) * 32 +
-                                   2 * (size_t)HS_MAX_B * HS_STATIC_MAX_V * 2;   // 1,572,864 bytes
+                                   2 * (size_t)HS_MAX_B * HS_STATIC_MAX_V * 2 + 256;   // 1,573,120 bytes
 static __device__ __align__(256) unsigned char scratch[HS_STATIC_BYTES];
 
 constexpr int HS_MAX_DEVICES = 64;
@@ -526,6 +598,14 @@ int vrl_int4_head_sample_bf16(const vrl_int4_problem *head, const void *noise, i
                               void *hip_stream) {
     return head_sample_launch(head, noise, sampled, logprob, B, cfg_weight, temperature, workspace, workspace_bytes,
                               hip_stream);
+}
+
+int vrl_int4_head_sample_ex_bf16(const vrl_int4_problem *head, const vrl_int4_head_extras *extras, const void *noise,
+                                 int64_t *sampled, float *logprob, int B, float cfg_weight, float temperature,
+                                 void *workspace, size_t workspace_bytes, void *hip_stream) {
+    if (!extras) return VRL_INT4_ENULL;
+    return head_sample_launch(head, noise, sampled, logprob, B, cfg_weight, temperature, workspace, workspace_bytes,
+                              hip_stream, extras);
 }
 
 }  // extern "C"

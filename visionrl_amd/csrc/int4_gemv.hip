@@ -463,9 +463,14 @@ struct DirectLora {   // adapters joined to a plan-free launch: down-projections
 };
 
 static int direct_launch(const vrl_int4_problem *problems, int n_problems, const vrl_int4_norm *norm,
-                         const DirectLora *lora, void *hip_stream) {
+                         const DirectLora *lora, void *hip_stream, const vrl_int4_epilogue *epilogue = nullptr) {
     if (!problems) return VRL_INT4_ENULL;
     if (n_problems < 1 || n_problems > DIRECT_MAX) return VRL_INT4_ESHAPE;
+    if (epilogue) {   // one plain problem: the bias belongs to its columns
+        if (n_problems != 1 || problems[0].fused_gate_up || lora) return VRL_INT4_ESHAPE;
+        if (epilogue->activation != VRL_INT4_ACT_NONE && epilogue->activation != VRL_INT4_ACT_GELU) return VRL_INT4_ESHAPE;
+        if (reinterpret_cast<uintptr_t>(epilogue->bias) & 1u) return VRL_INT4_EALIGN;
+    }
     bool fused_any = false;
     int max_nsc = 1, max_m = 1;
     long slab_tiles = 0;  // 16-column tiles x 16-row slabs of the launch
@@ -518,6 +523,11 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         args.norm.h_out = static_cast<uint16_t *>(norm->h_out);
         args.norm.eps = norm->eps;
         args.norm.enabled = 1;
+    }
+    if (epilogue && (epilogue->bias || epilogue->activation != VRL_INT4_ACT_NONE)) {
+        args.epi.bias = static_cast<const uint16_t *>(epilogue->bias);
+        args.epi.act = epilogue->activation;
+        args.epi.enabled = 1;
     }
     long workgroups = 0;
     size_t x_bytes = 0;
@@ -643,6 +653,12 @@ int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_pr
                                       const vrl_int4_norm *norm, void *hip_stream) {
     if (!norm) return VRL_INT4_ENULL;
     return direct_launch(problems, n_problems, norm, nullptr, hip_stream);
+}
+
+int vrl_int4_gemv_prepacked_epilogue_bf16(const vrl_int4_problem *problem, const vrl_int4_norm *norm,
+                                          const vrl_int4_epilogue *epilogue, void *hip_stream) {
+    if (!epilogue) return VRL_INT4_ENULL;
+    return direct_launch(problem, 1, norm, nullptr, hip_stream, epilogue);
 }
 
 size_t vrl_int4_grouped_plan_size(int n_problems) {

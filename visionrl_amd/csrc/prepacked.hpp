@@ -799,9 +799,48 @@ __device__ __forceinline__ void store_tile_lora(const DevProblem &p, int tile_lo
     }
 }
 
+// Bias and activation of a linear applied to the tile before it is stored (plan-free launches of one plain
+// problem): y = act(bf16(bf16(x . W^T) + bias)), the roundings of a bf16 module whose bias is added to its
+// output tensor and whose activation is a tensor op of its own (Janus' generation head is Linear, GELU, Linear:
+// vrl/models/families/janus_pro/policy.py:138-160 calls it).
+struct EpiArgs {
+    const uint16_t *bias;   // bf16 [N] or nullptr
+    int32_t act;            // 0: none; 1: GELU, x / 2 * (1 + erf(x / sqrt 2)) in fp32
+    int32_t enabled;
+};
+
+__device__ __forceinline__ float epi_round_bf16(float v) {
+    return bf16_bits_to_f32(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+}
+
+__device__ __forceinline__ float epi_apply(float acc, float bias, bool has_bias, int act) {
+    float v = epi_round_bf16(acc);
+    if (has_bias) v = epi_round_bf16(v + bias);
+    if (act == 1) v = v * 0.5f * (1.0f + erff(v * 0.70710678118654752440f));
+    return v;
+}
+
+// store_tile<1, false> with the epilogue
+__device__ __forceinline__ void store_tile_epi(const DevProblem &p, int tile_local, const f32x4_t &acc,
+                                               const EpiArgs &e) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int col = tile_local * 16 + (lane & 15);
+    if (col >= p.N) return;
+    const bool has_bias = e.bias != nullptr;
+    const float bias = has_bias ? bf16_bits_to_f32(as_global(e.bias)[col]) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = 4 * (lane >> 4) + i;
+        if (m < p.M)
+            as_global(p.y)[(long)m * p.N + col] =
+                (uint16_t)(pack_bf16_rne(epi_apply(acc[i], bias, has_bias, e.act), 0.0f) & 0xFFFFu);
+    }
+}
+
 template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG, bool UP = false>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
-                                                 const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{}) {
+                                                 const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{},
+                                                 const EpiArgs &epi = EpiArgs{}) {
     constexpr int RS = FUSED ? 2 : 1;
     static_assert(!XG || (TW == 1 && !NORM), "register-fed activations: one tile per workgroup, no norm");
     static_assert(!UP || (!FUSED && !NORM), "an adapter's up-projection joins a plain problem");
@@ -877,7 +916,12 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
                 if (up.fp32) store_tile_lora<true>(p, tile, acc[0][0], up, lora_ts, brows);
                 else store_tile_lora<false>(p, tile, acc[0][0], up, lora_ts, brows);
             } else {
-                store_tile<1, FUSED>(p, tile, acc);
+                if constexpr (!FUSED) {
+                    if (epi.enabled) store_tile_epi(p, tile, acc[0][0], epi);   // uniform over the launch
+                    else store_tile<1, false>(p, tile, acc);
+                } else {
+                    store_tile<1, FUSED>(p, tile, acc);
+                }
             }
         }
         work = work && next >= 0;
@@ -888,7 +932,8 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
 template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool UP = false>
 __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem,
-                                               const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{}) {
+                                               const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{},
+                                               const EpiArgs &epi = EpiArgs{}) {
     if constexpr (UP) {
         if (p.G == 128) split_segment_pp<false, KS, TW, 1, false, XG, true>(p, t0, t1, smem, norm, up);
         else if (p.G == 64) split_segment_pp<false, KS, TW, 2, false, XG, true>(p, t0, t1, smem, norm, up);
@@ -898,9 +943,9 @@ __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int 
         else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
         else split_segment_pp<FUSED, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
     } else {
-        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm);
-        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
-        else split_segment_pp<false, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm, up, epi);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm, up, epi);
+        else split_segment_pp<false, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm, up, epi);
     }
 }
 
@@ -948,6 +993,7 @@ struct DirectArgs {
     NormArgs norm;                // read by the NORM instantiations only
     LoraDownArgs ld;              // read by the LD instantiations only
     LoraUpArgs up;                // read by the UP instantiations only
+    EpiArgs epi;                  // bias / activation before the store (plain problems; enabled = 0: none)
 };
 
 template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD, bool UP>
@@ -967,7 +1013,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
     const int t0 = (g - p.tile_begin) * TW * a.rounds;
-    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW * a.rounds), smem, a.norm, a.up);
+    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW * a.rounds), smem, a.norm, a.up, a.epi);
 }
 
 }  // namespace

@@ -168,7 +168,11 @@ class NativeDecodeTrunk:
             return str(exc)
         return None
 
-    def __init__(self, trunk, cache, cur: torch.Tensor, mask: torch.Tensor, slot: torch.Tensor):
+    def __init__(self, trunk, cache, cur: torch.Tensor, mask: torch.Tensor, slot: torch.Tensor,
+                 final_norm: bool = True):
+        """``final_norm=False`` (hidden sizes up to 4096) leaves the model's last norm to the launch that
+        consumes the step's output: :attr:`final` then holds ``(x, residual, norm weight, eps)`` for a
+        launch that normalises while it stages its input, and :meth:`run` returns ``None``."""
         rows, one, hidden = cur.shape
         why = self.unsupported(trunk, rows, mask.shape[1])
         if why is not None:
@@ -205,6 +209,7 @@ class NativeDecodeTrunk:
         split_ws = ops.rope_attn_split_workspace(rows, H, D, dev) \
             if rows * H <= self.SPLIT_ATTENTION_PAIRS and self.max_len >= self.SPLIT_ATTENTION_FROM else None
         self._keep.append(split_ws)
+        self._split_ws = split_ws
         calls = []       # (function, argument tuple without the stream)
         state = {"x": cur.view(rows, hidden), "res": None, "flip": 0}   # x: sublayer output not yet added to res
 
@@ -306,9 +311,14 @@ class NativeDecodeTrunk:
             (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
             (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])
         w, eps = norm_weight(trunk.norm)
-        calls.append((lib.vrl_add_rmsnorm_bf16,
-                      (state["x"].data_ptr(), state["res"].data_ptr(), w.data_ptr(),
-                       streams[state["flip"]].data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+        self.final = None
+        if final_norm or not fuse_norm:
+            calls.append((lib.vrl_add_rmsnorm_bf16,
+                          (state["x"].data_ptr(), state["res"].data_ptr(), w.data_ptr(),
+                           streams[state["flip"]].data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+        else:
+            self.final = (state["x"], state["res"], w, eps)
+            self.normed = None
         self._calls = calls
         self.launches = len(calls)
 
@@ -319,5 +329,9 @@ class NativeDecodeTrunk:
             for fn, args in self._calls:
                 rc = fn(*args, stream)
                 if rc:
+                    # a step that stopped half-way may leave the split attention's arrival counters above zero,
+                    # and every later launch over that workspace would then merge too early: clear them
+                    if self._split_ws is not None and not torch.cuda.is_current_stream_capturing():
+                        self._split_ws.zero_()
                     _lib.check(rc, fn.__name__)
         return self.normed

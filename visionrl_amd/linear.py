@@ -40,12 +40,23 @@ def _version(t: torch.Tensor):
 
 
 def _source_state(*tensors):
-    """Identity and modification counters of the tensors a prepacked copy was made from."""
-    return tuple((t, _version(t)) for t in tensors)
+    """What identifies the tensors a prepacked copy was made from: a weak reference to each, its
+    modification counter and, for a tensor torch keeps no counter for (an inference tensor), the address
+    and shape of its data instead.  In-place writes to such a tensor go unnoticed: ``prepack_()`` again
+    after editing int4 buffers that were created under ``torch.inference_mode``."""
+    return tuple((weakref.ref(t), _version(t), (t.data_ptr(), tuple(t.shape))) for t in tensors)
 
 
 def _source_changed(state, *tensors) -> bool:
-    return any(t is not t0 or v0 is None or _version(t) != v0 for t, (t0, v0) in zip(tensors, state))
+    for t, (ref, v0, where) in zip(tensors, state):
+        if ref() is not t:
+            return True
+        if v0 is None:
+            if (t.data_ptr(), tuple(t.shape)) != where:
+                return True
+        elif _version(t) != v0:
+            return True
+    return False
 
 
 def _rows(x: torch.Tensor, in_features: int) -> torch.Tensor:

@@ -26,7 +26,7 @@ from .int4_format import check_packed
 __all__ = ["int4_gemv", "int4_dequant", "int4_gate_up_silu", "int4_gemv_into", "int4_prepack",
            "PrepackedWeight", "GroupedGemv", "DirectGemv", "int4_gemv_prepacked_into",
            "int4_gemv_prepacked_multi_into", "DirectCall", "cfg_sample", "head_sample", "head_sample_supported",
-           "head_sample_workspace", "add_rmsnorm", "rope_attn_split_workspace",
+           "head_sample_workspace", "EpilogueGemv", "add_rmsnorm", "rope_attn_split_workspace",
            "rope_attn_decode", "LoraAdd"]
 
 
@@ -461,6 +461,42 @@ def int4_gemv_prepacked_multi_into(ys, x: torch.Tensor, weights) -> None:
     _lib.check(rc, "vrl_int4_gemv_prepacked_bf16")
 
 
+class EpilogueGemv:
+    """One prepacked linear with its bias and a following GELU applied before the store, one plan-free launch:
+    ``y = act(bf16(bf16(x . W^T) + bias))``, optionally over ``weight * rmsnorm(x + residual)`` instead of ``x``.
+
+    The first half of Janus' two-layer image-token head (``Linear``, ``GELU``, ``Linear``; called through
+    ``gen_head`` at ``vrl/models/families/janus_pro/policy.py:138-160``) and any biased linear.  ``x`` is a
+    contiguous bf16 ``[M <= 32, K]`` tensor; ``bias`` bf16 ``[N]`` or ``None``; ``gelu`` the exact (erf) form of
+    ``torch.nn.GELU()``; ``norm = (residual | None, weight, eps)`` as in :class:`DirectGemv` (K <= 4096).  The
+    record is built once; the tensors captured here must stay alive and in place.
+    """
+
+    def __init__(self, x: torch.Tensor, weight: "PrepackedWeight", bias: torch.Tensor | None = None,
+                 gelu: bool = False, norm=None, out: torch.Tensor | None = None):
+        self._gemv = DirectGemv([(x, weight, False)], outputs=None if out is None else [out],
+                                norm=None if norm is None else (*norm, None))
+        self.device = self._gemv.device
+        if bias is not None:
+            if bias.dtype != torch.bfloat16 or tuple(bias.shape) != (weight.N,) or not bias.is_contiguous():
+                raise ValueError(f"bias must be contiguous bfloat16 [{weight.N}]")
+            _require_device("bias", bias, self.device)
+        self.epilogue = _lib.Epilogue()
+        self.epilogue.bias = bias.data_ptr() if bias is not None else None
+        self.epilogue.activation = _lib.ACT_GELU if gelu else _lib.ACT_NONE
+        self._keep = bias
+        self.output = self._gemv.outputs[0]
+
+    def launch(self) -> torch.Tensor:
+        g = self._gemv
+        with _on(self.device):
+            rc = _lib.load().vrl_int4_gemv_prepacked_epilogue_bf16(
+                g.table, ctypes.byref(g.norm) if g.norm is not None else None, ctypes.byref(self.epilogue),
+                _stream_handle(self.device))
+        _lib.check(rc, "vrl_int4_gemv_prepacked_epilogue_bf16")
+        return self.output
+
+
 def cfg_sample(logits: torch.Tensor, cfg_weight: float, temperature: float, *,
                generator: torch.Generator | None = None, noise: torch.Tensor | None = None):
     """CFG combine, softmax, one multinomial draw and its log-probability, in one launch.
@@ -518,7 +554,8 @@ def head_sample_workspace(B: int, V: int, device) -> torch.Tensor:
 
 def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, temperature: float, *,
                 generator: torch.Generator | None = None, noise: torch.Tensor | None = None,
-                logits_out: torch.Tensor | None = None, workspace: "torch.Tensor | str | None" = None, out=None):
+                logits_out: torch.Tensor | None = None, workspace: "torch.Tensor | str | None" = None, out=None,
+                bias: torch.Tensor | None = None, bookkeeping=None, embedding=None):
     """The image-token head and the sampling tail of a decode step in one launch.
 
     Stands for ``vrl/models/families/janus_pro/policy.py:684-693``: ``x`` is the bf16 ``[2B, K]``
@@ -530,6 +567,14 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     the string ``"static"`` for the library's own fixed scratch (``vrl_int4_head_sample_static_bf16``:
     B <= 16, V <= 16384, one call at a time per GPU); with ``noise`` and ``out = (sampled, logprob)``
     given as well, the call then allocates nothing.
+
+    The parts of the step around it, done by the same call when given (``vrl_int4_head_sample_ex_bf16``):
+    ``bias`` (bf16 ``[V]``) of a biased head, added to the rounded logits as the module adds it;
+    ``bookkeeping = (tokens int64 [B, L], logprobs float32 [B, L], position int64 [1], slot int64 [1] | None)``:
+    the draw and its log-probability are written at column ``position`` of the two buffers, ``position`` and
+    ``slot`` are incremented (``policy.py:695-696`` over a device-side position); ``embedding = (table bf16
+    [V, H], next bf16 [2B, H])``: rows ``b`` and ``B + b`` of ``next`` receive ``table[sampled[b]]``, the next
+    input embedding of both rows of the pair (``policy.py:698-700`` with ``prepare_gen_img_embeds`` tabulated).
     Raises ``ValueError`` for shapes the launch does not take (:func:`head_sample_supported`).
     """
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[0] % 2 != 0 or x.shape[0] < 2 or x.shape[1] != head.K:
@@ -566,8 +611,48 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     rec = _lib.Problem()
     rec.x, rec.qweight, rec.y = x.data_ptr(), head.blob.data_ptr(), (logits_out.data_ptr() if logits_out is not None else None)
     rec.M, rec.N, rec.K, rec.G, rec.prepacked = 2 * B, V, head.K, head.group_size, 1
+    extras = None
+    if bias is not None or bookkeeping is not None or embedding is not None:
+        if static:
+            raise ValueError("the library's fixed scratch serves the plain call only")
+        extras = _lib.HeadExtras()
+        if bias is not None:
+            if bias.dtype != torch.bfloat16 or tuple(bias.shape) != (V,) or not bias.is_contiguous():
+                raise ValueError(f"bias must be contiguous bfloat16 [{V}]")
+            _require_device("bias", bias, dev)
+            extras.bias = bias.data_ptr()
+        if bookkeeping is not None:
+            tokens, logprobs, position, slot = bookkeeping
+            if tokens.dtype != torch.int64 or logprobs.dtype != torch.float32 or tokens.dim() != 2 or \
+                    tokens.shape != logprobs.shape or tokens.shape[0] != B or not tokens.is_contiguous() or \
+                    not logprobs.is_contiguous():
+                raise ValueError(f"bookkeeping buffers must be contiguous int64 / float32 [{B}, L]")
+            for name, t in (("position", position), ("slot", slot)):
+                if t is not None and (t.dtype != torch.int64 or t.numel() != 1):
+                    raise ValueError(f"{name} must be an int64 device scalar")
+            for name, t in (("tokens", tokens), ("logprobs", logprobs), ("position", position), ("slot", slot)):
+                if t is not None:
+                    _require_device(name, t, dev)
+            extras.tokens, extras.logprobs, extras.position = tokens.data_ptr(), logprobs.data_ptr(), position.data_ptr()
+            extras.slot = slot.data_ptr() if slot is not None else None
+            extras.token_stride = tokens.shape[1]
+        if embedding is not None:
+            table, nxt = embedding
+            H = table.shape[-1]
+            if table.dtype != torch.bfloat16 or tuple(table.shape) != (V, H) or not table.is_contiguous() or H % 8:
+                raise ValueError(f"embedding table must be contiguous bfloat16 [{V}, H], H a multiple of 8")
+            if nxt.dtype != torch.bfloat16 or nxt.numel() != 2 * B * H or not nxt.is_contiguous():
+                raise ValueError(f"next embeddings must be contiguous bfloat16 with {2 * B} rows of {H}")
+            _require_device("embedding table", table, dev)
+            _require_device("next embeddings", nxt, dev)
+            extras.embed_table, extras.next_embeds, extras.embed_dim = table.data_ptr(), nxt.data_ptr(), H
     with _on(dev):
-        if static:   # the library's own scratch: the call allocates nothing
+        if extras is not None:
+            rc = _lib.load().vrl_int4_head_sample_ex_bf16(ctypes.byref(rec), ctypes.byref(extras), noise.data_ptr(),
+                                                          sampled.data_ptr(), logprob.data_ptr(), B, float(cfg_weight),
+                                                          float(temperature), workspace.data_ptr(), workspace.numel(),
+                                                          _stream_handle(dev))
+        elif static:   # the library's own scratch: the call allocates nothing
             rc = _lib.load().vrl_int4_head_sample_static_bf16(ctypes.byref(rec), noise.data_ptr(), sampled.data_ptr(),
                                                               logprob.data_ptr(), B, float(cfg_weight),
                                                               float(temperature), _stream_handle(dev))
@@ -737,6 +822,8 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
             rc = _lib.load().vrl_rope_attn_decode_bf16(*args, _stream_handle(dev))
         else:
             rc = _lib.load().vrl_rope_attn_decode_lora_bf16(*args, ctypes.byref(record), _stream_handle(dev))
+    if rc and split_workspace is not None and not torch.cuda.is_current_stream_capturing():
+        split_workspace.zero_()   # arrival counters a failed launch may have left above zero
     _lib.check(rc, "vrl_rope_attn_decode_bf16")
     return out
 
