@@ -789,7 +789,7 @@ class ValuDotLaunch:
     def __init__(self, problems):
         import ctypes
 
-        from visionrl_amd import _lib
+        from visionrl_amd import _lib, ops
 
         for x, pw, fused in problems:
             if x.shape[0] != 1 or fused or pw.group_size != 128:
