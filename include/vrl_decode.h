@@ -80,6 +80,20 @@ int vrl_rope_attn_decode_split_bf16(const void *q, const void *k, const void *v,
                                     void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
+ * vrl_rope_attn_decode_bf16 with one position per row: `positions` is int64 [M] in device memory and row m
+ * takes slot positions[m] (rotary tables, cache append, attended range), for a chunk whose rows advance at
+ * different times (the scheduler's partial batches: policy.py:631-645 steps a subset of the rows, which
+ * vrl/models/ar.py:42-110 cuts out of the cache and puts back; over a static cache every row keeps its own
+ * slot counter instead).  A row whose position lies outside [0, L_max) is left alone.  With `workspace`
+ * not NULL it is the split form (vrl_rope_attn_decode_split_bf16, same preconditions), else the plain one.
+ */
+int vrl_rope_attn_decode_rows_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                   void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                   const void *mask, const int64_t *positions, void *out,
+                                   int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                   void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
  * LoRA adapters on top of an int4 projection, for the decode step of a policy whose attention
  * projections carry PEFT adapters (vrl/models/families/janus_pro/policy.py:298-324: rank 32 on
  * q/k/v/o by default, policy.py:81-88); the wrapper computes
@@ -155,7 +169,7 @@ typedef struct vrl_attn_lora {
     int32_t r[3];            /* ranks (q, k, v): multiples of 8 up to 64 */
     int32_t offset[3];       /* first column of each adapter in t, a multiple of 4 */
     float scaling[3];
-    int32_t reserved;
+    int32_t position_per_row; /* 1: `position` of the call is int64 [M], one slot per row (vrl_rope_attn_decode_rows_bf16) */
     const void *o_A;         /* [o_r, n_heads * D] (type as weights_fp32 says), 16-byte aligned, or NULL */
     float *o_t;              /* [M, n_heads, o_r] float32, 16-byte aligned */
     int32_t o_r;             /* a multiple of 8 up to 64 */

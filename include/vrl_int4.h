@@ -256,6 +256,10 @@ int vrl_int4_head_sample_bf16(const vrl_int4_problem *head, const void *noise, i
  *   embed_table  bf16 [V, embed_dim], row t the input embedding of image token t (what
  *                prepare_gen_img_embeds returns for it, policy.py:698-700): rows b and B + b of next_embeds
  *                (bf16 [2B, embed_dim]) receive row sampled[b]; embed_dim a multiple of 8, 16-byte aligned rows
+ *   position_per_row = 1: position is int64 [B] and slot int64 [2B], one counter per batch row (pair of
+ *                rows), for a chunk whose rows advance at different times; `active` (uint8 [B], NULL: all) then
+ *                names the rows of this step's batch: only they are written, counted on and given a next input
+ *                (sampled / logprob are computed for every row; noise rows of the others are not used)
  * All of it is done by the call's second kernel, one workgroup per batch row.  workspace as for
  * vrl_int4_head_sample_bf16.
  */
@@ -269,6 +273,9 @@ typedef struct vrl_int4_head_extras {
     int64_t *slot;
     int32_t embed_dim;
     int32_t token_stride;
+    const uint8_t *active;
+    int32_t position_per_row;
+    int32_t reserved;   /* 0 */
 } vrl_int4_head_extras;
 
 int vrl_int4_head_sample_ex_bf16(const vrl_int4_problem *head, const vrl_int4_head_extras *extras, const void *noise,

@@ -739,3 +739,109 @@ def test_two_layer_head_logits_against_the_oracle():
     got = o.bf16_bits_to_f32(bf16_to_bits(logits)).astype(np.float64)
     # the linear's tolerance, and one more bf16 rounding for the sum with the bias
     assert (np.abs(got - (y2 + b2)) <= o.gemv_tolerance(y2, a2) + o.bf16_ulp(y2 + b2)).all()
+
+
+# ------------------------------------------------------------------ partial scheduler batches over the static cache
+@pytest.mark.gpu
+@pytest.mark.parametrize("head,batch_size", [("linear", 2), ("two_layer", 2), ("linear", 4)])
+def test_partial_batches_run_over_the_static_cache(int4_policy, head, batch_size, monkeypatch):
+    """A token scheduler that steps fewer rows than the chunk holds (``policy.py:631-645`` with ``row_indices``;
+    the reference cuts those rows out of its per-row caches, ``vrl/models/ar.py:42-110``): on the native path the
+    rows keep one static cache and a slot counter each.  Rows are independent given their draws, so the result
+    must be, bit for bit, what the same sampler gives when it steps every row together with the very draws the
+    partial batches used (recorded in the first run, injected in the second), and the draws are made per batch,
+    in the order of its rows, as ``torch.multinomial`` would make them for those rows alone."""
+    from visionrl_amd import ops
+
+    print("ar decode: partial scheduler batches,", head, batch_size, flush=True)
+    policy = int4_policy if head == "linear" else janus_shaped_policy(False)
+    B, n_img = 5, 9
+    inputs = make_inputs(B, 7, torch.bfloat16, "cuda:0", seed=71)
+    vocab = VOCAB_IMG
+    original = ops.head_sample
+    calls = []
+
+    def recording(x, packed, w, t, **kw):
+        calls.append((kw["active"].clone(), kw["noise"].clone()))
+        return original(x, packed, w, t, **kw)
+
+    monkeypatch.setattr(ops, "head_sample", recording)
+    sampler = install_static_ar_sampler(policy, graph=False)
+    torch.manual_seed(72)
+    (got_t, got_lp), results = scheduled_loop(policy, inputs, n_img, batch_size=batch_size)
+    torch.cuda.synchronize()
+    groups = [list(range(g, min(B, g + batch_size))) for g in range(0, B, batch_size)]
+    assert len(results) == n_img * len(groups) and len(calls) == len(results)
+    (sess,) = sampler._sessions.values()
+    assert sess.native_rows is not None and sess.native_rows.launches == 5 * LAYERS + 1
+    assert got_t.shape == (B, n_img) and int(sess.pos_rows.min()) == n_img and int(sess.pos_rows.max()) == n_img
+    assert sess.slot_rows.tolist() == [7 + n_img - 1] * (2 * B)
+    # the draws were made batch by batch, for the rows of the batch only, continuing one random stream
+    torch.manual_seed(72)
+    step = 0
+    assembled = torch.ones((n_img, B, vocab), dtype=torch.bfloat16, device="cuda:0")
+    for p in range(n_img):
+        for rows in groups:
+            active, noise = calls[step]
+            assert active.tolist() == [1 if r in rows else 0 for r in range(B)]
+            want = torch.empty((len(rows), vocab), dtype=torch.bfloat16, device="cuda:0").exponential_(1.0)
+            assert torch.equal(noise[rows], want)
+            assembled[p, rows] = want
+            res = results[step]
+            assert res.positions == [p] * len(rows) and res.sequence_ids == [f"s{r}" for r in rows]
+            assert torch.equal(res.token, got_t[rows, p]) and torch.equal(res.log_prob, got_lp[rows, p])
+            step += 1
+    # the same draws, every row stepped together
+    k = [0]
+
+    def injecting(x, packed, w, t, **kw):
+        kw["noise"] = assembled[k[0]].contiguous()
+        k[0] += 1
+        return original(x, packed, w, t, **kw)
+
+    monkeypatch.setattr(ops, "head_sample", injecting)
+    together = StaticARSampler(policy, graph=False)
+    want_t, want_lp = together.sample_image_tokens(*inputs, cfg_weight=5.0, temperature=1.0, image_token_num=n_img)
+    torch.cuda.synchronize()
+    assert k[0] == n_img and len(want_t.unique()) > n_img
+    assert torch.equal(got_t, want_t)
+    if head == "linear":
+        assert torch.equal(got_lp, want_lp)
+    else:   # stepping all rows together, the head's front is one launch with the last norm folded in
+        torch.testing.assert_close(got_lp, want_lp, rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.gpu
+def test_a_partial_batch_after_steps_of_the_whole_chunk(int4_policy):
+    """The scheduler may narrow its batch in the middle of a generation: the shared counters become one per row
+    where they stand, and the rows go on from there; repeated finalize calls return the same tokens."""
+    print("ar decode: whole-chunk steps, then partial batches", flush=True)
+    B, n_img = 4, 6
+    inputs = make_inputs(B, 7, torch.bfloat16, "cuda:0", seed=81)
+    install_static_ar_sampler(int4_policy, graph=True)
+    state = int4_policy.init_ar_state(*inputs, cfg_weight=5.0, temperature=1.0, image_token_num=n_img)
+    seqs = [Seq(r, n_img) for r in range(B)]
+    torch.manual_seed(82)
+    for _ in range(3):
+        int4_policy.step_ar(state, seqs)
+        for seq in seqs:
+            seq.position += 1
+    head_tokens = state.token_ids[:, :3].clone()
+    for p in range(3, n_img):
+        for rows in ([0, 1, 2], [3]):
+            batch = [seqs[r] for r in rows]
+            res = int4_policy.step_ar(state, batch)
+            assert res.positions == [p] * len(rows)
+            for seq in batch:
+                seq.position += 1
+    with pytest.raises(ValueError, match="finished"):
+        int4_policy.step_ar(state, [seqs[0]])
+    seqs[1].position = 2
+    with pytest.raises(ValueError, match="does not match"):
+        int4_policy.step_ar(state, [seqs[1]])                 # the sequence lags behind its row
+    tokens, logprobs = int4_policy.finalize_ar_state(state)
+    torch.cuda.synchronize()
+    assert state.finished and tokens.shape == (B, n_img) and torch.equal(tokens[:, :3], head_tokens)
+    assert bool((tokens >= 0).all()) and bool((tokens < VOCAB_IMG).all()) and bool((logprobs <= 0).all())
+    again = int4_policy.finalize_ar_state(state)
+    assert torch.equal(again[0], tokens) and torch.equal(again[1], logprobs)

@@ -256,6 +256,60 @@ def test_split_rope_attn_refuses_what_it_does_not_take(ops_mod):
     assert torch.equal(out, plain)
 
 
+@pytest.mark.parametrize("M,H,Hkv,D,L,split", [(6, 16, 16, 128, 640, False), (6, 16, 16, 128, 640, True),
+                                                (32, 16, 16, 128, 384, False), (4, 8, 2, 64, 96, False)])
+def test_rope_attn_with_one_position_per_row(ops_mod, M, H, Hkv, D, L, split):
+    """``vrl_rope_attn_decode_rows_bf16``: every row at its own slot (a chunk whose rows advance at different
+    times).  Row m of the launch equals, bit for bit, row m of the one-position launch at that row's slot over
+    the same cache; a row whose position lies outside the cache is left alone; the oracle agrees row by row."""
+    say("rope_attn, one position per row", M, H, Hkv, D, L, split)
+    rng = np.random.default_rng(M + L)
+    positions = rng.integers(0, L, size=M)
+    positions[0], positions[-1] = L - 1, 0
+    if split:
+        positions[1] = 600        # long enough for several workgroups per pair
+    c = attn_case(4700 + M, M, H, Hkv, D, L, 0)
+    t = {k: bits_to_bf16(c[k], DEV) for k in ("q", "k", "v", "kc", "vc", "cos", "sin")}
+    mask = torch.from_numpy(c["mask"]).to(DEV)
+    ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV) if split else None
+    kc, vc = t["kc"].clone(), t["vc"].clone()
+    pos = torch.from_numpy(positions.astype(np.int64)).to(DEV)
+    out = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc, vc, t["cos"], t["sin"], mask, pos, c["scaling"],
+                                   split_workspace=ws, per_row=True)
+    torch.cuda.synchronize()
+    for p in sorted(set(positions.tolist())):
+        rows = np.nonzero(positions == p)[0]
+        kc1, vc1 = t["kc"].clone(), t["vc"].clone()
+        ws1 = ops_mod.rope_attn_split_workspace(M, H, D, DEV) if split else None
+        one = ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc1, vc1, t["cos"], t["sin"], mask,
+                                       torch.tensor([p], dtype=torch.int64, device=DEV), c["scaling"],
+                                       split_workspace=ws1)
+        torch.cuda.synchronize()
+        assert torch.equal(out[rows], one[rows]), p
+        assert torch.equal(kc[rows], kc1[rows]) and torch.equal(vc[rows], vc1[rows]), p
+        want, _, _ = d.rope_attn_decode(c["q"], c["k"], c["v"], c["kc"], c["vc"], c["cos"], c["sin"], c["mask"], int(p),
+                                        H, Hkv, c["scaling"])
+        got = o.bf16_bits_to_f32(bf16_to_bits(out)).astype(np.float64)[rows]
+        tol = 0.51 * o.bf16_ulp(want[rows].astype(np.float32)) + 2e-5 * np.abs(want[rows]).max()
+        assert (np.abs(got - want[rows]) <= tol).all(), p
+    if split:
+        assert int(ws[: M * H * 4].view(torch.int32).abs().sum()) == 0
+    # a row outside the cache: nothing of it is written, the others as before
+    pos2 = pos.clone()
+    pos2[2] = L + 5
+    kc2, vc2 = t["kc"].clone(), t["vc"].clone()
+    out2 = torch.full_like(out, 7.0)
+    ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc2, vc2, t["cos"], t["sin"], mask, pos2, c["scaling"],
+                             out=out2, split_workspace=ws, per_row=True)
+    torch.cuda.synchronize()
+    keep = [m for m in range(M) if m != 2]
+    assert torch.equal(out2[keep], out[keep]) and bool((out2[2] == 7.0).all())
+    assert torch.equal(kc2[2], t["kc"][2]) and torch.equal(vc2[2], t["vc"][2])
+    with pytest.raises(ValueError):
+        ops_mod.rope_attn_decode(t["q"], t["k"], t["v"], kc2, vc2, t["cos"], t["sin"], mask, pos2[:1], c["scaling"],
+                                 per_row=True)
+
+
 def test_rope_attn_masks_and_strided_inputs(ops_mod):
     say("rope_attn masks, fused qkv buffer")
     M, H, D, L, p = 2, 4, 64, 32, 20

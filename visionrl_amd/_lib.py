@@ -36,6 +36,7 @@ SYMBOLS = (
     "vrl_int4_head_sample_static_bf16",
     "vrl_add_rmsnorm_bf16",
     "vrl_rope_attn_decode_bf16",
+    "vrl_rope_attn_decode_rows_bf16",
     "vrl_rope_attn_decode_split_workspace_bytes",
     "vrl_rope_attn_decode_split_bf16",
     "vrl_rope_attn_decode_lora_bf16",
@@ -108,6 +109,9 @@ class HeadExtras(ctypes.Structure):
         ("slot", ctypes.c_void_p),
         ("embed_dim", ctypes.c_int32),
         ("token_stride", ctypes.c_int32),
+        ("active", ctypes.c_void_p),
+        ("position_per_row", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -138,7 +142,7 @@ class AttnLora(ctypes.Structure):
         ("r", ctypes.c_int32 * 3),
         ("offset", ctypes.c_int32 * 3),
         ("scaling", ctypes.c_float * 3),
-        ("reserved", ctypes.c_int32),
+        ("position_per_row", ctypes.c_int32),
         ("o_A", ctypes.c_void_p),
         ("o_t", ctypes.c_void_p),
         ("o_r", ctypes.c_int32),
@@ -224,6 +228,9 @@ def _bind(lib):
     lib.vrl_rope_attn_decode_bf16.restype = ci
     lib.vrl_rope_attn_decode_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                               ci, ci, ci, ci, ci, ctypes.c_float, vp]
+    lib.vrl_rope_attn_decode_rows_bf16.restype = ci
+    lib.vrl_rope_attn_decode_rows_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
+                                                   ci, ci, ci, ci, ci, ctypes.c_float, vp, ctypes.c_size_t, vp]
     lib.vrl_rope_attn_decode_split_workspace_bytes.restype = ctypes.c_size_t
     lib.vrl_rope_attn_decode_split_workspace_bytes.argtypes = [ci, ci, ci]
     lib.vrl_rope_attn_decode_split_bf16.restype = ci

@@ -86,9 +86,12 @@ class StaticARState:
 
     released: bool = False         # finalized: the session's buffers may serve another generation
     final: Any = None              # (token ids, log-probabilities) as finalize_ar_state returned them
+    row_positions: Any = None      # per-row positions once the scheduler stepped a part of the rows (else None)
 
     @property
     def finished(self) -> bool:
+        if self.row_positions is not None:
+            return min(self.row_positions) >= self.image_token_num
         return self.position >= self.image_token_num
 
     @property
@@ -278,6 +281,71 @@ class _Session:
                 except (TypeError, ValueError):   # something the native launches do not take: module path
                     self.native, self.front_call = False, None
 
+    # -- rows that advance at different times (the scheduler's partial batches) -------------------------
+    def rows_mode_supported(self) -> bool:
+        """Whether a part of the rows can be stepped over the static cache: the native trunk and the one-call
+        head (the module trunk shares one cache position between the rows of a call)."""
+        s = self.sampler
+        packed = self._head_packed() if s.fused_tail and s.fused_head else None
+        return bool(s.native and self.cur.is_cuda and self.cur.dtype == torch.bfloat16 and packed is not None and
+                    ops.head_sample_supported(self.rows2, packed) and
+                    NativeDecodeTrunk.unsupported(s.trunk, self.rows2, self.max_len) is None)
+
+    def enter_rows_mode(self, prompt_len: int, position: int) -> None:
+        """Counters per row (cache slot of the 2B rows, image position of the B pairs) in place of the shared
+        ones, all at ``position``; the launch list over them is made with the first decode step."""
+        B, dev = self.rows2 // 2, self.cur.device
+        self.slot_rows = torch.full((self.rows2,), prompt_len + max(position - 1, 0), dtype=torch.long, device=dev)
+        self.pos_rows = torch.full((B,), position, dtype=torch.long, device=dev)
+        self.active = torch.zeros(B, dtype=torch.uint8, device=dev)
+        self.noise_rows = None
+        self.native_rows = None
+        self.prompt_hidden = None
+
+    def prefill_rows(self, embeds: torch.Tensor) -> None:
+        """The prompt pass of every row at once; nothing is drawn yet (a row's first token is drawn when the
+        scheduler steps it, so the random stream is used in the order of the reference's per-row loop)."""
+        out = self.sampler.trunk(inputs_embeds=embeds, attention_mask=self.mask, use_cache=True,
+                                 past_key_values=self.cache)
+        self.prompt_hidden = out.last_hidden_state[:, -1:, :].clone()
+
+    def step_rows(self, rows: list, first: bool) -> None:
+        """One token for the pairs ``rows``: the trunk runs over every row (a row outside the batch repeats its
+        last step into the same cache slot, which changes nothing), the head's call writes, counts and
+        embeds for the rows of the batch only."""
+        s = self.sampler
+        B = self.rows2 // 2
+        if first:
+            hidden = self.prompt_hidden
+        else:
+            if self.native_rows is None:
+                self.native_rows = NativeDecodeTrunk(s.trunk, self.cache, self.cur, self.mask_u8, self.slot_rows)
+            hidden = self.native_rows.run().view(self.rows2, 1, -1)
+        parts = self._head_parts()
+        packed = parts[1]._fresh_packed()
+        if parts[0] and not self._head_split_ok(parts, hidden):
+            raise RuntimeError("gen_head is not its last linear over its front modules")
+        front = self._front(parts, hidden).reshape(self.rows2, -1).contiguous()
+        idx = torch.tensor(rows, dtype=torch.long, device=self.cur.device)
+        self.active.zero_()
+        self.active[idx] = 1
+        # the draws of the batch, in its order, as torch.multinomial would make them for these rows alone
+        if self.noise_rows is None:
+            self.noise_rows = torch.ones((B, packed.N), dtype=torch.bfloat16, device=self.cur.device)
+        self.noise_rows[idx] = torch.empty((len(rows), packed.N), dtype=torch.bfloat16,
+                                           device=self.cur.device).exponential_(1.0)
+        if self.head_workspace is None:
+            self.head_workspace = ops.head_sample_workspace(B, packed.N, front.device)
+        table = s.embedding_table(packed.N, self.cur)
+        ops.head_sample(front, packed, self.cfg_weight, self.temperature, workspace=self.head_workspace,
+                        noise=self.noise_rows, out=(self.sampled, self.lp), bias=parts[1].bias,
+                        bookkeeping=(self.tokens, self.logprobs, self.pos_rows, None if first else self.slot_rows),
+                        embedding=None if table is None else (table, self.cur), per_row=True, active=self.active)
+        if table is None:
+            picked = self.sampled[idx]
+            nxt = s.base.prepare_gen_img_embeds(torch.cat([picked, picked], dim=0).unsqueeze(-1))
+            self.cur[torch.cat([idx, idx + B])] = nxt.reshape(2 * len(rows), 1, -1)
+
     def step(self) -> None:
         if self.native:
             hidden = self.native.run()
@@ -462,6 +530,37 @@ class StaticARSampler:
             sess.step()
         state.position += 1
 
+    def _advance_rows(self, state: "StaticARState", rows: list, position: int, sequences) -> "StaticARStepResult":
+        """One token for a part of the rows (``JanusProPolicy._sample_ar_step`` with ``row_indices``,
+        ``policy.py:624-731``), over the static cache with one slot counter per row."""
+        sess = state.session
+        if state.released:
+            raise ValueError("the state was finalized")
+        if len(set(rows)) != len(rows):
+            raise ValueError(f"duplicate Janus row indices: {rows}")
+        if state.row_positions is None:          # the first partial batch: counters per row from here on
+            if state.position == 0:
+                cond, uncond, cmask, umask = state.inputs
+                sess.begin(torch.cat([cmask, umask], dim=0))
+                sess.enter_rows_mode(cmask.shape[1], 0)
+                sess.prefill_rows(torch.cat([cond, uncond], dim=0))
+                state.inputs = None
+            else:
+                sess.enter_rows_mode(int(sess.slot.item()) - (state.position - 1), state.position)
+            state.row_positions = [state.position] * state.batch_size
+        if any(state.row_positions[row] != position for row in rows):
+            raise ValueError("requested position does not match row positions")
+        if position >= state.image_token_num:
+            raise ValueError("the generation has already finished sampling")
+        sess.step_rows(rows, first=position == 0)
+        for row in rows:
+            state.row_positions[row] += 1
+        state.position = min(state.row_positions)
+        idx = torch.tensor(rows, dtype=torch.long, device=sess.tokens.device)
+        return StaticARStepResult(sequence_ids=[str(seq.sample_id) for seq in sequences],
+                                  positions=[position] * len(rows),
+                                  token=sess.tokens[idx, position], log_prob=sess.logprobs[idx, position])
+
     @torch.no_grad()
     def step_ar(self, state: "StaticARState", sequences, *, generator=None) -> "StaticARStepResult":
         """One scheduled token step (``JanusProPolicy.step_ar``, ``policy.py:527-572``) for all rows at once.
@@ -483,15 +582,17 @@ class StaticARSampler:
         positions = [int(seq.position) for seq in sequences]
         if len(set(positions)) != 1:
             raise ValueError("ActiveSequence positions must match within one AR step")
-        if rows != list(range(B)):
-            if state.position == 0 and state.reference is not None:
-                cond, uncond, cmask, umask = state.inputs
-                state.delegate = state.reference[0](cond, uncond, cmask, umask, cfg_weight=state.cfg_weight,
-                                                    temperature=state.temperature,
-                                                    image_token_num=state.image_token_num)
-                return state.reference[1](state.delegate, sequences)
-            raise ValueError("the static decode loop steps all rows of a chunk together, in row order; "
-                             f"got rows {rows} of {B}")
+        if rows != list(range(B)) or state.row_positions is not None:
+            if state.row_positions is None and not state.session.rows_mode_supported():
+                if state.position == 0 and state.reference is not None:
+                    cond, uncond, cmask, umask = state.inputs
+                    state.delegate = state.reference[0](cond, uncond, cmask, umask, cfg_weight=state.cfg_weight,
+                                                        temperature=state.temperature,
+                                                        image_token_num=state.image_token_num)
+                    return state.reference[1](state.delegate, sequences)
+                raise ValueError("this policy's static decode loop steps all rows of a chunk together, in row "
+                                 f"order; got rows {rows} of {B}")
+            return self._advance_rows(state, rows, positions[0], sequences)
         if positions[0] != state.position:
             raise ValueError("ActiveSequence positions must match the state's position")
         p = state.position

@@ -118,6 +118,7 @@ struct AttnArgs {
     const uint16_t *cos, *sin;
     const uint8_t *mask;
     const long long *position;
+    int position_stride;     // 0: one position for every row; 1: position[m] is row m's
     uint16_t *out;
     int q_stride, kv_stride;
     int n_heads, n_kv_heads, L_max;
@@ -215,10 +216,10 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     __shared__ float s_new;                 // score of the new token's own slot
     __shared__ uint32_t s_before;           // SPLIT: workgroups of the pair that had arrived before this one
 
-    const long long p64 = *a.position;
-    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the grid
-    const int p = (int)p64;
     const int h = blockIdx.x, m = blockIdx.y;
+    const long long p64 = a.position[(long)m * a.position_stride];
+    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
+    const int p = (int)p64;
     const int group = a.n_heads / a.n_kv_heads;
     const int hk = h / group;
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
@@ -709,7 +710,8 @@ void launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
 int attn_decode(const void *q, const void *k, const void *v, int q_stride, int kv_stride, void *k_cache,
                 void *v_cache, const void *cos, const void *sin, const void *mask, const int64_t *position,
                 void *out, int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
-                const vrl_attn_lora *lora, void *hip_stream, void *workspace = nullptr, size_t workspace_bytes = 0) {
+                const vrl_attn_lora *lora, void *hip_stream, void *workspace = nullptr, size_t workspace_bytes = 0,
+                bool position_per_row = false) {
     if (!q || !k || !v || !k_cache || !v_cache || !cos || !sin || !mask || !position || !out) return VRL_INT4_ENULL;
     if (M < 1 || M > 65535 || n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || n_heads > 65535 ||
         (D != 64 && D != 128) || L_max < 1 || L_max > MAX_CACHE_LEN || q_stride < n_heads * D ||
@@ -730,6 +732,7 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
     a.sin = static_cast<const uint16_t *>(sin);
     a.mask = static_cast<const uint8_t *>(mask);
     a.position = reinterpret_cast<const long long *>(position);
+    a.position_stride = (position_per_row || (lora && lora->position_per_row)) ? 1 : 0;
     a.out = static_cast<uint16_t *>(out);
     a.q_stride = q_stride;
     a.kv_stride = kv_stride;
@@ -808,6 +811,15 @@ extern "C" int vrl_rope_attn_decode_split_bf16(const void *q, const void *k, con
     if (!workspace) return VRL_INT4_ENULL;
     return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, position, out, M, n_heads,
                        n_kv_heads, D, L_max, scaling, nullptr, hip_stream, workspace, workspace_bytes);
+}
+
+extern "C" int vrl_rope_attn_decode_rows_bf16(const void *q, const void *k, const void *v, int q_stride, int kv_stride,
+                                              void *k_cache, void *v_cache, const void *cos, const void *sin,
+                                              const void *mask, const int64_t *positions, void *out,
+                                              int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
+                                              void *workspace, size_t workspace_bytes, void *hip_stream) {
+    return attn_decode(q, k, v, q_stride, kv_stride, k_cache, v_cache, cos, sin, mask, positions, out, M, n_heads,
+                       n_kv_heads, D, L_max, scaling, nullptr, hip_stream, workspace, workspace_bytes, true);
 }
 
 extern "C" int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, int q_stride,

@@ -55,7 +55,9 @@ struct HeadArgs {
     long long *position;          // device scalar: column of tokens / logprobs, incremented by the call
     long long *slot;              // device scalar incremented by the call
     long long *position_seen;     // in the workspace: the position as the first kernel found it
+    const uint8_t *active;        // [B]: rows whose draw counts (null: all)
     int32_t embed_dim, token_stride;
+    int32_t per_row, reserved2;   // per_row: position is [B] and slot [2B], one counter per row
 };
 
 __device__ __forceinline__ float hs_round_bf16(float v) {
@@ -282,20 +284,27 @@ __global__ __launch_bounds__(MERGE_THREADS) void head_merge_kernel(HeadArgs a) {
         a.sampled[b] = bi;
         const float lp = hs_round_bf16(bc - cm - logf(cs));
         a.logprob[b] = lp;
-        if (a.position) {   // the step's bookkeeping (policy.py:695-696): token and log-probability at the position
-            const long long pos = *a.position_seen;
+        const bool counts = !a.active || a.active[b] != 0;   // a row outside the step's batch keeps its state
+        if (a.position && counts) {   // the step's bookkeeping (policy.py:695-696): token and log-probability at the position
+            const long long pos = a.per_row ? a.position[b] : *a.position_seen;
             if (pos >= 0 && pos < a.token_stride) {
                 if (a.tokens) a.tokens[(long)b * a.token_stride + pos] = bi;
                 if (a.logprobs) a.logprobs[(long)b * a.token_stride + pos] = lp;
             }
-            if (b == 0) {
+            if (a.per_row) {
+                a.position[b] = pos + 1;
+                if (a.slot) {   // the conditional and the unconditional row of the pair
+                    a.slot[b] += 1;
+                    a.slot[a.B + b] += 1;
+                }
+            } else if (b == 0) {
                 *a.position = pos + 1;
                 if (a.slot) *a.slot += 1;
             }
         }
         red_i[0] = bi;
     }
-    if (a.embed_table) {   // uniform: the next input of both rows of the pair (policy.py:698-700)
+    if (a.embed_table && (!a.active || a.active[b] != 0)) {   // uniform: the next input of both rows of the pair (policy.py:698-700)
         __syncthreads();
         const int token = red_i[0];
         const int words = a.embed_dim >> 3;   // 16-byte words per row
@@ -335,7 +344,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void head_sample_kernel(HeadArgs a) {
     const rsrc_t rsrc = pp_blob_rsrc(p);
     const int t0 = blockIdx.x * TW * a.rounds, t1 = min(a.tiles, t0 + TW * a.rounds);
     // the second kernel's workgroups all need the position this call writes at, and one of them moves it on
-    if (a.position && blockIdx.x == 0 && threadIdx.x == 0) *a.position_seen = *a.position;
+    if (a.position && !a.per_row && blockIdx.x == 0 && threadIdx.x == 0) *a.position_seen = *a.position;
     PPRing<1, GQ> ring;
     int tile = t0 + tw;
     bool work = sc0 < sc1 && tile < t1;   // wave-uniform
@@ -496,6 +505,7 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
                 return VRL_INT4_EALIGN;
         }
         if ((e.tokens || e.logprobs || e.slot) && !e.position) return VRL_INT4_ENULL;
+        if (e.active && !e.position_per_row) return VRL_INT4_ESHAPE;   // a partial batch needs a counter per row
         if (e.position && e.token_stride < 1) return VRL_INT4_ESHAPE;
         if ((reinterpret_cast<uintptr_t>(e.bias) & 1u) || (reinterpret_cast<uintptr_t>(e.tokens) & 7u) ||
             (reinterpret_cast<uintptr_t>(e.logprobs) & 3u) || (reinterpret_cast<uintptr_t>(e.position) & 7u) ||
@@ -511,6 +521,8 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
         args.position_seen = reinterpret_cast<long long *>(ws + lay.pos);
         args.embed_dim = e.embed_dim;
         args.token_stride = e.token_stride;
+        args.active = static_cast<const uint8_t *>(e.active);
+        args.per_row = e.position_per_row ? 1 : 0;
     }
     // as many workgroups as the device holds at once: a second round of workgroups would stage x again
     const long per_cu = std::max<long>(1, std::min<long>(16 / (ks * tw), (long)(160 * 1024 / std::max<size_t>(lds, 1024))));

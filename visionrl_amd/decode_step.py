@@ -135,7 +135,8 @@ class NativeDecodeTrunk:
     ``cache`` is the ``StaticCache`` the prompt pass already went through (its per-layer ``keys`` /
     ``values`` tensors are appended to in place), ``cur`` the ``[rows, 1, hidden]`` input embedding
     buffer, ``mask`` a uint8 ``[rows, L_max]`` buffer (0 = padding slot), ``slot`` an int64 device
-    scalar holding the cache slot the new token takes; :meth:`run` leaves ``slot`` untouched.
+    scalar holding the cache slot the new token takes, or an int64 ``[rows]`` tensor with one slot per
+    row (rows that advance at different times); :meth:`run` leaves ``slot`` untouched.
     """
 
     SPLIT_ATTENTION_FROM = 512   # cache slots from which the attention of few rows runs in its split form
@@ -181,8 +182,9 @@ class NativeDecodeTrunk:
             raise ValueError("cur must be a contiguous bfloat16 [rows, 1, hidden] device buffer")
         if mask.dtype != torch.uint8 or mask.shape[0] != rows or not mask.is_contiguous():
             raise ValueError("mask must be contiguous uint8 [rows, L_max]")
-        if slot.dtype != torch.int64 or slot.numel() != 1:
-            raise ValueError("slot must be an int64 device scalar")
+        if slot.dtype != torch.int64 or slot.numel() not in (1, rows) or not slot.is_contiguous():
+            raise ValueError("slot must be an int64 device scalar, or one slot per row")
+        per_row = slot.numel() != 1   # rows that advance at different times (a scheduler's partial batches)
         dev = cur.device
         conf = trunk.config
         self.device, self.rows, self.hidden, self.max_len = dev, rows, hidden, mask.shape[1]
@@ -301,7 +303,12 @@ class NativeDecodeTrunk:
                 calls[launch_at] = (lib.vrl_int4_gemv_prepacked_lora_up_bf16,
                                     (calls[launch_at][1][0], o_group.table, o_group.t.data_ptr(), H))
             if record is not None:
+                record.position_per_row = 1 if per_row else 0
                 calls[attn_at] = (lib.vrl_rope_attn_decode_lora_bf16, (*attn_args, ctypes.byref(record)))
+            elif per_row:
+                calls[attn_at] = (lib.vrl_rope_attn_decode_rows_bf16,
+                                  (*attn_args, split_ws.data_ptr() if split_ws is not None else None,
+                                   split_ws.numel() if split_ws is not None else 0))
             elif split_ws is not None:
                 calls[attn_at] = (lib.vrl_rope_attn_decode_split_bf16,
                                   (*attn_args, split_ws.data_ptr(), split_ws.numel()))

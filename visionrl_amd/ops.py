@@ -555,7 +555,8 @@ def head_sample_workspace(B: int, V: int, device) -> torch.Tensor:
 def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, temperature: float, *,
                 generator: torch.Generator | None = None, noise: torch.Tensor | None = None,
                 logits_out: torch.Tensor | None = None, workspace: "torch.Tensor | str | None" = None, out=None,
-                bias: torch.Tensor | None = None, bookkeeping=None, embedding=None):
+                bias: torch.Tensor | None = None, bookkeeping=None, embedding=None, per_row: bool = False,
+                active: torch.Tensor | None = None):
     """The image-token head and the sampling tail of a decode step in one launch.
 
     Stands for ``vrl/models/families/janus_pro/policy.py:684-693``: ``x`` is the bf16 ``[2B, K]``
@@ -575,6 +576,9 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
     ``slot`` are incremented (``policy.py:695-696`` over a device-side position); ``embedding = (table bf16
     [V, H], next bf16 [2B, H])``: rows ``b`` and ``B + b`` of ``next`` receive ``table[sampled[b]]``, the next
     input embedding of both rows of the pair (``policy.py:698-700`` with ``prepare_gen_img_embeds`` tabulated).
+    ``per_row``: ``position`` is int64 ``[B]`` and ``slot`` int64 ``[2B]``, one counter per row, for rows that
+    advance at different times; ``active`` (uint8 ``[B]``) then names the rows of this step's batch, the only
+    ones written, counted on and given a next input.
     Raises ``ValueError`` for shapes the launch does not take (:func:`head_sample_supported`).
     """
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[0] % 2 != 0 or x.shape[0] < 2 or x.shape[1] != head.K:
@@ -627,9 +631,15 @@ def head_sample(x: torch.Tensor, head: PrepackedWeight, cfg_weight: float, tempe
                     tokens.shape != logprobs.shape or tokens.shape[0] != B or not tokens.is_contiguous() or \
                     not logprobs.is_contiguous():
                 raise ValueError(f"bookkeeping buffers must be contiguous int64 / float32 [{B}, L]")
-            for name, t in (("position", position), ("slot", slot)):
-                if t is not None and (t.dtype != torch.int64 or t.numel() != 1):
-                    raise ValueError(f"{name} must be an int64 device scalar")
+            for name, t, n in (("position", position, B if per_row else 1), ("slot", slot, 2 * B if per_row else 1)):
+                if t is not None and (t.dtype != torch.int64 or t.numel() != n or not t.is_contiguous()):
+                    raise ValueError(f"{name} must be a contiguous int64 device tensor of {n} element(s)")
+            if active is not None:
+                if not per_row or active.dtype != torch.uint8 or active.numel() != B or not active.is_contiguous():
+                    raise ValueError(f"active goes with per_row and is a contiguous uint8 [{B}] tensor")
+                _require_device("active", active, dev)
+                extras.active = active.data_ptr()
+            extras.position_per_row = 1 if per_row else 0
             for name, t in (("tokens", tokens), ("logprobs", logprobs), ("position", position), ("slot", slot)):
                 if t is not None:
                     _require_device(name, t, dev)
@@ -755,13 +765,13 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
                      v_cache: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, mask: torch.Tensor,
                      position: torch.Tensor, scaling: float, *, out: torch.Tensor | None = None,
                      lora: "LoraAdd | None" = None, out_lora: "LoraAdd | None" = None,
-                     split_workspace: torch.Tensor | None = None) -> torch.Tensor:
+                     split_workspace: torch.Tensor | None = None, per_row: bool = False) -> torch.Tensor:
     """Rotary embedding, cache append and attention for one new token per row, one launch.
 
     ``q [M, H*D]``, ``k, v [M, Hkv*D]`` bf16 (rows may be strided views of one buffer), caches
     ``[M, Hkv, L, D]`` bf16 (the layout of transformers' ``StaticLayer``; slot ``position`` is
     written), ``cos, sin [L, D]`` bf16, ``mask [M, L]`` uint8, ``position`` an int64 device
-    scalar.  Stands for ``apply_rotary_pos_emb``, ``Cache.update`` and the attention of
+    scalar (``per_row``: int64 ``[M]``, one slot per row).  Stands for ``apply_rotary_pos_emb``, ``Cache.update`` and the attention of
     ``LlamaAttention.forward`` (reached from ``vrl/models/families/janus_pro/policy.py:673-678``).
     ``lora`` is a :class:`LoraAdd` over exactly the q, k, v outputs passed here whose down-projection
     was launched: the attention then adds the up-projections itself (q, k, v stay as they are).
@@ -791,8 +801,8 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
         _require_device(name, t, dev)
     if mask.dtype != torch.uint8 or tuple(mask.shape) != (M, L) or not mask.is_contiguous():
         raise ValueError(f"mask must be contiguous uint8 [{M}, {L}]")
-    if position.dtype != torch.int64 or position.numel() != 1:
-        raise ValueError("position must be an int64 tensor with one element")
+    if position.dtype != torch.int64 or position.numel() != (M if per_row else 1) or not position.is_contiguous():
+        raise ValueError("position must be an int64 tensor with one element (per_row: one per row)")
     for name, t in (("v_cache", v_cache), ("mask", mask), ("position", position)):
         _require_device(name, t, dev)
     if out is None:
@@ -814,8 +824,14 @@ def rope_attn_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache:
         if split_workspace.dtype != torch.uint8 or split_workspace.numel() < need or \
                 not split_workspace.is_contiguous() or split_workspace.device != dev:
             raise ValueError(f"split_workspace must be a contiguous uint8 tensor of {need} bytes on {dev}")
+    if per_row and record is not None:
+        record.position_per_row = 1
     with _on(dev):
-        if split_workspace is not None:
+        if per_row and record is None:   # one slot per row; the split form when a workspace is given
+            rc = _lib.load().vrl_rope_attn_decode_rows_bf16(
+                *args, split_workspace.data_ptr() if split_workspace is not None else None,
+                split_workspace.numel() if split_workspace is not None else 0, _stream_handle(dev))
+        elif split_workspace is not None:
             rc = _lib.load().vrl_rope_attn_decode_split_bf16(*args, split_workspace.data_ptr(),
                                                              split_workspace.numel(), _stream_handle(dev))
         elif record is None:
