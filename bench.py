@@ -275,6 +275,44 @@ def measure_set(items, steps: int, warmup: int):
     return out, total_bytes, grouped
 
 
+def fused_gate_up_launch(device, steps: int, warmup: int):
+    """Configuration 5a: fused gate||up with the SiLU epilogue, K=4096, N=2x11008, M=8, one grouped launch over 24
+    distinct weight sets (1.1 GB: beyond the memory-side cache); the outputs are compared with the unfused
+    float64 product afterwards."""
+    from visionrl_amd import ops
+    from visionrl_amd.int4_format import algorithmic_bytes
+
+    K, I, M = 4096, 11008, 8
+    sets, canon = [], []
+    for i in range(24):
+        qw, sc, qz = make_weights(5000 + i, K, 2 * I, GROUP, device)
+        sets.append(ops.int4_prepack(qw, sc, qz, GROUP))
+        if i < 2:
+            canon.append((qw, sc, qz))
+        del qw, sc, qz
+    x = make_x(5007, M, K, device)
+    nbytes = 24 * algorithmic_bytes(M, K, 2 * I, GROUP, fused_gate_up=True)
+    grouped = ops.GroupedGemv([(x, pw, True) for pw in sets])
+    ms, blocks = time_blocks(grouped.launch, steps, warmup, blocks=5, min_warm_ms=50.0)
+    worst = 0.0
+    for (qw, sc, qz), y in zip(canon, grouped.outputs):   # silu(gate) * up in float64 over the bit-exact weights
+        w = ops.int4_dequant(qw, sc, qz, GROUP).double()
+        acc, mag = x.double() @ w.t(), x.double().abs() @ w.abs().t()
+        gate, up = acc[:, :I], acc[:, I:]
+        ref = torch.nn.functional.silu(gate) * up
+        err = (y.double() - ref).abs()
+        # one bf16 rounding of the product, and the fp32 accumulation noise of either factor carried through
+        # (the slope of SiLU stays below 1.1)
+        tol = 2.0 ** -7 * ref.abs() + 2.0 ** -17 * (1.1 * mag[:, :I] * up.abs() +
+                                                     torch.nn.functional.silu(gate).abs() * mag[:, I:])
+        if not bool((err <= tol + 1e-30).all()):
+            raise RuntimeError("fused gate||up launch: outputs out of tolerance")
+        worst = max(worst, float((err / ref.abs().clamp_min(1e-6)).median()))
+    return {"ms_per_24_weight_sets": ms, "us_per_weight_set": ms * 1e3 / 24, "GBps": nbytes / (ms * 1e-3) / 1e9,
+            "pct_hbm_peak": 100.0 * nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "blocks_ms": blocks,
+            "algorithmic_bytes_per_launch": nbytes, "median_relative_error_of_checked_outputs": worst}
+
+
 def other_configs(device, steps: int, warmup: int):
     """The remaining benchmark configurations, one grouped launch each (prepacked layout)."""
     from visionrl_amd import ops
@@ -297,20 +335,7 @@ def other_configs(device, steps: int, warmup: int):
                                  "tolerance_counts": counts}
         del items, grouped
         torch.cuda.empty_cache()
-    # fused gate||up with the SiLU epilogue, K=4096, N=2x11008, M=8, over 24 distinct weight sets
-    K, I, M = 4096, 11008, 8
-    sets = []
-    for i in range(24):
-        qw, sc, qz = make_weights(5000 + i, K, 2 * I, GROUP, device)
-        sets.append(ops.int4_prepack(qw, sc, qz, GROUP))
-        del qw, sc, qz
-    x = make_x(5007, M, K, device)
-    nbytes = 24 * algorithmic_bytes(M, K, 2 * I, GROUP, fused_gate_up=True)
-    grouped = ops.GroupedGemv([(x, pw, True) for pw in sets])
-    ms, _ = time_blocks(grouped.launch, max(10, steps // 10), max(2, warmup // 10), blocks=5, min_warm_ms=50.0)
-    res["fused_gate_up_silu_k4096_i11008_m8"] = {"ms_per_24_weight_sets": ms, "us_per_weight_set": ms * 1e3 / 24,
-                                                  "GBps": nbytes / (ms * 1e-3) / 1e9}
-    del sets, grouped
+    res["fused_gate_up_silu_k4096_i11008_m8"] = fused_gate_up_launch(device, max(10, steps // 10), max(2, warmup // 10))
     torch.cuda.empty_cache()
     # group-size sweep, K=5632, N=2048, M=1: single launches over 48 distinct weight sets in a HIP graph
     sweep = {}
@@ -928,9 +953,13 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true",
                     help="run just the grouped decode-step launches (for profilers)")
-    ap.add_argument("--rows", type=int, default=1, choices=(1, 32),
+    ap.add_argument("--rows", type=int, default=1, choices=(1, 8, 16, 32),
                     help="with --only-headline: 1 = the M=1 set (default), 32 = the rollout-batch set plus the "
-                         "image-token head")
+                         "image-token head; with --shapes 7b: 1, 8 or 16 rows")
+    ap.add_argument("--shapes", default="1b", choices=("1b", "7b", "5a"),
+                    help="with --only-headline: 1b = the Janus-Pro-1B set (default); 7b = the 7B-class set plus its "
+                         "head (configuration 4); 5a = the fused gate||up launch over 24 weight sets, K=4096, "
+                         "N=2x11008, M=8 (configuration 5a)")
     ap.add_argument("--valu-dot", action="store_true",
                     help="with --only-headline (M=1): the comparison build whose dot product runs on the vector unit")
     ap.add_argument("--single-calls", action="store_true",
@@ -1019,8 +1048,17 @@ def main():
         print(json.dumps({"stream_read": stream_read(device, 642_539_520, args.steps, args.warmup)}))
         return
 
-    if args.only_headline and args.rows == 32:
+    if args.only_headline and args.shapes == "5a":
+        print(json.dumps(fused_gate_up_launch(device, args.steps, args.warmup)))
+        return
+    if args.only_headline and args.shapes == "7b":
+        if args.rows == 32:
+            raise SystemExit("the 7B-class configuration is quoted at 1, 8 and 16 rows")
+        items = build_set(4, args.rows, device, with_head=True, hidden=4096, inter=11008, layers=30, head=16384)
+    elif args.only_headline and args.rows == 32:
         items = build_set(3, 32, device, with_head=True)
+    elif args.only_headline and args.rows != 1:
+        raise SystemExit("the 1B set is quoted at 1 and 32 rows")
     else:
         items = build_set(2, 1, device, with_head=False)
     torch.cuda.synchronize()
@@ -1032,7 +1070,8 @@ def main():
         nbytes = sum(it["bytes"] for it in items)
         counts = {}
         worst = check_outputs(items, grouped.outputs, "grouped launch", counts)
-        print(json.dumps({"rows": args.rows, "valu_dot": bool(args.valu_dot), "ms_per_step": ms, "blocks_ms": per_block,
+        print(json.dumps({"shapes": args.shapes, "rows": args.rows, "valu_dot": bool(args.valu_dot), "ms_per_step": ms,
+                          "blocks_ms": per_block,
                           "algorithmic_bytes_per_step": nbytes, "GBps": nbytes / (ms * 1e-3) / 1e9,
                           "outputs_checked": len(items), "worst_backward_error": worst, "tolerance_counts": counts}))
         return
