@@ -332,10 +332,15 @@ def other_configs(device, steps: int, warmup: int):
                                  "blocks_ms": per_block, "algorithmic_bytes_per_step": nbytes, "gemvs": len(items),
                                  "worst_backward_error": check_outputs(items, grouped.outputs, f"7B-class set, M={M}",
                                                                        counts),
-                                 "tolerance_counts": counts}
+                                 "tolerance_counts": counts,
+                                 # HBM bytes per launch by rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this launch
+                                 # (profiles/gemv_stream_kernel_7b_class_m1_m8_m16.txt), not measured in this run
+                                 "traffic": load_traffic(f"gemv_stream_kernel_7b_m{M}")}
         del items, grouped
         torch.cuda.empty_cache()
     res["fused_gate_up_silu_k4096_i11008_m8"] = fused_gate_up_launch(device, max(10, steps // 10), max(2, warmup // 10))
+    # profiles/gemv_stream_kernel_fused_gate_up_k4096_i11008_m8.txt
+    res["fused_gate_up_silu_k4096_i11008_m8"]["traffic"] = load_traffic("gemv_stream_kernel_5a")
     torch.cuda.empty_cache()
     # group-size sweep, K=5632, N=2048, M=1: single launches over 48 distinct weight sets in a HIP graph
     sweep = {}
