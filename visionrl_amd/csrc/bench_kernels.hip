@@ -60,11 +60,9 @@ int vrl_bench_stream_read(const void *buf, size_t bytes, void *sink, int waves_p
     const uint32_t waves = (uint32_t)cus * (uint32_t)waves_per_cu / 4u * 4u;
     uint64_t per_wave = (bytes + waves - 1) / waves;
     per_wave = (per_wave + 4095) / 4096 * 4096;
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(stream_read_kernel<4>, dim3(waves / 4), dim3(4 * WAVE), 0,
+    return vrl_launch(&stream_read_kernel<4>, dim3(waves / 4), dim3(4 * WAVE), 0,
                        reinterpret_cast<hipStream_t>(hip_stream), buf, (uint32_t)bytes, (uint32_t)per_wave,
                        static_cast<uint32_t *>(sink));
-    return (int)hipGetLastError();
 }
 
 // One grouped launch over `plan_dev` (the device copy of a plan made by vrl_int4_grouped_plan_build of the
@@ -80,11 +78,9 @@ int vrl_bench_gemv_grouped_valu_dot_bf16(const void *plan_dev, const vrl_int4_pl
     const uint8_t *base = static_cast<const uint8_t *>(plan_dev);
     const DevProblem *recs = reinterpret_cast<const DevProblem *>(base + 16);   // behind the plan's 16-byte header
     const int2 *block_tab = reinterpret_cast<const int2 *>(recs + info->n_problems);
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL((gemv_stream_kernel<4, 1, false, true, false, false, 1, true>), dim3(info->grid),
+    return vrl_launch(&gemv_stream_kernel<4, 1, false, true, false, false, 1, true>, dim3(info->grid),
                        dim3(4 * WAVE), (size_t)info->lds_bytes, reinterpret_cast<hipStream_t>(hip_stream), recs,
                        block_tab, info->n_problems);
-    return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -17,6 +17,7 @@
 #include <stdint.h>
 
 #include "../../include/vrl_int4.h"
+#include "launch.hpp"
 #include "wave_reduce.hpp"
 
 namespace {
@@ -277,9 +278,7 @@ extern "C" int vrl_cfg_sample_bf16(const void *logits, const void *noise, int64_
                   : V <= THREADS * 8 ? &cfg_sample_resident_kernel<1>
                   : V <= THREADS * 16 ? &cfg_sample_resident_kernel<2>
                                       : &cfg_sample_kernel<8>;
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
+    return vrl_launch(kernel, dim3(B), dim3(THREADS), 0, reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint16_t *>(logits), static_cast<const uint16_t *>(noise),
                        reinterpret_cast<long long *>(sampled), logprob, B, V, cfg_weight, 1.0f / temperature);
-    return (int)hipGetLastError();
 }

@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "../../include/vrl_int4.h"
+#include "launch.hpp"
 #include "wave_reduce.hpp"
 
 namespace {

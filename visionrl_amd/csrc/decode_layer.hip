@@ -18,6 +18,7 @@
 
 #include "../../include/vrl_decode.h"
 #include "../../include/vrl_int4.h"
+#include "launch.hpp"
 #include "lora.hpp"
 #include "wave_reduce.hpp"
 
@@ -617,18 +618,16 @@ __global__ __launch_bounds__(UP_THREADS) void lora_up_add_kernel(const float *__
 }
 
 template <bool FP32, int MB>
-void launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_t stream) {
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL((lora_down_kernel<FP32, MB>), dim3(a.off[a.n], (a.M + MB - 1) / MB), dim3(THREADS), 0, stream,
-                       x, a, t);
+int launch_lora_down(const uint16_t *x, const LoraArgs &a, float *t, hipStream_t stream) {
+    return vrl_launch(&lora_down_kernel<FP32, MB>, dim3(a.off[a.n], (a.M + MB - 1) / MB), dim3(THREADS), 0, stream,
+                      x, a, t);
 }
 
 template <bool FP32, int RB>
-void launch_lora_up(const float *t, int parts, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL((lora_up_add_kernel<FP32, RB>),
-                       dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n, (a.M + UP_ROWS - 1) / UP_ROWS),
-                       dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, parts, a);
+int launch_lora_up(const float *t, int parts, const LoraArgs &a, int max_n, int max_r, hipStream_t stream) {
+    return vrl_launch(&lora_up_add_kernel<FP32, RB>,
+                      dim3((max_n + UP_THREADS - 1) / UP_THREADS, a.n, (a.M + UP_ROWS - 1) / UP_ROWS),
+                      dim3(UP_THREADS), (size_t)UP_ROWS * max_r * sizeof(float), stream, t, parts, a);
 }
 
 bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
@@ -650,29 +649,24 @@ extern "C" int vrl_add_rmsnorm_bf16(const void *x, const void *residual, const v
     auto ws = static_cast<const uint16_t *>(weight);
     auto hs = static_cast<uint16_t *>(h_out);
     auto ys = static_cast<uint16_t *>(y);
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    if (residual)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<true>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
-    else
-        hipLaunchKernelGGL(add_rmsnorm_kernel<false>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
-    return (int)hipGetLastError();
+    if (residual) return vrl_launch(&add_rmsnorm_kernel<true>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
+    return vrl_launch(&add_rmsnorm_kernel<false>, dim3(M), dim3(THREADS), lds, stream, xs, rs, ws, hs, ys, K, eps);
 }
 
 namespace {
 template <int LORA, bool STREAMED>
-void launch_attn_build(const AttnArgs &a, int M, int D, hipStream_t stream) {
+int launch_attn_build(const AttnArgs &a, int M, int D, hipStream_t stream) {
     const bool many = (long)a.n_heads * M >= 512;
     const dim3 grid(a.n_heads, M);
     // few workgroups: 16 waves each (256 slots per trip); many: 8 waves, several workgroups per CU
     // (a deeper unroll of the 16-wave form, 512 slots per trip, measured slower)
     if (D == 128 && many)
-        hipLaunchKernelGGL((rope_attn_decode_kernel<128, 8, 4, LORA, STREAMED>), grid, dim3(8 * WAVE), 0, stream, a);
-    else if (D == 128)
-        hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4, LORA, STREAMED>), grid, dim3(16 * WAVE), 0, stream, a);
-    else if (many)
-        hipLaunchKernelGGL((rope_attn_decode_kernel<64, 8, 4, LORA, STREAMED>), grid, dim3(8 * WAVE), 0, stream, a);
-    else
-        hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4, LORA, STREAMED>), grid, dim3(16 * WAVE), 0, stream, a);
+        return vrl_launch(&rope_attn_decode_kernel<128, 8, 4, LORA, STREAMED>, grid, dim3(8 * WAVE), 0, stream, a);
+    if (D == 128)
+        return vrl_launch(&rope_attn_decode_kernel<128, 16, 4, LORA, STREAMED>, grid, dim3(16 * WAVE), 0, stream, a);
+    if (many)
+        return vrl_launch(&rope_attn_decode_kernel<64, 8, 4, LORA, STREAMED>, grid, dim3(8 * WAVE), 0, stream, a);
+    return vrl_launch(&rope_attn_decode_kernel<64, 16, 4, LORA, STREAMED>, grid, dim3(16 * WAVE), 0, stream, a);
 }
 
 // keys and values of one layer beyond this many bytes are read with non-temporal loads: a model's
@@ -684,27 +678,25 @@ int attn_splits(long pairs) { return pairs <= 32 ? 8 : (pairs <= 64 ? 4 : (pairs
 size_t attn_counter_bytes(long pairs) { return (size_t)(pairs * sizeof(uint32_t) + 255) / 256 * 256; }
 
 template <bool STREAMED>
-void launch_attn_split(const AttnArgs &a, int M, int D, int splits, hipStream_t stream) {
+int launch_attn_split(const AttnArgs &a, int M, int D, int splits, hipStream_t stream) {
     const dim3 grid(a.n_heads, M, splits);
     if (D == 128)
-        hipLaunchKernelGGL((rope_attn_decode_kernel<128, 16, 4, 0, STREAMED, true>), grid, dim3(16 * WAVE), 0, stream, a);
-    else
-        hipLaunchKernelGGL((rope_attn_decode_kernel<64, 16, 4, 0, STREAMED, true>), grid, dim3(16 * WAVE), 0, stream, a);
+        return vrl_launch(&rope_attn_decode_kernel<128, 16, 4, 0, STREAMED, true>, grid, dim3(16 * WAVE), 0, stream, a);
+    return vrl_launch(&rope_attn_decode_kernel<64, 16, 4, 0, STREAMED, true>, grid, dim3(16 * WAVE), 0, stream, a);
 }
 
 template <int LORA>
-void launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
+int launch_attn(const AttnArgs &a, int M, int D, hipStream_t stream) {
     const long cache_bytes = (long)M * a.n_kv_heads * a.L_max * D * 2 * 2;
     if constexpr (LORA == 0) {
         const int splits = a.partials ? attn_splits((long)a.n_heads * M) : 1;
         if (splits > 1) {
-            if (cache_bytes > STREAMED_CACHE_BYTES) launch_attn_split<true>(a, M, D, splits, stream);
-            else launch_attn_split<false>(a, M, D, splits, stream);
-            return;
+            if (cache_bytes > STREAMED_CACHE_BYTES) return launch_attn_split<true>(a, M, D, splits, stream);
+            return launch_attn_split<false>(a, M, D, splits, stream);
         }
     }
-    if (cache_bytes > STREAMED_CACHE_BYTES) launch_attn_build<LORA, true>(a, M, D, stream);
-    else launch_attn_build<LORA, false>(a, M, D, stream);
+    if (cache_bytes > STREAMED_CACHE_BYTES) return launch_attn_build<LORA, true>(a, M, D, stream);
+    return launch_attn_build<LORA, false>(a, M, D, stream);
 }
 
 int attn_decode(const void *q, const void *k, const void *v, int q_stride, int kv_stride, void *k_cache,
@@ -750,10 +742,7 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
         a.arrived = static_cast<uint32_t *>(workspace);
         a.partials = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + attn_counter_bytes(pairs));
     }
-    if (!lora) {
-        launch_attn<0>(a, M, D, stream);
-        return (int)hipGetLastError();
-    }
+    if (!lora) return launch_attn<0>(a, M, D, stream);
     const void *bs[3] = {lora->q_B, lora->k_B, lora->v_B};
     bool any = false;
     for (int i = 0; i < 3; ++i) {
@@ -782,9 +771,8 @@ int attn_decode(const void *q, const void *k, const void *v, int q_stride, int k
     if (!any) return VRL_INT4_ENULL;
     a.t = lora->t;
     a.t_stride = lora->t_stride;
-    if (lora->weights_fp32) launch_attn<1>(a, M, D, stream);
-    else launch_attn<2>(a, M, D, stream);
-    return (int)hipGetLastError();
+    if (lora->weights_fp32) return launch_attn<1>(a, M, D, stream);
+    return launch_attn<2>(a, M, D, stream);
 }
 }  // namespace
 
@@ -844,9 +832,8 @@ extern "C" int vrl_lora_down_bf16(const void *x, int M, int K, const vrl_lora_ad
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     auto xs = static_cast<const uint16_t *>(x);
     const bool fp32 = a.ad[0].weights_fp32 != 0;
-    if (M <= 8) fp32 ? launch_lora_down<true, 8>(xs, a, t, stream) : launch_lora_down<false, 8>(xs, a, t, stream);
-    else fp32 ? launch_lora_down<true, 16>(xs, a, t, stream) : launch_lora_down<false, 16>(xs, a, t, stream);
-    return (int)hipGetLastError();
+    if (M <= 8) return fp32 ? launch_lora_down<true, 8>(xs, a, t, stream) : launch_lora_down<false, 8>(xs, a, t, stream);
+    return fp32 ? launch_lora_down<true, 16>(xs, a, t, stream) : launch_lora_down<false, 16>(xs, a, t, stream);
 }
 
 extern "C" int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vrl_lora_adapter *adapters,
@@ -865,9 +852,8 @@ extern "C" int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vr
     }
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     const bool fp32 = a.ad[0].weights_fp32 != 0;
-    if (fp32) max_r <= 32 ? launch_lora_up<true, 32>(t, t_parts, a, max_n, max_r, stream)
-                          : launch_lora_up<true, 64>(t, t_parts, a, max_n, max_r, stream);
-    else max_r <= 32 ? launch_lora_up<false, 32>(t, t_parts, a, max_n, max_r, stream)
-                     : launch_lora_up<false, 64>(t, t_parts, a, max_n, max_r, stream);
-    return (int)hipGetLastError();
+    if (fp32) return max_r <= 32 ? launch_lora_up<true, 32>(t, t_parts, a, max_n, max_r, stream)
+                                 : launch_lora_up<true, 64>(t, t_parts, a, max_n, max_r, stream);
+    return max_r <= 32 ? launch_lora_up<false, 32>(t, t_parts, a, max_n, max_r, stream)
+                       : launch_lora_up<false, 64>(t, t_parts, a, max_n, max_r, stream);
 }

@@ -426,9 +426,7 @@ int launch_head(const HeadArgs &args, int workgroups, size_t lds, hipStream_t st
             raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
-    return (int)hipGetLastError();
+    return vrl_launch(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
 }
 
 template <int KS, int TW, int MB>
@@ -545,12 +543,9 @@ int head_sample_launch(const vrl_int4_problem *head, const void *noise, int64_t 
     }
     if (rc != VRL_INT4_OK) return rc;
     // the rows: one workgroup each
-    (void)hipGetLastError();
     if (args.tiles <= 4 * MERGE_THREADS)
-        hipLaunchKernelGGL(head_merge_kernel<4>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
-    else
-        hipLaunchKernelGGL(head_merge_kernel<16>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
-    return (int)hipGetLastError();
+        return vrl_launch(&head_merge_kernel<4>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
+    return vrl_launch(&head_merge_kernel<16>, dim3(B), dim3(MERGE_THREADS), 0, stream, args);
 }
 
 // ---------------------------------------------------------------------------------------------

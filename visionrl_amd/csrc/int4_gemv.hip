@@ -134,10 +134,8 @@ int launch_tile(const DevProblem &p, hipStream_t stream) {
     const int cols_per_tile = p.fused ? 16 * (R / 2) : 16 * R;
     const int tiles = (out_cols + cols_per_tile - 1) / cols_per_tile;
     const size_t smem = tile_smem_bytes<R, MB>(p.M, p.kc);
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL((gemv_tile_kernel<R, MB, TILE_WPB>), dim3(tiles), dim3(TILE_WPB * WAVE), smem,
+    return vrl_launch(&gemv_tile_kernel<R, MB, TILE_WPB>, dim3(tiles), dim3(TILE_WPB * WAVE), smem,
                        stream, p);
-    return (int)hipGetLastError();
 }
 
 int launch_problem(DevProblem p, hipStream_t stream) {
@@ -145,10 +143,8 @@ int launch_problem(DevProblem p, hipStream_t stream) {
     if (!tile_path_ok(p)) {
         // the generic kernel walks activation rows itself, any M
         const int waves = 4;
-        (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-        hipLaunchKernelGGL(gemv_generic_kernel, dim3((out_cols + waves - 1) / waves),
+        return vrl_launch(&gemv_generic_kernel, dim3((out_cols + waves - 1) / waves),
                            dim3(waves * WAVE), 0, stream, p);
-        return (int)hipGetLastError();
     }
     p.kc = staged_k(p.M, p.K);
     // widest tile that still gives every CU two workgroups; narrow tiles otherwise
@@ -225,10 +221,8 @@ int launch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *
         info->grid = per_cu;
         return VRL_INT4_OK;
     }
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes,
+    return vrl_launch(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes,
                        stream, recs, block_begin, info->n_problems);
-    return (int)hipGetLastError();
 }
 
 // prepacked-only plans: fused or not, staged passes or not (only the widest workgroups ever
@@ -286,10 +280,8 @@ int launch_split(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *b
         info->grid = per_cu;
         return VRL_INT4_OK;
     }
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes, stream, recs,
+    return vrl_launch(kernel, dim3(info->grid), dim3(WPB * WAVE), (size_t)info->lds_bytes, stream, recs,
                        block_tab, info->n_problems);
-    return (int)hipGetLastError();
 }
 
 template <int WPB>
@@ -315,16 +307,17 @@ int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_
             raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
-    return (int)hipGetLastError();
+    return vrl_launch(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
 }
 
 template <bool FUSED, bool NORM>
 int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int workgroups, size_t lds,
                         hipStream_t stream) {
     if constexpr (!NORM) {
-        if (xg && ks == 16) return launch_direct<FUSED, 16, 1, false, true>(args, workgroups, lds, stream);
+        if constexpr (!FUSED) {
+            if (xg && ks == 16) return launch_direct<false, 16, 1, false, true>(args, workgroups, lds, stream);
+        }
+        if (xg && ks == 16) return VRL_INT4_EPLAN;
         if (xg && ks == 8) return launch_direct<FUSED, 8, 1, false, true>(args, workgroups, lds, stream);
         if (xg) return launch_direct<FUSED, 4, 1, false, true>(args, workgroups, lds, stream);
     }
@@ -342,8 +335,8 @@ int launch_direct_up(const DirectArgs &args, int ks, bool xg, int workgroups, si
                            : launch_direct<false, 4, 1, false, false, false, true>(args, workgroups, lds, stream);
     if (ks == 8) return xg ? launch_direct<false, 8, 1, false, true, false, true>(args, workgroups, lds, stream)
                            : launch_direct<false, 8, 1, false, false, false, true>(args, workgroups, lds, stream);
-    return xg ? launch_direct<false, 16, 1, false, true, false, true>(args, workgroups, lds, stream)
-              : launch_direct<false, 16, 1, false, false, false, true>(args, workgroups, lds, stream);
+    if (xg) return VRL_INT4_EPLAN;   // never chosen: see the choice of xg in direct_launch
+    return launch_direct<false, 16, 1, false, false, false, true>(args, workgroups, lds, stream);
 }
 
 // with the adapters' down-projection as extra workgroups: plain (staged, unfused) problems only
@@ -424,12 +417,10 @@ int vrl_int4_dequant_bf16(const void *qweight, const void *scales, const void *q
     long blocks = (total + 255) / 256;
     const long cap = (long)device_cu_count() * 32;
     if (blocks > cap) blocks = cap;
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
+    return vrl_launch(&dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
                        static_cast<const uint32_t *>(qzeros), static_cast<uint16_t *>(w), N, K, G);
-    return (int)hipGetLastError();
 }
 
 size_t vrl_int4_prepacked_bytes(int N, int K, int G) {
@@ -446,12 +437,10 @@ int vrl_int4_prepack(const void *qweight, const void *scales, const void *qzeros
     long blocks = (total + 255) / 256;
     const long cap = (long)device_cu_count() * 32;
     if (blocks > cap) blocks = cap;
-    (void)hipGetLastError();  // what an earlier call left behind is not this launch's status
-    hipLaunchKernelGGL(prepack_kernel, dim3((unsigned)blocks), dim3(256), 0,
+    return vrl_launch(&prepack_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(hip_stream),
                        static_cast<const uint32_t *>(qweight), static_cast<const uint16_t *>(scales),
                        static_cast<const uint32_t *>(qzeros), static_cast<u32x4_t *>(packed), N, K, G);
-    return (int)hipGetLastError();
 }
 
 struct DirectLora {   // adapters joined to a plan-free launch: down-projections (up false) or one up-projection
@@ -498,8 +487,10 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // rows of the longest K that LDS holds beside a 16-wave workgroup's partial tiles
     const long staged_rows = (long)((DIRECT_LDS_CAP - (size_t)15 * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t)) /
                                     ((size_t)(max_nsc * PP_SC + XPAD) * 2));
+    // (the 16-wave register-fed form is not built for fused gate|up records or with an adapter's up-projection:
+    // its accumulators and operands did not fit the registers, and the staged form serves those launches)
     const bool xg = !norm && !lora_down &&
-                    (ks == 16 ? max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows)
+                    (ks == 16 ? !fused_any && !lora_up && (max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows))
                               : max_nsc <= ks && max_m >= 8 && slab_tiles <= 2L * device_cu_count());
     const int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
