@@ -185,11 +185,15 @@ int vrl_int4_gemv_prepacked_norm_bf16(const vrl_int4_problem *problems, int n_pr
  * applied to the activations on their way in (the trunk's final norm in front of the head).
  * bias: bf16 [N] or NULL.  activation: VRL_INT4_ACT_NONE, or VRL_INT4_ACT_GELU for
  * x / 2 * (1 + erf(x / sqrt(2))) evaluated in fp32 on the bf16 value and rounded to bf16 (torch.nn.GELU()).
+ * residual: bf16 [M, N] or NULL, added last: y = bf16(residual + that) — the `residual + hidden_states` that
+ * follows o_proj and down_proj in LlamaDecoderLayer.forward (reached from policy.py:673-678), so that the
+ * residual stream is written by the launch that produces the sublayer's output; it may be the memory of y.
  */
 #define VRL_INT4_ACT_NONE 0
 #define VRL_INT4_ACT_GELU 1
 typedef struct vrl_int4_epilogue {
     const void *bias;
+    const void *residual;
     int32_t activation;
     int32_t reserved;   /* 0 */
 } vrl_int4_epilogue;

@@ -206,7 +206,9 @@ def test_head_sample_with_bias_bookkeeping_and_next_embeddings(ops_mod, B, K, V)
 
 @pytest.mark.parametrize("M,K,N,G,norm", [(2, 2048, 2048, 128, False), (2, 2048, 2048, 128, True),
                                           (32, 2048, 2048, 128, True), (8, 4096, 4096, 128, True),
-                                          (5, 1024, 1536, 64, False)])
+                                          (5, 1024, 1536, 64, False), (32, 5632, 2048, 128, False),
+                                          (16, 2048, 2048, 128, False), (2, 5632, 2048, 128, False),
+                                          (32, 11008, 4096, 128, False)])
 def test_linear_with_bias_and_gelu_in_one_launch(ops_mod, M, K, N, G, norm):
     """``vrl_int4_gemv_prepacked_epilogue_bf16`` (the front of a two-layer head): bit for bit what the plain
     launch followed by the tensor ops gives (bias added to the bf16 output, exact GELU in fp32 on the bf16
@@ -234,5 +236,20 @@ def test_linear_with_bias_and_gelu_in_one_launch(ops_mod, M, K, N, G, norm):
         want = torch.nn.functional.gelu(want) if gelu else want
         torch.cuda.synchronize()
         assert torch.equal(got, want), (b is not None, gelu, (got.float() - want.float()).abs().max().item())
+    # the sublayer's output joining a residual stream in the same launch (o_proj, down_proj of a decoder layer):
+    # bf16(residual + bf16(x . W^T)); also into the residual's own memory
+    stream = torch.randn((M, N), generator=gen, device=DEV).to(torch.bfloat16)
+    got = ops_mod.EpilogueGemv(d["x"], pw, residual=stream, norm=norm_args).launch()
+    torch.cuda.synchronize()
+    assert torch.equal(got, stream + base)
+    got = ops_mod.EpilogueGemv(d["x"], pw, bias, gelu=True, residual=stream, norm=norm_args).launch()
+    torch.cuda.synchronize()
+    assert torch.equal(got, stream + torch.nn.functional.gelu(base + bias))
+    in_place = stream.clone()
+    ops_mod.EpilogueGemv(d["x"], pw, residual=in_place, out=in_place, norm=norm_args).launch()
+    torch.cuda.synchronize()
+    assert torch.equal(in_place, stream + base)
     with pytest.raises(ValueError):
         ops_mod.EpilogueGemv(d["x"], pw, bias[:-1].contiguous())
+    with pytest.raises(ValueError):
+        ops_mod.EpilogueGemv(d["x"], pw, residual=stream[:, :-8].contiguous())

@@ -88,6 +88,7 @@ class Epilogue(ctypes.Structure):
 
     _fields_ = [
         ("bias", ctypes.c_void_p),
+        ("residual", ctypes.c_void_p),
         ("activation", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
     ]

@@ -291,9 +291,9 @@ int launch_split_variant(vrl_int4_plan_info *info, const DevProblem *recs, const
                                            : launch_split<false, WPB>(info, recs, block_tab, stream);
 }
 
-template <bool FUSED, int KS, int TW, bool NORM, bool XG = false, bool LD = false, bool UP = false>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG = false, bool LD = false, bool UP = false, bool EPI = false>
 int launch_direct(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
-    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG, LD, UP>;
+    auto kernel = &gemv_split_direct_kernel<FUSED, KS, TW, NORM, XG, LD, UP, EPI>;
     if (lds > 64 * 1024) {
         // once per instantiation and device: the attribute belongs to the function on that device
         static std::atomic<uint64_t> raised{0};
@@ -326,6 +326,23 @@ int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int wor
     if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1, NORM>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2, NORM>(args, workgroups, lds, stream);
     if (ks == 16 && tw == 1) return launch_direct<FUSED, 16, 1, NORM>(args, workgroups, lds, stream);
+    return VRL_INT4_EPLAN;
+}
+
+// with bias, activation or residual applied before the store: one plain problem
+template <bool NORM>
+int launch_direct_epilogue(const DirectArgs &args, int ks, int tw, bool xg, int workgroups, size_t lds,
+                           hipStream_t stream) {
+    if constexpr (!NORM) {
+        if (xg && ks == 16) return launch_direct<false, 16, 1, false, true, false, false, true>(args, workgroups, lds, stream);
+        if (xg && ks == 8) return launch_direct<false, 8, 1, false, true, false, false, true>(args, workgroups, lds, stream);
+        if (xg) return launch_direct<false, 4, 1, false, true, false, false, true>(args, workgroups, lds, stream);
+    }
+    if (ks == 4 && tw == 1) return launch_direct<false, 4, 1, NORM, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 4) return launch_direct<false, 4, 4, NORM, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 1) return launch_direct<false, 8, 1, NORM, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 8 && tw == 2) return launch_direct<false, 8, 2, NORM, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 16 && tw == 1) return launch_direct<false, 16, 1, NORM, false, false, false, true>(args, workgroups, lds, stream);
     return VRL_INT4_EPLAN;
 }
 
@@ -458,7 +475,8 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     if (epilogue) {   // one plain problem: the bias belongs to its columns
         if (n_problems != 1 || problems[0].fused_gate_up || lora) return VRL_INT4_ESHAPE;
         if (epilogue->activation != VRL_INT4_ACT_NONE && epilogue->activation != VRL_INT4_ACT_GELU) return VRL_INT4_ESHAPE;
-        if (reinterpret_cast<uintptr_t>(epilogue->bias) & 1u) return VRL_INT4_EALIGN;
+        if ((reinterpret_cast<uintptr_t>(epilogue->bias) | reinterpret_cast<uintptr_t>(epilogue->residual)) & 1u)
+            return VRL_INT4_EALIGN;
     }
     bool fused_any = false;
     int max_nsc = 1, max_m = 1;
@@ -515,8 +533,10 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         args.norm.eps = norm->eps;
         args.norm.enabled = 1;
     }
-    if (epilogue && (epilogue->bias || epilogue->activation != VRL_INT4_ACT_NONE)) {
+    if (epilogue && (epilogue->bias || epilogue->residual || epilogue->activation != VRL_INT4_ACT_NONE)) {
         args.epi.bias = static_cast<const uint16_t *>(epilogue->bias);
+        args.epi.residual = static_cast<const uint16_t *>(epilogue->residual);
+        args.epi.y0 = static_cast<const uint16_t *>(problems[0].y);
         args.epi.act = epilogue->activation;
         args.epi.enabled = 1;
     }
@@ -563,8 +583,9 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // More workgroups than the device holds at once (16 waves and 160 KB of LDS per CU) would run in
     // waves of workgroups, each staging x and ramping up again: a workgroup then walks several sets of
     // TW tiles, the next set's first loads issued under the current one's last.
+    // (a register-fed launch with an epilogue keeps one tile per workgroup: its build walks no second set)
     args.rounds = 1;
-    if (!lora_up) {
+    if (!lora_up && !(xg && args.epi.enabled)) {
         const long per_cu = std::max<long>(1, std::min<long>(16 / (ks * tw), (long)(160 * 1024 / std::max<size_t>(lds, 1024))));
         const long capacity = per_cu * device_cu_count();
         args.rounds = (int)std::min<long>(8, (workgroups + capacity - 1) / capacity);
@@ -614,6 +635,9 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         lds = std::max(lds, (size_t)ks * tw * 16 * sizeof(float));
         return launch_direct_lora(args, ks, tw, (int)workgroups, lds, stream);
     }
+    if (args.epi.enabled)
+        return norm ? launch_direct_epilogue<true>(args, ks, tw, false, (int)workgroups, lds, stream)
+                    : launch_direct_epilogue<false>(args, ks, tw, xg, (int)workgroups, lds, stream);
     if (norm)
         return fused_any ? launch_direct_shape<true, true>(args, ks, tw, false, (int)workgroups, lds, stream)
                          : launch_direct_shape<false, true>(args, ks, tw, false, (int)workgroups, lds, stream);

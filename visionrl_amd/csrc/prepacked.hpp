@@ -802,10 +802,14 @@ __device__ __forceinline__ void store_tile_lora(const DevProblem &p, int tile_lo
 // Bias and activation of a linear applied to the tile before it is stored (plan-free launches of one plain
 // problem): y = act(bf16(bf16(x . W^T) + bias)), the roundings of a bf16 module whose bias is added to its
 // output tensor and whose activation is a tensor op of its own (Janus' generation head is Linear, GELU, Linear:
-// vrl/models/families/janus_pro/policy.py:138-160 calls it).
+// vrl/models/families/janus_pro/policy.py:138-160 calls it).  Last, a residual stream may be added:
+// y = bf16(residual + that), the `hidden_states = residual + hidden_states` that follows o_proj and down_proj in
+// LlamaDecoderLayer.forward (reached from policy.py:673-678), so that the launch after it reads one tensor.
 struct EpiArgs {
-    const uint16_t *bias;   // bf16 [N] or nullptr
-    int32_t act;            // 0: none; 1: GELU, x / 2 * (1 + erf(x / sqrt 2)) in fp32
+    const uint16_t *bias;      // bf16 [N] or nullptr
+    const uint16_t *residual;  // bf16 [M, N] added last (the residual stream a sublayer's output joins), or nullptr
+    const uint16_t *y0;        // the problem's y: a record's rows of `residual` lie where its rows of y lie
+    int32_t act;               // 0: none; 1: GELU, x / 2 * (1 + erf(x / sqrt 2)) in fp32
     int32_t enabled;
 };
 
@@ -820,9 +824,27 @@ __device__ __forceinline__ float epi_apply(float acc, float bias, bool has_bias,
     return v;
 }
 
+// What the lane's four outputs of a tile add from the residual stream, requested before the tile's weights are
+// streamed so that the values wait in registers when the tile is stored (rows past M repeat the last one).
+struct EpiResidual {
+    uint16_t v[4];
+};
+__device__ __forceinline__ EpiResidual epi_residual(const DevProblem &p, int tile_local, const EpiArgs &e) {
+    EpiResidual r = {{0, 0, 0, 0}};
+    if (e.residual) {   // uniform over the launch
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int col = min(tile_local * 16 + (lane & 15), p.N - 1);
+        const uint16_t *rows = e.residual + (p.y - e.y0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            r.v[i] = as_global(rows)[(long)min(4 * (lane >> 4) + i, p.M - 1) * p.N + col];
+    }
+    return r;
+}
+
 // store_tile<1, false> with the epilogue
 __device__ __forceinline__ void store_tile_epi(const DevProblem &p, int tile_local, const f32x4_t &acc,
-                                               const EpiArgs &e) {
+                                               const EpiArgs &e, const EpiResidual &res) {
     const int lane = threadIdx.x & (WAVE - 1);
     const int col = tile_local * 16 + (lane & 15);
     if (col >= p.N) return;
@@ -831,17 +853,20 @@ __device__ __forceinline__ void store_tile_epi(const DevProblem &p, int tile_loc
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = 4 * (lane >> 4) + i;
-        if (m < p.M)
-            as_global(p.y)[(long)m * p.N + col] =
-                (uint16_t)(pack_bf16_rne(epi_apply(acc[i], bias, has_bias, e.act), 0.0f) & 0xFFFFu);
+        if (m < p.M) {
+            float v = epi_apply(acc[i], bias, has_bias, e.act);
+            if (e.residual) v = epi_round_bf16(epi_round_bf16(v) + bf16_bits_to_f32(res.v[i]));
+            as_global(p.y)[(long)m * p.N + col] = (uint16_t)(pack_bf16_rne(v, 0.0f) & 0xFFFFu);
+        }
     }
 }
 
-template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG, bool UP = false>
+template <bool FUSED, int KS, int TW, int GQ, bool NORM, bool XG, bool UP = false, bool EPI = false>
 __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, int t1, uint8_t *smem,
                                                  const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{},
                                                  const EpiArgs &epi = EpiArgs{}) {
     constexpr int RS = FUSED ? 2 : 1;
+    static_assert(!EPI || (!FUSED && !UP), "bias, activation and residual join a plain problem");
     static_assert(!XG || (TW == 1 && !NORM), "register-fed activations: one tile per workgroup, no norm");
     static_assert(!UP || (!FUSED && !NORM), "an adapter's up-projection joins a plain problem");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -890,7 +915,9 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
     }
     for (int base = t0; base < t1; base += TW) {
         tile = base + tw;
-        const int next = tile + TW < t1 ? tile + TW : -1;
+        // a register-fed launch with an epilogue walks one tile per workgroup (the host sees to it): the
+        // registers that would hold the next tile's activations are the epilogue's
+        const int next = (XG && EPI) ? -1 : (tile + TW < t1 ? tile + TW : -1);
         f32x4_t acc[RS][1];
 #pragma unroll
         for (int r = 0; r < RS; ++r) acc[r][0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -905,6 +932,12 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
 #pragma unroll
             for (int r = 0; r < RS; ++r) red[((kw - 1) * RS + r) * WAVE + lane] = acc[r][0];
         }
+        // what the tile adds from the residual stream is requested here, when the wave's operands have left
+        // the registers, and arrives while the partial tiles meet
+        EpiResidual joins = {{0, 0, 0, 0}};
+        if constexpr (EPI) {
+            if (kw == 0 && tile < t1) joins = epi_residual(p, tile, epi);
+        }
         __syncthreads();
         if (kw == 0 && tile < t1) {
 #pragma unroll
@@ -916,25 +949,26 @@ __device__ __forceinline__ void split_segment_pp(const DevProblem &p, int t0, in
                 if (up.fp32) store_tile_lora<true>(p, tile, acc[0][0], up, lora_ts, brows);
                 else store_tile_lora<false>(p, tile, acc[0][0], up, lora_ts, brows);
             } else {
-                if constexpr (!FUSED) {
-                    if (epi.enabled) store_tile_epi(p, tile, acc[0][0], epi);   // uniform over the launch
-                    else store_tile<1, false>(p, tile, acc);
-                } else {
-                    store_tile<1, FUSED>(p, tile, acc);
-                }
+                if constexpr (EPI) store_tile_epi(p, tile, acc[0][0], epi, joins);
+                else store_tile<1, FUSED>(p, tile, acc);
             }
         }
+        if constexpr (XG && EPI) break;
         work = work && next >= 0;
         if (base + TW < t1) __syncthreads();  // the partial tiles are read before they are rewritten
     }
 }
 
 // the latency kernels take any of the three group sizes in one build (they are not register-critical)
-template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool UP = false>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool UP = false, bool EPI = false>
 __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int t1, uint8_t *smem,
                                                const NormArgs &norm, const LoraUpArgs &up = LoraUpArgs{},
                                                const EpiArgs &epi = EpiArgs{}) {
-    if constexpr (UP) {
+    if constexpr (EPI) {
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG, false, true>(p, t0, t1, smem, norm, up, epi);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG, false, true>(p, t0, t1, smem, norm, up, epi);
+        else split_segment_pp<false, KS, TW, 4, NORM, XG, false, true>(p, t0, t1, smem, norm, up, epi);
+    } else if constexpr (UP) {
         if (p.G == 128) split_segment_pp<false, KS, TW, 1, false, XG, true>(p, t0, t1, smem, norm, up);
         else if (p.G == 64) split_segment_pp<false, KS, TW, 2, false, XG, true>(p, t0, t1, smem, norm, up);
         else split_segment_pp<false, KS, TW, 4, false, XG, true>(p, t0, t1, smem, norm, up);
@@ -943,9 +977,9 @@ __device__ __forceinline__ void split_by_group(const DevProblem &p, int t0, int 
         else if (p.G == 64) split_segment_pp<FUSED, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
         else split_segment_pp<FUSED, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
     } else {
-        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm, up, epi);
-        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm, up, epi);
-        else split_segment_pp<false, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm, up, epi);
+        if (p.G == 128) split_segment_pp<false, KS, TW, 1, NORM, XG>(p, t0, t1, smem, norm);
+        else if (p.G == 64) split_segment_pp<false, KS, TW, 2, NORM, XG>(p, t0, t1, smem, norm);
+        else split_segment_pp<false, KS, TW, 4, NORM, XG>(p, t0, t1, smem, norm);
     }
 }
 
@@ -993,10 +1027,10 @@ struct DirectArgs {
     NormArgs norm;                // read by the NORM instantiations only
     LoraDownArgs ld;              // read by the LD instantiations only
     LoraUpArgs up;                // read by the UP instantiations only
-    EpiArgs epi;                  // bias / activation before the store (plain problems; enabled = 0: none)
+    EpiArgs epi;                  // read by the EPI instantiations only: bias, activation, residual before the store
 };
 
-template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD, bool UP>
+template <bool FUSED, int KS, int TW, bool NORM, bool XG, bool LD, bool UP, bool EPI = false>
 __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     int g = blockIdx.x;
@@ -1013,7 +1047,7 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
         if (k < a.n && a.recs[k].tile_begin <= g) p = a.recs[k];  // scalar selects, no indexing
     const int tiles = ((p.fused ? p.N / 2 : p.N) + 15) / 16;
     const int t0 = (g - p.tile_begin) * TW * a.rounds;
-    split_by_group<FUSED, KS, TW, NORM, XG, UP>(p, t0, min(tiles, t0 + TW * a.rounds), smem, a.norm, a.up, a.epi);
+    split_by_group<FUSED, KS, TW, NORM, XG, UP, EPI>(p, t0, min(tiles, t0 + TW * a.rounds), smem, a.norm, a.up, a.epi);
 }
 
 }  // namespace

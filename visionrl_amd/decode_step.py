@@ -198,7 +198,8 @@ class NativeDecodeTrunk:
         self.cos, self.sin = cos[0].contiguous(), sin[0].contiguous()
         new = lambda n: torch.empty((rows, n), dtype=torch.bfloat16, device=dev)
         # the residual stream alternates between two buffers: a launch that adds to it reads one and
-        # writes the other (its workgroups read the old stream while one of them writes the new one)
+        # writes the other (the input embedding is the first stream and must stay as it is; a normalising
+        # launch's workgroups read the old stream while one of them writes the new one)
         streams = [new(hidden), new(hidden)]
         self.normed, self.attn = new(hidden), new(H * D)
         self._keep = [cache, cur, mask, slot, streams]
@@ -222,7 +223,18 @@ class NativeDecodeTrunk:
             self._keep.append(w)
             return w, float(module.variance_epsilon)
 
-        def gemv(problems, norm=None):
+        def gemv(problems, norm=None, joins=None):
+            if joins is not None:
+                # the sublayer's output joins the residual stream in the launch that produces it
+                # (`hidden_states = residual + hidden_states`): the next norm then reads one tensor
+                (x, pw, _), = problems
+                out = streams[state["flip"]]
+                state["flip"] ^= 1
+                launch = ops.EpilogueGemv(x, pw, residual=joins, out=out)
+                self._keep.append(launch)
+                calls.append((lib.vrl_int4_gemv_prepacked_epilogue_bf16,
+                              (launch._gemv.table, None, ctypes.byref(launch.epilogue))))
+                return [launch.output]
             launch = ops.DirectGemv(problems, norm=norm)
             self._keep.append(launch)
             if norm is None:
@@ -252,17 +264,21 @@ class NativeDecodeTrunk:
             return launch
 
         def normed_gemv(module, weights, fused, adapters=(), up=True):
-            """h = res + x; the linears over norm(h); afterwards res = h.  Returns (outputs, adapter group)."""
+            """h = res + x (h = x where x already holds the stream); the linears over norm(h); afterwards res = h.
+            Returns (outputs, adapter group)."""
             w, eps = norm_weight(module)
-            h_out = streams[state["flip"]]
-            state["flip"] ^= 1
+            h_out = None
+            if state["res"] is not None:
+                h_out = streams[state["flip"]]
+                state["flip"] ^= 1
             group = None
             if fuse_norm and not any(ad is not None for ad in adapters):
                 outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
             else:
                 calls.append((lib.vrl_add_rmsnorm_bf16,
                               (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,
-                               w.data_ptr(), h_out.data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+                               w.data_ptr(), h_out.data_ptr() if h_out is not None else None,
+                               self.normed.data_ptr(), rows, hidden, eps)))
                 # the adapters read the normalised row, so it is written out; their down-projection and the
                 # base projections share one launch
                 launch_at = len(calls)
@@ -271,7 +287,7 @@ class NativeDecodeTrunk:
                 if group is not None and not fused:
                     calls[launch_at] = (lib.vrl_int4_gemv_prepacked_lora_bf16,
                                         (*calls[launch_at][1], group.table, len(group.table), group.t.data_ptr()))
-            state["res"] = h_out
+            state["res"] = h_out if h_out is not None else state["x"]
             return outs, group
 
         for i, layer in enumerate(trunk.layers):
@@ -296,7 +312,11 @@ class NativeDecodeTrunk:
             attn_at = len(calls)
             calls.append(None)
             launch_at = len(calls)
-            outs = gemv([(self.attn, proj["o_proj"][0], False)])
+            # o_proj's output joins the residual stream in its own launch, unless an adapter's launch form stores it
+            joins = state["res"] if proj["o_proj"][1] is None else None
+            outs = gemv([(self.attn, proj["o_proj"][0], False)], joins=joins)
+            if joins is not None:
+                state["res"] = None
             o_group = lora(self.attn, outs, [proj["o_proj"][1]], up=False, parts=H)
             if o_group is not None:   # o_proj's launch adds the up-projection itself
                 record = o_group.attn_output_record(record)
@@ -316,13 +336,16 @@ class NativeDecodeTrunk:
                 calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args)
             (state["x"],) = outs
             (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
-            (state["x"],) = gemv([(act, mlp.down_proj._packed, False)])
+            (state["x"],) = gemv([(act, mlp.down_proj._packed, False)], joins=state["res"])
+            state["res"] = None
         w, eps = norm_weight(trunk.norm)
         self.final = None
         if final_norm or not fuse_norm:
+            res = state["res"]
             calls.append((lib.vrl_add_rmsnorm_bf16,
-                          (state["x"].data_ptr(), state["res"].data_ptr(), w.data_ptr(),
-                           streams[state["flip"]].data_ptr(), self.normed.data_ptr(), rows, hidden, eps)))
+                          (state["x"].data_ptr(), res.data_ptr() if res is not None else None, w.data_ptr(),
+                           streams[state["flip"]].data_ptr() if res is not None else None,
+                           self.normed.data_ptr(), rows, hidden, eps)))
         else:
             self.final = (state["x"], state["res"], w, eps)
             self.normed = None

@@ -468,12 +468,15 @@ class EpilogueGemv:
     The first half of Janus' two-layer image-token head (``Linear``, ``GELU``, ``Linear``; called through
     ``gen_head`` at ``vrl/models/families/janus_pro/policy.py:138-160``) and any biased linear.  ``x`` is a
     contiguous bf16 ``[M <= 32, K]`` tensor; ``bias`` bf16 ``[N]`` or ``None``; ``gelu`` the exact (erf) form of
-    ``torch.nn.GELU()``; ``norm = (residual | None, weight, eps)`` as in :class:`DirectGemv` (K <= 4096).  The
-    record is built once; the tensors captured here must stay alive and in place.
+    ``torch.nn.GELU()``; ``norm = (residual | None, weight, eps)`` as in :class:`DirectGemv` (K <= 4096);
+    ``residual`` (bf16 ``[M, N]``) is added last, ``y = bf16(residual + ...)``: the residual stream that the
+    outputs of ``o_proj`` and ``down_proj`` join in a decoder layer.  The record is built once; the tensors
+    captured here must stay alive and in place.
     """
 
     def __init__(self, x: torch.Tensor, weight: "PrepackedWeight", bias: torch.Tensor | None = None,
-                 gelu: bool = False, norm=None, out: torch.Tensor | None = None):
+                 gelu: bool = False, norm=None, out: torch.Tensor | None = None,
+                 residual: torch.Tensor | None = None):
         self._gemv = DirectGemv([(x, weight, False)], outputs=None if out is None else [out],
                                 norm=None if norm is None else (*norm, None))
         self.device = self._gemv.device
@@ -481,11 +484,16 @@ class EpilogueGemv:
             if bias.dtype != torch.bfloat16 or tuple(bias.shape) != (weight.N,) or not bias.is_contiguous():
                 raise ValueError(f"bias must be contiguous bfloat16 [{weight.N}]")
             _require_device("bias", bias, self.device)
+        self.output = self._gemv.outputs[0]
+        if residual is not None:
+            if residual.dtype != torch.bfloat16 or residual.shape != self.output.shape or not residual.is_contiguous():
+                raise ValueError(f"residual must be contiguous bfloat16 {tuple(self.output.shape)}")
+            _require_device("residual", residual, self.device)
         self.epilogue = _lib.Epilogue()
         self.epilogue.bias = bias.data_ptr() if bias is not None else None
+        self.epilogue.residual = residual.data_ptr() if residual is not None else None
         self.epilogue.activation = _lib.ACT_GELU if gelu else _lib.ACT_NONE
-        self._keep = bias
-        self.output = self._gemv.outputs[0]
+        self._keep = (bias, residual)
 
     def launch(self) -> torch.Tensor:
         g = self._gemv
