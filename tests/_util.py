@@ -82,3 +82,24 @@ def assert_gemv_close(y_bits: np.ndarray, ops: dict, G: int, what: str = ""):
     y = oracle.bf16_bits_to_f32(y_bits).astype(np.float64)
     y_ref, a_ref = oracle.gemv_and_abs_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
     return check_gemv(y, y_ref, a_ref, what)
+
+
+def assert_gate_up_close(y_bits: np.ndarray, ops: dict, G: int, what: str = ""):
+    """The fused ``SiLU(gate) * up`` output (bf16 bit patterns) against the oracle's float64 value.
+
+    Two bf16 steps or 1e-2 relative, plus what the GEMV rule grants each fp32 accumulator (``2^-18 * sum|x w|``)
+    carried through the product: ``|SiLU'(g)| |u| e_g + |SiLU(g)| e_u``.  That term decides only where the gate or
+    the up sum cancelled (about one output in 10^5); a wrong weight or index moves outputs by whole units.
+    """
+    acc, a = oracle.gemv_and_abs_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    inter = acc.shape[1] // 2
+    g, u = acc[:, :inter], acc[:, inter:]
+    sig = 1.0 / (1.0 + np.exp(-g))
+    silu, dsilu = g * sig, sig * (1.0 + g * (1.0 - sig))
+    ref = silu * u
+    noise = 2.0 ** -18 * (np.abs(dsilu * u) * a[:, :inter] + np.abs(silu) * a[:, inter:])
+    tol = np.maximum(2 * oracle.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5 + noise
+    got = oracle.bf16_bits_to_f32(y_bits).astype(np.float64)
+    assert got.shape == ref.shape, what
+    bad = np.abs(got - ref) > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} outputs beyond tolerance"

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import int4_oracle as o
-from tests._util import assert_gemv_close, bf16_to_bits, bits_to_bf16, to_device
+from tests._util import assert_gate_up_close, assert_gemv_close, bf16_to_bits, bits_to_bf16, to_device
 
 pytestmark = pytest.mark.gpu
 
@@ -542,6 +542,69 @@ def test_direct_prepacked_parity(ops_mod, M, K, N, fused):
     got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
     tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
     assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all()
+
+
+# 17 to 32 rows of K > 2048 with enough tiles: activations staged in passes over K, either one record for all the
+# rows (K up to 4096, 512 tiles or more) or records of 16 rows with eight waves per tile (256 tiles or more)
+ROWS32_SHAPES = [
+    # M, K, N, fused, G
+    (32, 4096, 8192, False, 128), (17, 2560, 8200, False, 128), (24, 4096, 2 * 8192, True, 128),
+    (32, 3072, 8192, False, 64), (32, 4096, 2 * 8192, True, 32),
+    (32, 11008, 4096, False, 128), (20, 4096, 4100, False, 128), (32, 8704, 4096, False, 64),
+    (31, 4608, 4096, False, 32),
+]
+
+
+@pytest.mark.parametrize("M,K,N,fused,G", ROWS32_SHAPES)
+def test_direct_prepacked_parity_rows_17_to_32_long_k(ops_mod, M, K, N, fused, G):
+    say("direct prepacked, passes over K", M, K, N, fused, G)
+    ops = o.make_operands(9400 + M + K + N + G, M, K, N, G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    (y,) = ops_mod.DirectGemv([(d["x"], pw, fused)]).launch()
+    torch.cuda.synchronize()
+    if not fused:
+        assert_gemv_close(bf16_to_bits(y), ops, G, f"direct M{M} K{K} N{N} G{G}")
+        # rows do not depend on how many travel together: the first rows alone take the 16-row forms
+        (y8,) = ops_mod.DirectGemv([(d["x"][:8].contiguous(), pw, False)]).launch()
+        torch.cuda.synchronize()
+        assert_gemv_close(bf16_to_bits(y8), {**ops, "x_bits": ops["x_bits"][:8]}, G, "first rows alone")
+        return
+    assert_gate_up_close(bf16_to_bits(y), ops, G, f"direct fused M{M} K{K} N{N} G{G}")
+
+
+def test_direct_rows32_group_of_three_and_one_hot(ops_mod):
+    """A q|k|v-like group at 32 rows of K = 4096 (one record per problem for all rows): each output against the
+    oracle, and one-hot activations return the exact weight columns in both row blocks."""
+    say("direct group, 32 rows")
+    G, M, K = 128, 32, 4096
+    probs, checks = [], []
+    for i, N in enumerate((4096, 4096, 1024)):
+        ops = o.make_operands(9500 + i, M, K, N, G)
+        d = to_device(ops, DEV)
+        if i:
+            d["x"] = probs[0][0]
+            ops = {**ops, "x_bits": checks[0]["x_bits"]}
+        probs.append((d["x"], ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G), False))
+        checks.append(ops)
+    outs = [y.clone() for y in ops_mod.DirectGemv(probs).launch()]
+    torch.cuda.synchronize()
+    for y, ops in zip(outs, checks):
+        assert_gemv_close(bf16_to_bits(y), ops, G, "direct group, 32 rows")
+    ops = o.make_operands(9510, M, K, 8192, G, "loguniform")
+    w = o.dequant_bf16(ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
+    d = to_device(ops, DEV)
+    pw = ops_mod.int4_prepack(d["qweight"], d["scales"], d["qzeros"], G)
+    x = np.zeros((M, K), dtype=np.float32)
+    ks = [(131 * m + 7) % K for m in range(M)]
+    for m in range(M):
+        x[m, ks[m]] = 1.0
+    (y,) = ops_mod.DirectGemv([(bits_to_bf16(o.f32_to_bf16_bits(x), DEV), pw, False)]).launch()
+    torch.cuda.synchronize()
+    y = bf16_to_bits(y)
+    for m in range(M):
+        want = w[:, ks[m]]
+        assert ((y[m] == want) | (((y[m] | want) & 0x7FFF) == 0)).all(), m
 
 
 def test_direct_group_matches_single_launches_and_plan(ops_mod):

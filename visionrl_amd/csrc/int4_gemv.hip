@@ -35,6 +35,7 @@
 #include <atomic>
 
 #include "stream_kernel.hpp"
+#include "rows32.hpp"
 
 namespace {
 
@@ -329,6 +330,24 @@ int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int wor
     return VRL_INT4_EPLAN;
 }
 
+// records of 17 to 32 rows: four waves per tile, four tiles per workgroup
+constexpr size_t ROWS32_LDS_CAP = 160 * 1024;
+template <bool FUSED, int KS, int TW, int MB>
+int launch_rows32(const DirectArgs &args, int workgroups, size_t lds, hipStream_t stream) {
+    auto kernel = &gemv_rows32_direct_kernel<FUSED, KS, TW, MB>;
+    static std::atomic<uint64_t> raised{0};   // once per instantiation and device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(raised.load(std::memory_order_relaxed) & bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)ROWS32_LDS_CAP);
+        if (e != hipSuccess) return (int)e;
+        raised.fetch_or(bit, std::memory_order_relaxed);
+    }
+    return vrl_launch(kernel, dim3(workgroups), dim3(KS * TW * WAVE), lds, stream, args);
+}
+
 // with bias, activation or residual applied before the store: one plain problem
 template <bool NORM>
 int launch_direct_epilogue(const DirectArgs &args, int ks, int tw, bool xg, int workgroups, size_t lds,
@@ -539,6 +558,55 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
         args.epi.y0 = static_cast<const uint16_t *>(problems[0].y);
         args.epi.act = epilogue->activation;
         args.epi.enabled = 1;
+    }
+    if (max_m > MAX_TILE_M && max_m <= 2 * MAX_TILE_M && max_nsc > 4 && !norm && !lora && !args.epi.enabled) {
+        // 17 to 32 rows of K > 2048: two forms of gemv_rows32_direct_kernel, K in passes of what LDS holds of the rows.
+        // (a) One record per problem holds all its rows (a weight word is read and rebuilt once for both blocks of
+        // 16 rows): four waves per tile, four tiles per workgroup.  (b) Records of 16 rows, eight waves per tile, two
+        // tiles per workgroup, fused records excepted.  Measured at 32 rows against two register-fed or staged
+        // slabs (7B-class layer): q|k|v (a) 14.6, (b) 23.2, slabs 23.7 us; gate|up (a) 21.1, slabs 32.2 us; o_proj
+        // (a) 13.2, (b) 8.2, slabs 12.8 us; down_proj, K = 11008: (a) 30.8 (six passes), (b) 17.1 (three), slabs
+        // 29.9 us (every tile's workgroup fetches all of x there: 180 MB from L2); and a form of (a) that fetches
+        // its operands into registers 11.7 / 27.0 us for o_proj / down_proj.  With few tiles the slabs win
+        // (K = 5632, N = 2048: (b) 10.1, slabs 9.8 us), and at K = 2048 they run side by side (7.5 against 8.9 us).
+        const long cus = device_cu_count();
+        const bool whole = max_nsc <= 8 && slab_tiles >= 4 * cus;
+        const bool slabs16 = !whole && !fused_any && slab_tiles >= 2 * cus;
+        if (whole || slabs16) {
+            const int ks = whole ? 4 : 8, tw = whole ? 4 : 2, rows = whole ? 2 * MAX_TILE_M : MAX_TILE_M;
+            const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
+            long sc_pass = ((long)((ROWS32_LDS_CAP - red) / ((size_t)std::min(rows, max_m) * 2)) - XPAD) / PP_SC;
+            sc_pass -= sc_pass % ks;
+            if (sc_pass > max_nsc) sc_pass = max_nsc;
+            if (sc_pass >= 1) {
+                long wgs = 0;
+                for (int i = 0; i < n_problems; ++i) {
+                    const vrl_int4_problem &q = problems[i];
+                    const int out_cols = q.fused_gate_up ? q.N / 2 : q.N;
+                    for (int m0 = 0; m0 < q.M; m0 += rows) {
+                        if (args.n == DIRECT_MAX) return VRL_INT4_ESHAPE;
+                        DevProblem &p = args.recs[args.n++];
+                        p.x = static_cast<const uint16_t *>(q.x) + (long)m0 * q.K;
+                        p.qweight = static_cast<const uint32_t *>(q.qweight);
+                        p.y = static_cast<uint16_t *>(q.y) + (long)m0 * out_cols;
+                        p.M = std::min<int>(rows, q.M - m0);
+                        p.N = q.N; p.K = q.K; p.G = q.G;
+                        p.fused = q.fused_gate_up ? 1 : 0;
+                        p.prepacked = 1;
+                        p.kc = (int)std::min<long>(sc_pass, pp_nsc(q.K)) * PP_SC;
+                        p.tile_begin = (int)wgs;
+                        wgs += ((out_cols + 15) / 16 + tw - 1) / tw;
+                    }
+                }
+                if (wgs > (1L << 20)) return VRL_INT4_ESHAPE;
+                const size_t lds = (size_t)std::min(rows, max_m) * ((size_t)sc_pass * PP_SC + XPAD) * 2 + red;
+                hipStream_t s32 = reinterpret_cast<hipStream_t>(hip_stream);
+                args.rounds = 1;
+                if (!whole) return launch_rows32<false, 8, 2, 1>(args, (int)wgs, lds, s32);
+                return fused_any ? launch_rows32<true, 4, 4, 2>(args, (int)wgs, lds, s32)
+                                 : launch_rows32<false, 4, 4, 2>(args, (int)wgs, lds, s32);
+            }
+        }
     }
     long workgroups = 0;
     size_t x_bytes = 0;

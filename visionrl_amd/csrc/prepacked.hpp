@@ -571,9 +571,13 @@ __device__ __forceinline__ void stream_rows_pp(const DevProblem &p, rsrc_t rsrc,
         if constexpr (XG) {
             if (*xpre_sc != sc) {  // wave-uniform; never with one super-chunk per wave
                 const int kb = sc * PP_SC + kq * 128;
-                const uint32_t vo = (lc < p.M && kb < p.K) ? (uint32_t)(lc * p.K + kb) * 2u : PP_OUT_OF_RANGE;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) xpre[0][i] = __builtin_amdgcn_raw_buffer_load_b128(*xr, vo + 16u * i, 0, 0);
+                for (int b = 0; b < MB; ++b) {
+                    const int row = 16 * b + lc;
+                    const uint32_t vo = (row < p.M && kb < p.K) ? (uint32_t)(row * p.K + kb) * 2u : PP_OUT_OF_RANGE;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) xpre[b][i] = __builtin_amdgcn_raw_buffer_load_b128(*xr, vo + 16u * i, 0, 0);
+                }
                 *xpre_sc = sc;
             }
         }

@@ -204,7 +204,12 @@ class NativeDecodeTrunk:
         self.normed, self.attn = new(hidden), new(H * D)
         self._keep = [cache, cur, mask, slot, streams]
         lib = _lib.load()
-        fuse_norm = hidden <= 4096   # the linears normalise their input while staging it
+        # The linears normalise their input while staging it, where that is the faster form: every workgroup of
+        # such a launch normalises all the rows it stages, which for wide rows and many of them costs more than
+        # a norm launch of its own in front of a launch that reads every weight once (hidden 4096: q|k|v 30.0
+        # against 2.9 + 14.6 us at 32 rows; at 16 rows the two forms tie, below that and at hidden 2048 the
+        # fused form wins).  That norm launch then adds the residual stream as well.
+        fuse_norm = hidden <= 4096 and (hidden <= 2048 or rows <= 16)
         # With few (row, head) pairs and a cache that grows long the attention divides a pair's cached slots
         # over several workgroups (one workspace for all layers: the launches are ordered by the stream).
         # Its exchange costs about 1.5 us per launch, which pays from about 400 cached slots on (at 2 rows
@@ -313,7 +318,7 @@ class NativeDecodeTrunk:
             calls.append(None)
             launch_at = len(calls)
             # o_proj's output joins the residual stream in its own launch, unless an adapter's launch form stores it
-            joins = state["res"] if proj["o_proj"][1] is None else None
+            joins = state["res"] if proj["o_proj"][1] is None and fuse_norm else None
             outs = gemv([(self.attn, proj["o_proj"][0], False)], joins=joins)
             if joins is not None:
                 state["res"] = None
@@ -336,11 +341,12 @@ class NativeDecodeTrunk:
                 calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args)
             (state["x"],) = outs
             (act,), _ = normed_gemv(layer.post_attention_layernorm, [mlp.gate_up._packed], True)
-            (state["x"],) = gemv([(act, mlp.down_proj._packed, False)], joins=state["res"])
-            state["res"] = None
+            (state["x"],) = gemv([(act, mlp.down_proj._packed, False)], joins=state["res"] if fuse_norm else None)
+            if fuse_norm:
+                state["res"] = None
         w, eps = norm_weight(trunk.norm)
         self.final = None
-        if final_norm or not fuse_norm:
+        if final_norm or hidden > 4096:
             res = state["res"]
             calls.append((lib.vrl_add_rmsnorm_bf16,
                           (state["x"].data_ptr(), res.data_ptr() if res is not None else None, w.data_ptr(),
