@@ -323,6 +323,7 @@ int launch_direct_shape(const DirectArgs &args, int ks, int tw, bool xg, int wor
         if (xg) return launch_direct<FUSED, 4, 1, false, true>(args, workgroups, lds, stream);
     }
     if (ks == 4 && tw == 1) return launch_direct<FUSED, 4, 1, NORM>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 2) return launch_direct<FUSED, 4, 2, NORM>(args, workgroups, lds, stream);
     if (ks == 4 && tw == 4) return launch_direct<FUSED, 4, 4, NORM>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 1) return launch_direct<FUSED, 8, 1, NORM>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 2) return launch_direct<FUSED, 8, 2, NORM>(args, workgroups, lds, stream);
@@ -358,6 +359,7 @@ int launch_direct_epilogue(const DirectArgs &args, int ks, int tw, bool xg, int 
         if (xg) return launch_direct<false, 4, 1, false, true, false, false, true>(args, workgroups, lds, stream);
     }
     if (ks == 4 && tw == 1) return launch_direct<false, 4, 1, NORM, false, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 2) return launch_direct<false, 4, 2, NORM, false, false, false, true>(args, workgroups, lds, stream);
     if (ks == 4 && tw == 4) return launch_direct<false, 4, 4, NORM, false, false, false, true>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 1) return launch_direct<false, 8, 1, NORM, false, false, false, true>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 2) return launch_direct<false, 8, 2, NORM, false, false, false, true>(args, workgroups, lds, stream);
@@ -378,6 +380,7 @@ int launch_direct_up(const DirectArgs &args, int ks, bool xg, int workgroups, si
 // with the adapters' down-projection as extra workgroups: plain (staged, unfused) problems only
 int launch_direct_lora(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
     if (ks == 4 && tw == 1) return launch_direct<false, 4, 1, false, false, true>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 2) return launch_direct<false, 4, 2, false, false, true>(args, workgroups, lds, stream);
     if (ks == 4 && tw == 4) return launch_direct<false, 4, 4, false, false, true>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 1) return launch_direct<false, 8, 1, false, false, true>(args, workgroups, lds, stream);
     if (ks == 8 && tw == 2) return launch_direct<false, 8, 2, false, false, true>(args, workgroups, lds, stream);
@@ -529,7 +532,16 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     const bool xg = !norm && !lora_down &&
                     (ks == 16 ? !fused_any && !lora_up && (max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows))
                               : max_nsc <= ks && max_m >= 8 && slab_tiles <= 2L * device_cu_count());
-    const int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
+    // Tiles per workgroup.  One staging of x serves them, but fewer workgroups share the launch: up to 16 rows
+    // of a launch with many tiles (q|k|v, gate|up) two tiles per workgroup measured best at every row count
+    // (K = 2048, 384 tiles, fused norm: 5.9 / 6.5 / 7.8 us at 2 / 8 / 16 rows against 6.1 / 7.9 / 10.9 us with one
+    // and 7.1 / 8.0 / 8.7 us with four; K = 4096, 768 tiles: 10.3 / 12.4 / 13.9 against 11.3 / 14.1 / 25.0 us with
+    // one), except that fused records of 12 or more rows of K > 2048 fill LDS with one workgroup per CU
+    // either way and then three sets of one tile beat two sets of two (688 tiles: 18.9 against 26.0 us).  With
+    // few tiles (o_proj: 128 or 256) one tile per workgroup below 8 rows (4.2 against 4.9 us at 2 rows).
+    int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
+    if (!xg && !lora_up && max_m <= MAX_TILE_M && ks <= 8 && slab_tiles >= 5L * device_cu_count() / 4)
+        tw = (ks == 8 && fused_any && max_m >= 12) ? 1 : 2;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
