@@ -381,12 +381,18 @@ NORM_FUSED_CASES = [
     # through the registers in halves), incl. a K that is no multiple of 512 and the 7B-class shapes
     (16, 4096, [256, 128], False, True), (32, 4096, [2 * 1024], True, True), (5, 3072, [64], False, True),
     (7, 2560, [48], False, False), (32, 4096, [4096], False, True),
+    # launches of many tiles take other workgroup shapes: wide rows with four waves per tile (two super-chunks each)
+    # and four tiles per workgroup, fused records of 12+ rows with one tile, two slabs of rows, and rows of up to
+    # 2048 values at 13 to 16 rows with eight waves per tile
+    (8, 4096, [4096, 4096, 1024], False, True), (16, 4096, [4096, 4096], False, True),
+    (4, 4096, [2 * 5632], True, True), (14, 4096, [2 * 5632], True, False), (24, 4096, [4096, 2048], False, True),
+    (20, 4096, [2 * 5632], True, True), (14, 2048, [2048, 2048, 2048], False, True), (16, 2048, [2 * 5632], True, True),
 ]
 
 
 @pytest.mark.parametrize("M,K,Ns,fused,with_residual", NORM_FUSED_CASES)
 def test_norm_fused_launch_parity(ops_mod, M, K, Ns, fused, with_residual):
-    from tests._util import assert_gemv_close, to_device
+    from tests._util import assert_gate_up_close, assert_gemv_close, to_device
 
     say("norm-fused launch", M, K, Ns, fused, with_residual)
     G = 128
@@ -409,10 +415,7 @@ def test_norm_fused_launch_parity(ops_mod, M, K, Ns, fused, with_residual):
         if not fused:
             assert_gemv_close(bf16_to_bits(y), ops, G, "norm-fused")
             continue
-        ref = o.gate_up_silu_f64(ops["x_bits"], ops["qweight"], ops["scales_bits"], ops["qzeros"], G)
-        got = o.bf16_bits_to_f32(bf16_to_bits(y)).astype(np.float64)
-        tol = np.maximum(2 * o.bf16_ulp(ref), 1e-2 * np.abs(ref)) + 1e-5
-        assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all()
+        assert_gate_up_close(bf16_to_bits(y), ops, G, "norm-fused gate|up")
     # against the two-launch form on the device: same h, outputs within a rounding of the normalised row
     h2, normed = ops_mod.add_rmsnorm(xt, wt, 1e-6, rt if with_residual else None)
     two = ops_mod.DirectGemv([(normed, pw, f) for _, pw, f in probs]).launch()

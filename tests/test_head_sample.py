@@ -208,7 +208,9 @@ def test_head_sample_with_bias_bookkeeping_and_next_embeddings(ops_mod, B, K, V)
                                           (32, 2048, 2048, 128, True), (8, 4096, 4096, 128, True),
                                           (5, 1024, 1536, 64, False), (32, 5632, 2048, 128, False),
                                           (16, 2048, 2048, 128, False), (2, 5632, 2048, 128, False),
-                                          (32, 11008, 4096, 128, False)])
+                                          (32, 11008, 4096, 128, False), (32, 4096, 4096, 128, False),
+                                          (24, 3072, 2048, 64, False), (6, 2048, 2048, 128, False),
+                                          (12, 5632, 2048, 128, False)])
 def test_linear_with_bias_and_gelu_in_one_launch(ops_mod, M, K, N, G, norm):
     """``vrl_int4_gemv_prepacked_epilogue_bf16`` (the front of a two-layer head): bit for bit what the plain
     launch followed by the tensor ops gives (bias added to the bf16 output, exact GELU in fp32 on the bf16

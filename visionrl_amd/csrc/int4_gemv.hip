@@ -517,7 +517,7 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     }
     // KS waves split K of a tile (one super-chunk each where K allows); with 8 or more
     // activation rows a workgroup carries several tiles so that one staging of x serves them
-    const int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
+    int ks = max_nsc > 8 ? 16 : (max_nsc > 4 ? 8 : 4);
     // The waves can fetch their own activations, with nothing staged and one tile per workgroup.  Long K
     // does with one super-chunk per wave, and with two when staging would need more than one slab of
     // rows (the second fetch waits for the first super-chunk's arithmetic); shorter K with 8+ rows and one
@@ -529,9 +529,9 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
                                     ((size_t)(max_nsc * PP_SC + XPAD) * 2));
     // (the 16-wave register-fed form is not built for fused gate|up records or with an adapter's up-projection:
     // its accumulators and operands did not fit the registers, and the staged form serves those launches)
-    const bool xg = !norm && !lora_down &&
-                    (ks == 16 ? !fused_any && !lora_up && (max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows))
-                              : max_nsc <= ks && max_m >= 8 && slab_tiles <= 2L * device_cu_count());
+    bool xg = !norm && !lora_down &&
+              (ks == 16 ? !fused_any && !lora_up && (max_nsc <= ks || (max_nsc <= 2 * ks && max_m > staged_rows))
+                        : max_nsc <= ks && max_m >= 8 && slab_tiles <= 2L * device_cu_count());
     // Tiles per workgroup.  One staging of x serves them, but fewer workgroups share the launch: up to 16 rows
     // of a launch with many tiles (q|k|v, gate|up) two tiles per workgroup measured best at every row count
     // (K = 2048, 384 tiles, fused norm: 5.9 / 6.5 / 7.8 us at 2 / 8 / 16 rows against 6.1 / 7.9 / 10.9 us with one
@@ -540,8 +540,39 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // either way and then three sets of one tile beat two sets of two (688 tiles: 18.9 against 26.0 us).  With
     // few tiles (o_proj: 128 or 256) one tile per workgroup below 8 rows (4.2 against 4.9 us at 2 rows).
     int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
-    if (!xg && !lora_up && max_m <= MAX_TILE_M && ks <= 8 && slab_tiles >= 5L * device_cu_count() / 4)
+    const bool many_tiles = slab_tiles >= 5L * device_cu_count() / 4;
+    if (!xg && !lora_up && max_m <= MAX_TILE_M && ks <= 8 && many_tiles)
         tw = (ks == 8 && fused_any && max_m >= 12) ? 1 : 2;
+    // Three more measured preferences, all about how the rows get into LDS.  A register-fed wave asks for its
+    // rows' fragments sixteen bytes at a time, one cache line per lane and instruction: with 8 or more rows that
+    // is slower than staging with coalesced loads, where LDS holds the rows in one or two slabs (K = 5632,
+    // N = 2048: 6.9 / 7.7 us staged against 7.8 / 9.9 us register-fed at 8 / 16 rows; a tie at 2 to 4 rows).
+    if (xg && ks == 16 && !lora_up && max_m >= 6 && max_m <= MAX_TILE_M && max_nsc <= 16 && max_m <= 2 * staged_rows)
+        xg = false;
+    // Staging is shared by all waves of a workgroup, so few tiles of short K are served faster by sixteen waves
+    // of which only the first few stream (K = 2048, N = 2048 at 4 / 8 / 16 rows: 4.6 / 4.8 / 5.2 against 5.0 /
+    // 5.0 / 5.3 us; K = 4096, N = 4096 at 8 / 16 rows: 6.3 / 7.3 against 6.8 / 8.2 us register-fed).
+    if (!norm && !lora && !fused_any && !many_tiles && ks <= 8 && max_m >= 4 && max_m <= MAX_TILE_M &&
+        max_m <= staged_rows) {
+        ks = 16;
+        tw = 1;
+        xg = false;
+    }
+    // A normalising launch over rows of 2049 to 4096 values: four waves per tile (two super-chunks each) and four
+    // tiles per workgroup up to 8 rows (768 tiles: 10.2 / 10.8 / 11.9 us at 2 / 4 / 8 rows against 10.9 / 11.3 /
+    // 12.5 us; 688 fused tiles: 15.3 / 16.4 / 17.5 against 16.5 / 17.7 / 18.9 us), and for plain records up to 16
+    // (13.5 against 14.1 us); rows of up to 2048 values at 13 to 16 rows: eight waves per tile, half of them
+    // streaming (384 tiles: 7.6 against 8.0 us; 352 fused tiles: 9.7 against 10.2 us).
+    // At 17 to 32 rows (two slabs): 17.9 against 29.8 us for 768 tiles, and four waves per tile with two tiles per
+    // workgroup for fused records (688 tiles: 27.5 against 38.3 us).
+    if (norm && !lora && many_tiles) {
+        if (ks == 8 && (max_m <= 8 || !fused_any)) ks = 4, tw = 4;
+        else if (ks == 8 && max_m > MAX_TILE_M) ks = 4, tw = 2;
+        else if (ks == 4 && max_m > 12 && max_m <= MAX_TILE_M) ks = 8, tw = 2;
+    }
+    // Few tiles of 17 to 32 rows of K up to 4096 with an epilogue (the passes over K above serve plain launches):
+    // staged, two tiles per workgroup, against register-fed slabs 8.5 against 13.1 us (K = 4096, N = 4096).
+    if (xg && ks == 8 && max_m > MAX_TILE_M && !lora && MAX_TILE_M <= staged_rows) xg = false, tw = 2;
     const size_t red = (size_t)tw * (ks - 1) * (fused_any ? 2 : 1) * WAVE * sizeof(f32x4_t);
     // activations go in slabs of at most 16 rows that fit LDS beside the partial tiles; one record per slab
     DirectArgs args;
