@@ -845,3 +845,41 @@ def test_a_partial_batch_after_steps_of_the_whole_chunk(int4_policy):
     assert bool((tokens >= 0).all()) and bool((tokens < VOCAB_IMG).all()) and bool((logprobs <= 0).all())
     again = int4_policy.finalize_ar_state(state)
     assert torch.equal(again[0], tokens) and torch.equal(again[1], logprobs)
+
+
+@pytest.mark.gpu
+def test_recording_keeps_the_garbage_collector_out_and_sessions_die_with_their_sampler(int4_policy, monkeypatch):
+    """A finalizer that frees device resources in the middle of a stream capture ends the process: the cyclic
+    collector is off while a step is recorded (and back on afterwards), and a sampler holds its sessions without a
+    reference cycle, so dropping it frees them (their recorded graphs included) at once."""
+    import gc
+    import weakref
+
+    from visionrl_amd import ar_decode
+
+    print("ar decode: no garbage collection inside a recording", flush=True)
+    seen = []
+    step = ar_decode._Session.step
+
+    def watched(self):
+        if torch.cuda.is_current_stream_capturing():
+            seen.append(gc.isenabled())
+        return step(self)
+
+    monkeypatch.setattr(ar_decode._Session, "step", watched)
+    cond, uncond, cmask, umask = make_inputs(2, 6, torch.bfloat16, "cuda:0", seed=81)
+    sampler = StaticARSampler(int4_policy)
+    assert gc.isenabled()
+    sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=6)
+    torch.cuda.synchronize()
+    assert seen == [False] and gc.isenabled()
+    (sess,) = sampler._sessions.values()
+    assert sess.graph is not None
+    gone = weakref.ref(sess)
+    del sess
+    gc.disable()
+    try:
+        del sampler
+        assert gone() is None        # freed by reference counting alone
+    finally:
+        gc.enable()

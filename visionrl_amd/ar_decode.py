@@ -37,6 +37,7 @@ policy's own step functions.
 from __future__ import annotations
 
 import dataclasses
+import gc
 import types
 import weakref
 from typing import Any
@@ -120,7 +121,9 @@ class _Session:
                  mask_dtype: torch.dtype):
         from transformers.cache_utils import StaticCache
 
-        self.sampler = sampler
+        self._sampler = weakref.ref(sampler)   # no cycle with the sampler's table of sessions: a dropped sampler frees
+                                               # its sessions (recorded graphs included) at once, not in some later
+                                               # garbage collection that may fall into another session's recording
         self.rows2, self.max_len = rows2, max_len
         self.cfg_weight, self.temperature = float(cfg_weight), float(temperature)
         trunk = sampler.trunk
@@ -356,10 +359,26 @@ class _Session:
             hidden = out.last_hidden_state[:, -1:, :]
         self.tail(hidden, advance_slot=True)
 
+    @property
+    def sampler(self) -> "StaticARSampler":
+        sampler = self._sampler()
+        if sampler is None:
+            raise RuntimeError("the sampler this session belongs to no longer exists")
+        return sampler
+
     def capture(self) -> None:
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self.step()
+        # No cyclic garbage collection while the stream records: a finalizer that releases device resources (another
+        # recorded graph, say) in the middle of a recording ends the process.  torch.cuda.graph collects once itself
+        # before the recording begins.
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                self.step()
+        finally:
+            if collecting:
+                gc.enable()
         self.graph = graph
 
 
