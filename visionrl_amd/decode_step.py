@@ -9,9 +9,10 @@ the arithmetic in it.  :class:`NativeDecodeTrunk` runs the same layer as five la
     [add + RMSNorm ->] q|k|v (one int4 launch) -> rotary + cache append + attention -> o_proj
     -> [add + RMSNorm ->] gate|up + SiLU (one int4 launch) -> down_proj
 
-where the residual add of the previous sublayer and the norm are applied by the int4 launch that
-follows them while it stages its input (for hidden sizes up to 4096; a launch of their own
-otherwise), over the same
+where the norm is applied by the int4 launch that follows it while it stages its input, and the
+residual add by the launch that produces the sublayer's output as it stores (hidden sizes up to
+4096; above that, and for rows wider than 2048 at more than 16 rows, add and norm are a launch of
+their own: measured faster there), over the same
 ``StaticCache`` tensors the prompt pass filled (``[rows, kv_heads, L_max, head_dim]``), the cache
 slot of the new token held in device memory, and every buffer preallocated, so that the whole
 step can be recorded as one HIP graph.  Arithmetic follows the library's roundings (each tensor
