@@ -525,6 +525,7 @@ def test_graph_replays_equal_eager_steps_with_lora():
 @pytest.mark.parametrize("B,kv_heads,lora,hidden,inter,heads", [
     (1, 16, False, 2048, 5632, 16), (16, 16, False, 2048, 5632, 16), (16, 4, True, 2048, 5632, 16),
     (1, 32, False, 4096, 11008, 32), (16, 32, True, 4096, 11008, 32),      # the 7B-class layer
+    (24, 16, False, 2048, 5632, 16), (32, 4, False, 2048, 5632, 16),       # 48 and 64 rows: two launches per linear
 ])
 def test_native_trunk_at_janus_layer_shapes(B, kv_heads, lora, hidden, inter, heads):
     """Two decoder layers of the Janus-Pro-1B geometry (2048 hidden, 16 heads of 128, 5632 intermediate,

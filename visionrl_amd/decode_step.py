@@ -140,6 +140,8 @@ class NativeDecodeTrunk:
     row (rows that advance at different times); :meth:`run` leaves ``slot`` untouched.
     """
 
+    ROW_BLOCK = 32               # rows one plan-free launch takes; more rows go as several launches per linear,
+    MAX_ROWS = 64                # each reading the weights again (beyond this a dequantised GEMM is the better form)
     SPLIT_ATTENTION_FROM = 512   # cache slots from which the attention of few rows runs in its split form
     SPLIT_ATTENTION_PAIRS = 128  # (row, head) pairs up to which the library splits a pair's slots
 
@@ -162,10 +164,15 @@ class NativeDecodeTrunk:
                 if not isinstance(mlp, Int4LlamaMLP) or getattr(mlp.gate_up, "_packed", None) is None:
                     return f"layers[{i}].mlp is not a prepacked fused int4 MLP"
                 packed.append(_plain_int4(mlp.down_proj, f"layers[{i}].mlp.down_proj"))
-                if rows > min(w.direct_rows(False, 3) for w in packed[:3]) or \
-                        rows > min(w.direct_rows() for w in packed[3:]) or \
-                        rows > mlp.gate_up._packed.direct_rows(True):
-                    return f"{rows} rows exceed what one plan-free launch takes"
+                block = min(rows, NativeDecodeTrunk.ROW_BLOCK)   # more rows go as several launches per linear
+                if rows > NativeDecodeTrunk.MAX_ROWS or \
+                        block > min(w.direct_rows(False, 3) for w in packed[:3]) or \
+                        block > min(w.direct_rows() for w in packed[3:]) or \
+                        block > mlp.gate_up._packed.direct_rows(True):
+                    return f"{rows} rows exceed what the plan-free launches take"
+                if rows > NativeDecodeTrunk.ROW_BLOCK and any(
+                        _projection(getattr(attn, n), n)[1] is not None for n in ("q_proj", "k_proj", "v_proj", "o_proj")):
+                    return f"{rows} rows with adapters (their launches take up to {NativeDecodeTrunk.ROW_BLOCK})"
         except (AttributeError, TypeError) as exc:
             return str(exc)
         return None
@@ -229,26 +236,39 @@ class NativeDecodeTrunk:
             self._keep.append(w)
             return w, float(module.variance_epsilon)
 
+        blocks = [(r0, min(rows, r0 + self.ROW_BLOCK)) for r0 in range(0, rows, self.ROW_BLOCK)]
+
         def gemv(problems, norm=None, joins=None):
+            """The launches of one linear group over all rows: one per block of ROW_BLOCK rows."""
+            cut = lambda t, r0, r1: None if t is None else (t if len(blocks) == 1 else t[r0:r1])
             if joins is not None:
                 # the sublayer's output joins the residual stream in the launch that produces it
                 # (`hidden_states = residual + hidden_states`): the next norm then reads one tensor
                 (x, pw, _), = problems
                 out = streams[state["flip"]]
                 state["flip"] ^= 1
-                launch = ops.EpilogueGemv(x, pw, residual=joins, out=out)
+                for r0, r1 in blocks:
+                    launch = ops.EpilogueGemv(cut(x, r0, r1), pw, residual=cut(joins, r0, r1), out=cut(out, r0, r1))
+                    self._keep.append(launch)
+                    calls.append((lib.vrl_int4_gemv_prepacked_epilogue_bf16,
+                                  (launch._gemv.table, None, ctypes.byref(launch.epilogue))))
+                return [out]
+            outs = [new(pw.N // 2 if fused else pw.N) for _, pw, fused in problems] if len(blocks) > 1 else None
+            for r0, r1 in blocks:
+                xs = {}   # one view per input tensor and block: a normalising launch wants the same object for all
+                part = [(xs.setdefault(id(x), cut(x, r0, r1)), pw, fused) for x, pw, fused in problems]
+                launch = ops.DirectGemv(part, outputs=None if outs is None else [y[r0:r1] for y in outs],
+                                        norm=None if norm is None else
+                                        (cut(norm[0], r0, r1), norm[1], norm[2], cut(norm[3], r0, r1)))
                 self._keep.append(launch)
-                calls.append((lib.vrl_int4_gemv_prepacked_epilogue_bf16,
-                              (launch._gemv.table, None, ctypes.byref(launch.epilogue))))
-                return [launch.output]
-            launch = ops.DirectGemv(problems, norm=norm)
-            self._keep.append(launch)
-            if norm is None:
-                calls.append((lib.vrl_int4_gemv_prepacked_bf16, (launch.table, len(launch.table))))
-            else:
-                calls.append((lib.vrl_int4_gemv_prepacked_norm_bf16,
-                              (launch.table, len(launch.table), ctypes.byref(launch.norm))))
-            return launch.outputs
+                if norm is None:
+                    calls.append((lib.vrl_int4_gemv_prepacked_bf16, (launch.table, len(launch.table))))
+                else:
+                    calls.append((lib.vrl_int4_gemv_prepacked_norm_bf16,
+                                  (launch.table, len(launch.table), ctypes.byref(launch.norm))))
+                if outs is None:
+                    outs = launch.outputs
+            return outs
 
         def lora(x, outs, adapters, up=True, down=True, parts=1):
             """outs[i] += adapter i applied to x, for the projections that carry one: a down-projection
