@@ -182,6 +182,40 @@ int vrl_rope_attn_decode_lora_bf16(const void *q, const void *k, const void *v, 
                                    int M, int n_heads, int n_kv_heads, int D, int L_max, float scaling,
                                    const vrl_attn_lora *lora, void *hip_stream);
 
+/*
+ * The launches of a decode step issued from one host call.  A step of the native decoder layer is a list of
+ * some 120 calls of the entry points above and of vrl_int4.h, and a host loop in an interpreted language needs
+ * about as long to issue them as the device needs to run them.  A record names the entry point (`kind`) and
+ * holds its arguments in the order of its declaration: pointers in p[], integers (int, size_t) in i[], floats
+ * in f[]; `hip_stream` is the stream of every call.  The calls are issued in order; the first that fails ends
+ * the walk: its return value is returned and, if `failed_at` is not NULL, its index is written there (nothing
+ * is written when all succeed).  The records, and whatever they point to, stay the caller's.
+ * No counterpart in the reference, whose step is the model's forward (policy.py:673-678).
+ */
+enum {
+    VRL_CALL_GEMV = 1,          /* vrl_int4_gemv_prepacked_bf16 */
+    VRL_CALL_GEMV_NORM = 2,     /* vrl_int4_gemv_prepacked_norm_bf16 */
+    VRL_CALL_GEMV_EPILOGUE = 3, /* vrl_int4_gemv_prepacked_epilogue_bf16 */
+    VRL_CALL_GEMV_LORA = 4,     /* vrl_int4_gemv_prepacked_lora_bf16 */
+    VRL_CALL_GEMV_LORA_UP = 5,  /* vrl_int4_gemv_prepacked_lora_up_bf16 */
+    VRL_CALL_ADD_RMSNORM = 6,   /* vrl_add_rmsnorm_bf16 */
+    VRL_CALL_ATTN = 7,          /* vrl_rope_attn_decode_bf16 */
+    VRL_CALL_ATTN_SPLIT = 8,    /* vrl_rope_attn_decode_split_bf16 */
+    VRL_CALL_ATTN_ROWS = 9,     /* vrl_rope_attn_decode_rows_bf16 */
+    VRL_CALL_ATTN_LORA = 10,    /* vrl_rope_attn_decode_lora_bf16 */
+    VRL_CALL_LORA_DOWN = 11,    /* vrl_lora_down_bf16 */
+    VRL_CALL_LORA_UP_ADD = 12   /* vrl_lora_up_add_bf16 */
+};
+typedef struct vrl_step_call {
+    int32_t kind;
+    int32_t reserved;        /* 0 */
+    const void *p[12];
+    int64_t i[8];
+    float f[2];
+} vrl_step_call;
+
+int vrl_decode_run_calls(const vrl_step_call *calls, int n_calls, int *failed_at, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

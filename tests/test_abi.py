@@ -378,3 +378,31 @@ def test_head_sample_extras_validation(lib):
     assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need, None) == 1002
     ex.position = p
     assert f(ctypes.byref(head), ctypes.byref(ex), p, p, p, 1, 5.0, 1.0, p, need - 256, None) == 1001  # workspace too small
+
+
+def test_step_call_records_hold_the_arguments_by_type_and_the_walk_reports_the_failing_call():
+    """``vrl_decode_run_calls``: arguments go to the pointer / integer / float slots in declaration order; a NULL
+    list, a negative count and an unknown kind are refused before anything is launched, the index of the call
+    that failed is reported."""
+    import ctypes
+
+    lib = _lib.load()
+    norm = _lib.Norm()
+    table = _lib.step_calls([
+        (lib.vrl_add_rmsnorm_bf16, (16, 32, 48, None, 80, 7, 2048, 0.5)),
+        (lib.vrl_int4_gemv_prepacked_norm_bf16, ((_lib.Problem * 2)(), 2, ctypes.byref(norm))),
+    ])
+    assert table[0].kind == 6 and list(table[0].p[:5]) == [16, 32, 48, None, 80]
+    assert list(table[0].i[:2]) == [7, 2048] and table[0].f[0] == 0.5
+    assert table[1].kind == 2 and table[1].i[0] == 2 and table[1].p[1] == ctypes.addressof(norm)
+    with pytest.raises(ValueError):
+        _lib.step_calls([(lib.vrl_add_rmsnorm_bf16, (1, 2, 3))])
+    failed = ctypes.c_int(-1)
+    assert lib.vrl_decode_run_calls(None, 1, ctypes.byref(failed), None) == 1003
+    assert lib.vrl_decode_run_calls(table, -1, ctypes.byref(failed), None) == 1001
+    assert lib.vrl_decode_run_calls(table, 0, ctypes.byref(failed), None) == 0 and failed.value == -1
+    bad = (_lib.StepCall * 2)()
+    bad[0].kind, bad[1].kind = 6, 99      # a norm over NULL tensors, then an unknown entry point
+    assert lib.vrl_decode_run_calls(bad, 2, ctypes.byref(failed), None) == 1003 and failed.value == 0
+    bad[0].kind = 99
+    assert lib.vrl_decode_run_calls(bad, 2, None, None) == 1001

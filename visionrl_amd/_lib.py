@@ -44,7 +44,54 @@ SYMBOLS = (
     "vrl_lora_up_add_bf16",
     "vrl_int4_gemv_prepacked_lora_bf16",
     "vrl_int4_gemv_prepacked_lora_up_bf16",
+    "vrl_decode_run_calls",
 )
+
+
+class StepCall(ctypes.Structure):
+    """Mirror of ``vrl_step_call`` (include/vrl_decode.h): one call of a decode step's launch list."""
+
+    _fields_ = [("kind", ctypes.c_int32), ("reserved", ctypes.c_int32), ("p", ctypes.c_void_p * 12),
+                ("i", ctypes.c_int64 * 8), ("f", ctypes.c_float * 2)]
+
+
+# vrl_step_call.kind of the entry points a launch list may hold
+STEP_CALL_KINDS = {
+    "vrl_int4_gemv_prepacked_bf16": 1, "vrl_int4_gemv_prepacked_norm_bf16": 2,
+    "vrl_int4_gemv_prepacked_epilogue_bf16": 3, "vrl_int4_gemv_prepacked_lora_bf16": 4,
+    "vrl_int4_gemv_prepacked_lora_up_bf16": 5, "vrl_add_rmsnorm_bf16": 6, "vrl_rope_attn_decode_bf16": 7,
+    "vrl_rope_attn_decode_split_bf16": 8, "vrl_rope_attn_decode_rows_bf16": 9,
+    "vrl_rope_attn_decode_lora_bf16": 10, "vrl_lora_down_bf16": 11, "vrl_lora_up_add_bf16": 12,
+}
+
+
+def step_calls(calls) -> "ctypes.Array":
+    """``[(library function, arguments without the stream), ...]`` as an array of ``vrl_step_call`` records:
+    every argument goes to the slot list of its declared type, in order (pointers, integers, floats).  The
+    objects the arguments refer to must be kept alive by the caller."""
+    table = (StepCall * len(calls))()
+    for rec, (fn, args) in zip(table, calls):
+        if len(args) != len(fn.argtypes) - 1:
+            raise ValueError(f"{fn.__name__} takes {len(fn.argtypes) - 1} arguments before the stream")
+        rec.kind = STEP_CALL_KINDS[fn.__name__]
+        n_p = n_i = n_f = 0
+        for kind, value in zip(fn.argtypes[:-1], args):
+            if kind is ctypes.c_float:
+                rec.f[n_f] = float(value)
+                n_f += 1
+            elif kind in (ctypes.c_int, ctypes.c_size_t, ctypes.c_int64):
+                rec.i[n_i] = int(value)
+                n_i += 1
+            else:   # c_void_p or a typed pointer: an address, None, a ctypes object or a byref() of one
+                if value is None:
+                    address = None
+                elif isinstance(value, int):
+                    address = value
+                else:
+                    address = ctypes.addressof(getattr(value, "_obj", value))
+                rec.p[n_p] = address
+                n_p += 1
+    return table
 
 
 class Int4LibraryError(RuntimeError):
@@ -233,6 +280,8 @@ def _bind(lib):
     lib.vrl_rope_attn_decode_rows_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                                    ci, ci, ci, ci, ci, ctypes.c_float, vp, ctypes.c_size_t, vp]
     lib.vrl_rope_attn_decode_split_workspace_bytes.restype = ctypes.c_size_t
+    lib.vrl_decode_run_calls.argtypes = [ctypes.POINTER(StepCall), ci, ctypes.POINTER(ctypes.c_int), vp]
+    lib.vrl_decode_run_calls.restype = ci
     lib.vrl_rope_attn_decode_split_workspace_bytes.argtypes = [ci, ci, ci]
     lib.vrl_rope_attn_decode_split_bf16.restype = ci
     lib.vrl_rope_attn_decode_split_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,

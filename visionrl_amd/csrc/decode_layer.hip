@@ -857,3 +857,82 @@ extern "C" int vrl_lora_up_add_bf16(const float *t, int t_parts, int M, const vr
     return max_r <= 32 ? launch_lora_up<false, 32>(t, t_parts, a, max_n, max_r, stream)
                        : launch_lora_up<false, 64>(t, t_parts, a, max_n, max_r, stream);
 }
+
+// ---------------------------------------------------------------- a step's launches from one host call
+extern "C" int vrl_decode_run_calls(const vrl_step_call *calls, int n_calls, int *failed_at, void *hip_stream) {
+    if (!calls) return VRL_INT4_ENULL;
+    if (n_calls < 0) return VRL_INT4_ESHAPE;
+    for (int n = 0; n < n_calls; ++n) {
+        const vrl_step_call &c = calls[n];
+        const void *const *p = c.p;
+        const int64_t *i = c.i;
+        void *s = hip_stream;
+        auto w = [&](int k) { return const_cast<void *>(p[k]); };   // a pointer the callee writes through
+        int rc;
+        switch (c.kind) {
+            case VRL_CALL_GEMV:
+                rc = vrl_int4_gemv_prepacked_bf16(static_cast<const vrl_int4_problem *>(p[0]), (int)i[0], s);
+                break;
+            case VRL_CALL_GEMV_NORM:
+                rc = vrl_int4_gemv_prepacked_norm_bf16(static_cast<const vrl_int4_problem *>(p[0]), (int)i[0],
+                                                       static_cast<const vrl_int4_norm *>(p[1]), s);
+                break;
+            case VRL_CALL_GEMV_EPILOGUE:
+                rc = vrl_int4_gemv_prepacked_epilogue_bf16(static_cast<const vrl_int4_problem *>(p[0]),
+                                                           static_cast<const vrl_int4_norm *>(p[1]),
+                                                           static_cast<const vrl_int4_epilogue *>(p[2]), s);
+                break;
+            case VRL_CALL_GEMV_LORA:
+                rc = vrl_int4_gemv_prepacked_lora_bf16(static_cast<const vrl_int4_problem *>(p[0]), (int)i[0],
+                                                       static_cast<const vrl_lora_adapter *>(p[1]), (int)i[1],
+                                                       static_cast<float *>(w(2)), s);
+                break;
+            case VRL_CALL_GEMV_LORA_UP:
+                rc = vrl_int4_gemv_prepacked_lora_up_bf16(static_cast<const vrl_int4_problem *>(p[0]),
+                                                          static_cast<const vrl_lora_adapter *>(p[1]),
+                                                          static_cast<const float *>(p[2]), (int)i[0], s);
+                break;
+            case VRL_CALL_ADD_RMSNORM:
+                rc = vrl_add_rmsnorm_bf16(p[0], p[1], p[2], w(3), w(4), (int)i[0], (int)i[1], c.f[0], s);
+                break;
+            case VRL_CALL_ATTN:
+                rc = vrl_rope_attn_decode_bf16(p[0], p[1], p[2], (int)i[0], (int)i[1], w(3), w(4), p[5], p[6], p[7],
+                                               static_cast<const int64_t *>(p[8]), w(9), (int)i[2], (int)i[3],
+                                               (int)i[4], (int)i[5], (int)i[6], c.f[0], s);
+                break;
+            case VRL_CALL_ATTN_SPLIT:
+                rc = vrl_rope_attn_decode_split_bf16(p[0], p[1], p[2], (int)i[0], (int)i[1], w(3), w(4), p[5], p[6],
+                                                     p[7], static_cast<const int64_t *>(p[8]), w(9), (int)i[2],
+                                                     (int)i[3], (int)i[4], (int)i[5], (int)i[6], c.f[0], w(10),
+                                                     (size_t)i[7], s);
+                break;
+            case VRL_CALL_ATTN_ROWS:
+                rc = vrl_rope_attn_decode_rows_bf16(p[0], p[1], p[2], (int)i[0], (int)i[1], w(3), w(4), p[5], p[6],
+                                                    p[7], static_cast<const int64_t *>(p[8]), w(9), (int)i[2],
+                                                    (int)i[3], (int)i[4], (int)i[5], (int)i[6], c.f[0], w(10),
+                                                    (size_t)i[7], s);
+                break;
+            case VRL_CALL_ATTN_LORA:
+                rc = vrl_rope_attn_decode_lora_bf16(p[0], p[1], p[2], (int)i[0], (int)i[1], w(3), w(4), p[5], p[6],
+                                                    p[7], static_cast<const int64_t *>(p[8]), w(9), (int)i[2],
+                                                    (int)i[3], (int)i[4], (int)i[5], (int)i[6], c.f[0],
+                                                    static_cast<const vrl_attn_lora *>(p[10]), s);
+                break;
+            case VRL_CALL_LORA_DOWN:
+                rc = vrl_lora_down_bf16(p[0], (int)i[0], (int)i[1], static_cast<const vrl_lora_adapter *>(p[1]),
+                                        (int)i[2], static_cast<float *>(w(2)), s);
+                break;
+            case VRL_CALL_LORA_UP_ADD:
+                rc = vrl_lora_up_add_bf16(static_cast<const float *>(p[0]), (int)i[0], (int)i[1],
+                                          static_cast<const vrl_lora_adapter *>(p[1]), (int)i[2], s);
+                break;
+            default:
+                rc = VRL_INT4_ESHAPE;
+        }
+        if (rc != 0) {
+            if (failed_at) *failed_at = n;
+            return rc;
+        }
+    }
+    return 0;
+}

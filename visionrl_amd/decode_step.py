@@ -378,17 +378,19 @@ class NativeDecodeTrunk:
             self.normed = None
         self._calls = calls
         self.launches = len(calls)
+        # the same list as records of the library's own walk over it: one host call per step
+        self._table = _lib.step_calls(calls)
+        self._failed_at = ctypes.c_int(-1)
 
     def run(self) -> torch.Tensor:
         """Enqueue the step on the current stream; returns the ``[rows, hidden]`` output buffer."""
         stream = torch.cuda.current_stream(self.device).cuda_stream
         with ops._on(self.device):
-            for fn, args in self._calls:
-                rc = fn(*args, stream)
-                if rc:
-                    # a step that stopped half-way may leave the split attention's arrival counters above zero,
-                    # and every later launch over that workspace would then merge too early: clear them
-                    if self._split_ws is not None and not torch.cuda.is_current_stream_capturing():
-                        self._split_ws.zero_()
-                    _lib.check(rc, fn.__name__)
+            rc = _lib.load().vrl_decode_run_calls(self._table, len(self._table), ctypes.byref(self._failed_at), stream)
+        if rc:
+            # a step that stopped half-way may leave the split attention's arrival counters above zero,
+            # and every later launch over that workspace would then merge too early: clear them
+            if self._split_ws is not None and not torch.cuda.is_current_stream_capturing():
+                self._split_ws.zero_()
+            _lib.check(rc, self._calls[self._failed_at.value][0].__name__)
         return self.normed
