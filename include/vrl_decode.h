@@ -136,6 +136,17 @@ int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_pr
                                       void *hip_stream);
 
 /*
+ * The launch above with the residual add and RMSNorm of vrl_int4_gemv_prepacked_norm_bf16 applied to the shared
+ * input first, for both the base projections and the adapters (which read the normalised rows, as the wrapper's
+ * lora_A does: input_layernorm precedes q|k|v in LlamaDecoderLayer.forward): a decoder layer under adapters then
+ * needs no norm launch of its own in front of q|k|v.  `norm` as for vrl_int4_gemv_prepacked_norm_bf16; K <= 2048,
+ * M <= 16 (the adapters' workgroups keep their rows in registers).
+ */
+int vrl_int4_gemv_prepacked_norm_lora_bf16(const vrl_int4_problem *problems, int n_problems,
+                                           const vrl_int4_norm *norm, const vrl_lora_adapter *adapters,
+                                           int n_adapters, float *t, void *hip_stream);
+
+/*
  * vrl_int4_gemv_prepacked_bf16 of one problem and vrl_lora_up_add_bf16 of its adapter in one launch:
  *   y[m,n] = bf16( bf16(x . W^T)[m,n] + scaling * sum_j t[m,j] * B[n,j] )
  * with t [M, t_parts, r] as for vrl_lora_up_add_bf16 (the down-projection of the same x, e.g. the
@@ -204,7 +215,8 @@ enum {
     VRL_CALL_ATTN_ROWS = 9,     /* vrl_rope_attn_decode_rows_bf16 */
     VRL_CALL_ATTN_LORA = 10,    /* vrl_rope_attn_decode_lora_bf16 */
     VRL_CALL_LORA_DOWN = 11,    /* vrl_lora_down_bf16 */
-    VRL_CALL_LORA_UP_ADD = 12   /* vrl_lora_up_add_bf16 */
+    VRL_CALL_LORA_UP_ADD = 12,  /* vrl_lora_up_add_bf16 */
+    VRL_CALL_GEMV_NORM_LORA = 13 /* vrl_int4_gemv_prepacked_norm_lora_bf16 */
 };
 typedef struct vrl_step_call {
     int32_t kind;

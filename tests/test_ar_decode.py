@@ -441,7 +441,7 @@ def lora_policy(dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_native_trunk_with_lora_adapters_tracks_the_module_trunk(dtype):
-    """As above with adapters on q/k/v/o: the native layer adds them with two launches per group; a
+    """As above with adapters on q/k/v/o: the native layer adds them inside its five launches; a
     weight sync in place (``load_lora_state``) reaches it without rebuilding anything."""
     from visionrl_amd.policy_glue import load_lora_state
 
@@ -458,7 +458,7 @@ def test_native_trunk_with_lora_adapters_tracks_the_module_trunk(dtype):
         sessions.append(sess)
     nat, mod = sessions
     assert nat.native and not mod.native
-    assert nat.native.launches == (5 + 1) * LAYERS + 1   # the first norm as a launch of its own
+    assert nat.native.launches == 5 * LAYERS + 1   # the adapters' workgroups of q|k|v normalise their rows themselves
     trunk = policy._lm_trunk()
     gen = torch.Generator(device="cuda:0").manual_seed(62)
 

@@ -655,6 +655,54 @@ def test_down_projection_rides_with_the_base_launch(ops_mod, M, K, Ns, ranks, fp
     assert np.abs(group.t.cpu().numpy() - t64).max() <= (2.0 ** -7 if not fp32 else 2.0 ** -16) * max(1.0, np.abs(t64).max())
 
 
+@pytest.mark.parametrize("M,K,Ns,ranks,fp32,with_residual", [
+    (2, 2048, (2048, 2048, 2048), (32, 32, 32), True, False), (8, 2048, (2048, 512, 512), (32, 16, 16), True, True),
+    (16, 2048, (2048, 2048, 2048), (32, 32, 32), False, True), (5, 640, (96, 48), (8, 24), False, False),
+    (1, 1536, (64,), (64,), True, True)])
+def test_norm_and_down_projection_ride_with_the_base_launch(ops_mod, M, K, Ns, ranks, fp32, with_residual):
+    """``DirectGemv(norm=...).launch(lora_down=group)``: residual add, RMSNorm, the base projections and the
+    adapters' down-projections of the normalised rows in one launch, against the norm launch followed by the
+    base launch with its down-projection workgroups: the same ``h``, base outputs and ``t`` within what a last-bit
+    difference in a row's scale (sums of squares added in another order) can move them."""
+    from tests._util import to_device
+    say("norm + base launch with down-projection", M, K, Ns, ranks, fp32, with_residual)
+    rng = np.random.default_rng(3 * M + K)
+    dtype = torch.float32 if fp32 else torch.bfloat16
+    x, res = bits_to_bf16(rand_bits(rng, (M, K)), DEV), bits_to_bf16(rand_bits(rng, (M, K), 4.0), DEV)
+    wn = bits_to_bf16(rand_bits(rng, (K,), 0.5), DEV)
+    gen = torch.Generator().manual_seed(K + M)
+    packed, ads = [], []
+    for i, (N, r) in enumerate(zip(Ns, ranks)):
+        w = to_device(o.make_operands(950 + i, M, K, N, 128), DEV)
+        packed.append(ops_mod.int4_prepack(w["qweight"], w["scales"], w["qzeros"], 128))
+        A = (torch.randn(r, K, generator=gen) * K ** -0.5).to(dtype).to(DEV)
+        B = (torch.randn(N, r, generator=gen) * 0.2).to(dtype).to(DEV)
+        ads.append((A, B))
+    h_want, normed = ops_mod.add_rmsnorm(x, wn, 1e-6, res if with_residual else None)
+    two = ops_mod.DirectGemv([(normed, pw, False) for pw in packed])
+    g2 = ops_mod.LoraAdd(normed, [(A, B, 1.0, y) for (A, B), y in zip(ads, two.outputs)])
+    want_y = [y.clone() for y in two.launch(lora_down=g2)]
+    h_out = torch.zeros_like(x)
+    one = ops_mod.DirectGemv([(x, pw, False) for pw in packed],
+                             norm=(res if with_residual else None, wn, 1e-6, h_out if with_residual else None))
+    g1 = ops_mod.LoraAdd(x, [(A, B, 1.0, y) for (A, B), y in zip(ads, one.outputs)])
+    g1.t.fill_(float("nan"))
+    got_y = one.launch(lora_down=g1)
+    torch.cuda.synchronize()
+    if with_residual:
+        assert torch.equal(h_out, h_want)
+    for a, b in zip(got_y, want_y):
+        close = (a.float() - b.float()).abs() <= 2.0 ** -6 * b.float().abs() + 2.0 ** -7
+        assert close.all() and (a != b).float().mean().item() < 0.02
+    scale = max(1.0, g2.t.abs().max().item())
+    assert torch.isfinite(g1.t).all() and (g1.t - g2.t).abs().max().item() <= 2.0 ** -6 * scale
+    if M <= 16:
+        with pytest.raises(ValueError):   # more rows than the adapters' workgroups keep in registers
+            big = torch.zeros((17, K), dtype=torch.bfloat16, device=DEV)
+            launch = ops_mod.DirectGemv([(big, packed[0], False)], norm=(None, wn, 1e-6, None))
+            launch.launch(lora_down=ops_mod.LoraAdd(big, [(*ads[0], 1.0, launch.outputs[0])]))
+
+
 @pytest.mark.parametrize("M,K,N,r,parts,fp32", [(2, 2048, 2048, 32, 16, True), (32, 2048, 2048, 32, 16, True),
                                                 (7, 512, 100, 8, 1, False), (16, 4096, 4096, 64, 32, True),
                                                 (20, 5632, 2048, 16, 3, False), (1, 256, 48, 8, 1, True),

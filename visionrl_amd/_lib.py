@@ -45,6 +45,7 @@ SYMBOLS = (
     "vrl_int4_gemv_prepacked_lora_bf16",
     "vrl_int4_gemv_prepacked_lora_up_bf16",
     "vrl_decode_run_calls",
+    "vrl_int4_gemv_prepacked_norm_lora_bf16",
 )
 
 
@@ -62,6 +63,7 @@ STEP_CALL_KINDS = {
     "vrl_int4_gemv_prepacked_lora_up_bf16": 5, "vrl_add_rmsnorm_bf16": 6, "vrl_rope_attn_decode_bf16": 7,
     "vrl_rope_attn_decode_split_bf16": 8, "vrl_rope_attn_decode_rows_bf16": 9,
     "vrl_rope_attn_decode_lora_bf16": 10, "vrl_lora_down_bf16": 11, "vrl_lora_up_add_bf16": 12,
+    "vrl_int4_gemv_prepacked_norm_lora_bf16": 13,
 }
 
 
@@ -280,6 +282,9 @@ def _bind(lib):
     lib.vrl_rope_attn_decode_rows_bf16.argtypes = [vp, vp, vp, ci, ci, vp, vp, vp, vp, vp, vp, vp,
                                                    ci, ci, ci, ci, ci, ctypes.c_float, vp, ctypes.c_size_t, vp]
     lib.vrl_rope_attn_decode_split_workspace_bytes.restype = ctypes.c_size_t
+    lib.vrl_int4_gemv_prepacked_norm_lora_bf16.restype = ci
+    lib.vrl_int4_gemv_prepacked_norm_lora_bf16.argtypes = [ctypes.POINTER(Problem), ci, ctypes.POINTER(Norm),
+                                                           ctypes.POINTER(LoraAdapter), ci, vp, vp]
     lib.vrl_decode_run_calls.argtypes = [ctypes.POINTER(StepCall), ci, ctypes.POINTER(ctypes.c_int), vp]
     lib.vrl_decode_run_calls.restype = ci
     lib.vrl_rope_attn_decode_split_workspace_bytes.argtypes = [ci, ci, ci]

@@ -926,6 +926,12 @@ extern "C" int vrl_decode_run_calls(const vrl_step_call *calls, int n_calls, int
                 rc = vrl_lora_up_add_bf16(static_cast<const float *>(p[0]), (int)i[0], (int)i[1],
                                           static_cast<const vrl_lora_adapter *>(p[1]), (int)i[2], s);
                 break;
+            case VRL_CALL_GEMV_NORM_LORA:
+                rc = vrl_int4_gemv_prepacked_norm_lora_bf16(static_cast<const vrl_int4_problem *>(p[0]), (int)i[0],
+                                                            static_cast<const vrl_int4_norm *>(p[1]),
+                                                            static_cast<const vrl_lora_adapter *>(p[2]), (int)i[1],
+                                                            static_cast<float *>(w(3)), s);
+                break;
             default:
                 rc = VRL_INT4_ESHAPE;
         }

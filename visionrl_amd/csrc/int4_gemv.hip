@@ -388,6 +388,13 @@ int launch_direct_lora(const DirectArgs &args, int ks, int tw, int workgroups, s
     return VRL_INT4_EPLAN;
 }
 
+// the same with residual add and RMSNorm applied to the shared input (rows of up to 2048 values: four waves per tile)
+int launch_direct_lora_norm(const DirectArgs &args, int ks, int tw, int workgroups, size_t lds, hipStream_t stream) {
+    if (ks == 4 && tw == 1) return launch_direct<false, 4, 1, true, false, true>(args, workgroups, lds, stream);
+    if (ks == 4 && tw == 2) return launch_direct<false, 4, 2, true, false, true>(args, workgroups, lds, stream);
+    return VRL_INT4_EPLAN;   // (sixteen-wave workgroups leave the adapters' rows too few registers: not built)
+}
+
 int dispatch_stream(vrl_int4_plan_info *info, const DevProblem *recs, const int2 *block_tab,
                     hipStream_t stream) {
     const bool mb2 = (info->variant & VARIANT_MB2) != 0;
@@ -541,6 +548,7 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     // few tiles (o_proj: 128 or 256) one tile per workgroup below 8 rows (4.2 against 4.9 us at 2 rows).
     int tw = (max_m >= 8 && !xg && !lora_up) ? 16 / ks : 1;
     const bool many_tiles = slab_tiles >= 5L * device_cu_count() / 4;
+    if (norm && lora_down && tw > 2) tw = 2;   // the build of that launch with four tiles per workgroup spills
     if (!xg && !lora_up && max_m <= MAX_TILE_M && ks <= 8 && many_tiles)
         tw = (ks == 8 && fused_any && max_m >= 12) ? 1 : 2;
     // Three more measured preferences, all about how the rows get into LDS.  A register-fed wave asks for its
@@ -738,13 +746,16 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
             if (problems[i].x != q0.x || problems[i].M != q0.M || problems[i].K != q0.K) return VRL_INT4_ESHAPE;
         const int rc = lora_args(args.ld.a, q0.M, q0.K, lora->adapters, lora->n_adapters, false);
         if (rc != VRL_INT4_OK) return rc;
+        // with a norm the adapters' workgroups normalise the rows themselves, a lane holding one piece of each
+        if (norm && (q0.K > NORM_MAX_K / 2 || ks != 4 || q0.M > MAX_TILE_M)) return VRL_INT4_ESHAPE;
         args.ld.x = static_cast<const uint16_t *>(q0.x);
         args.ld.t = lora->t;
         args.ld.fp32 = args.ld.a.ad[0].weights_fp32 != 0;
         args.ld.wgs = lora_down_workgroups(args.ld.a, ks * tw);
         workgroups += args.ld.wgs;
         lds = std::max(lds, (size_t)ks * tw * 16 * sizeof(float));
-        return launch_direct_lora(args, ks, tw, (int)workgroups, lds, stream);
+        return norm ? launch_direct_lora_norm(args, ks, tw, (int)workgroups, lds, stream)
+                    : launch_direct_lora(args, ks, tw, (int)workgroups, lds, stream);
     }
     if (args.epi.enabled)
         return norm ? launch_direct_epilogue<true>(args, ks, tw, false, (int)workgroups, lds, stream)
@@ -766,6 +777,14 @@ int vrl_int4_gemv_prepacked_lora_bf16(const vrl_int4_problem *problems, int n_pr
     if (!adapters) return VRL_INT4_ENULL;
     const DirectLora lora{adapters, n_adapters, t, false, 1};
     return direct_launch(problems, n_problems, nullptr, &lora, hip_stream);
+}
+
+int vrl_int4_gemv_prepacked_norm_lora_bf16(const vrl_int4_problem *problems, int n_problems,
+                                           const vrl_int4_norm *norm, const vrl_lora_adapter *adapters,
+                                           int n_adapters, float *t, void *hip_stream) {
+    if (!norm || !adapters) return VRL_INT4_ENULL;
+    const DirectLora lora{adapters, n_adapters, t, false, 1};
+    return direct_launch(problems, n_problems, norm, &lora, hip_stream);
 }
 
 int vrl_int4_gemv_prepacked_lora_up_bf16(const vrl_int4_problem *problem, const vrl_lora_adapter *adapter,

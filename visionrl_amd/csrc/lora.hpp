@@ -58,6 +58,124 @@ __device__ __forceinline__ void load8(const void *base, long index, float (&f)[8
 // group).  Written without data-dependent branches: rows past the end repeat the last one (clamped
 // index), which costs arithmetic but keeps every load of a lane in flight at once.  Every thread of
 // the workgroup must call it (it holds a workgroup barrier); groups with `active` false only wait.
+// NORMED (K <= 2048: a lane holds one piece of every row): x is a sublayer output and the adapter reads
+//   weight * bf16(h * rsqrt(mean(h^2) + eps)),  h = residual ? bf16(x + residual) : x
+// instead, the residual add and RMSNorm that precede q|k|v in LlamaDecoderLayer.forward, with the tensor ops'
+// roundings: the rows stay in registers while their sums of squares meet in `part`.
+struct LoraNorm {
+    const uint16_t *residual;  // same shape as x, or nullptr
+    const uint16_t *weight;    // [K]
+    float eps;
+};
+
+template <bool FP32, int MB>
+__device__ __forceinline__ void lora_down_item_normed(const uint16_t *x, const LoraArgs &a, const LoraNorm &nrm,
+                                                      float *t, bool active, int col, int m_lo, int gw, int lane,
+                                                      float *part) {
+    const int total = a.off[a.n];
+    const int k = (gw * LORA_WAVE + lane) * 8;
+    const bool in = active && k < a.K;
+    int rows = 0;
+    float af[8];
+    uint32_t h[MB][4], wv[4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) af[e] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wv[e] = 0u;
+#pragma unroll
+    for (int u = 0; u < MB; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[u][e] = 0u;
+    if (active) {  // uniform over the group's waves
+        int i = 0;
+#pragma unroll
+        for (int q = 1; q < LORA_MAX_ADAPTERS; ++q)
+            if (q < a.n && a.off[q] <= col) i = q;
+        const void *A = a.ad[0].A;
+        int first = 0;
+#pragma unroll
+        for (int q = 1; q < LORA_MAX_ADAPTERS; ++q)
+            if (q == i) A = a.ad[q].A, first = a.off[q];
+        rows = min(MB, a.M - m_lo);
+        if (in) {
+            load8<FP32>(A, (long)(col - first) * a.K + k, af);
+            const uint4 w4 = *reinterpret_cast<const uint4 *>(nrm.weight + k);
+            wv[0] = w4.x, wv[1] = w4.y, wv[2] = w4.z, wv[3] = w4.w;
+            uint4 xr[MB], rr[MB];
+#pragma unroll
+            for (int u = 0; u < MB; ++u) {
+                const long at = (long)(m_lo + (u < rows ? u : rows - 1)) * a.K + k;
+                xr[u] = *reinterpret_cast<const uint4 *>(x + at);
+                rr[u] = nrm.residual ? *reinterpret_cast<const uint4 *>(nrm.residual + at) : uint4{0u, 0u, 0u, 0u};
+            }
+            __builtin_amdgcn_sched_barrier(0);  // all requests before the first use
+#pragma unroll
+            for (int u = 0; u < MB; ++u) {
+                const uint32_t xw[4] = {xr[u].x, xr[u].y, xr[u].z, xr[u].w};
+                const uint32_t rw[4] = {rr[u].x, rr[u].y, rr[u].z, rr[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (nrm.residual) {   // uniform
+                        const float lo = lora_round_bf16(lora_bf16(rw[e] & 0xFFFFu) + lora_bf16(xw[e] & 0xFFFFu));
+                        const float hi = lora_round_bf16(lora_bf16(rw[e] >> 16) + lora_bf16(xw[e] >> 16));
+                        h[u][e] = (__builtin_bit_cast(uint32_t, lo) >> 16) | (__builtin_bit_cast(uint32_t, hi) & 0xFFFF0000u);
+                    } else {
+                        h[u][e] = xw[e];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < MB; ++u) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float lo = lora_bf16(h[u][e] & 0xFFFFu), hi = lora_bf16(h[u][e] >> 16);
+                ss += lo * lo;
+                ss += hi * hi;
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) part[gw * MB + u] = ss;
+        }
+    }
+    __syncthreads();
+    float acc[MB];
+    if (active) {
+        const float inv_k = 1.0f / (float)a.K;
+#pragma unroll
+        for (int u = 0; u < MB; ++u) {
+            float ss = part[u];
+#pragma unroll
+            for (int w = 1; w < LORA_DOWN_WAVES; ++w) ss += part[w * MB + u];
+            const float r = rsqrtf(ss * inv_k + nrm.eps);
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float lo = lora_round_bf16(lora_bf16(wv[e] & 0xFFFFu) * lora_round_bf16(lora_bf16(h[u][e] & 0xFFFFu) * r));
+                const float hi = lora_round_bf16(lora_bf16(wv[e] >> 16) * lora_round_bf16(lora_bf16(h[u][e] >> 16) * r));
+                sum += lo * af[2 * e] + hi * af[2 * e + 1];
+            }
+            acc[u] = sum;
+        }
+    }
+    __syncthreads();  // the sums of squares are read before the partial products take their place
+    if (active) {
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const float v = wave_sum(acc[m]);
+            if (lane == 0) part[gw * MB + m] = v;
+        }
+    }
+    __syncthreads();
+    if (active && gw == 0 && lane < rows) {
+        float v = part[lane];
+#pragma unroll
+        for (int w = 1; w < LORA_DOWN_WAVES; ++w) v += part[w * MB + lane];
+        if (!FP32) v = lora_round_bf16(v);  // lora_A's output tensor is bf16 then
+        t[(long)(m_lo + lane) * total + col] = v;
+    }
+}
+
 template <bool FP32, int MB>
 __device__ __forceinline__ void lora_down_item(const uint16_t *x, const LoraArgs &a, float *t, bool active,
                                                int col, int m_lo, int gw, int lane, float *part) {
@@ -113,9 +231,9 @@ __device__ __forceinline__ void lora_down_item(const uint16_t *x, const LoraArgs
 
 // A workgroup of NW waves (a multiple of four) as NW / 4 groups: group `grp` takes item
 // wg * (NW / 4) + grp of the r_total x row-block items; `smem` holds NW x 16 floats.
-template <int NW>
+template <int NW, bool NORMED = false>
 __device__ __forceinline__ void lora_down_workgroup(const uint16_t *x, const LoraArgs &a, float *t, bool fp32,
-                                                    int wg, float *smem) {
+                                                    int wg, float *smem, const LoraNorm &nrm = LoraNorm{}) {
     static_assert(NW % LORA_DOWN_WAVES == 0, "whole groups of four waves");
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & (LORA_WAVE - 1);
     const int grp = wave / LORA_DOWN_WAVES, gw = wave % LORA_DOWN_WAVES;
@@ -126,6 +244,16 @@ __device__ __forceinline__ void lora_down_workgroup(const uint16_t *x, const Lor
     const bool active = item < items;
     const int col = item % total, m_lo = (item / total) * mb;
     float *part = smem + grp * LORA_DOWN_WAVES * 16;
+    if constexpr (NORMED) {
+        if (mb == 8) {
+            if (fp32) lora_down_item_normed<true, 8>(x, a, nrm, t, active, col, m_lo, gw, lane, part);
+            else lora_down_item_normed<false, 8>(x, a, nrm, t, active, col, m_lo, gw, lane, part);
+        } else {
+            if (fp32) lora_down_item_normed<true, 16>(x, a, nrm, t, active, col, m_lo, gw, lane, part);
+            else lora_down_item_normed<false, 16>(x, a, nrm, t, active, col, m_lo, gw, lane, part);
+        }
+        return;
+    }
     if (mb == 8) {
         if (fp32) lora_down_item<true, 8>(x, a, t, active, col, m_lo, gw, lane, part);
         else lora_down_item<false, 8>(x, a, t, active, col, m_lo, gw, lane, part);

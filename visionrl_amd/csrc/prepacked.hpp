@@ -1040,7 +1040,11 @@ __global__ __launch_bounds__(KS *TW *WAVE) void gemv_split_direct_kernel(DirectA
     int g = blockIdx.x;
     if constexpr (LD) {
         if (g < a.ld.wgs) {  // uniform over the workgroup
-            lora_down_workgroup<KS * TW>(a.ld.x, a.ld.a, a.ld.t, a.ld.fp32 != 0, g, reinterpret_cast<float *>(smem));
+            if constexpr (NORM)   // the adapters read the normalised rows, as the tiles do
+                lora_down_workgroup<KS * TW, true>(a.ld.x, a.ld.a, a.ld.t, a.ld.fp32 != 0, g, reinterpret_cast<float *>(smem),
+                                                   LoraNorm{a.norm.residual, a.norm.weight, a.norm.eps});
+            else
+                lora_down_workgroup<KS * TW>(a.ld.x, a.ld.a, a.ld.t, a.ld.fp32 != 0, g, reinterpret_cast<float *>(smem));
             return;
         }
         g -= a.ld.wgs;

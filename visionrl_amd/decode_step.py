@@ -21,7 +21,9 @@ op in fp32, rounded to bf16); the attention keeps its probabilities in fp32.
 Needs a trunk whose projections were swapped for prepacked :class:`Int4Linear` modules with the
 fused MLP (``apply_int4_to_policy`` defaults).  Attention projections may carry one active LoRA
 adapter each (the reference's default, ``policy.py:81-88``, ``:298-324``): their layer then takes
-the norm as a launch of its own (the adapters read the normalised row): six launches.  The
+the norm as a launch of its own (the adapters read the normalised row) when the rows are wider than
+2048 values or more than 8: six launches; otherwise the adapters' workgroups of the q|k|v launch
+normalise the rows themselves (up to 8 rows).  The
 down-projections of the q|k|v adapters ride with the q|k|v launch as extra workgroups and their
 up-projections are added by the attention launch as it reads q, k, v; the attention launch also leaves
 o_proj's down-projection behind, one piece per head, and o_proj's launch adds the up-projection before
@@ -298,8 +300,21 @@ class NativeDecodeTrunk:
                 h_out = streams[state["flip"]]
                 state["flip"] ^= 1
             group = None
-            if fuse_norm and not any(ad is not None for ad in adapters):
+            with_adapters = any(ad is not None for ad in adapters)
+            if fuse_norm and not with_adapters:
                 outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
+            elif fuse_norm and not fused and hidden <= 2048 and rows <= 8:
+                # rows of up to 2048 values, at most 8 of them: the adapters' down-projection workgroups of the
+                # q|k|v launch normalise the rows themselves, so the layer needs no norm launch of its own here
+                # either (7.7 against 3.5 + 6.0 us at 2 rows; a step with adapters, same box, alternating:
+                # 0.98-1.00 against 1.00-1.02 ms at B=1, 1.11 against 1.13-1.16 ms at B=4; with 16 rows those
+                # workgroups become the launch's longest, 1.34 against 1.29 ms at B=8, and at 32 rows they hold
+                # more rows than their registers take)
+                launch_at = len(calls)
+                outs = gemv([(state["x"], pw, fused) for pw in weights], norm=(state["res"], w, eps, h_out))
+                group = lora(state["x"], outs, adapters, up, down=False)
+                calls[launch_at] = (lib.vrl_int4_gemv_prepacked_norm_lora_bf16,
+                                    (*calls[launch_at][1], group.table, len(group.table), group.t.data_ptr()))
             else:
                 calls.append((lib.vrl_add_rmsnorm_bf16,
                               (state["x"].data_ptr(), state["res"].data_ptr() if state["res"] is not None else None,

@@ -397,11 +397,16 @@ class DirectGemv:
                 rc = lib.vrl_int4_gemv_prepacked_lora_up_bf16(self.table, lora_up.table, lora_up.t.data_ptr(),
                                                               lora_up.parts, _stream_handle(self.device))
             elif lora_down is not None:
-                if self.norm is not None or lora_down.parts != 1:
-                    raise ValueError("the adapters' down-projection joins a launch without a norm, in one piece")
-                rc = lib.vrl_int4_gemv_prepacked_lora_bf16(self.table, len(self.table), lora_down.table,
-                                                           len(lora_down.table), lora_down.t.data_ptr(),
-                                                           _stream_handle(self.device))
+                if lora_down.parts != 1:
+                    raise ValueError("the adapters' down-projection joins the launch in one piece")
+                if self.norm is not None:   # base projections and adapters over the normalised rows (K <= 2048)
+                    rc = lib.vrl_int4_gemv_prepacked_norm_lora_bf16(
+                        self.table, len(self.table), ctypes.byref(self.norm), lora_down.table, len(lora_down.table),
+                        lora_down.t.data_ptr(), _stream_handle(self.device))
+                else:
+                    rc = lib.vrl_int4_gemv_prepacked_lora_bf16(self.table, len(self.table), lora_down.table,
+                                                               len(lora_down.table), lora_down.t.data_ptr(),
+                                                               _stream_handle(self.device))
             elif self.norm is not None:
                 rc = lib.vrl_int4_gemv_prepacked_norm_bf16(self.table, len(self.table), ctypes.byref(self.norm),
                                                            _stream_handle(self.device))
