@@ -576,8 +576,11 @@ static int direct_launch(const vrl_int4_problem *problems, int n_problems, const
     if (norm && !lora && many_tiles) {
         if (ks == 8 && (max_m <= 8 || !fused_any)) ks = 4, tw = 4;
         else if (ks == 8 && max_m > MAX_TILE_M) ks = 4, tw = 2;
-        else if (ks == 4 && max_m > 12 && max_m <= MAX_TILE_M) ks = 8, tw = 2;
+        else if (ks == 4 && max_m > 12) ks = 8, tw = 2;   // also two slabs: 9.2 against 9.4 us, fused 12.2 against 12.7
     }
+    // Long K at 17 to 32 rows, register-fed: four waves per tile that walk three super-chunks each leave the CU's
+    // L1 fewer fragment requests at a time than sixteen waves with one (K = 5632, N = 2048: 9.2 against 9.9 us).
+    if (xg && ks == 16 && max_m > MAX_TILE_M && max_nsc <= 12 && !lora) ks = 4;
     // Few tiles of 17 to 32 rows of K up to 4096 with an epilogue (the passes over K above serve plain launches):
     // staged, two tiles per workgroup, against register-fed slabs 8.5 against 13.1 us (K = 4096, N = 4096).
     if (xg && ks == 8 && max_m > MAX_TILE_M && !lora && MAX_TILE_M <= staged_rows) xg = false, tw = 2;
