@@ -334,6 +334,35 @@ def test_rope_attn_masks_and_strided_inputs(ops_mod):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("M,H,Hkv,D,L,p", [(2, 16, 16, 128, 640, 0), (2, 16, 16, 128, 640, 1), (2, 16, 16, 128, 640, 37),
+                                           (2, 16, 16, 128, 640, 127), (2, 16, 16, 128, 640, 128),
+                                           (2, 16, 16, 128, 640, 129), (3, 4, 2, 64, 40, 33), (2, 8, 2, 128, 24, 5)])
+def test_rope_attn_ignores_what_the_slots_past_the_position_hold(ops_mod, M, H, Hkv, D, L, p):
+    """Slots at and past the row's position have not been written by this sequence: whatever bits they hold
+    (infinities and NaNs included, which a weight of zero would not silence) the result and the slots
+    themselves are what a cache of ordinary values there gives, for the one-workgroup and the split form."""
+    say("rope_attn poisoned tail", M, H, Hkv, D, L, p)
+    c = attn_case(7000 + p + L, M, H, Hkv, D, L, p)
+    want, kc_want, vc_want = run_attn(ops_mod, c)
+    poison = np.array([0x7FC0, 0x7F80, 0xFF80, 0xFFFF], dtype=np.uint16)
+    bad = dict(c)
+    bad["kc"], bad["vc"] = c["kc"].copy(), c["vc"].copy()
+    tail = bad["kc"][:, :, p:, :]
+    bad["kc"][:, :, p:, :] = poison[np.arange(tail.size).reshape(tail.shape) % 4]
+    bad["vc"][:, :, p:, :] = poison[(np.arange(tail.size).reshape(tail.shape) + 1) % 4]
+    bad["mask"] = np.zeros_like(c["mask"])         # nor does the mask past the position matter
+    bad["mask"][:, :p + 1] = c["mask"][:, :p + 1]
+    out, kc, vc = run_attn(ops_mod, bad)
+    assert torch.equal(out, want)
+    assert torch.equal(kc[:, :, :p + 1], kc_want[:, :, :p + 1]) and torch.equal(vc[:, :, :p + 1], vc_want[:, :, :p + 1])
+    assert (bf16_to_bits(kc)[:, :, p + 1:] == bad["kc"][:, :, p + 1:]).all()
+    ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV)
+    split_want, _, _ = run_attn_split(ops_mod, c, ws)
+    split_out, _, _ = run_attn_split(ops_mod, bad, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(split_out, split_want)
+
+
 def test_position_outside_the_cache_is_a_no_op(ops_mod):
     say("rope_attn position out of range")
     c = attn_case(8, 2, 2, 2, 64, 16, 3)

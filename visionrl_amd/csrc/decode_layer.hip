@@ -218,9 +218,6 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     __shared__ uint32_t s_before;           // SPLIT: workgroups of the pair that had arrived before this one
 
     const int h = blockIdx.x, m = blockIdx.y;
-    const long long p64 = a.position[(long)m * a.position_stride];
-    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
-    const int p = (int)p64;
     const int group = a.n_heads / a.n_kv_heads;
     const int hk = h / group;
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
@@ -230,6 +227,24 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     const uint16_t *kc = a.k_cache + cache_base + l16 * VEC;
     const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
     constexpr int STEP = 4 * ATT_WAVES * ATT_UNROLL;  // slots the workgroup visits per batch
+    RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
+    bool live[ATT_UNROLL];
+    if constexpr (!SPLIT) {
+        // Which slots the first batch visits does not depend on the row's position, only how many of them
+        // count: they are requested before the position is known (it comes from memory, and a request
+        // that waited for it would start a round trip later) and the slots at or past it are dropped below.
+#pragma unroll
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const int j = u * 4 * ATT_WAVES + wave * 4 + sub;
+            const int jj = j < a.L_max ? j : a.L_max - 1;
+            kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
+            vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
+            live[u] = mask[jj] != 0;
+        }
+    }
+    const long long p64 = a.position[(long)m * a.position_stride];
+    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
+    const int p = (int)p64;
     // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
     // multiple of 64 slots (what the workgroup's waves visit together)
     const int n_split = SPLIT ? (int)gridDim.z : 1, split = SPLIT ? (int)blockIdx.z : 0;
@@ -242,8 +257,6 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
 
     // The cached slots do not depend on the new token: the first batch of keys and values is
     // requested before anything else and arrives while the query is rotated.
-    RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
-    bool live[ATT_UNROLL];
     auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs j_hi > j_lo
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
@@ -254,7 +267,22 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             live[u] = j < j_hi && mask[jj] != 0;
         }
     };
-    if (j_hi > j_lo) request(j_lo);
+    if constexpr (SPLIT) {
+        if (j_hi > j_lo) request(j_lo);
+    } else {
+        // a slot at or past the position may hold anything (also what is not a number): it gets weight zero
+        // below, and zeros in place of its values keep 0 * value at zero
+#pragma unroll
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const bool inside = u * 4 * ATT_WAVES + wave * 4 + sub < j_hi;
+            live[u] = live[u] && inside;
+#pragma unroll
+            for (int i = 0; i < VEC / 2; ++i) {
+                kraw[u].w[i] = inside ? kraw[u].w[i] : 0u;
+                vraw[u].w[i] = inside ? vraw[u].w[i] : 0u;
+            }
+        }
+    }
 
     // The adapter of the projection that follows: thread (j, l16) holds the lane's VEC columns of row j
     // of A (rows j, j + OJ, ... if the rank exceeds OJ; the first is requested here, ahead of its use).
