@@ -229,34 +229,11 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     constexpr int STEP = 4 * ATT_WAVES * ATT_UNROLL;  // slots the workgroup visits per batch
     RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
     bool live[ATT_UNROLL];
-    if constexpr (!SPLIT) {
-        // Which slots the first batch visits does not depend on the row's position, only how many of them
-        // count: they are requested before the position is known (it comes from memory, and a request
-        // that waited for it would start a round trip later) and the slots at or past it are dropped below.
-#pragma unroll
-        for (int u = 0; u < ATT_UNROLL; ++u) {
-            const int j = u * 4 * ATT_WAVES + wave * 4 + sub;
-            const int jj = j < a.L_max ? j : a.L_max - 1;
-            kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
-            vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
-            live[u] = mask[jj] != 0;
-        }
-    }
-    const long long p64 = a.position[(long)m * a.position_stride];
-    if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
-    const int p = (int)p64;
     // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
     // multiple of 64 slots (what the workgroup's waves visit together)
     const int n_split = SPLIT ? (int)gridDim.z : 1, split = SPLIT ? (int)blockIdx.z : 0;
-    int j_lo = 0, j_hi = p;
-    if constexpr (SPLIT) {
-        const int share = ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
-        j_lo = min(p, split * share);
-        j_hi = min(p, j_lo + share);
-    }
-
-    // The cached slots do not depend on the new token: the first batch of keys and values is
-    // requested before anything else and arrives while the query is rotated.
+    const long long p64 = a.position[(long)m * a.position_stride];
+    int p = 0, j_lo = 0, j_hi = 0;
     auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs j_hi > j_lo
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
@@ -267,20 +244,27 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             live[u] = j < j_hi && mask[jj] != 0;
         }
     };
+    // The cached slots do not depend on the new token: the first batch of keys and values is
+    // requested before anything else and arrives while the query is rotated.
     if constexpr (SPLIT) {
+        if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
+        p = (int)p64;
+        const int share = ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
+        j_lo = min(p, split * share);
+        j_hi = min(p, j_lo + share);
         if (j_hi > j_lo) request(j_lo);
     } else {
-        // a slot at or past the position may hold anything (also what is not a number): it gets weight zero
-        // below, and zeros in place of its values keep 0 * value at zero
+        // Which slots the first batch visits does not depend on the row's position, only how many of them
+        // count, and neither do the new token's query, key and value: all are requested before the position
+        // is looked at (it comes from memory, and what waited for it would start a round trip later); the
+        // slots at or past it are dropped before the batch is used.
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
-            const bool inside = u * 4 * ATT_WAVES + wave * 4 + sub < j_hi;
-            live[u] = live[u] && inside;
-#pragma unroll
-            for (int i = 0; i < VEC / 2; ++i) {
-                kraw[u].w[i] = inside ? kraw[u].w[i] : 0u;
-                vraw[u].w[i] = inside ? vraw[u].w[i] : 0u;
-            }
+            const int j = u * 4 * ATT_WAVES + wave * 4 + sub;
+            const int jj = j < a.L_max ? j : a.L_max - 1;
+            kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
+            vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
+            live[u] = mask[jj] != 0;
         }
     }
 
@@ -397,6 +381,11 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         }
     }
     if constexpr (LORA != 0) __syncthreads();  // everyone has read its pair before the rotated values go in
+    if constexpr (!SPLIT) {
+        if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
+        p = (int)p64;
+        j_hi = p;
+    }
     if (tid < D) {
         const float sign = tid < D / 2 ? -1.0f : 1.0f;  // rotate_half: (-x2, x1)
         const float c = bf16_to_f32(a.cos[(long)p * D + tid]), s = bf16_to_f32(a.sin[(long)p * D + tid]);
@@ -428,6 +417,20 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         if (lane == 0) s_new = (mask[p] && split == 0) ? dot * a.scaling : -INFINITY;  // one workgroup of a pair counts it
     }
 
+    if constexpr (!SPLIT) {
+        // a slot at or past the position may hold anything (also what is not a number): it gets weight zero
+        // below, and zeros in place of its values keep 0 * value at zero
+#pragma unroll
+        for (int u = 0; u < ATT_UNROLL; ++u) {
+            const bool inside = u * 4 * ATT_WAVES + wave * 4 + sub < j_hi;
+            live[u] = live[u] && inside;
+#pragma unroll
+            for (int i = 0; i < VEC / 2; ++i) {
+                kraw[u].w[i] = inside ? kraw[u].w[i] : 0u;
+                vraw[u].w[i] = inside ? vraw[u].w[i] : 0u;
+            }
+        }
+    }
     Partial<VEC> st;
     st.m = -INFINITY;
     st.l = 0.0f;
