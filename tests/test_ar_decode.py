@@ -287,18 +287,19 @@ def int4_policy():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("native", [False, True, "split"])
-def test_graph_replays_equal_eager_steps(int4_policy, native, monkeypatch):
+@pytest.mark.parametrize("native", [False, True, "split", "crossing"])
+def test_graph_replays_equal_eager_steps(int4_policy, native):
     """Every replayed step against the same step run eagerly: tokens and log-probabilities bit for bit,
-    over two calls (the second reuses the recorded graph) with eager work and syncs in between."""
+    over two calls (the second reuses the recorded graph) with eager work and syncs in between.
+    "split": prompts of more than 512 slots, where the attention of few rows divides a pair's slots over several
+    workgroups; "crossing": the generation begins below 512 filled slots and ends above, so it is replayed from
+    two recordings (one-workgroup launches first, split launches from slot 512 on)."""
     print("ar decode: graph vs eager, native trunk", native, flush=True)
-    if native == "split":   # the attention's split form whatever the cache length
-        from visionrl_amd.decode_step import NativeDecodeTrunk
-        monkeypatch.setattr(NativeDecodeTrunk, "SPLIT_ATTENTION_FROM", 0)
-        native = True
+    longer = {"split": 523, "crossing": 492}.get(native, 0)
+    form, native = native, bool(native)
     eager = StaticARSampler(int4_policy, graph=False, native=native)
     graphed = StaticARSampler(int4_policy, graph=True, native=native)
-    for call, (n_text, n_img, seed) in enumerate(((7, 24, 21), (11, 20, 22), (7, 24, 21))):
+    for call, (n_text, n_img, seed) in enumerate(((7 + longer, 24, 21), (11 + longer, 20, 22), (7 + longer, 24, 21))):
         cond, uncond, cmask, umask = make_inputs(3, n_text, torch.bfloat16, "cuda:0", seed=seed)
         torch.manual_seed(seed)
         want_t, want_lp = eager.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=n_img)
@@ -311,6 +312,32 @@ def test_graph_replays_equal_eager_steps(int4_policy, native, monkeypatch):
         assert len(want_t.unique()) > n_img // 2
     (sess,) = graphed._sessions.values()
     assert sess.graph is not None and bool(sess.native) == native
+    assert (sess.graph_short is not None) == (form == "crossing")
+    if form in ("split", "crossing"):
+        assert sess.native.short_form(511) and not sess.native.short_form(512)
+
+
+@pytest.mark.gpu
+def test_short_cache_launch_list_equals_the_default_one(int4_policy, monkeypatch):
+    """While no row has 512 filled slots the split launches leave a pair to one workgroup, and the launch list
+    with one-workgroup launches in their place does the same arithmetic: same tokens, same log-probabilities
+    bit for bit, whichever list the steps run from."""
+    print("ar decode: short-cache launch list vs default list", flush=True)
+    from visionrl_amd.decode_step import NativeDecodeTrunk
+    cond, uncond, cmask, umask = make_inputs(3, 470, torch.bfloat16, "cuda:0", seed=77)
+    results = []
+    for use_short in (True, False):
+        if not use_short:
+            monkeypatch.setattr(NativeDecodeTrunk, "short_form", lambda self, cached: False)
+        sampler = StaticARSampler(int4_policy, graph=False, native=True)
+        torch.manual_seed(5)
+        results.append(sampler.sample_image_tokens(cond, uncond, cmask, umask, image_token_num=40))
+        torch.cuda.synchronize()
+        (sess,) = sampler._sessions.values()
+        assert sess.native and sess.native._table_short is not None and sess.max_len == 512
+    (t_short, lp_short), (t_long, lp_long) = results
+    assert torch.equal(t_short, t_long) and torch.equal(lp_short, lp_long)
+    assert len(t_short.unique()) > 20
 
 
 @pytest.mark.gpu
@@ -335,15 +362,12 @@ def test_fused_static_path_samples_what_the_reference_loop_samples(int4_policy, 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("side,split", [("left", False), ("right", False), ("left", True)])
-def test_native_trunk_tracks_the_module_trunk(int4_policy, side, split, monkeypatch):
+def test_native_trunk_tracks_the_module_trunk(int4_policy, side, split):
     """Teacher-forced: both trunks consume the same inputs step after step, each over its own cache;
     hidden states and appended cache rows stay within bf16 roundings of each other (also with the
     attention in its split form, which long caches of few rows take)."""
     print("ar decode: native trunk vs module trunk", flush=True)
-    if split:
-        from visionrl_amd.decode_step import NativeDecodeTrunk
-        monkeypatch.setattr(NativeDecodeTrunk, "SPLIT_ATTENTION_FROM", 0)
-    rows, n_text, steps = 6, 7, 12
+    rows, n_text, steps = 6, 517 if split else 7, 12   # the split form divides a pair from 512 filled slots on
     cond, uncond, cmask, umask = make_inputs(rows // 2, n_text, torch.bfloat16, "cuda:0", seed=41, side=side)
     sessions = []
     for native in (True, False):
@@ -862,10 +886,10 @@ def test_recording_keeps_the_garbage_collector_out_and_sessions_die_with_their_s
     seen = []
     step = ar_decode._Session.step
 
-    def watched(self):
+    def watched(self, *args):
         if torch.cuda.is_current_stream_capturing():
             seen.append(gc.isenabled())
-        return step(self)
+        return step(self, *args)
 
     monkeypatch.setattr(ar_decode._Session, "step", watched)
     cond, uncond, cmask, umask = make_inputs(2, 6, torch.bfloat16, "cuda:0", seed=81)

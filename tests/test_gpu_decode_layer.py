@@ -97,7 +97,10 @@ def test_rope_attn_decode_parity(ops_mod, M, H, Hkv, D, L, p):
 
 SPLIT_CASES = [
     # M, H, Hkv, D, L, p: 8 workgroups per pair up to 32 pairs, 4 up to 64, 2 up to 128; ranges of multiples of 64
-    # slots: empty ranges, one partly filled range, exact multiples, a long cache
+    # slots: empty ranges, one partly filled range, exact multiples, a long cache.  Below 512 cached slots the
+    # launch leaves a pair to its first workgroup (no exchange): both sides of that line, and on it
+    (2, 16, 16, 128, 896, 511), (2, 16, 16, 128, 896, 513), (2, 16, 16, 128, 896, 600), (4, 16, 16, 128, 640, 600),
+    (8, 16, 16, 128, 640, 639), (3, 4, 2, 64, 1024, 577),
     (2, 16, 16, 128, 896, 0), (2, 16, 16, 128, 896, 1), (2, 16, 16, 128, 896, 63), (2, 16, 16, 128, 896, 64),
     (2, 16, 16, 128, 896, 65), (2, 16, 16, 128, 896, 330), (2, 16, 16, 128, 896, 512), (2, 16, 16, 128, 896, 830),
     (2, 16, 16, 128, 896, 895), (4, 16, 16, 128, 384, 300), (8, 16, 16, 128, 384, 383), (1, 6, 3, 64, 48, 47),
@@ -142,7 +145,7 @@ def test_split_rope_attn_launches_share_one_workspace(ops_mod):
     checked afterwards: a launch must read what its own workgroups wrote, never what an earlier launch
     left in the workspace or in a cache; masked slots and an all-masked row included."""
     say("rope_attn split, repeated launches")
-    M, H, D, L = 2, 16, 128, 640
+    M, H, D, L = 2, 16, 128, 1280    # positions on both sides of the 512 slots from which a pair is divided
     ws = ops_mod.rope_attn_split_workspace(M, H, D, DEV)
     rng = np.random.default_rng(77)
     runs = []
@@ -208,9 +211,10 @@ def test_split_rope_attn_tracks_the_one_workgroup_form_over_many_launches(ops_mo
 def test_split_rope_attn_in_a_graph_equals_eager(ops_mod):
     """Recorded once, replayed with eager launches and synchronisations between the replays, the position
     advancing as in a decode loop: every replay equals the eager launch bit for bit (the merge runs in
-    index order whichever workgroup arrives last)."""
+    index order whichever workgroup arrives last).  The position crosses the 512 slots from which the launch
+    divides a pair: the one recorded launch serves both sides."""
     say("rope_attn split, graph replay")
-    M, H, D, L = 2, 16, 128, 512
+    M, H, D, L = 2, 16, 128, 896
     c = attn_case(4100, M, H, H, D, L, 200)
     t = {k: bits_to_bf16(c[k], DEV) for k in ("q", "k", "v", "kc", "vc", "cos", "sin")}
     mask = torch.from_numpy(c["mask"]).to(DEV)
@@ -228,7 +232,7 @@ def test_split_rope_attn_in_a_graph_equals_eager(ops_mod):
     gen = torch.Generator(device=DEV).manual_seed(9)
     kc_e, vc_e = kc_g.clone(), vc_g.clone()
     for step in range(6):
-        pos.fill_(201 + 37 * step)
+        pos.fill_(421 + 37 * step)     # 421 ... 606
         for name in ("q", "k", "v"):
             t[name].copy_((torch.randn(t[name].shape, generator=gen, device=DEV) * 0.7).to(torch.bfloat16))
         want = call(kc_e, vc_e, ws_eager, None)
@@ -336,7 +340,8 @@ def test_rope_attn_masks_and_strided_inputs(ops_mod):
 
 @pytest.mark.parametrize("M,H,Hkv,D,L,p", [(2, 16, 16, 128, 640, 0), (2, 16, 16, 128, 640, 1), (2, 16, 16, 128, 640, 37),
                                            (2, 16, 16, 128, 640, 127), (2, 16, 16, 128, 640, 128),
-                                           (2, 16, 16, 128, 640, 129), (3, 4, 2, 64, 40, 33), (2, 8, 2, 128, 24, 5)])
+                                           (2, 16, 16, 128, 640, 129), (2, 16, 16, 128, 640, 600),
+                                           (3, 4, 2, 64, 40, 33), (2, 8, 2, 128, 24, 5)])
 def test_rope_attn_ignores_what_the_slots_past_the_position_hold(ops_mod, M, H, Hkv, D, L, p):
     """Slots at and past the row's position have not been written by this sequence: whatever bits they hold
     (infinities and NaNs included, which a weight of zero would not silence) the result and the slots

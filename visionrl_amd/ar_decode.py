@@ -137,6 +137,9 @@ class _Session:
         self.slot = torch.zeros(1, dtype=torch.long, device=device)   # cache slot of the next new token
         self.native = None     # NativeDecodeTrunk once the cache exists, False if the trunk does not qualify
         self.graph = None
+        self.graph_short = None   # the step with the launch list for a cache that is still short, where there is one
+        self.eager_steps = [0, 0]  # eager decode steps so far with the default / the short list (a recording's warm-up)
+        self.prompt_len = 0        # slots the prompt pass filled
         self.owner = None      # weak reference to the state whose generation the buffers hold
         self.head_workspace = None   # of the fused head + tail launch
         self.signature = None  # of the trunk's modules and adapter state the launch list / graph were made for
@@ -181,7 +184,8 @@ class _Session:
     def begin(self, mask: torch.Tensor) -> None:
         signature = (trunk_signature(self.sampler.trunk), id(self._head_packed()), id(self._front_packed()))
         if signature != self.signature:   # modules swapped, adapters merged / disabled / switched: start over
-            self.signature, self.native, self.graph = signature, None, None
+            self.signature, self.native, self.graph, self.graph_short = signature, None, None, None
+            self.eager_steps = [0, 0]
             self.head_workspace = None    # sized for the head it was made for
             self.front_call = None
         self.cache.reset()
@@ -189,6 +193,7 @@ class _Session:
         self.mask[:, :mask.shape[1]].copy_(mask)
         self.mask_u8.copy_(self.mask != 0)
         self.slot.fill_(mask.shape[1])
+        self.prompt_len = int(mask.shape[1])
         self.img_pos.zero_()
 
     def _front(self, parts, hidden: torch.Tensor) -> torch.Tensor:
@@ -349,9 +354,14 @@ class _Session:
             nxt = s.base.prepare_gen_img_embeds(torch.cat([picked, picked], dim=0).unsqueeze(-1))
             self.cur[torch.cat([idx, idx + B])] = nxt.reshape(2 * len(rows), 1, -1)
 
-    def step(self) -> None:
+    def short_form(self, position: int) -> bool:
+        """Whether the decode step that samples image token ``position`` (>= 1) takes the native trunk's launch
+        list for a short cache: the slots filled by then are the prompt's and one per earlier step."""
+        return bool(self.native) and self.native.short_form(self.prompt_len + position - 1)
+
+    def step(self, short: bool = False) -> None:
         if self.native:
-            hidden = self.native.run()
+            hidden = self.native.run(short)
             hidden = hidden.view(self.rows2, 1, -1) if hidden is not None else None
         else:
             out = self.sampler.trunk(inputs_embeds=self.cur, attention_mask=self.mask, use_cache=True,
@@ -366,7 +376,7 @@ class _Session:
             raise RuntimeError("the sampler this session belongs to no longer exists")
         return sampler
 
-    def capture(self) -> None:
+    def capture(self, short: bool = False) -> None:
         graph = torch.cuda.CUDAGraph()
         # No cyclic garbage collection while the stream records: a finalizer that releases device resources (another
         # recorded graph, say) in the middle of a recording ends the process.  torch.cuda.graph collects once itself
@@ -375,11 +385,14 @@ class _Session:
         gc.disable()
         try:
             with torch.cuda.graph(graph):
-                self.step()
+                self.step(short)
         finally:
             if collecting:
                 gc.enable()
-        self.graph = graph
+        if short:
+            self.graph_short = graph
+        else:
+            self.graph = graph
 
 
 class StaticARSampler:
@@ -539,14 +552,20 @@ class StaticARSampler:
             sess.prefill(torch.cat([cond, uncond], dim=0))
             state.inputs = None
         elif self.graph and sess.cur.is_cuda:
-            if sess.graph is None and state.position >= 2:
-                sess.capture()           # after one eager decode step: records, does not run
-            if sess.graph is None:
-                sess.step()              # a real step, and the warm-up the capture needs
+            # two recordings where the native trunk has a launch list of its own for a short cache: the
+            # step is replayed from the one that fits the slots filled so far
+            short = sess.short_form(state.position)
+            graph = sess.graph_short if short else sess.graph
+            if graph is None and sess.eager_steps[short] >= 1:
+                sess.capture(short)      # after one eager decode step of that form: records, does not run
+                graph = sess.graph_short if short else sess.graph
+            if graph is None:
+                sess.step(short)         # a real step, and the warm-up the capture needs
+                sess.eager_steps[short] += 1
             else:
-                sess.graph.replay()
+                graph.replay()
         else:
-            sess.step()
+            sess.step(sess.short_form(state.position))
         state.position += 1
 
     def _advance_rows(self, state: "StaticARState", rows: list, position: int, sequences) -> "StaticARStepResult":

@@ -112,6 +112,10 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_kernel(const uint16_t *x,
 
 // ---------------------------------------------------------------- rotary + cache append + attention
 constexpr int ATTN_MAX_SPLITS = 8;   // workgroups that share the cached slots of one (row, head) in the split form
+// A row with fewer cached slots than this is left to the first workgroup of each of its pairs by a split launch
+// (the exchange of the split form costs more than it saves there: a decode step at 2 rows takes 0.82 against
+// 0.85 ms at 450 slots, 0.86 against 0.86 at 530, 0.91 against 0.86 at 610).
+constexpr int ATTN_SPLIT_FROM = 512;
 
 struct AttnArgs {
     const uint16_t *q, *k, *v;
@@ -230,10 +234,20 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
     bool live[ATT_UNROLL];
     // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
-    // multiple of 64 slots (what the workgroup's waves visit together)
+    // multiple of 64 slots (what the workgroup's waves visit together).  A split launch over a cache that is
+    // still short (fewer than ATTN_SPLIT_FROM slots filled: the launch is captured once for a whole
+    // generation, which begins short) leaves a pair to its first workgroup: `whole`.
     const int n_split = SPLIT ? (int)gridDim.z : 1, split = SPLIT ? (int)blockIdx.z : 0;
     const long long p64 = a.position[(long)m * a.position_stride];
     int p = 0, j_lo = 0, j_hi = 0;
+    bool whole = !SPLIT;
+    auto slot_range = [&]() {   // needs p64
+        p = (int)p64;
+        whole = !SPLIT || p < ATTN_SPLIT_FROM;
+        const int share = whole ? p : ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
+        j_lo = min(p, split * share);
+        j_hi = min(p, j_lo + share);
+    };
     auto request = [&](int j0) {  // slot j0 + u * 4 * ATT_WAVES + wave * 4 + sub for u = 0..ATT_UNROLL-1; needs j_hi > j_lo
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
@@ -245,19 +259,14 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         }
     };
     // The cached slots do not depend on the new token: the first batch of keys and values is
-    // requested before anything else and arrives while the query is rotated.
-    if constexpr (SPLIT) {
-        if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
-        p = (int)p64;
-        const int share = ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
-        j_lo = min(p, split * share);
-        j_hi = min(p, j_lo + share);
-        if (j_hi > j_lo) request(j_lo);
-    } else {
-        // Which slots the first batch visits does not depend on the row's position, only how many of them
-        // count, and neither do the new token's query, key and value: all are requested before the position
-        // is looked at (it comes from memory, and what waited for it would start a round trip later); the
-        // slots at or past it are dropped before the batch is used.
+    // requested before anything else and arrives while the query is rotated.  A pair's first (or only)
+    // workgroup begins at slot 0 wherever the row stands: which slots its first batch visits does not depend
+    // on the position, only how many of them count, and neither do the new token's query, key and value, so
+    // all are requested before the position is looked at (it comes from memory, and what waited for it
+    // would start a round trip later); the slots at or past the range's end are dropped before the batch
+    // is used.
+    const bool ahead = split == 0;   // uniform
+    if (ahead) {
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             const int j = u * 4 * ATT_WAVES + wave * 4 + sub;
@@ -266,6 +275,11 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
             live[u] = mask[jj] != 0;
         }
+    } else {
+        if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
+        slot_range();
+        if (whole) return;                      // the pair's first workgroup has it all
+        if (j_hi > j_lo) request(j_lo);
     }
 
     // The adapter of the projection that follows: thread (j, l16) holds the lane's VEC columns of row j
@@ -381,10 +395,9 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         }
     }
     if constexpr (LORA != 0) __syncthreads();  // everyone has read its pair before the rotated values go in
-    if constexpr (!SPLIT) {
+    if (ahead) {
         if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
-        p = (int)p64;
-        j_hi = p;
+        slot_range();
     }
     if (tid < D) {
         const float sign = tid < D / 2 ? -1.0f : 1.0f;  // rotate_half: (-x2, x1)
@@ -417,9 +430,9 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         if (lane == 0) s_new = (mask[p] && split == 0) ? dot * a.scaling : -INFINITY;  // one workgroup of a pair counts it
     }
 
-    if constexpr (!SPLIT) {
-        // a slot at or past the position may hold anything (also what is not a number): it gets weight zero
-        // below, and zeros in place of its values keep 0 * value at zero
+    if (ahead) {
+        // a slot at or past the range's end may hold anything (also what is not a number): it gets weight
+        // zero below, and zeros in place of its values keep 0 * value at zero
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             const bool inside = u * 4 * ATT_WAVES + wave * 4 + sub < j_hi;
@@ -504,9 +517,9 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
                 o += c * pacc[w][tid];
                 sum += c * pl[w];
             }
-            if constexpr (!SPLIT) o /= sum;
+            if (whole) o /= sum;
         }
-        if constexpr (SPLIT) {
+        if (!whole) {
             // this workgroup's state: o and sum relative to mx (zeros and -inf if it saw nothing attendable)
             float *mine = a.partials + (((long)m * a.n_heads + h) * n_split + split) * (D + 2);
             __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -531,7 +544,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             if constexpr (LORA != 0) qs[tid] = bf16_to_f32(bits);  // what the next projection reads
         }
     }
-    if constexpr (SPLIT) {
+    if (!whole) {
         uint32_t *count = a.arrived + (long)m * a.n_heads + h;
         __syncthreads();
         if (tid == 0) s_before = __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -222,13 +222,16 @@ class NativeDecodeTrunk:
         fuse_norm = hidden <= 4096 and (hidden <= 2048 or rows <= 16)
         # With few (row, head) pairs and a cache that grows long the attention divides a pair's cached slots
         # over several workgroups (one workspace for all layers: the launches are ordered by the stream).
-        # Its exchange costs about 1.5 us per launch, which pays from about 400 cached slots on (at 2 rows
-        # a step takes 0.87 / 0.89 / 0.90 ms at 330 / 590 / 830 slots against 0.84 / 0.94 / 1.02 ms).
+        # Its exchange costs about 1.5 us per launch, which pays from about 500 cached slots on (at 2 rows a
+        # step takes 0.85 / 0.86 / 0.86 / 0.88 ms at 450 / 530 / 610 / 830 slots against 0.82 / 0.86 / 0.91 /
+        # 0.96 ms); the launch is recorded once for a whole generation, and while a row has fewer than 512
+        # slots filled it leaves each of the row's pairs to one workgroup, as the other form does.
         split_ws = ops.rope_attn_split_workspace(rows, H, D, dev) \
             if rows * H <= self.SPLIT_ATTENTION_PAIRS and self.max_len >= self.SPLIT_ATTENTION_FROM else None
         self._keep.append(split_ws)
         self._split_ws = split_ws
         calls = []       # (function, argument tuple without the stream)
+        short_form = []  # (index, call): the one-workgroup attention launches that stand in while the cache is short
         state = {"x": cur.view(rows, hidden), "res": None, "flip": 0}   # x: sublayer output not yet added to res
 
         def norm_weight(module):
@@ -373,6 +376,7 @@ class NativeDecodeTrunk:
             elif split_ws is not None:
                 calls[attn_at] = (lib.vrl_rope_attn_decode_split_bf16,
                                   (*attn_args, split_ws.data_ptr(), split_ws.numel()))
+                short_form.append((attn_at, (lib.vrl_rope_attn_decode_bf16, attn_args)))
             else:
                 calls[attn_at] = (lib.vrl_rope_attn_decode_bf16, attn_args)
             (state["x"],) = outs
@@ -395,17 +399,36 @@ class NativeDecodeTrunk:
         self.launches = len(calls)
         # the same list as records of the library's own walk over it: one host call per step
         self._table = _lib.step_calls(calls)
+        # The split launches leave a row with fewer than SPLIT_ATTENTION_FROM cached slots to one workgroup per
+        # pair themselves, but the workgroups that then have nothing to do still cost about 1 us per launch
+        # (7.2 against 6.2 us at 150 slots, 9.0 against 7.8 at 330).  A caller that knows on the host how far
+        # the rows have come (the sampling loop does) asks for the list with the one-workgroup launches instead.
+        self._calls_short = self._table_short = None
+        if short_form:
+            self._calls_short = list(calls)
+            for at, call in short_form:
+                self._calls_short[at] = call
+            self._table_short = _lib.step_calls(self._calls_short)
         self._failed_at = ctypes.c_int(-1)
 
-    def run(self) -> torch.Tensor:
-        """Enqueue the step on the current stream; returns the ``[rows, hidden]`` output buffer."""
+    def short_form(self, cached_slots: int) -> bool:
+        """Whether :meth:`run` has a launch list of its own for a step that finds ``cached_slots`` filled slots
+        (the most any row holds): the split attention's one-workgroup stand-in below ``SPLIT_ATTENTION_FROM``."""
+        return self._table_short is not None and 0 <= cached_slots < self.SPLIT_ATTENTION_FROM
+
+    def run(self, short: bool = False) -> torch.Tensor:
+        """Enqueue the step on the current stream; returns the ``[rows, hidden]`` output buffer.  ``short``: the
+        list :meth:`short_form` speaks of (the caller vouches that no row has reached ``SPLIT_ATTENTION_FROM``
+        cached slots; the results are those of the default list either way, up to the order of fp32 sums)."""
         stream = torch.cuda.current_stream(self.device).cuda_stream
+        short = short and self._table_short is not None
+        table, calls = (self._table_short, self._calls_short) if short else (self._table, self._calls)
         with ops._on(self.device):
-            rc = _lib.load().vrl_decode_run_calls(self._table, len(self._table), ctypes.byref(self._failed_at), stream)
+            rc = _lib.load().vrl_decode_run_calls(table, len(table), ctypes.byref(self._failed_at), stream)
         if rc:
             # a step that stopped half-way may leave the split attention's arrival counters above zero,
             # and every later launch over that workspace would then merge too early: clear them
             if self._split_ws is not None and not torch.cuda.is_current_stream_capturing():
                 self._split_ws.zero_()
-            _lib.check(rc, self._calls[self._failed_at.value][0].__name__)
+            _lib.check(rc, calls[self._failed_at.value][0].__name__)
         return self.normed
