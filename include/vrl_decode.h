@@ -67,10 +67,10 @@ int vrl_rope_attn_decode_bf16(const void *q, const void *k, const void *v, int q
  * a long cache is read by many compute units instead of one per pair; each leaves its running softmax
  * state in `workspace`, and whichever finishes last merges them in index order and writes `out`
  * (deterministic; no workgroup waits for another).  Results equal the launch above up to the order of
- * the fp32 sums.  A row at a position below 512 is left to one workgroup per pair, with the launch above's
- * arithmetic (one recorded launch serves a generation from its first slot on); the workgroups that then
- * have nothing to do cost about 1 us per launch, so a caller that knows on the host that every row is below
- * 512 does better with the launch above.  `workspace`: vrl_rope_attn_decode_split_workspace_bytes(M, n_heads, D) bytes of device
+ * the fp32 sums.  A row at a position below 512 (768 where a pair has two workgroups) is left to one
+ * workgroup per pair, with the launch above's arithmetic (one recorded launch serves a generation from its
+ * first slot on); the workgroups that then have nothing to do cost about 1 us per launch, so a caller that
+ * knows on the host that every row is below that line does better with the launch above.  `workspace`: vrl_rope_attn_decode_split_workspace_bytes(M, n_heads, D) bytes of device
  * memory, 256-byte aligned, whose first M * n_heads * 4 bytes are zero before the first launch (every
  * launch leaves them zero again); launches that share a workspace must be ordered by the stream.
  * No counterpart in the reference (its attention is the library's, policy.py:673-678).

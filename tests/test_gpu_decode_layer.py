@@ -101,6 +101,8 @@ SPLIT_CASES = [
     # launch leaves a pair to its first workgroup (no exchange): both sides of that line, and on it
     (2, 16, 16, 128, 896, 511), (2, 16, 16, 128, 896, 513), (2, 16, 16, 128, 896, 600), (4, 16, 16, 128, 640, 600),
     (8, 16, 16, 128, 640, 639), (3, 4, 2, 64, 1024, 577),
+    # two workgroups per pair (65 to 128 pairs) divide a pair from 768 slots on
+    (8, 16, 16, 128, 1024, 767), (8, 16, 16, 128, 1024, 768), (8, 16, 16, 128, 1024, 1000),
     (2, 16, 16, 128, 896, 0), (2, 16, 16, 128, 896, 1), (2, 16, 16, 128, 896, 63), (2, 16, 16, 128, 896, 64),
     (2, 16, 16, 128, 896, 65), (2, 16, 16, 128, 896, 330), (2, 16, 16, 128, 896, 512), (2, 16, 16, 128, 896, 830),
     (2, 16, 16, 128, 896, 895), (4, 16, 16, 128, 384, 300), (8, 16, 16, 128, 384, 383), (1, 6, 3, 64, 48, 47),

@@ -116,6 +116,9 @@ constexpr int ATTN_MAX_SPLITS = 8;   // workgroups that share the cached slots o
 // (the exchange of the split form costs more than it saves there: a decode step at 2 rows takes 0.82 against
 // 0.85 ms at 450 slots, 0.86 against 0.86 at 530, 0.91 against 0.86 at 610).
 constexpr int ATTN_SPLIT_FROM = 512;
+// ... and with two workgroups per pair (65 to 128 pairs: half the compute units are busy without it) from 768:
+// a decode step at 8 rows takes 1.07 against 1.03 ms at 580 slots and 1.10 against 1.11 ms at 810.
+constexpr int ATTN_SPLIT_FROM_TWO = 768;
 
 struct AttnArgs {
     const uint16_t *q, *k, *v;
@@ -235,7 +238,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     bool live[ATT_UNROLL];
     // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
     // multiple of 64 slots (what the workgroup's waves visit together).  A split launch over a cache that is
-    // still short (fewer than ATTN_SPLIT_FROM slots filled: the launch is captured once for a whole
+    // still short (fewer than ATTN_SPLIT_FROM slots filled, ATTN_SPLIT_FROM_TWO with two workgroups per pair: the launch is captured once for a whole
     // generation, which begins short) leaves a pair to its first workgroup: `whole`.
     const int n_split = SPLIT ? (int)gridDim.z : 1, split = SPLIT ? (int)blockIdx.z : 0;
     const long long p64 = a.position[(long)m * a.position_stride];
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     bool whole = !SPLIT;
     auto slot_range = [&]() {   // needs p64
         p = (int)p64;
-        whole = !SPLIT || p < ATTN_SPLIT_FROM;
+        whole = !SPLIT || p < (n_split > 2 ? ATTN_SPLIT_FROM : ATTN_SPLIT_FROM_TWO);
         const int share = whole ? p : ((p + n_split - 1) / n_split + 4 * ATT_WAVES - 1) / (4 * ATT_WAVES) * (4 * ATT_WAVES);
         j_lo = min(p, split * share);
         j_hi = min(p, j_lo + share);

@@ -145,6 +145,7 @@ class NativeDecodeTrunk:
     ROW_BLOCK = 32               # rows one plan-free launch takes; more rows go as several launches per linear,
     MAX_ROWS = 64                # each reading the weights again (beyond this a dequantised GEMM is the better form)
     SPLIT_ATTENTION_FROM = 512   # cache slots from which the attention of few rows runs in its split form
+    SPLIT_ATTENTION_FROM_TWO = 768   # ... where the library gives a pair two workgroups (65 to 128 pairs)
     SPLIT_ATTENTION_PAIRS = 128  # (row, head) pairs up to which the library splits a pair's slots
 
     @staticmethod
@@ -226,8 +227,11 @@ class NativeDecodeTrunk:
         # step takes 0.85 / 0.86 / 0.86 / 0.88 ms at 450 / 530 / 610 / 830 slots against 0.82 / 0.86 / 0.91 /
         # 0.96 ms); the launch is recorded once for a whole generation, and while a row has fewer than 512
         # slots filled it leaves each of the row's pairs to one workgroup, as the other form does.
+        # (the library's own lines: 512 slots with 8 or 4 workgroups per pair, 768 with two, where half the
+        # compute units are busy without the split: 1.07 against 1.03 ms per step at 8 rows and 580 slots)
+        self._split_from = self.SPLIT_ATTENTION_FROM if rows * H <= 64 else self.SPLIT_ATTENTION_FROM_TWO
         split_ws = ops.rope_attn_split_workspace(rows, H, D, dev) \
-            if rows * H <= self.SPLIT_ATTENTION_PAIRS and self.max_len >= self.SPLIT_ATTENTION_FROM else None
+            if rows * H <= self.SPLIT_ATTENTION_PAIRS and self.max_len >= self._split_from else None
         self._keep.append(split_ws)
         self._split_ws = split_ws
         calls = []       # (function, argument tuple without the stream)
@@ -413,13 +417,14 @@ class NativeDecodeTrunk:
 
     def short_form(self, cached_slots: int) -> bool:
         """Whether :meth:`run` has a launch list of its own for a step that finds ``cached_slots`` filled slots
-        (the most any row holds): the split attention's one-workgroup stand-in below ``SPLIT_ATTENTION_FROM``."""
-        return self._table_short is not None and 0 <= cached_slots < self.SPLIT_ATTENTION_FROM
+        (the most any row holds): the split attention's one-workgroup stand-in below ``SPLIT_ATTENTION_FROM``
+        (``SPLIT_ATTENTION_FROM_TWO`` for 65 to 128 pairs)."""
+        return self._table_short is not None and 0 <= cached_slots < self._split_from
 
     def run(self, short: bool = False) -> torch.Tensor:
         """Enqueue the step on the current stream; returns the ``[rows, hidden]`` output buffer.  ``short``: the
-        list :meth:`short_form` speaks of (the caller vouches that no row has reached ``SPLIT_ATTENTION_FROM``
-        cached slots; the results are those of the default list either way, up to the order of fp32 sums)."""
+        list :meth:`short_form` speaks of (the caller vouches that no row has as many cached slots as the split
+        form begins at; the results are those of the default list either way, up to the order of fp32 sums)."""
         stream = torch.cuda.current_stream(self.device).cuda_stream
         short = short and self._table_short is not None
         table, calls = (self._table_short, self._calls_short) if short else (self._table, self._calls)
