@@ -235,7 +235,14 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
     const uint16_t *vc = a.v_cache + cache_base + l16 * VEC;
     constexpr int STEP = 4 * ATT_WAVES * ATT_UNROLL;  // slots the workgroup visits per batch
     RawVec<VEC> kraw[ATT_UNROLL], vraw[ATT_UNROLL];
+    // Whether a slot counts: its flag computed where the slot is requested (the compiler then waits there for the
+    // mask byte, and with it for every load issued before: one round trip per slot of a batch), or the mask bytes
+    // kept as loaded until the batch is used (MASK_LATE: one round trip per batch).  Per launch, from HIP graphs of
+    // 24: 16.9 -> 16.3 us for the 8-wave workgroups of 32 rows and 9.3 -> 8.9 us in the split form, but 7.0 ->
+    // 7.5 us for the 16-wave one-workgroup form at 2 rows and 8.5 -> 9.0 us at 8, which keeps the early flags.
+    constexpr bool MASK_LATE = SPLIT || ATT_WAVES < 16;
     bool live[ATT_UNROLL];
+    uint8_t mraw[ATT_UNROLL];
     // the workgroup's share of the cached slots 0..p-1: all of them, or the z-th of gridDim.z ranges of a
     // multiple of 64 slots (what the workgroup's waves visit together).  A split launch over a cache that is
     // still short (fewer than ATTN_SPLIT_FROM slots filled, ATTN_SPLIT_FROM_TWO with two workgroups per pair: the launch is captured once for a whole
@@ -258,7 +265,8 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             const int jj = j < j_hi ? j : j_hi - 1;  // slots past the end repeat the last one and are not counted
             kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
             vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
-            live[u] = j < j_hi && mask[jj] != 0;
+            if constexpr (MASK_LATE) mraw[u] = mask[jj];
+            else live[u] = j < j_hi && mask[jj] != 0;
         }
     };
     // The cached slots do not depend on the new token: the first batch of keys and values is
@@ -276,7 +284,8 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             const int jj = j < a.L_max ? j : a.L_max - 1;
             kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
             vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
-            live[u] = mask[jj] != 0;
+            if constexpr (MASK_LATE) mraw[u] = mask[jj];
+            else live[u] = mask[jj] != 0;
         }
     } else {
         if (p64 < 0 || p64 >= a.L_max) return;  // uniform over the workgroups of the row
@@ -439,7 +448,7 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
 #pragma unroll
         for (int u = 0; u < ATT_UNROLL; ++u) {
             const bool inside = u * 4 * ATT_WAVES + wave * 4 + sub < j_hi;
-            live[u] = live[u] && inside;
+            if constexpr (!MASK_LATE) live[u] = live[u] && inside;
 #pragma unroll
             for (int i = 0; i < VEC / 2; ++i) {
                 kraw[u].w[i] = inside ? kraw[u].w[i] : 0u;
@@ -467,7 +476,8 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
             for (int i = 0; i < VEC / 2; ++i)
                 dot = __builtin_amdgcn_fdot2_f32_bf16(qpair[i], __builtin_bit_cast(bf16x2_t, kraw[u].w[i]), dot, false);
             dot = row16_sum(dot);  // the sixteen lanes that share the slot
-            sc[u] = live[u] ? dot * a.scaling : -INFINITY;
+            const bool counts = MASK_LATE ? (j0 + u * 4 * ATT_WAVES + wave * 4 + sub < j_hi) & (mraw[u] != 0) : live[u];
+            sc[u] = counts ? dot * a.scaling : -INFINITY;
             mx = fmaxf(mx, sc[u]);
         }
         const float ref = mx == -INFINITY ? 0.0f : mx;  // nothing attendable yet: keep zeros, avoid inf - inf
