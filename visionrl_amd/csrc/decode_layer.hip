@@ -263,10 +263,18 @@ __global__ __launch_bounds__(ATT_WAVES *WAVE) void rope_attn_decode_kernel(AttnA
         for (int u = 0; u < ATT_UNROLL; ++u) {
             const int j = j0 + u * 4 * ATT_WAVES + wave * 4 + sub;
             const int jj = j < j_hi ? j : j_hi - 1;  // slots past the end repeat the last one and are not counted
-            kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
-            vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
-            if constexpr (MASK_LATE) mraw[u] = mask[jj];
-            else live[u] = j < j_hi && mask[jj] != 0;
+            // SPLIT: a range is often shorter than a batch, and a whole group of slots past its end (uniform) asks
+            // for nothing (8.9 -> 8.6 us per launch at 600 slots; the other builds measure slower with the branch)
+            if (!SPLIT || j0 + u * 4 * ATT_WAVES < j_hi) {
+                kraw[u] = load_raw<VEC, STREAMED>(kc + (long)jj * D);
+                vraw[u] = load_raw<VEC, STREAMED>(vc + (long)jj * D);
+                if constexpr (MASK_LATE) mraw[u] = mask[jj];
+                else live[u] = j < j_hi && mask[jj] != 0;
+            } else {
+#pragma unroll
+                for (int i = 0; i < VEC / 2; ++i) kraw[u].w[i] = vraw[u].w[i] = 0u;
+                mraw[u] = 0;
+            }
         }
     };
     // The cached slots do not depend on the new token: the first batch of keys and values is
